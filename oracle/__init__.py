@@ -1,0 +1,229 @@
+"""ctypes view of the CPU oracle (oracle/qlinear_oracle.c).  TEST INFRASTRUCTURE ONLY.
+
+Only tests/, the smoke check and the bench's CPU-baseline leg may import this module; the product path never does.
+Arrays are numpy; bf16 and f16 tensors travel as uint16 bit patterns.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libqlinear_oracle.so")
+F32, F16, BF16 = 0, 1, 2
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            from . import build as _b
+            _b.build()
+        L = C.CDLL(_LIB_PATH)
+        vp, i64, i32, f32 = C.c_void_p, C.c_int64, C.c_int, C.c_float
+        L.orc_f32_to_bf16.restype = C.c_uint16; L.orc_f32_to_bf16.argtypes = [f32]
+        L.orc_f32_to_f16.restype = C.c_uint16; L.orc_f32_to_f16.argtypes = [f32]
+        L.orc_bf16_to_f32.restype = f32; L.orc_bf16_to_f32.argtypes = [C.c_uint16]
+        L.orc_f16_to_f32.restype = f32; L.orc_f16_to_f32.argtypes = [C.c_uint16]
+        L.orc_e4m3_to_f32.restype = f32; L.orc_e4m3_to_f32.argtypes = [C.c_uint8]
+        L.orc_fht.restype = i32; L.orc_fht.argtypes = [vp, i32, i32]
+        L.orc_quant_rows.restype = i32; L.orc_quant_rows.argtypes = [i32, vp, i64, vp, vp, i32, i32, i32]
+        L.orc_rotate_rows_f32.restype = i32; L.orc_rotate_rows_f32.argtypes = [vp, i64, vp, i32, i32]
+        L.orc_sd_quant_rows.restype = i32; L.orc_sd_quant_rows.argtypes = [vp, i64, vp, vp, i32, i32, i32]
+        L.orc_int8_gemm_acc.restype = None; L.orc_int8_gemm_acc.argtypes = [vp, vp, vp, i64, i64, i64]
+        L.orc_epilogue.restype = None; L.orc_epilogue.argtypes = [vp, vp, vp, vp, vp, i64, i64, i32, i32]
+        L.orc_epilogue_residual.restype = None
+        L.orc_epilogue_residual.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i32, i32]
+        L.orc_int8_gemm.restype = i32; L.orc_int8_gemm.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, i32, i32]
+        L.orc_int8_gemm_residual.restype = i32
+        L.orc_int8_gemm_residual.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i32, i32]
+        L.orc_w6_decode.restype = i32; L.orc_w6_decode.argtypes = [vp, vp, vp, i64, i32, i32]
+        L.orc_w6_pack_planes.restype = None; L.orc_w6_pack_planes.argtypes = [vp, vp, i64, i32]
+        L.orc_w6_pack_words.restype = None; L.orc_w6_pack_words.argtypes = [vp, vp, i64, i32]
+        L.orc_w6_unpack_words.restype = None; L.orc_w6_unpack_words.argtypes = [vp, vp, i64, i32]
+        L.orc_w6a8_group_gemm.restype = i32
+        L.orc_w6a8_group_gemm.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i32]
+        L.orc_linear_w8a8.restype = i32
+        L.orc_linear_w8a8.argtypes = [i32, vp, i64, i32, vp, vp, vp, vp, i32, i32, i32, i32, i32, vp]
+        L.orc_set_threads.restype = None; L.orc_set_threads.argtypes = [i32]
+        _lib = L
+    return _lib
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def _c(a, dt=None):
+    a = np.ascontiguousarray(a)
+    if dt is not None:
+        assert a.dtype == dt, (a.dtype, dt)
+    return a
+
+
+_OUT_NP = {F32: np.float32, F16: np.uint16, BF16: np.uint16}
+_IN_NP = {F32: np.float32, F16: np.uint16, BF16: np.uint16}
+
+
+def bf16_bits(x):
+    """float32 array -> bf16 bit patterns (RNE), elementwise through the oracle's scalar routine semantics."""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    nan = (u & 0x7fffffff) > 0x7f800000
+    r = ((u + (0x7fff + ((u >> 16) & 1))) >> 16).astype(np.uint16)
+    r[nan] = ((u[nan] >> 16) | 0x40).astype(np.uint16)
+    return r
+
+
+def bf16_to_f32(b):
+    return (np.ascontiguousarray(b, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def f16_bits(x):
+    return np.ascontiguousarray(x, dtype=np.float32).astype(np.float16).view(np.uint16)
+
+
+def f16_to_f32(b):
+    return np.ascontiguousarray(b, dtype=np.uint16).view(np.float16).astype(np.float32)
+
+
+def to_f32(a, dt):
+    return a.astype(np.float32) if dt == F32 else bf16_to_f32(a) if dt == BF16 else f16_to_f32(a)
+
+
+def fht(row, g):
+    r = np.array(row, dtype=np.float32, copy=True).reshape(-1)
+    rc = lib().orc_fht(_p(r), r.size, g)
+    assert rc == 0, rc
+    return r.reshape(np.shape(row))
+
+
+def quant_rows(dtype, x, K, rotate, x_stride=None):
+    """x: [M, x_stride] array (uint16 bits for bf16, float32 for f32). Returns (rc, q int8 [M,K], scales f32 [M])."""
+    x = _c(x, _IN_NP[dtype])
+    M = x.shape[0]
+    x_stride = x.shape[1] if x_stride is None else x_stride
+    q = np.zeros((M, K), np.int8)
+    s = np.zeros((M,), np.float32)
+    rc = lib().orc_quant_rows(dtype, _p(x), x_stride, _p(q), _p(s), M, K, rotate)
+    return rc, q, s
+
+
+def rotate_rows_f32(x, K, x_stride=None):
+    x = _c(x, np.float32)
+    M = x.shape[0]
+    x_stride = x.shape[1] if x_stride is None else x_stride
+    out = np.zeros((M, K), np.float32)
+    rc = lib().orc_rotate_rows_f32(_p(x), x_stride, _p(out), M, K)
+    return rc, out
+
+
+def sd_quant_rows(x, K, rotate, x_stride=None):
+    x = _c(x, np.uint16)
+    M = x.shape[0]
+    x_stride = x.shape[1] if x_stride is None else x_stride
+    q = np.zeros((M, K), np.int8)
+    s = np.zeros((M,), np.float32)
+    rc = lib().orc_sd_quant_rows(_p(x), x_stride, _p(q), _p(s), M, K, rotate)
+    return rc, q, s
+
+
+def int8_gemm_acc(A, W):
+    A = _c(A, np.int8); W = _c(W, np.int8)
+    M, K = A.shape
+    N = W.shape[0]
+    acc = np.zeros((M, N), np.int32)
+    lib().orc_int8_gemm_acc(_p(A), _p(W), _p(acc), M, N, K)
+    return acc
+
+
+def epilogue(acc, xs, ws, bias, out_dt, fma):
+    acc = _c(acc, np.int32); xs = _c(xs, np.float32); ws = _c(ws, np.float32)
+    bias = None if bias is None else _c(bias, _OUT_NP[out_dt])
+    M, N = acc.shape
+    D = np.zeros((M, N), _OUT_NP[out_dt])
+    lib().orc_epilogue(_p(acc), _p(xs), _p(ws), _p(bias), _p(D), M, N, out_dt, int(fma))
+    return D
+
+
+def epilogue_residual(acc, xs, ws, bias, rscale, resid, out_dt, fma):
+    acc = _c(acc, np.int32); xs = _c(xs, np.float32); ws = _c(ws, np.float32)
+    bias = None if bias is None else _c(bias, _OUT_NP[out_dt])
+    rscale = _c(rscale, _OUT_NP[out_dt]); resid = _c(resid, _OUT_NP[out_dt])
+    M, N = acc.shape
+    D = np.zeros((M, N), _OUT_NP[out_dt])
+    lib().orc_epilogue_residual(_p(acc), _p(xs), _p(ws), _p(bias), _p(rscale), _p(resid), _p(D), M, N, out_dt,
+                                int(fma))
+    return D
+
+
+def int8_gemm(A, W, xs, ws, bias, out_dt, fma=1):
+    acc = int8_gemm_acc(A, W)
+    return epilogue(acc, xs, ws, bias, out_dt, fma)
+
+
+def int8_gemm_residual(A, W, xs, ws, bias, rscale, resid, out_dt, fma=1):
+    acc = int8_gemm_acc(A, W)
+    return epilogue_residual(acc, xs, ws, bias, rscale, resid, out_dt, fma)
+
+
+def e4m3_table():
+    L = lib()
+    return np.array([L.orc_e4m3_to_f32(i) for i in range(256)], np.float32)
+
+
+def w6_decode(q, s_rel, N, K, G):
+    q = _c(q, np.uint8); s_rel = _c(s_rel, np.uint8)
+    out = np.zeros((N, K), np.int8)
+    rc = lib().orc_w6_decode(_p(q), _p(s_rel), _p(out), N, K, G)
+    return rc, out
+
+
+def w6_pack_planes(codes):
+    codes = _c(codes, np.uint8)
+    N, K = codes.shape
+    q = np.zeros((N, K * 3 // 4), np.uint8)
+    lib().orc_w6_pack_planes(_p(codes), _p(q), N, K)
+    return q
+
+
+def w6_pack_words(qv):
+    qv = _c(qv, np.int8)
+    N, K = qv.shape
+    p = np.zeros((N, K * 3 // 4), np.uint8)
+    lib().orc_w6_pack_words(_p(qv), _p(p), N, K)
+    return p
+
+
+def w6_unpack_words(p, K):
+    p = _c(p, np.uint8)
+    N = p.shape[0]
+    qv = np.zeros((N, K), np.int8)
+    lib().orc_w6_unpack_words(_p(p), _p(qv), N, K)
+    return qv
+
+
+def w6a8_group_gemm(A, packed, xs, sw, bias, out_dt, want_partials=False):
+    A = _c(A, np.int8); packed = _c(packed, np.uint8); xs = _c(xs, np.float32); sw = _c(sw, np.float32)
+    bias = None if bias is None else _c(bias, _OUT_NP[out_dt])
+    M, K = A.shape
+    N = packed.shape[0]
+    D = np.zeros((M, N), _OUT_NP[out_dt])
+    part = np.zeros((M, N, K // 128), np.int32) if want_partials else None
+    rc = lib().orc_w6a8_group_gemm(_p(A), _p(packed), _p(xs), _p(sw), _p(bias), _p(D), _p(part), M, N, K, out_dt)
+    return rc, D, part
+
+
+def linear_w8a8(dtype, x, rotate, W, ws, bias, out_dt, fma=1, threads=None):
+    """Whole linear on the CPU; returns (rc, D, threads_used)."""
+    x = _c(x, _IN_NP[dtype]); W = _c(W, np.int8); ws = _c(ws, np.float32)
+    bias = None if bias is None else _c(bias, _OUT_NP[out_dt])
+    M, K = x.shape
+    N = W.shape[0]
+    if threads is not None:
+        lib().orc_set_threads(threads)
+    D = np.zeros((M, N), _OUT_NP[out_dt])
+    t = C.c_int(0)
+    rc = lib().orc_linear_w8a8(dtype, _p(x), K, rotate, _p(W), _p(ws), _p(bias), _p(D), M, N, K, out_dt, int(fma),
+                               C.byref(t))
+    return rc, D, t.value

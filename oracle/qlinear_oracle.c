@@ -1,0 +1,426 @@
+/*
+ * CPU oracle for the quantized-linear hot path.  TEST INFRASTRUCTURE ONLY.
+ *
+ * This file is a plain-C restatement of the arithmetic of the reference's W8A8 / W6A8 linear, written from its
+ * source text.  It exists so that the HIP kernels can be checked bit-for-bit on the same inputs.  Nothing in the
+ * product (the HIP library, its host wrappers) may call, link or import it: only the tests, the smoke check and
+ * the bench's CPU-baseline leg do, and only as the checker / the reported CPU number.
+ *
+ * Every function cites the reference lines it follows (paths relative to the reference checkout).
+ * Build with -ffp-contract=off: an FMA appears only where `fmaf` is written.
+ *
+ * Parity status of each function (what pins it, see tests/test_oracle_*.py):
+ *   orc_bf16_round / orc_f16_round     pinned: exhaustive/sampled against torch.bfloat16 / numpy.float16 casts
+ *   orc_fht                            g=64,256 pinned: dense Kronecker matrix, H=H^T, H.H=I, exact on small integers;
+ *                                      g=128 is this build's own definition (the reference has no 128 transform)
+ *   orc_quant_rows / orc_sd_quant_rows pinned: torch bf16/f16 tensor arithmetic (divide, round, clamp), closed-form
+ *                                      special rows (zero row, single outlier, +-127.5 ties, inf, NaN)
+ *   orc_int8_gemm_acc                  pinned: numpy int64 matmul, torch._int_mm
+ *   orc_epilogue[_residual]            pinned for the non-fused form: numpy float32 ops; the fused form against exact
+ *                                      rational arithmetic.  Which of the two the reference's CUTLASS/nvcc build
+ *                                      produces is PARITY UNPINNED (only a run of the reference could tell); both
+ *                                      are provided and differ by at most one ulp of the output type.
+ *   orc_e4m3_to_f32 / orc_w6_decode    pinned: exhaustive 256 bytes against torch.float8_e4m3fn; exhaustive
+ *                                      64 codes x 256 scales against the definition; pack/unpack round trip
+ *   orc_w6a8_group_gemm                this build's own format (no reference counterpart); integer partials pinned by
+ *                                      numpy int64
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define ORC_API __attribute__((visibility("default")))
+
+enum { ORC_F32 = 0, ORC_F16 = 1, ORC_BF16 = 2 }; /* csrc/common.cuh:15 */
+
+static inline uint32_t f2u(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+static inline float u2f(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+
+/* ---------------------------------------------------------------------------------------------
+ * Rounding helpers: rnd<T> of csrc/common.cuh:25-28 (round to T with RNE, widen back to float).
+ * ------------------------------------------------------------------------------------------- */
+ORC_API uint16_t orc_f32_to_bf16(float v) {
+    uint32_t u = f2u(v);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u); /* quiet NaN */
+    /* integer form used by tests/sparse_attn_match_comfy.rs:20-23 */
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+ORC_API float orc_bf16_to_f32(uint16_t h) { return u2f((uint32_t)h << 16); }
+ORC_API float orc_bf16_round(float v) { return orc_bf16_to_f32(orc_f32_to_bf16(v)); }
+
+ORC_API uint16_t orc_f32_to_f16(float v) {
+    const uint32_t u = f2u(v);
+    const uint16_t sign = (uint16_t)((u >> 16) & 0x8000u);
+    const uint32_t a = u & 0x7fffffffu;
+    if (a > 0x7f800000u) return (uint16_t)(sign | 0x7e00u);          /* NaN */
+    if (a >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u);         /* >= 65520 rounds to inf */
+    if (a < 0x33000001u) return sign;                                 /* <= 2^-25 rounds to 0 (tie to even) */
+    int e = (int)(a >> 23) - 127;
+    uint32_t man = (a & 0x7fffffu) | 0x800000u;                       /* 24-bit significand */
+    int shift;                                                        /* bits dropped from `man` */
+    uint32_t base;
+    if (e < -14) { shift = 13 + (-14 - e); base = 0; }                /* half subnormal */
+    else { shift = 13; base = (uint32_t)(e + 15) << 10; man &= 0x7fffffu; }
+    uint32_t keep = man >> shift;
+    const uint32_t rem = man & ((1u << shift) - 1u), half = 1u << (shift - 1);
+    if (rem > half || (rem == half && (keep & 1u))) ++keep;           /* RNE; a carry ripples into the exponent */
+    return (uint16_t)(sign | (base + keep));
+}
+ORC_API float orc_f16_to_f32(uint16_t h) {
+    const uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    const int e = (h >> 10) & 0x1f;
+    const uint32_t m = h & 0x3ffu;
+    if (e == 31) return u2f(sign | 0x7f800000u | (m << 13));
+    if (e == 0) {
+        const float f = ldexpf((float)m, -24);
+        return (h & 0x8000u) ? -f : f;
+    }
+    return u2f(sign | ((uint32_t)(e + 112) << 23) | (m << 13));
+}
+ORC_API float orc_f16_round(float v) { return orc_f16_to_f32(orc_f32_to_f16(v)); }
+
+static inline float rnd_t(int dt, float v) {
+    return dt == ORC_BF16 ? orc_bf16_round(v) : dt == ORC_F16 ? orc_f16_round(v) : v;
+}
+static inline float ld_t(int dt, const void* p, int64_t i) {
+    return dt == ORC_BF16 ? orc_bf16_to_f32(((const uint16_t*)p)[i])
+         : dt == ORC_F16  ? orc_f16_to_f32(((const uint16_t*)p)[i])
+                          : ((const float*)p)[i];
+}
+static inline void st_t(int dt, void* p, int64_t i, float v) {
+    if (dt == ORC_BF16) ((uint16_t*)p)[i] = orc_f32_to_bf16(v);
+    else if (dt == ORC_F16) ((uint16_t*)p)[i] = orc_f32_to_f16(v);
+    else ((float*)p)[i] = v;
+}
+/* fmaxf/fminf as the device code uses them: a NaN operand is dropped (csrc/kernels.cu:224,255). */
+static inline float fmax_dev(float a, float b) { return isnan(a) ? b : isnan(b) ? a : (a > b ? a : b); }
+static inline float fmin_dev(float a, float b) { return isnan(a) ? b : isnan(b) ? a : (a < b ? a : b); }
+
+/* ---------------------------------------------------------------------------------------------
+ * ConvRot group transform.  h4_row: csrc/common.cuh:99-106 (left-to-right adds).  Staged order:
+ * fht256_rows_smem csrc/common.cuh:110-126 (4 radix-4 stages, strides 1,4,16,64, each scaled by 0.5) and
+ * fht64_rows_smem csrc/sd.cu:560-576 (3 stages).  g = 128 has no reference form: it is defined here as the three
+ * radix-4 stages of each 64-block followed by one radix-2 stage at stride 64 scaled by 1/sqrt(2).
+ * ------------------------------------------------------------------------------------------- */
+static inline float h4_row(int d, float x0, float x1, float x2, float x3) {
+    switch (d) {
+        case 0: return x0 + x1 + x2 - x3;
+        case 1: return x0 + x1 - x2 + x3;
+        case 2: return x0 - x1 + x2 + x3;
+        default: return -x0 + x1 + x2 + x3;
+    }
+}
+ORC_API int orc_fht(float* row, int K, int g) {
+    if (g != 64 && g != 128 && g != 256) return -1;
+    if (K % g) return -1;
+    const int blk = g == 256 ? 256 : 64;          /* width the radix-4 stages span */
+    const int nstage = g == 256 ? 4 : 3;
+    for (int stage = 0; stage < nstage; ++stage) {
+        const int s = 1 << (2 * stage);
+        for (int b = 0; b < K / 4; ++b) {
+            const int grp = b / (blk / 4), r = b % (blk / 4);
+            const int i0 = grp * blk + (r / s) * (4 * s) + (r % s);
+            const float x0 = row[i0], x1 = row[i0 + s], x2 = row[i0 + 2 * s], x3 = row[i0 + 3 * s];
+            row[i0] = 0.5f * h4_row(0, x0, x1, x2, x3);
+            row[i0 + s] = 0.5f * h4_row(1, x0, x1, x2, x3);
+            row[i0 + 2 * s] = 0.5f * h4_row(2, x0, x1, x2, x3);
+            row[i0 + 3 * s] = 0.5f * h4_row(3, x0, x1, x2, x3);
+        }
+    }
+    if (g == 128) {
+        const float c = 0.70710678118654752f;
+        for (int base = 0; base < K; base += 128)
+            for (int i = 0; i < 64; ++i) {
+                const float a = row[base + i], b = row[base + 64 + i];
+                row[base + i] = (a + b) * c;
+                row[base + 64 + i] = (a - b) * c;
+            }
+    }
+    return 0;
+}
+
+/* `rotate` argument of the drop-in boundary: 0 none; 1 or 256 -> 256 (the reference's flag, csrc/kernels.cu:193);
+ * 64 and 128 are this build's extension. */
+static int rotate_group(int rotate) {
+    if (rotate == 0) return 0;
+    if (rotate == 64 || rotate == 128) return rotate;
+    return 256;
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * gpu_quant_rows, PRO_PLAIN: csrc/kernels.cu:271-298 (argument checks), :184-258 (rotation, amax, scale, codes).
+ * x is T[M, x_stride], T = bf16 or f32.  The K % 256 check of the reference is relaxed to K % 64 when no 256-wide
+ * rotation is asked for (the reference returns -1 there; every reference-valid call behaves identically).
+ * ------------------------------------------------------------------------------------------- */
+static int quant_check(int dtype, int K, int rotate) {
+    const int g = rotate_group(rotate);
+    const int need = (g == 256 || g == 0) ? (g == 0 ? 64 : 256) : g;
+    if (K <= 0 || (K % need) != 0) return -1;
+    if (dtype != ORC_BF16 && dtype != ORC_F32) return -4;
+    if (K > 32768) return -2; /* more than 32 warps of 4 groups, csrc/kernels.cu:263-265 */
+    return 0;
+}
+ORC_API int orc_quant_rows(int dtype, const void* x, int64_t x_stride, int8_t* q, float* scales, int M, int K,
+                           int rotate) {
+    const int rc = quant_check(dtype, K, rotate);
+    if (rc) return rc;
+    const int g = rotate_group(rotate);
+    const float tmax = dtype == ORC_BF16 ? 3.38953139e38f : 3.402823466e+38f; /* csrc/kernels.cu:48-50 */
+#pragma omp parallel
+    {
+        float* v = (float*)malloc(sizeof(float) * (size_t)K);
+#pragma omp for schedule(static)
+        for (int m = 0; m < M; ++m) {
+            for (int k = 0; k < K; ++k) v[k] = ld_t(dtype, x, (int64_t)m * x_stride + k);
+            if (g) orc_fht(v, K, g);
+            float amax = 0.f;
+            for (int k = 0; k < K; ++k) amax = fmax_dev(amax, fabsf(v[k]));
+            const float scale = fmax_dev(fmin_dev(amax, tmax) * (1.f / 127.f), 1.0e-30f); /* :241 */
+            scales[m] = scale;
+            const float st = rnd_t(dtype, scale);                                           /* :243 */
+            for (int k = 0; k < K; ++k) {
+                const float t = rnd_t(dtype, rnd_t(dtype, v[k]) / st);                      /* :254 */
+                q[(int64_t)m * K + k] = (int8_t)fmin_dev(127.f, fmax_dev(-128.f, nearbyintf(t)));
+            }
+        }
+        free(v);
+    }
+    return 0;
+}
+
+/* gpu_rotate_rows_f32, PRO_PLAIN: csrc/kernels.cu:316-327 with :227-238 (rotation always on, f32 in, f32 out). */
+ORC_API int orc_rotate_rows_f32(const float* x, int64_t x_stride, float* out, int M, int K) {
+    if (K <= 0 || (K % 256) != 0) return -1;
+    if (K > 32768) return -2;
+    for (int m = 0; m < M; ++m) {
+        float* o = out + (int64_t)m * K;
+        for (int k = 0; k < K; ++k) o[k] = x[(int64_t)m * x_stride + k];
+        orc_fht(o, K, 256);
+    }
+    return 0;
+}
+
+/* gpu_sd_quant_rows: csrc/sd.cu:578-606 (fp16 rows; rotate in {0,64,256}). */
+ORC_API int orc_sd_quant_rows(const uint16_t* x, int64_t x_stride, int8_t* q, float* scales, int M, int K,
+                              int rotate) {
+    if ((rotate != 0 && rotate != 64 && rotate != 256) || (rotate && K % rotate)) return -1; /* :600 */
+#pragma omp parallel
+    {
+        float* row = (float*)malloc(sizeof(float) * (size_t)(K > 0 ? K : 1));
+#pragma omp for schedule(static)
+        for (int m = 0; m < M; ++m) {
+            for (int k = 0; k < K; ++k) row[k] = orc_f16_to_f32(x[(int64_t)m * x_stride + k]);
+            if (rotate) orc_fht(row, K, rotate);
+            float mx = 0.f;
+            for (int k = 0; k < K; ++k) mx = fmax_dev(mx, fabsf(orc_f16_round(row[k])));     /* :587 */
+            const float scale = fmax_dev(mx, 1e-30f) / 127.f;                                /* :589 */
+            scales[m] = scale;
+            const float sh = orc_f16_round(scale);
+            const float st = sh > 0.f ? sh : scale;                                          /* :593 */
+            for (int k = 0; k < K; ++k) {
+                const float t = orc_f16_round(orc_f16_round(row[k]) / st);
+                q[(int64_t)m * K + k] = (int8_t)fmin_dev(127.f, fmax_dev(-128.f, nearbyintf(t)));
+            }
+        }
+        free(row);
+    }
+    return 0;
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * int8 x int8 -> int32 GEMM, A[M,K] . W[N,K]^T: csrc/vendor/cutlass_gemm_int8.cu:70-75,105 (exact for K <= 13824).
+ * ------------------------------------------------------------------------------------------- */
+ORC_API void orc_int8_gemm_acc(const int8_t* A, const int8_t* W, int32_t* acc, int64_t M, int64_t N, int64_t K) {
+#pragma omp parallel for schedule(static)
+    for (int64_t m = 0; m < M; ++m)
+        for (int64_t n = 0; n < N; ++n) {
+            const int8_t* a = A + m * K;
+            const int8_t* w = W + n * K;
+            int32_t s = 0;
+            for (int64_t k = 0; k < K; ++k) s += (int32_t)a[k] * (int32_t)w[k];
+            acc[m * N + n] = s;
+        }
+}
+
+/* Dequant epilogue: csrc/vendor/cutlass_gemm_int8.cu:84-95.  t0 = float(acc)*xs[m]; t1 = t0*ws[n];
+ * t2 = t1 + float(bias[n]) (bias read in the output type, null = 0); D = Out(t2).  `fma` selects the contracted form
+ * fmaf(t0, ws, bias) that nvcc may emit for the last two nodes. */
+static inline float epi_plain(int32_t acc, float xs, float ws, float b, int fma) {
+    const float t0 = (float)acc * xs;
+    return fma ? fmaf(t0, ws, b) : (t0 * ws) + b;
+}
+ORC_API void orc_epilogue(const int32_t* acc, const float* xs, const float* ws, const void* bias, void* D, int64_t M,
+                          int64_t N, int out_dt, int fma) {
+#pragma omp parallel for schedule(static)
+    for (int64_t m = 0; m < M; ++m)
+        for (int64_t n = 0; n < N; ++n) {
+            const float b = bias ? ld_t(out_dt, bias, n) : 0.f;
+            st_t(out_dt, D, m * N + n, epi_plain(acc[m * N + n], xs[m], ws[n], b, fma));
+        }
+}
+/* Residual epilogue: csrc/vendor/cutlass_gemm_int8.cu:149-161.  z = Out(plain epilogue);
+ * D = Out(float(z)*float(rscale[n]) + float(resid[m,n])).  D may alias resid (csrc/gemm.cu:131). */
+ORC_API void orc_epilogue_residual(const int32_t* acc, const float* xs, const float* ws, const void* bias,
+                                   const void* rscale, const void* resid, void* D, int64_t M, int64_t N, int out_dt,
+                                   int fma) {
+#pragma omp parallel for schedule(static)
+    for (int64_t m = 0; m < M; ++m)
+        for (int64_t n = 0; n < N; ++n) {
+            const float b = bias ? ld_t(out_dt, bias, n) : 0.f;
+            const float z = rnd_t(out_dt, epi_plain(acc[m * N + n], xs[m], ws[n], b, fma));
+            const float rs = ld_t(out_dt, rscale, n), r = ld_t(out_dt, resid, m * N + n);
+            st_t(out_dt, D, m * N + n, fma ? fmaf(z, rs, r) : (z * rs) + r);
+        }
+}
+
+/* gpu_int8_gemm: csrc/gemm.cu:124-129 -> launch_cutlass_int8_dequant csrc/vendor/cutlass_gemm_int8.cu:373-388.
+ * Returns 0, or -200 for an unknown output type.  M, N or K == 0 returns 0 and writes nothing (:377). */
+ORC_API int orc_int8_gemm(const int8_t* A, const int8_t* W, const float* xs, const float* ws, const void* bias, void* D,
+                          int64_t M, int64_t N, int64_t K, int out_dt, int fma) {
+    if (M == 0 || N == 0 || K == 0) return 0;
+    if (out_dt < 0 || out_dt > 2) return -200;
+    int32_t* acc = (int32_t*)malloc(sizeof(int32_t) * (size_t)(M * N));
+    orc_int8_gemm_acc(A, W, acc, M, N, K);
+    orc_epilogue(acc, xs, ws, bias, D, M, N, out_dt, fma);
+    free(acc);
+    return 0;
+}
+/* gpu_int8_gemm_residual: csrc/gemm.cu:132-140 -> launch_cutlass_int8_dequant_residual
+ * csrc/vendor/cutlass_gemm_int8.cu:348-371: M or N == 0 -> ok; K == 0 or a null rscale/resid -> refused (-201). */
+ORC_API int orc_int8_gemm_residual(const int8_t* A, const int8_t* W, const float* xs, const float* ws, const void* bias,
+                                   const void* rscale, const void* resid, void* D, int64_t M, int64_t N, int64_t K,
+                                   int out_dt, int fma) {
+    if (M == 0 || N == 0) return 0;
+    if (K == 0 || !rscale || !resid) return -201;
+    if (out_dt < 0 || out_dt > 2) return -201;
+    int32_t* acc = (int32_t*)malloc(sizeof(int32_t) * (size_t)(M * N));
+    orc_int8_gemm_acc(A, W, acc, M, N, K);
+    orc_epilogue_residual(acc, xs, ws, bias, rscale, resid, D, M, N, out_dt, fma);
+    free(acc);
+    return 0;
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * W6 decode, reference format: csrc/h3.cu:5 (e4m3), :11-46.  Row n = K/2 nibble bytes then K/4 top-bit bytes;
+ * s_rel is fp8-e4m3 [N, K/G]; out = clamp(rint((c-32)*s), -127, 127).
+ * ------------------------------------------------------------------------------------------- */
+ORC_API float orc_e4m3_to_f32(uint8_t v) {
+    const int s = v >> 7, e = (v >> 3) & 0xf, m = v & 7;
+    float f;
+    if (e == 15 && m == 7) f = NAN;                         /* S.1111.111 is the only NaN; there is no infinity */
+    else if (e == 0) f = ldexpf((float)m, -9);              /* subnormal: m/8 * 2^-6 */
+    else f = ldexpf((float)(8 + m), e - 10);                /* (1 + m/8) * 2^(e-7) */
+    return s ? -f : f;
+}
+ORC_API int orc_w6_decode(const uint8_t* q, const uint8_t* s_rel, int8_t* out, int64_t N, int K, int G) {
+    if (K % 32 || G % 16) return -1; /* csrc/h3.cu:41 */
+    for (int64_t n = 0; n < N; ++n) {
+        const uint8_t* lo = q + n * (K * 3 / 4);
+        const uint8_t* hi = lo + K / 2;
+        for (int e = 0; e < K; ++e) {
+            const unsigned nib = (lo[e / 2] >> (4 * (e & 1))) & 0xFu;
+            const unsigned top = (hi[e / 4] >> (2 * (e & 3))) & 3u;
+            const unsigned c = nib | (top << 4);
+            const float s = orc_e4m3_to_f32(s_rel[n * (K / G) + e / G]);
+            out[n * K + e] = (int8_t)fmin_dev(127.f, fmax_dev(-127.f, nearbyintf(((float)c - 32.f) * s)));
+        }
+    }
+    return 0;
+}
+/* Packer for the reference two-plane layout (the inverse of the unpack above; layout from
+ * csrc/vendor/w6a8_requant.cu:138-150).  codes[N,K] hold c = q+32 in 0..63. */
+ORC_API void orc_w6_pack_planes(const uint8_t* codes, uint8_t* q, int64_t N, int K) {
+    for (int64_t n = 0; n < N; ++n) {
+        uint8_t* lo = q + n * (K * 3 / 4);
+        uint8_t* hi = lo + K / 2;
+        memset(lo, 0, (size_t)(K * 3 / 4));
+        for (int e = 0; e < K; ++e) {
+            const unsigned c = codes[n * K + e] & 63u;
+            lo[e / 2] |= (uint8_t)((c & 0xFu) << (4 * (e & 1)));
+            hi[e / 4] |= (uint8_t)((c >> 4) << (2 * (e & 3)));
+        }
+    }
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * W6A8 with per-group weight scales: this build's own format (the reference has none like it).
+ * Weights: 4 codes per 3 bytes along K, 24-bit little-endian word u0 | u1<<6 | u2<<12 | u3<<18 with u = q + 32,
+ * q in [-31,31]; sw f32 [N, K/128].  For each output: p_g = sum over group g of A*q (int32, exact);
+ * accf = fmaf((float)p_g, sw[n,g], accf) for g ascending from accf = 0; y = Out(fmaf(accf, xs[m], bias[n])).
+ * ------------------------------------------------------------------------------------------- */
+ORC_API void orc_w6_pack_words(const int8_t* qv, uint8_t* packed, int64_t N, int K) {
+    for (int64_t n = 0; n < N; ++n)
+        for (int k = 0; k < K; k += 4) {
+            uint32_t w = 0;
+            for (int j = 0; j < 4; ++j) w |= (uint32_t)((qv[n * K + k + j] + 32) & 63) << (6 * j);
+            uint8_t* p = packed + n * (K * 3 / 4) + (k / 4) * 3;
+            p[0] = (uint8_t)w; p[1] = (uint8_t)(w >> 8); p[2] = (uint8_t)(w >> 16);
+        }
+}
+ORC_API void orc_w6_unpack_words(const uint8_t* packed, int8_t* qv, int64_t N, int K) {
+    for (int64_t n = 0; n < N; ++n)
+        for (int k = 0; k < K; k += 4) {
+            const uint8_t* p = packed + n * (K * 3 / 4) + (k / 4) * 3;
+            const uint32_t w = (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16);
+            for (int j = 0; j < 4; ++j) qv[n * K + k + j] = (int8_t)((int)((w >> (6 * j)) & 63u) - 32);
+        }
+}
+ORC_API int orc_w6a8_group_gemm(const int8_t* A, const uint8_t* packed, const float* xs, const float* sw,
+                                const void* bias, void* D, int32_t* partials, int64_t M, int64_t N, int64_t K,
+                                int out_dt) {
+    if (K % 128) return -1;
+    if (out_dt < 0 || out_dt > 2) return -200;
+    if (M == 0 || N == 0) return 0;
+    const int64_t ng = K / 128;
+    int8_t* w = (int8_t*)malloc((size_t)(N * K));
+    orc_w6_unpack_words(packed, w, N, (int)K);
+#pragma omp parallel for schedule(static)
+    for (int64_t m = 0; m < M; ++m)
+        for (int64_t n = 0; n < N; ++n) {
+            float accf = 0.f;
+            for (int64_t g = 0; g < ng; ++g) {
+                int32_t p = 0;
+                for (int64_t k = g * 128; k < (g + 1) * 128; ++k) p += (int32_t)A[m * K + k] * (int32_t)w[n * K + k];
+                if (partials) partials[(m * N + n) * ng + g] = p;
+                accf = fmaf((float)p, sw[n * ng + g], accf);
+            }
+            const float b = bias ? ld_t(out_dt, bias, n) : 0.f;
+            st_t(out_dt, D, m * N + n, fmaf(accf, xs[m], b));
+        }
+    free(w);
+    return 0;
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * The whole linear on the CPU (quantize -> GEMM -> epilogue), for the bench's CPU-baseline leg.  Row-parallel with
+ * OpenMP; returns the thread count it ran with through *threads.
+ * ------------------------------------------------------------------------------------------- */
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+ORC_API int orc_linear_w8a8(int dtype, const void* x, int64_t x_stride, int rotate, const int8_t* W, const float* ws,
+                            const void* bias, void* D, int M, int N, int K, int out_dt, int fma, int* threads) {
+    int8_t* q = (int8_t*)malloc((size_t)M * (size_t)K);
+    float* xs = (float*)malloc(sizeof(float) * (size_t)M);
+    int rc = orc_quant_rows(dtype, x, x_stride, q, xs, M, K, rotate);
+    if (!rc) rc = orc_int8_gemm(q, W, xs, ws, bias, D, M, N, K, out_dt, fma);
+    free(q);
+    free(xs);
+    if (threads) {
+#ifdef _OPENMP
+        *threads = omp_get_max_threads();
+#else
+        *threads = 1;
+#endif
+    }
+    return rc;
+}
+ORC_API void orc_set_threads(int n) {
+#ifdef _OPENMP
+    omp_set_num_threads(n > 0 ? n : 1);
+#else
+    (void)n;
+#endif
+}
