@@ -1,0 +1,160 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-linear hot path on one MI355X.
+
+A step is one W8A8 linear over one batch of synthetic activations already resident in HBM: per-token int8
+quantization with the ConvRot rotation (gpu_quant_rows), then the int8 GEMM with the fused dequant/bias epilogue
+(gpu_int8_gemm).  The default workload is the one the headline metric is quoted on: the image-DiT MLP up-projection,
+M=4608 tokens, K=3072, N=12288, bf16 in and out, Hadamard block 128.
+
+Prints ONE JSON line: whole-step throughput in TOPS (2*M*N*K per step), the roofline of the dominant kernel (the int8
+GEMM against the dense int8 MFMA peak) from HIP events recorded inside the timed region, the CPU oracle timed on a
+bounded row sample, and the memory-bound skinny (M=256) linears as HBM GB/s.
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, 5.0 POP/s
+PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, 8 TB/s
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--shape", default="4608,3072,12288", help="M,K,N of the timed linear")
+    ap.add_argument("--rotate", type=int, default=128, help="Hadamard block (0 = none, 64, 128, 256)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-skinny", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
+    return ap.parse_args()
+
+
+def make_inputs(torch, synth, M, K, N, seed=0, dev="cuda:0", kind="t3"):
+    import numpy as np
+    x = synth.bf16_bits(synth.activations(seed, M, K, kind))
+    W, ws, bias = synth.w8_weights(seed, N, K)
+    bias = synth.bf16_bits(bias)
+    host = dict(x=x, W=W, ws=ws, bias=bias)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    devs = dict(x=t(x.view(np.int16)).view(torch.bfloat16), W=t(W), ws=t(ws),
+                bias=t(bias.view(np.int16)).view(torch.bfloat16))
+    return host, devs
+
+
+def time_linear(torch, ffi, d, M, K, N, rotate, steps, warmup, nbuf=1):
+    """Times `steps` linears; returns (ms_total, ms_quant_avg, ms_gemm_avg).  nbuf > 1 rotates among copies of the
+    weights so that a memory-bound shape cannot live in the 256 MB last-level cache."""
+    st = torch.cuda.current_stream()
+    s = st.cuda_stream
+    q = torch.empty((M, K), dtype=torch.int8, device="cuda:0")
+    xs = torch.empty((M,), dtype=torch.float32, device="cuda:0")
+    D = torch.empty((M, N), dtype=torch.bfloat16, device="cuda:0")
+    Ws = [d["W"]] + [d["W"].clone() for _ in range(nbuf - 1)]
+
+    def step(i, evs=None):
+        W = Ws[i % nbuf]
+        if evs: evs[0].record(st)
+        ffi.k("gpu_quant_rows", ffi.DT_BF16, ffi.PRO_PLAIN, d["x"].data_ptr(), K, 0, 0, 0, 0, 0.0, 0, 0, q.data_ptr(),
+              xs.data_ptr(), M, K, rotate, s)
+        if evs: evs[1].record(st)
+        ffi.k("gpu_int8_gemm", q.data_ptr(), W.data_ptr(), xs.data_ptr(), d["ws"].data_ptr(), d["bias"].data_ptr(),
+              D.data_ptr(), M, N, K, ffi.DT_BF16, s)
+        if evs: evs[2].record(st)
+
+    for i in range(warmup):
+        step(i)
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        step(i, evs[i])
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    gpu_ms = evs[0][0].elapsed_time(evs[-1][2])
+    tq = sum(e[0].elapsed_time(e[1]) for e in evs) / steps
+    tg = sum(e[1].elapsed_time(e[2]) for e in evs) / steps
+    return max(gpu_ms, 0.0), wall_ms, tq, tg
+
+
+def cpu_baseline(host, M, K, N, rotate, target_s):
+    """The oracle's whole linear (quantize, int32 GEMM, epilogue) on a row sample sized for about `target_s` seconds."""
+    import oracle
+    threads = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
+    rows = min(M, 64)
+    t0 = time.perf_counter()
+    rc, _, used = oracle.linear_w8a8(oracle.BF16, host["x"][:rows], rotate, host["W"], host["ws"], host["bias"], oracle.BF16,
+                                     threads=threads)
+    dt = time.perf_counter() - t0
+    assert rc == 0
+    rows2 = int(min(M, max(rows, rows * target_s / max(dt, 1e-3))))
+    rows2 -= rows2 % threads if rows2 > threads else 0
+    t0 = time.perf_counter()
+    rc, _, used = oracle.linear_w8a8(oracle.BF16, host["x"][:rows2], rotate, host["W"], host["ws"], host["bias"], oracle.BF16,
+                                     threads=threads)
+    dt = time.perf_counter() - t0
+    assert rc == 0
+    return {"value": 2.0 * rows2 * N * K / dt / 1e12, "unit": "TOPS", "cores": used, "kind": "port",
+            "sample": "first %d of %d rows, whole linear (quantize + int32 GEMM + epilogue), %.1f s" % (rows2, M, dt)}
+
+
+def main():
+    a = parse()
+    if a.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)" % a.gpus, file=sys.stderr)
+        sys.exit(2)
+    import torch
+    ffi = importlib.import_module("comfyui-backend-but-rust_amd.ffi")
+    synth = importlib.import_module("comfyui-backend-but-rust_amd.synth")
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    M, K, N = (int(v) for v in a.shape.split(","))
+    host, d = make_inputs(torch, synth, M, K, N)
+    gpu_ms, wall_ms, tq, tg = time_linear(torch, ffi, d, M, K, N, a.rotate, a.steps, a.warmup)
+    ops = 2.0 * M * N * K
+    ms_per_step = wall_ms / a.steps
+    value = ops / (ms_per_step * 1e-3) / 1e12
+    gemm_tops = ops / (tg * 1e-3) / 1e12
+    quant_bytes = M * K * 2 + M * K + M * 4
+    out = {
+        "metric": "W8A8 linear TOPS @M%d K%d N%d (quantize + int8 GEMM + dequant epilogue)" % (M, K, N),
+        "value": round(value, 2), "unit": "TOPS", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8", "data": "synthetic",
+        "config": {"workload": "image-DiT MLP up-projection W8A8 linear, bf16 activations M=%d K=%d -> N=%d, Hadamard "
+                               "block %d, per-channel scales, bf16 bias and output" % (M, K, N, a.rotate),
+                   "M": M, "K": K, "N": N, "rotate": a.rotate},
+        "roofline": {"bound": "mfma", "kernel": "int8_gemm_kernel (gpu_int8_gemm)", "achieved": round(gemm_tops, 2),
+                     "peak": PEAK_INT8_TOPS, "unit": "TFLOP/s", "frac": round(gemm_tops / PEAK_INT8_TOPS, 4),
+                     "traffic": None, "avg_launch_us": round(tg * 1e3, 2)},
+        "kernels": {"quant_rows_us": round(tq * 1e3, 2), "quant_rows_GBs": round(quant_bytes / (tq * 1e-3) / 1e9, 1),
+                    "int8_gemm_us": round(tg * 1e3, 2), "gpu_ms_total": round(gpu_ms, 4)},
+    }
+    if not a.no_skinny:
+        sk = []
+        for (m, k, n) in ((256, 4096, 24576), (256, 12288, 4096)):
+            h2, d2 = make_inputs(torch, synth, m, k, n, seed=1, kind="normal")
+            nbuf = max(2, int(600e6 // (n * k)) + 1)
+            _, wall2, tq2, tg2 = time_linear(torch, ffi, d2, m, k, n, a.rotate, a.steps, a.warmup, nbuf=nbuf)
+            gemm_bytes = m * k + m * 4 + n * k + n * 4 + n * 2 + m * n * 2
+            sk.append({"M": m, "K": k, "N": n, "int8_gemm_us": round(tg2 * 1e3, 2),
+                       "GBs": round(gemm_bytes / (tg2 * 1e-3) / 1e9, 1),
+                       "frac_hbm": round(gemm_bytes / (tg2 * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                       "quant_rows_us": round(tq2 * 1e3, 2), "weight_copies_rotated": nbuf})
+            del h2, d2
+        out["skinny"] = sk
+    if not a.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(host, M, K, N, a.rotate, a.cpu_seconds)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,55 @@
+"""Build libgpu_kernels.so (the C-ABI library of the gfx950 kernels) in-tree with hipcc.
+
+hipcc cross-compiles for gfx950 without a GPU.  Objects are built in parallel, one per .hip file, then linked.
+"""
+import concurrent.futures
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+OUT = os.path.join(HERE, "libgpu_kernels.so")
+ARCH = os.environ.get("HIP_ARCH", "gfx950")
+SOURCES = ["quant_rows.hip", "int8_gemm.hip", "w6.hip"]
+FLAGS = [
+    "--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
+    # exact arithmetic: no contraction except where fmaf is written, IEEE divide, no fast-math
+    "-ffp-contract=off", "-fno-fast-math", "-fhip-fp32-correctly-rounded-divide-sqrt",
+    # keep the compiler from forming packed-fp32 instructions
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+
+def _compile(src):
+    obj = os.path.join(CSRC, os.path.splitext(src)[0] + ".o")
+    cmd = ["hipcc", *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc failed for %s:\n%s" % (src, err))
+    if err.strip():
+        sys.stderr.write(err + "\n")
+    return obj
+
+
+def stale():
+    if not os.path.exists(OUT):
+        return True
+    t = os.path.getmtime(OUT)
+    deps = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".hip", ".hpp"))]
+    deps.append(os.path.join(os.path.dirname(HERE), "include", "gpu_api.h"))
+    return any(os.path.getmtime(d) > t for d in deps)
+
+
+def build(force=True):
+    if not force and not stale():
+        return OUT
+    with concurrent.futures.ThreadPoolExecutor(max_workers=len(SOURCES)) as ex:
+        objs = list(ex.map(_compile, SOURCES))
+    subprocess.check_call(["hipcc", "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", OUT, *objs])
+    return OUT
+
+
+if __name__ == "__main__":
+    print(build(force="--if-stale" not in sys.argv))

@@ -1,0 +1,336 @@
+// Per-row absmax int8 quantization with the optional ConvRot group rotation, for gfx950 (wave64).
+//
+// Arithmetic follows the reference's quantizers exactly (csrc/kernels.cu:184-258 for bf16/f32 rows,
+// csrc/sd.cu:578-598 for fp16 rows, csrc/common.cuh:99-126 for the staged radix-4 Hadamard butterflies): same
+// float operation order, same rounding points.  The structure does not: a row is cut into chunks of 1024 values, one
+// wave per chunk, each lane holding 16 consecutive values in registers.  Radix-4 stages with strides 1 and 4 run inside
+// a lane; for the wider strides the chunk makes one trip through a wave-private LDS tile so that those butterflies are
+// again lane-local, then returns to row order for the 16-byte code stores.
+#include "common.hpp"
+
+namespace {
+
+enum { MODE_BF16 = 0, MODE_F32 = 1, MODE_SD_F16 = 2, MODE_ROT_F32 = 3 };
+
+struct QuantArgs {
+    const void* x;
+    int64_t x_stride;  // elements between rows
+    int8_t* q;         // [M, K]
+    float* scales;     // [M]
+    float* out_f;      // MODE_ROT_F32: rotated rows [M, K]
+    int M, K;
+    int wpr;           // waves per row
+    int rpb;           // rows per block
+};
+
+constexpr int kChunk = 1024;           // values per wave-chunk (64 lanes x 16)
+constexpr int kLdsPerWave = 1024 + 64; // floats: one chunk plus 16 pad floats per 256
+
+// LDS position of chunk element e.  Each lane's 16 consecutive values are four 16-byte vectors; vector i of lane L is
+// rotated to slot (i + L/2) & 3 so that 8 neighbouring lanes cover all 32 banks in a 128-bit access, and every 256
+// elements are padded by 16 floats so that the stride-16 accesses of the second phase spread over both bank halves.
+__device__ __forceinline__ int lds_pos(int e) {
+    const int L = e >> 4, i = (e >> 2) & 3, j = e & 3;
+    return (L << 4) + (((i + (L >> 1)) & 3) << 2) + j + ((e >> 8) << 4);
+}
+
+// h4_row x 4 outputs with the reference's left-to-right adds, scaled by 0.5 (csrc/common.cuh:99-106,119-122).
+__device__ __forceinline__ void bfly4(float& a, float& b, float& c, float& d) {
+    const float x0 = a, x1 = b, x2 = c, x3 = d;
+    a = 0.5f * (x0 + x1 + x2 - x3);
+    b = 0.5f * (x0 + x1 - x2 + x3);
+    c = 0.5f * (x0 - x1 + x2 + x3);
+    d = 0.5f * (-x0 + x1 + x2 + x3);
+}
+
+template <int MODE> __device__ __forceinline__ void load16(const void* x, int64_t off, float* v) {
+    if (MODE == MODE_BF16) {
+        const uint4* p = reinterpret_cast<const uint4*>((const uint16_t*)x + off);
+        const uint4 a = p[0], b = p[1];
+        const uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            v[2 * i] = u2f(w[i] << 16);
+            v[2 * i + 1] = u2f(w[i] & 0xffff0000u);
+        }
+    } else if (MODE == MODE_SD_F16) {
+        const uint4* p = reinterpret_cast<const uint4*>((const uint16_t*)x + off);
+        const uint4 a = p[0], b = p[1];
+        const uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            v[2 * i] = f16_to_f((uint16_t)(w[i] & 0xffffu));
+            v[2 * i + 1] = f16_to_f((uint16_t)(w[i] >> 16));
+        }
+    } else {
+        const float4* p = reinterpret_cast<const float4*>((const float*)x + off);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float4 f = p[i];
+            v[4 * i] = f.x; v[4 * i + 1] = f.y; v[4 * i + 2] = f.z; v[4 * i + 3] = f.w;
+        }
+    }
+}
+
+// Rotate one chunk held as v[16] per lane (element 16*lane + i).  wl is the wave's LDS tile.  Uniform over the block.
+template <int G> __device__ __forceinline__ void rotate_chunk(float* v, float* wl, int lane) {
+    // strides 1 and 4: inside the lane
+#pragma unroll
+    for (int i = 0; i < 4; ++i) bfly4(v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) bfly4(v[j], v[j + 4], v[j + 8], v[j + 12]);
+    // to LDS in row order
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        *reinterpret_cast<float4*>(wl + lds_pos(16 * lane + 4 * i)) = make_float4(v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]);
+    __syncthreads();
+    if (G == 256) {
+        // lane (R = lane/16, b = lane%16) takes elements R*256 + a*16 + b, a = 0..15: strides 16 and 64 are lane-local
+        const int base = (lane >> 4) * 256 + (lane & 15);
+        float w[16];
+#pragma unroll
+        for (int a = 0; a < 16; ++a) w[a] = wl[lds_pos(base + a * 16)];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) bfly4(w[4 * i], w[4 * i + 1], w[4 * i + 2], w[4 * i + 3]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) bfly4(w[j], w[j + 4], w[j + 8], w[j + 12]);
+#pragma unroll
+        for (int a = 0; a < 16; ++a) wl[lds_pos(base + a * 16)] = w[a];
+    } else if (G == 64) {
+        // lane (Q = lane/4, p = lane%4) takes elements Q*64 + d*16 + 4p + j: stride 16 is lane-local
+        const int base = (lane >> 2) * 64 + (lane & 3) * 4;
+        float4 w[4];
+#pragma unroll
+        for (int d = 0; d < 4; ++d) w[d] = *reinterpret_cast<float4*>(wl + lds_pos(base + d * 16));
+        bfly4(w[0].x, w[1].x, w[2].x, w[3].x);
+        bfly4(w[0].y, w[1].y, w[2].y, w[3].y);
+        bfly4(w[0].z, w[1].z, w[2].z, w[3].z);
+        bfly4(w[0].w, w[1].w, w[2].w, w[3].w);
+#pragma unroll
+        for (int d = 0; d < 4; ++d) *reinterpret_cast<float4*>(wl + lds_pos(base + d * 16)) = w[d];
+    } else {
+        // G == 128: lane (O = lane/8, p = lane%8) takes O*128 + t*64 + d*16 + 2p + j: stride 16 (radix 4) and the
+        // closing radix-2 stage at stride 64, scaled by 1/sqrt(2)
+        const int base = (lane >> 3) * 128 + (lane & 7) * 2;
+        float2 w[2][4];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int d = 0; d < 4; ++d) w[t][d] = *reinterpret_cast<float2*>(wl + lds_pos(base + t * 64 + d * 16));
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            bfly4(w[t][0].x, w[t][1].x, w[t][2].x, w[t][3].x);
+            bfly4(w[t][0].y, w[t][1].y, w[t][2].y, w[t][3].y);
+        }
+        const float c = 0.70710678118654752f;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            const float ax = w[0][d].x, bx = w[1][d].x, ay = w[0][d].y, by = w[1][d].y;
+            w[0][d].x = (ax + bx) * c; w[1][d].x = (ax - bx) * c;
+            w[0][d].y = (ay + by) * c; w[1][d].y = (ay - by) * c;
+        }
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int d = 0; d < 4; ++d) *reinterpret_cast<float2*>(wl + lds_pos(base + t * 64 + d * 16)) = w[t][d];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float4 f = *reinterpret_cast<float4*>(wl + lds_pos(16 * lane + 4 * i));
+        v[4 * i] = f.x; v[4 * i + 1] = f.y; v[4 * i + 2] = f.z; v[4 * i + 3] = f.w;
+    }
+    __syncthreads();
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+
+template <int MODE, int G, int C>
+__global__ void __launch_bounds__(512) quant_rows_kernel(QuantArgs p) {
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    __shared__ float red[8];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int rloc = wave / p.wpr, wr = wave - rloc * p.wpr;
+    const int64_t m = (int64_t)blockIdx.x * p.rpb + rloc;
+    const bool row_ok = m < p.M;
+    float* wl = lds + wave * kLdsPerWave;
+
+    float v[C][16];
+    float amax = 0.f;
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+        const int e0 = (wr + c * p.wpr) * kChunk + lane * 16;
+        const bool act = row_ok && e0 < p.K;
+        if (act) {
+            load16<MODE>(p.x, m * p.x_stride + e0, v[c]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) v[c][i] = 0.f;
+        }
+        if (G != 0) rotate_chunk<G>(v[c], wl, lane);
+        if (MODE == MODE_ROT_F32) {
+            if (act) {
+                float4* o = reinterpret_cast<float4*>(p.out_f + m * (int64_t)p.K + e0);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) o[i] = make_float4(v[c][4 * i], v[c][4 * i + 1], v[c][4 * i + 2], v[c][4 * i + 3]);
+            }
+        } else if (MODE == MODE_SD_F16) {
+            // the maximum is taken over the half-rounded row (csrc/sd.cu:587)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) amax = fmaxf(amax, fabsf(rnd_dt<DT_F16>(v[c][i])));
+        } else {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) amax = fmaxf(amax, fabsf(v[c][i]));
+        }
+    }
+    if (MODE == MODE_ROT_F32) return;
+
+    amax = wave_max(amax);
+    if (p.wpr > 1) {  // uniform over the block
+        if (lane == 0) red[wave] = amax;
+        __syncthreads();
+        amax = 0.f;
+        for (int i = 0; i < p.wpr; ++i) amax = fmaxf(amax, red[rloc * p.wpr + i]);
+    }
+
+    float scale, st, rinv = 0.f;
+    if (MODE == MODE_SD_F16) {
+        scale = fmaxf(amax, 1e-30f) / 127.f;                       // csrc/sd.cu:589
+        const float sh = rnd_dt<DT_F16>(scale);
+        st = sh > 0.f ? sh : scale;                                // :593
+    } else if (MODE == MODE_BF16) {
+        scale = fmaxf(fminf(amax, 3.38953139e38f) * (1.f / 127.f), 1.0e-30f);  // csrc/kernels.cu:241
+        st = rnd_dt<DT_BF16>(scale);
+        rinv = __builtin_amdgcn_rcpf(st);
+    } else {
+        scale = fmaxf(fminf(amax, 3.402823466e+38f) * (1.f / 127.f), 1.0e-30f);
+        st = scale;
+    }
+    if (row_ok && wr == 0 && lane == 0) p.scales[m] = scale;
+
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+        const int e0 = (wr + c * p.wpr) * kChunk + lane * 16;
+        if (!(row_ok && e0 < p.K)) continue;
+        uint32_t w[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            uint32_t acc = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float x = v[c][4 * i + j];
+                float t;
+                if (MODE == MODE_BF16) {
+                    // Both operands carry 8 significant bits, so their exact quotient is never closer than 2^-17
+                    // (relative) to a bf16 rounding boundary: a 1-ulp reciprocal times the numerator rounds to the
+                    // same bf16 value as the IEEE quotient does.
+                    t = rnd_dt<DT_BF16>(rnd_dt<DT_BF16>(x) * rinv);
+                } else if (MODE == MODE_SD_F16) {
+                    t = rnd_dt<DT_F16>(rnd_dt<DT_F16>(x) / st);
+                } else {
+                    t = x / st;
+                }
+                const int qi = (int)fminf(127.f, fmaxf(-128.f, nearbyintf(t)));
+                acc |= ((uint32_t)qi & 0xffu) << (8 * j);
+            }
+            w[i] = acc;
+        }
+        *reinterpret_cast<uint4*>(p.q + m * (int64_t)p.K + e0) = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+}
+
+template <int MODE, int G, int C>
+int launch(const QuantArgs& a, int nw, hipStream_t st) {
+    const int grid = (a.M + a.rpb - 1) / a.rpb;
+    const size_t smem = G ? (size_t)nw * kLdsPerWave * sizeof(float) : 0;
+    hipLaunchKernelGGL((quant_rows_kernel<MODE, G, C>), dim3(grid), dim3(nw * 64), smem, st, a);
+    KCHECK();
+    return 0;
+}
+
+template <int MODE, int G>
+int launch_c(const QuantArgs& a, int nw, int C, hipStream_t st) {
+    switch (C) {
+        case 1: return launch<MODE, G, 1>(a, nw, st);
+        case 2: return launch<MODE, G, 2>(a, nw, st);
+        case 3: return launch<MODE, G, 3>(a, nw, st);
+        default: return launch<MODE, G, 4>(a, nw, st);
+    }
+}
+
+// g: rotation group width (0, 64, 128, 256).  Picks waves per row so that a wave holds at most 4 chunks.
+template <int MODE>
+int run_quant(QuantArgs a, int g, hipStream_t st) {
+    if (a.M <= 0) return 0;
+    const int nchunks = (a.K + kChunk - 1) / kChunk;
+    int wpr = 1;
+    while ((nchunks + wpr - 1) / wpr > 4) wpr *= 2;
+    if (wpr > 8) return -2;
+    const int C = (nchunks + wpr - 1) / wpr;
+    const int nw = wpr < 4 ? 4 : wpr;
+    a.wpr = wpr;
+    a.rpb = nw / wpr;
+    switch (g) {
+        case 0: return launch_c<MODE, 0>(a, nw, C, st);
+        case 64: return launch_c<MODE, 64>(a, nw, C, st);
+        case 128: if (MODE == MODE_SD_F16 || MODE == MODE_ROT_F32) return -1; return launch_c<MODE == MODE_F32 || MODE == MODE_BF16 ? MODE : MODE_BF16, 128>(a, nw, C, st);
+        default: return launch_c<MODE, 256>(a, nw, C, st);
+    }
+}
+
+int rotate_group(int rotate) { return rotate == 0 ? 0 : (rotate == 64 || rotate == 128) ? rotate : 256; }
+
+bool known_prologue(int p) { return p >= PRO_PLAIN && p <= PRO_SITU_FAST && p != PRO_LN_AFFINE_SILU; }
+
+}  // namespace
+
+GPU_API int gpu_quant_rows(int dtype, int prologue, const void* x, int64_t x_stride, const void* g, int64_t g_stride,
+                           int64_t up_offset, const float* norm_w, float eps, const void* mod_scale,
+                           const void* mod_shift, int8_t* q, float* scales, int M, int K, int rotate, void* stream) {
+    (void)g; (void)g_stride; (void)up_offset; (void)norm_w; (void)eps; (void)mod_scale; (void)mod_shift;
+    const int grp = rotate_group(rotate);
+    const int need = grp == 0 ? 64 : grp;
+    if (K <= 0 || (K % need) != 0) return -1;
+    if (dtype != DT_BF16 && dtype != DT_F32) return -4;
+    if (!known_prologue(prologue)) return -3;   // the id list of csrc/kernels.cu:280-292
+    if (K > 32768) return -2;
+    if (prologue != PRO_PLAIN) return -30;
+    QuantArgs a{x, x_stride, q, scales, nullptr, M, K, 1, 1};
+    hipStream_t st = (hipStream_t)stream;
+    return dtype == DT_BF16 ? run_quant<MODE_BF16>(a, grp, st) : run_quant<MODE_F32>(a, grp, st);
+}
+
+GPU_API int gpu_quant_rows_b(int dtype, int prologue, const void* x, int64_t x_stride, const float* norm_w,
+                             const float* norm_b, float eps, const void* mod_scale, const void* mod_shift, int8_t* q,
+                             float* scales, int M, int K, int rotate, void* stream) {
+    (void)x; (void)x_stride; (void)norm_w; (void)norm_b; (void)eps; (void)mod_scale; (void)mod_shift; (void)q;
+    (void)scales; (void)M; (void)rotate; (void)stream;
+    if ((K % 256) != 0) return -1;
+    if (dtype != DT_BF16) return -4;
+    if (prologue != PRO_LN_MOD && prologue != PRO_LN_AFFINE) return -3;
+    return -30;
+}
+
+GPU_API int gpu_rotate_rows_f32(int prologue, const float* x, int64_t x_stride, int64_t up_offset, const float* norm_w,
+                                float eps, float* out, int M, int K, void* stream) {
+    (void)up_offset; (void)norm_w; (void)eps;
+    if (K <= 0 || (K % 256) != 0) return -1;
+    if (prologue != PRO_PLAIN && prologue != PRO_RMS && prologue != PRO_SWIGLU) return -3;
+    if (K > 32768) return -2;
+    if (prologue != PRO_PLAIN) return -30;
+    QuantArgs a{x, x_stride, nullptr, nullptr, out, M, K, 1, 1};
+    return run_quant<MODE_ROT_F32>(a, 256, (hipStream_t)stream);
+}
+
+GPU_API int gpu_sd_quant_rows(const void* x, int64_t x_stride, int8_t* q, float* scales, int M, int K, int rotate,
+                              void* stream) {
+    if ((rotate != 0 && rotate != 64 && rotate != 256) || (rotate && K % rotate)) return -1;
+    if (K <= 0 || (K % 16) != 0) return -1;   // 16 values per lane
+    if (K > 32768) return -2;
+    QuantArgs a{x, x_stride, q, scales, nullptr, M, K, 1, 1};
+    return run_quant<MODE_SD_F16>(a, rotate, (hipStream_t)stream);
+}

@@ -1,0 +1,85 @@
+"""Host-side call pattern of one quantized linear, as the reference's model code issues it (src/dit.rs:550-555,
+src/unet.rs:436-456, src/h3.rs:1208-1251): quantize rows, then the fused int8 GEMM.  torch supplies device memory and
+the stream; all arithmetic happens in libgpu_kernels.so.
+"""
+import torch
+
+from . import ffi
+
+_TORCH_DT = {torch.float32: ffi.DT_F32, torch.float16: ffi.DT_F16, torch.bfloat16: ffi.DT_BF16}
+_DT_TORCH = {v: k for k, v in _TORCH_DT.items()}
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t):
+    return 0 if t is None else t.data_ptr()
+
+
+def quant_rows(x, rotate=0, K=None, q=None, scales=None):
+    """x: [M, x_stride] bf16 or f32 CUDA tensor -> (q int8 [M,K], scales f32 [M])."""
+    M, x_stride = x.shape
+    K = x_stride if K is None else K
+    q = torch.empty((M, K), dtype=torch.int8, device=x.device) if q is None else q
+    scales = torch.empty((M,), dtype=torch.float32, device=x.device) if scales is None else scales
+    ffi.k("gpu_quant_rows", _TORCH_DT[x.dtype], ffi.PRO_PLAIN, _ptr(x), x.stride(0), 0, 0, 0, 0, 0.0, 0, 0, _ptr(q),
+          _ptr(scales), M, K, rotate, _stream())
+    return q, scales
+
+
+def sd_quant_rows(x, rotate=0, K=None):
+    M, x_stride = x.shape
+    K = x_stride if K is None else K
+    q = torch.empty((M, K), dtype=torch.int8, device=x.device)
+    scales = torch.empty((M,), dtype=torch.float32, device=x.device)
+    ffi.k("gpu_sd_quant_rows", _ptr(x), x.stride(0), _ptr(q), _ptr(scales), M, K, rotate, _stream())
+    return q, scales
+
+
+def rotate_rows_f32(x, K=None):
+    M, x_stride = x.shape
+    K = x_stride if K is None else K
+    out = torch.empty((M, K), dtype=torch.float32, device=x.device)
+    ffi.k("gpu_rotate_rows_f32", ffi.PRO_PLAIN, _ptr(x), x.stride(0), 0, 0, 0.0, _ptr(out), M, K, _stream())
+    return out
+
+
+def int8_gemm(A, W, xs, ws, bias=None, out_dtype=torch.bfloat16, D=None):
+    M, K = A.shape
+    N = W.shape[0]
+    D = torch.empty((M, N), dtype=out_dtype, device=A.device) if D is None else D
+    ffi.k("gpu_int8_gemm", _ptr(A), _ptr(W), _ptr(xs), _ptr(ws), _ptr(bias), _ptr(D), M, N, K, _TORCH_DT[out_dtype],
+          _stream())
+    return D
+
+
+def int8_gemm_residual(A, W, xs, ws, bias, rscale, resid, D=None):
+    """D = resid + rscale * (...); pass D=resid for the in-place form the DiT block uses."""
+    M, K = A.shape
+    N = W.shape[0]
+    D = torch.empty_like(resid) if D is None else D
+    ffi.k("gpu_int8_gemm_residual", _ptr(A), _ptr(W), _ptr(xs), _ptr(ws), _ptr(bias), _ptr(rscale), _ptr(resid), _ptr(D),
+          M, N, K, _TORCH_DT[resid.dtype], _stream())
+    return D
+
+
+def int8_gemm_acc(A, W):
+    M, K = A.shape
+    N = W.shape[0]
+    acc = torch.empty((M, N), dtype=torch.int32, device=A.device)
+    ffi.k("gpu_int8_gemm_acc", _ptr(A), _ptr(W), _ptr(acc), M, N, K, _stream())
+    return acc
+
+
+def w6_decode(wq, s_rel, N, K, G):
+    out = torch.empty((N, K), dtype=torch.int8, device=wq.device)
+    ffi.k("gpu_w6_decode", _ptr(wq), _ptr(s_rel), _ptr(out), N, K, G, _stream())
+    return out
+
+
+def linear_w8a8(x, W, ws, bias=None, rotate=0, out_dtype=None):
+    """One W8A8 linear: y = dequant(quant(x) . W^T)."""
+    q, xs = quant_rows(x, rotate)
+    return int8_gemm(q, W, xs, ws, bias, x.dtype if out_dtype is None else out_dtype)

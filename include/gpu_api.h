@@ -1,0 +1,99 @@
+/*
+ * C ABI of the MI355X (gfx950) quantized-linear kernels: libgpu_kernels.so.
+ *
+ * The first block of entry points has the reference's names, argument order and C types, so the reference's Rust
+ * declarations (src/ffi.rs) bind to this library unchanged; each prototype cites the declaration it replaces.
+ * All pointers are device pointers unless stated; `stream` is a hipStream_t passed as void* (null = default stream).
+ * Every call is asynchronous on `stream`, allocates nothing that outlives it, keeps no state between calls and
+ * never throws.
+ *
+ * Return convention (src/ffi.rs:336-344, csrc/common.cuh:128): 0 = ok; > 0 = a hipError_t from the launch
+ * (hipGetErrorString names it); < 0 = the launcher refused the arguments, with the reference's codes:
+ *   quantizers  -1 shape (K granularity), -2 row too long (K > 32768), -3 prologue id, -4 dtype
+ *   int8 GEMM   -200 (plain) / -201 (residual): unknown out_dt, null rscale/resid, K == 0 for the residual form,
+ *               or a shape the kernels cannot run (K % 16 != 0)
+ *   w6 decode   -1 (K % 32 or G % 16)
+ *   -30         a prologue id that exists in the reference but is not built in this library yet
+ */
+#ifndef GPU_API_H
+#define GPU_API_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* dtype codes: csrc/common.cuh:15, src/ffi.rs:11-13 */
+enum { DT_F32 = 0, DT_F16 = 1, DT_BF16 = 2 };
+
+/* prologue ids: csrc/kernels.cu:13-15, src/ffi.rs:15-29 */
+enum {
+    PRO_PLAIN = 0, PRO_RMS = 1, PRO_GATE = 2, PRO_SWIGLU = 3, PRO_LAYERNORM = 4, PRO_SILU = 5, PRO_GELU = 6,
+    PRO_ADALN = 7, PRO_SITU = 8, PRO_LN_MOD = 9, PRO_LN_AFFINE = 10, PRO_GELU_TANH = 11, PRO_LN_AFFINE_SILU = 12,
+    PRO_SITU_FAST = 13
+};
+
+/* Row prologue -> optional ConvRot rotation -> dynamic per-row absmax int8 quantization.
+ * Replaces gpu_quant_rows, src/ffi.rs:74-75 / csrc/kernels.cu:271-298.
+ * x: T[M, x_stride] (T = bf16 or f32 by `dtype`; rows 16-byte aligned); q: int8 [M, K]; scales: f32 [M].
+ * rotate: 0 = none; 1 or 256 = the reference's 256-wide normalized Hadamard; 64 and 128 select a 64- or 128-wide
+ * group (an extension: the reference treats the argument as a flag).  K must be a multiple of 256 (of 64 when
+ * rotate is 0 or 64, of 128 when rotate is 128). */
+int gpu_quant_rows(int dtype, int prologue, const void* x, int64_t x_stride, const void* g, int64_t g_stride,
+                   int64_t up_offset, const float* norm_w, float eps, const void* mod_scale, const void* mod_shift,
+                   int8_t* q, float* scales, int M, int K, int rotate, void* stream);
+
+/* gpu_quant_rows with a LayerNorm bias.  Replaces gpu_quant_rows_b, src/ffi.rs:246-247 / csrc/kernels.cu:301-313. */
+int gpu_quant_rows_b(int dtype, int prologue, const void* x, int64_t x_stride, const float* norm_w,
+                     const float* norm_b, float eps, const void* mod_scale, const void* mod_shift, int8_t* q,
+                     float* scales, int M, int K, int rotate, void* stream);
+
+/* Same prologues + 256-wide rotation, fp32 in and out, no quantization.
+ * Replaces gpu_rotate_rows_f32, src/ffi.rs:35-36 / csrc/kernels.cu:316-327. */
+int gpu_rotate_rows_f32(int prologue, const float* x, int64_t x_stride, int64_t up_offset, const float* norm_w,
+                        float eps, float* out, int M, int K, void* stream);
+
+/* fp16 rows -> optional 64/256 rotation -> int8 rows + scales (the SD/SDXL UNet quantizer).
+ * Replaces gpu_sd_quant_rows, src/ffi.rs:252 / csrc/sd.cu:599-606.  rotate in {0, 64, 256}, K % 16 == 0. */
+int gpu_sd_quant_rows(const void* x, int64_t x_stride, int8_t* q, float* scales, int M, int K, int rotate,
+                      void* stream);
+
+/* D[M,N] = Out((A[M,K] . W[N,K]^T) * xs[m] * ws[n] + bias[n]).
+ * Replaces gpu_int8_gemm, src/ffi.rs:38 / csrc/gemm.cu:124-129.
+ * A, W int8 row-major (K contiguous); xs f32 [M]; ws f32 [N]; bias Out[N] or null; D Out[M,N]; out_dt a DT_* code. */
+int gpu_int8_gemm(const int8_t* A, const int8_t* W, const float* xs, const float* ws, const void* bias, void* D,
+                  int64_t M, int64_t N, int64_t K, int out_dt, void* stream);
+
+/* D = Out(float(Out(acc*xs*ws + bias)) * rscale[n] + resid[m,n]); D may alias resid.
+ * Replaces gpu_int8_gemm_residual, src/ffi.rs:39-40 / csrc/gemm.cu:132-140. */
+int gpu_int8_gemm_residual(const int8_t* A, const int8_t* W, const float* xs, const float* ws, const void* bias,
+                           const void* rscale, const void* resid, void* D, int64_t M, int64_t N, int64_t K,
+                           int out_dt, void* stream);
+
+/* Packed 6-bit weights (two planes per row: K/2 nibble bytes, then K/4 top-bit bytes) with fp8-e4m3 scales
+ * s_rel[N, K/G] -> int8 [N, K].  Replaces gpu_w6_decode, src/ffi.rs:121 / csrc/h3.cu:40-46. */
+int gpu_w6_decode(const void* q, const void* s_rel, void* out, int64_t N, int K, int G, void* stream);
+
+/* ---------------------------------------------------------------------------------------------------------------
+ * Additions with no counterpart in the reference.
+ * ------------------------------------------------------------------------------------------------------------- */
+
+/* The int32 accumulators of gpu_int8_gemm, before the epilogue: acc[M,N] = A . W^T.  For bit-exact checks. */
+int gpu_int8_gemm_acc(const int8_t* A, const int8_t* W, int32_t* acc, int64_t M, int64_t N, int64_t K, void* stream);
+
+/* Test and tuning hook: force the GEMM tile configuration (0 = 256x256, 1 = 128x128, 2 = 64x64, -1 = automatic). */
+int gpu_int8_gemm_force_config(int cfg);
+
+/* Writes, for each of the 64 lanes and 16 accumulator registers of one v_mfma_i32_32x32x32_i8, the (row of src0,
+ * row of src1) pair that the register holds, as out[lane*16 + r] = i*32 + j.  A start-up self check of the operand
+ * layout the GEMM kernels assume; out is int32 [1024]. */
+int gpu_mfma_layout_probe(int32_t* out, void* stream);
+
+/* Library build tag (a static string). */
+const char* gpu_kernels_build_info(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GPU_API_H */

@@ -1,0 +1,335 @@
+"""Parity of the HIP kernels with the CPU oracle, through the C ABI, on a real MI355X.
+
+Bars: int8 codes, per-row scales and int32 accumulators bit-exact; bf16/f16/f32 outputs bit-exact against the oracle's
+fused-multiply-add epilogue and within one unit in the last place of the output type of its unfused form.
+"""
+import hashlib
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oracle import BF16, F16, F32
+from conftest import ROOT, pkg
+
+pytestmark = pytest.mark.gpu
+
+ffi = pkg("ffi")
+ql = pkg("qlinear")
+synth = pkg("synth")
+DEV = "cuda:0"
+TDT = {BF16: torch.bfloat16, F16: torch.float16, F32: torch.float32}
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+def dev_bits(bits, dt):
+    """numpy array (uint16 bits for bf16/f16, float32 for f32) -> CUDA tensor of that dtype."""
+    if dt == F32:
+        return torch.from_numpy(np.ascontiguousarray(bits, dtype=np.float32)).to(DEV)
+    return torch.from_numpy(np.ascontiguousarray(bits).view(np.int16)).to(DEV).view(TDT[dt])
+
+
+def host_bits(t):
+    if t.dtype == torch.float32:
+        return t.cpu().numpy()
+    return t.view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+def ulp_close(a_bits, b_bits, dt):
+    a = oracle.to_f32(a_bits, dt).astype(np.float64)
+    b = oracle.to_f32(b_bits, dt).astype(np.float64)
+    ulp = {BF16: 2.0 ** -7, F16: 2.0 ** -10, F32: 2.0 ** -23}[dt]
+    return (np.abs(a - b) <= ulp * np.maximum(np.abs(a), np.abs(b)) + 1e-30).all()
+
+
+# ------------------------------------------------------------------------------------------------ MFMA layout
+def test_mfma_operand_layout_is_what_the_gemm_assumes():
+    out = torch.zeros(1024, dtype=torch.int32, device=DEV)
+    ffi.k("gpu_mfma_layout_probe", out.data_ptr(), 0)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy().reshape(64, 16)
+    lane = np.arange(64)[:, None]
+    r = np.arange(16)[None, :]
+    i = 8 * (r // 4) + 4 * (lane // 32) + (r % 4)
+    j = lane % 32 + 0 * r
+    want = i * 32 + j
+    if not np.array_equal(got, want):
+        say("probe (i,j) for lane 0:", [(int(v) // 32, int(v) % 32) for v in got[0]])
+        say("probe (i,j) for lane 1:", [(int(v) // 32, int(v) % 32) for v in got[1]])
+        say("probe (i,j) for lane 32:", [(int(v) // 32, int(v) % 32) for v in got[32]])
+    assert np.array_equal(got, want)
+
+
+# ------------------------------------------------------------------------------------------------ quantizers
+QUANT_CASES = [
+    # (M, K, rotate, kind)
+    (256, 1024, 0, "normal"), (7, 256, 1, "normal"), (5, 256, 0, "t3"), (33, 1024, 256, "t3"), (3, 640, 0, "normal"),
+    (9, 640, 64, "normal"), (4, 384, 128, "t3"), (130, 3072, 1, "t3"), (66, 3072, 128, "t3"), (5, 4096, 1, "normal"),
+    (3, 5120, 1, "t3"), (2, 12288, 1, "t3"), (2, 12288, 128, "t3"), (1, 13824, 0, "normal"), (1, 32768, 1, "normal"),
+    (2, 16384, 64, "normal"), (1, 6144, 1, "t3"),
+]
+
+
+@pytest.mark.parametrize("M,K,rotate,kind", QUANT_CASES)
+def test_quant_rows_bf16_bit_exact(M, K, rotate, kind):
+    say("quant_rows bf16", M, K, rotate, kind)
+    xb = synth.bf16_bits(synth.activations(100 + K + rotate, M, K, kind, (3, K - 1)))
+    rc, q, s = oracle.quant_rows(BF16, xb, K, rotate)
+    assert rc == 0
+    qd, sd = ql.quant_rows(dev_bits(xb, BF16), rotate)
+    torch.cuda.synchronize()
+    assert np.array_equal(sd.cpu().numpy().view(np.uint32), s.view(np.uint32))
+    assert np.array_equal(qd.cpu().numpy(), q)
+
+
+@pytest.mark.parametrize("M,K,rotate", [(5, 256, 0), (4, 1024, 1), (3, 2304, 64), (2, 8192, 1), (3, 512, 128)])
+def test_quant_rows_f32_bit_exact(M, K, rotate):
+    say("quant_rows f32", M, K, rotate)
+    x = synth.activations(200 + K, M, K, "t3")
+    rc, q, s = oracle.quant_rows(F32, x, K, rotate)
+    assert rc == 0
+    qd, sd = ql.quant_rows(dev(x), rotate)
+    torch.cuda.synchronize()
+    assert np.array_equal(sd.cpu().numpy().view(np.uint32), s.view(np.uint32))
+    assert np.array_equal(qd.cpu().numpy(), q)
+
+
+def test_quant_rows_special_rows_and_stride():
+    K = 512
+    rows = np.zeros((8, K), np.float32)
+    rows[1, 7] = 20.0; rows[1, 9] = -20.0; rows[1, 11] = 10.0
+    rows[2, 0] = np.inf; rows[2, 1] = -np.inf; rows[2, 2] = 1.0
+    rows[3, 0] = np.nan; rows[3, 1] = 2.0; rows[3, 2] = -1.0
+    rows[4, :] = 1e-35
+    rows[5, 0] = 131.0; rows[5, 1] = -131.0                      # a +-127.5 tie row if one exists for this amax
+    for A in range(128, 256):                                    # find an amax whose quotient rounds to 127.5
+        a = np.float32(A)
+        st = oracle.bf16_to_f32(oracle.bf16_bits(np.array([a * np.float32(1 / 127)])))[0]
+        if oracle.bf16_to_f32(oracle.bf16_bits(np.array([a / st], np.float32)))[0] == np.float32(127.5):
+            rows[5, 0] = a; rows[5, 1] = -a
+            break
+    rows[6] = synth.normal(9, 1, K) * np.float32(3e37)           # near the top of the range
+    rows[7] = synth.normal(9, 2, K) * np.float32(1e-30)
+    xb = oracle.bf16_bits(rows)
+    for rotate in (0, 1):
+        rc, q, s = oracle.quant_rows(BF16, xb, K, rotate)
+        qd, sd = ql.quant_rows(dev_bits(xb, BF16), rotate)
+        torch.cuda.synchronize()
+        assert np.array_equal(sd.cpu().numpy().view(np.uint32), s.view(np.uint32)), rotate
+        assert np.array_equal(qd.cpu().numpy(), q), rotate
+        if rotate == 0:
+            assert q[5, 0] == 127 and q[5, 1] == -128
+    # rows that are a window of a wider buffer (x_stride > K), as the SwiGLU call sites read them (src/dit.rs:605)
+    wide = synth.bf16_bits(synth.activations(10, 6, 3 * K, "normal"))
+    rc, q, s = oracle.quant_rows(BF16, wide, K, 1, x_stride=3 * K)
+    xd = dev_bits(wide, BF16)
+    qd, sd = ql.quant_rows(xd, 1, K=K)
+    torch.cuda.synchronize()
+    assert np.array_equal(qd.cpu().numpy(), q) and np.array_equal(sd.cpu().numpy(), s)
+
+
+@pytest.mark.parametrize("M,K,rotate", [(8, 640, 0), (70, 640, 64), (9, 1280, 256), (5, 2560, 256), (3, 5120, 64), (2, 320, 64)])
+def test_sd_quant_rows_bit_exact(M, K, rotate):
+    say("sd_quant_rows", M, K, rotate)
+    xb = synth.f16_bits(synth.activations(300 + K, M, K, "normal", (5,)))
+    xb[0, :] = 0
+    rc, q, s = oracle.sd_quant_rows(xb, K, rotate)
+    assert rc == 0
+    qd, sd = ql.sd_quant_rows(dev_bits(xb, F16), rotate)
+    torch.cuda.synchronize()
+    assert np.array_equal(sd.cpu().numpy().view(np.uint32), s.view(np.uint32))
+    assert np.array_equal(qd.cpu().numpy(), q)
+
+
+def test_rotate_rows_f32_bit_exact():
+    x = synth.activations(400, 6, 3 * 1024, "t3")
+    rc, out = oracle.rotate_rows_f32(x, 1024, x_stride=3 * 1024)
+    got = ql.rotate_rows_f32(dev(x), K=1024)
+    torch.cuda.synchronize()
+    assert np.array_equal(got.cpu().numpy().view(np.uint32), out.view(np.uint32))
+
+
+def test_rotated_quant_golden_fixture():
+    g = json.load(open(os.path.join(ROOT, "tests", "golden", "rotated_quant.json")))
+    xb = synth.bf16_bits(synth.activations(11, 8, 1024, "t3"))
+    assert hashlib.sha256(xb.tobytes()).hexdigest() == g["x_sha256"]
+    for grp in (64, 128, 256):
+        qd, sd = ql.quant_rows(dev_bits(xb, BF16), grp)
+        torch.cuda.synchronize()
+        q = qd.cpu().numpy()
+        s = sd.cpu().numpy().view(np.uint32)
+        assert hashlib.sha256(q.tobytes()).hexdigest() == g["q_g%d_sha256" % grp]
+        assert hashlib.sha256(s.tobytes()).hexdigest() == g["xs_bits_g%d_sha256" % grp]
+        assert q.reshape(-1)[::g["stride"]].tolist() == g["q_g%d_sample" % grp]
+
+
+# ------------------------------------------------------------------------------------------------ GEMM
+def rand_i8(seed, stream, M, K, lo=-128, hi=127):
+    return synth.randint(seed, stream, M * K, lo, hi).astype(np.int8).reshape(M, K)
+
+
+ACC_CASES = [(1, 96, 256), (3, 32, 16), (64, 64, 64), (65, 72, 48), (100, 104, 320), (130, 260, 80), (257, 96, 3072),
+             (300, 520, 192), (33, 8, 1024)]
+
+
+@pytest.mark.parametrize("cfg", [2, 1, 0])
+@pytest.mark.parametrize("M,N,K", ACC_CASES)
+def test_int8_gemm_acc_bit_exact(M, N, K, cfg):
+    say("gemm_acc", M, N, K, "cfg", cfg)
+    A = rand_i8(1, 500 + M, M, K)
+    W = rand_i8(1, 600 + N, N, K)
+    A[0, :] = -128
+    W[0, :] = -128                                           # the extreme product, K * 2^14
+    want = oracle.int8_gemm_acc(A, W)
+    ffi.raw("gpu_int8_gemm_force_config", cfg)
+    try:
+        got = ql.int8_gemm_acc(dev(A), dev(W))
+        torch.cuda.synchronize()
+    finally:
+        ffi.raw("gpu_int8_gemm_force_config", -1)
+    assert np.array_equal(got.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("out_dt", [BF16, F16, F32])
+@pytest.mark.parametrize("M,N,K,with_bias", [(37, 96, 256, True), (130, 264, 192, False), (256, 1024, 1024, True)])
+def test_int8_gemm_epilogue(M, N, K, with_bias, out_dt):
+    say("gemm", M, N, K, with_bias, out_dt)
+    A = rand_i8(2, 1, M, K, -127, 127)
+    W = rand_i8(2, 2, N, K, -127, 127)
+    xs = synth.uniform(2, 3, M, 0.005, 0.2)
+    ws = synth.uniform(2, 4, N, 1e-3, 1e-2)
+    tob = {BF16: oracle.bf16_bits, F16: oracle.f16_bits, F32: lambda a: a.astype(np.float32)}[out_dt]
+    bias = tob(synth.normal(2, 5, N) * np.float32(0.02)) if with_bias else None
+    want = oracle.int8_gemm(A, W, xs, ws, bias, out_dt, fma=1)
+    loose = oracle.int8_gemm(A, W, xs, ws, bias, out_dt, fma=0)
+    for cfg in (-1, 0, 1, 2):
+        ffi.raw("gpu_int8_gemm_force_config", cfg)
+        try:
+            got = ql.int8_gemm(dev(A), dev(W), dev(xs), dev(ws), None if bias is None else dev_bits(bias, out_dt), TDT[out_dt])
+            torch.cuda.synchronize()
+        finally:
+            ffi.raw("gpu_int8_gemm_force_config", -1)
+        gb = host_bits(got)
+        assert np.array_equal(gb.view(np.uint32 if out_dt == F32 else np.uint16), want.view(np.uint32 if out_dt == F32 else np.uint16)), cfg
+        assert ulp_close(gb, loose, out_dt)
+
+
+@pytest.mark.parametrize("out_dt", [BF16, F16, F32])
+def test_int8_gemm_residual_in_place(out_dt):
+    M, N, K = 150, 136, 256
+    A = rand_i8(3, 1, M, K, -127, 127)
+    W = rand_i8(3, 2, N, K, -127, 127)
+    xs = synth.uniform(3, 3, M, 0.005, 0.2)
+    ws = synth.uniform(3, 4, N, 1e-3, 1e-2)
+    tob = {BF16: oracle.bf16_bits, F16: oracle.f16_bits, F32: lambda a: a.astype(np.float32)}[out_dt]
+    bias = tob(synth.normal(3, 5, N) * np.float32(0.02))
+    rscale = tob(synth.normal(3, 6, N))
+    resid = tob(synth.normal(3, 7, M * N).reshape(M, N))
+    want = oracle.int8_gemm_residual(A, W, xs, ws, bias, rscale, resid, out_dt, fma=1)
+    loose = oracle.int8_gemm_residual(A, W, xs, ws, bias, rscale, resid, out_dt, fma=0)
+    x = dev_bits(resid, out_dt)                      # D aliases resid, as in src/dit.rs:592
+    ql.int8_gemm_residual(dev(A), dev(W), dev(xs), dev(ws), dev_bits(bias, out_dt), dev_bits(rscale, out_dt), x, D=x)
+    torch.cuda.synchronize()
+    gb = host_bits(x)
+    view = np.uint32 if out_dt == F32 else np.uint16
+    assert np.array_equal(gb.view(view), want.view(view))
+    # two roundings: the unfused form can differ by one ulp of z scaled by rscale, plus one ulp of the result
+    a = oracle.to_f32(gb, out_dt).astype(np.float64)
+    b = oracle.to_f32(loose, out_dt).astype(np.float64)
+    ulp = {BF16: 2.0 ** -7, F16: 2.0 ** -10, F32: 2.0 ** -23}[out_dt]
+    assert (np.abs(a - b) <= 4 * ulp * (np.abs(a) + np.abs(b) + 1.0)).all()
+    # without bias, out of place
+    want2 = oracle.int8_gemm_residual(A, W, xs, ws, None, rscale, resid, out_dt, fma=1)
+    got2 = ql.int8_gemm_residual(dev(A), dev(W), dev(xs), dev(ws), None, dev_bits(rscale, out_dt), dev_bits(resid, out_dt))
+    torch.cuda.synchronize()
+    assert np.array_equal(host_bits(got2).view(view), want2.view(view))
+
+
+def test_config0_end_to_end_matches_golden_fixture():
+    g = json.load(open(os.path.join(ROOT, "tests", "golden", "config0_w8a8.json")))
+    c = synth.config0(0)
+    dig = lambda a: hashlib.sha256(np.ascontiguousarray(a).tobytes()).hexdigest()
+    assert dig(c["x"]) == g["x_sha256"] and dig(c["W"]) == g["W_sha256"]
+    x = dev_bits(c["x"], BF16)
+    W, ws, bias = dev(c["W"]), dev(c["ws"]), dev_bits(c["bias"], BF16)
+    q, xs = ql.quant_rows(x, 0)
+    acc = ql.int8_gemm_acc(q, W)
+    d = ql.int8_gemm(q, W, xs, ws, bias, torch.bfloat16)
+    d2 = ql.linear_w8a8(x, W, ws, bias, rotate=0)
+    torch.cuda.synchronize()
+    s = g["stride"]
+    assert dig(q.cpu().numpy()) == g["q_sha256"] and q.cpu().numpy().reshape(-1)[::s].tolist() == g["q_sample"]
+    assert dig(xs.cpu().numpy().view(np.uint32)) == g["xs_bits_sha256"]
+    assert dig(acc.cpu().numpy()) == g["acc_sha256"] and acc.cpu().numpy().reshape(-1)[::s].tolist() == g["acc_sample"]
+    db = host_bits(d)
+    assert dig(db) == g["d_fma_bits_sha256"] and db.reshape(-1)[::s].tolist() == g["d_fma_bits_sample"]
+    assert np.array_equal(host_bits(d2), db)
+    nofma = np.array(g["d_nofma_bits_sample"], np.uint16)
+    assert ulp_close(db.reshape(-1)[::s], nofma, BF16)
+
+
+# ------------------------------------------------------------------------------------------------ W6
+def test_w6_decode_exhaustive_and_random():
+    K, G = 64, 16
+    codes = np.arange(64, dtype=np.uint8)[None, :].repeat(256, axis=0)
+    wq = oracle.w6_pack_planes(codes)
+    s_rel = np.arange(256, dtype=np.uint8)[:, None].repeat(K // G, axis=1)
+    rc, want = oracle.w6_decode(wq, s_rel, 256, K, G)
+    got = ql.w6_decode(dev(wq), dev(s_rel), 256, K, G)
+    torch.cuda.synchronize()
+    assert np.array_equal(got.cpu().numpy(), want)
+    N, K, G = 77, 5376, 32
+    codes = (synth.w6_codes(6, N, K).astype(np.int16) + 32).astype(np.uint8)
+    wq = oracle.w6_pack_planes(codes)
+    s_rel = synth.w6_srel_bytes(6, N, K, G)
+    rc, want = oracle.w6_decode(wq, s_rel, N, K, G)
+    got = ql.w6_decode(dev(wq), dev(s_rel), N, K, G)
+    torch.cuda.synchronize()
+    assert np.array_equal(got.cpu().numpy(), want)
+
+
+# ------------------------------------------------------------------------------------------------ full-size shapes
+FULL = [  # (name, M, K, N, rotate, kind)
+    ("dit mlp up", 4608, 3072, 12288, 128, "t3"),
+    ("dit mlp down", 4608, 12288, 3072, 1, "t3"),
+    ("skinny gate+up", 256, 4096, 24576, 128, "normal"),
+    ("skinny down", 256, 12288, 4096, 1, "normal"),
+    ("sdxl geglu", 8192, 640, 5120, 0, "normal"),
+]
+
+
+@pytest.mark.parametrize("name,M,K,N,rotate,kind", FULL)
+def test_full_size_linear_rows_against_oracle(name, M, K, N, rotate, kind):
+    """At the benchmark sizes the oracle is too slow for the whole output: check the quantizer on every row, the GEMM on
+    a spread of rows (bit-exact), and a checksum identity over the whole int32 result: sum_n acc[m,n] = A[m,:] . sum_n W[n,:]."""
+    say("full size", name, M, K, N, rotate)
+    xb = synth.bf16_bits(synth.activations(7, M, K, kind, synth.outlier_columns(7, K, 0.001)))
+    W, ws, bias32 = synth.w8_weights(7, N, K)
+    bias = synth.bf16_bits(bias32)
+    rc, q, xs = oracle.quant_rows(BF16, xb, K, rotate)
+    assert rc == 0
+    x = dev_bits(xb, BF16)
+    Wd, wsd, bd = dev(W), dev(ws), dev_bits(bias, BF16)
+    qd, xsd = ql.quant_rows(x, rotate)
+    d = ql.int8_gemm(qd, Wd, xsd, wsd, bd, torch.bfloat16)
+    acc = ql.int8_gemm_acc(qd, Wd)
+    torch.cuda.synchronize()
+    assert np.array_equal(qd.cpu().numpy(), q) and np.array_equal(xsd.cpu().numpy(), xs)
+    rows = sorted(set([0, 1, 31, 32, 127, 128, 255, M // 2, M - 129, M - 2, M - 1]))
+    want = oracle.int8_gemm(q[rows], W, xs[rows], ws, bias, BF16, fma=1)
+    got = host_bits(d[torch.tensor(rows, device=DEV)])
+    assert np.array_equal(got, want)
+    colsum = W.astype(np.int64).sum(axis=0)
+    want_rowsum = q.astype(np.int64) @ colsum
+    got_rowsum = acc.to(torch.int64).sum(dim=1).cpu().numpy()
+    assert np.array_equal(got_rowsum, want_rowsum)

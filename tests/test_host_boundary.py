@@ -1,0 +1,117 @@
+"""CPU-only checks of the drop-in boundary: the library loads, exports every symbol the header declares, and refuses bad
+arguments with the reference's return codes before touching the GPU."""
+import ctypes
+import json
+import os
+import re
+
+import numpy as np
+import pytest
+
+import oracle
+from conftest import ROOT, pkg
+
+ffi = pkg("ffi")
+
+
+def header_functions():
+    text = open(os.path.join(ROOT, "include", "gpu_api.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return re.findall(r"\b(gpu_[a-z0-9_]+)\s*\(", text)
+
+
+def test_library_exports_every_declared_symbol():
+    names = header_functions()
+    assert {"gpu_quant_rows", "gpu_quant_rows_b", "gpu_rotate_rows_f32", "gpu_sd_quant_rows", "gpu_int8_gemm",
+            "gpu_int8_gemm_residual", "gpu_w6_decode"} <= set(names)
+    lib = ctypes.CDLL(ffi.LIB_PATH)
+    for n in names:
+        assert hasattr(lib, n), n
+    for n in ffi.SIGNATURES:
+        assert n in names, "ffi.py binds %s, which the header does not declare" % n
+    assert "gfx950" in ffi.build_info()
+
+
+def test_header_constants_match_reference_codes():
+    text = open(os.path.join(ROOT, "include", "gpu_api.h")).read()
+    assert re.search(r"DT_F32 = 0, DT_F16 = 1, DT_BF16 = 2", text)
+    assert (ffi.PRO_PLAIN, ffi.PRO_RMS, ffi.PRO_GATE, ffi.PRO_SWIGLU, ffi.PRO_ADALN, ffi.PRO_SITU_FAST) == (0, 1, 2, 3, 7, 13)
+    for name, val in (("PRO_LN_MOD", 9), ("PRO_LN_AFFINE", 10), ("PRO_GELU_TANH", 11), ("PRO_LN_AFFINE_SILU", 12)):
+        assert re.search(r"%s = %d\b" % (name, val), text)
+
+
+def q(dtype=2, pro=0, K=256, rotate=0, M=4):
+    return ffi.raw("gpu_quant_rows", dtype, pro, 0, K, 0, 0, 0, 0, 0.0, 0, 0, 0, 0, M, K, rotate, 0)
+
+
+def test_quant_rows_refusals_match_reference_order():
+    assert q(K=200) == -1                       # csrc/kernels.cu:275
+    assert q(K=320, rotate=1) == -1
+    assert q(K=192, rotate=128) == -1
+    assert q(dtype=1) == -4                     # :297
+    assert q(dtype=1, pro=99) == -4             # dtype is looked at before the prologue id
+    assert q(pro=99) == -3 and q(pro=12) == -3  # :292 (LN_AFFINE_SILU is not in the quantizer's list)
+    assert q(K=32768 + 256) == -2               # :265
+    assert q(pro=ffi.PRO_RMS) == -30            # known prologue, not built here
+    assert q(M=0) == 0
+    # the oracle agrees on the shared codes
+    x = np.zeros((1, 512), np.uint16)
+    assert oracle.quant_rows(oracle.BF16, x, 200, 0)[0] == -1
+    assert oracle.quant_rows(oracle.F16, x, 256, 0)[0] == -4
+
+
+def test_other_entry_point_refusals():
+    assert ffi.raw("gpu_quant_rows_b", 2, ffi.PRO_LN_MOD, 0, 300, 0, 0, 0.0, 0, 0, 0, 0, 1, 300, 0, 0) == -1
+    assert ffi.raw("gpu_quant_rows_b", 0, ffi.PRO_LN_MOD, 0, 256, 0, 0, 0.0, 0, 0, 0, 0, 1, 256, 0, 0) == -4
+    assert ffi.raw("gpu_quant_rows_b", 2, ffi.PRO_RMS, 0, 256, 0, 0, 0.0, 0, 0, 0, 0, 1, 256, 0, 0) == -3
+    assert ffi.raw("gpu_rotate_rows_f32", ffi.PRO_PLAIN, 0, 320, 0, 0, 0.0, 0, 1, 320, 0) == -1
+    assert ffi.raw("gpu_rotate_rows_f32", ffi.PRO_GATE, 0, 256, 0, 0, 0.0, 0, 1, 256, 0) == -3
+    assert ffi.raw("gpu_sd_quant_rows", 0, 640, 0, 0, 1, 640, 128, 0) == -1     # csrc/sd.cu:600
+    assert ffi.raw("gpu_sd_quant_rows", 0, 640, 0, 0, 1, 640, 256, 0) == -1
+    assert ffi.raw("gpu_w6_decode", 0, 0, 0, 4, 48, 32, 0) == -1                # csrc/h3.cu:41
+    assert ffi.raw("gpu_w6_decode", 0, 0, 0, 4, 64, 8, 0) == -1
+    assert ffi.raw("gpu_w6_decode", 0, 0, 0, 0, 64, 32, 0) == 0
+
+
+def test_gemm_refusals_and_empty_shapes():
+    g = lambda M, N, K, dt=2: ffi.raw("gpu_int8_gemm", 0, 0, 0, 0, 0, 0, M, N, K, dt, 0)
+    assert g(0, 8, 16) == 0 and g(8, 0, 16) == 0 and g(8, 8, 0) == 0       # csrc/vendor/cutlass_gemm_int8.cu:377
+    assert g(8, 8, 16, dt=5) == -200                                         # csrc/gemm.cu:126
+    assert g(8, 8, 24) == -200
+    r = lambda M, N, K, rs=1, res=1, dt=2: ffi.raw("gpu_int8_gemm_residual", 0, 0, 0, 0, 0, rs, res, 0, M, N, K, dt, 0)
+    assert r(0, 8, 16) == 0 and r(8, 0, 16) == 0                             # :353
+    assert r(8, 8, 0) == -201                                                # :355, csrc/gemm.cu:137
+    assert r(8, 8, 16, rs=0) == -201 and r(8, 8, 16, res=0) == -201          # :357
+    assert r(8, 8, 16, dt=9) == -201
+
+
+def test_ok_and_k_raise_like_the_reference():
+    ffi.ok(0, "anything")
+    with pytest.raises(ffi.KernelError, match="gpu_quant_rows failed with code -1"):
+        ffi.k("gpu_quant_rows", 2, 0, 0, 200, 0, 0, 0, 0, 0.0, 0, 0, 0, 0, 4, 200, 0, 0)
+    with pytest.raises(ffi.KernelError, match="x failed: "):
+        ffi.ok(1, "x")
+
+
+def test_oracle_reproduces_golden_fixtures(synth):
+    import hashlib
+    dig = lambda a: hashlib.sha256(np.ascontiguousarray(a).tobytes()).hexdigest()
+    g = json.load(open(os.path.join(ROOT, "tests", "golden", "config0_w8a8.json")))
+    c = synth.config0(0)
+    assert dig(c["x"]) == g["x_sha256"] and dig(c["W"]) == g["W_sha256"] and dig(c["ws"]) == g["ws_sha256"]
+    rc, qq, xs = oracle.quant_rows(oracle.BF16, c["x"], c["K"], 0)
+    acc = oracle.int8_gemm_acc(qq, c["W"])
+    assert dig(qq) == g["q_sha256"] and dig(xs.view(np.uint32)) == g["xs_bits_sha256"] and dig(acc) == g["acc_sha256"]
+    assert qq.reshape(-1)[::g["stride"]].tolist() == g["q_sample"]
+    d = oracle.epilogue(acc, xs, c["ws"], c["bias"], oracle.BF16, fma=1)
+    assert dig(d) == g["d_fma_bits_sha256"] and d.reshape(-1)[::g["stride"]].tolist() == g["d_fma_bits_sample"]
+    # the plain formula of the config text (scale = absmax/127, RNE, float product) lands within 1 code of the bf16 path
+    x = synth.bf16_to_f32(c["x"])
+    plain = np.clip(np.rint(x / (np.abs(x).max(1, keepdims=True) / np.float32(127))), -127, 127)
+    assert np.abs(plain - qq).max() <= 1
+    r = json.load(open(os.path.join(ROOT, "tests", "golden", "rotated_quant.json")))
+    xr = synth.bf16_bits(synth.activations(11, 8, 1024, "t3"))
+    assert dig(xr) == r["x_sha256"]
+    for grp in (64, 128, 256):
+        rc, q2, s2 = oracle.quant_rows(oracle.BF16, xr, 1024, grp)
+        assert dig(q2) == r["q_g%d_sha256" % grp] and dig(s2.view(np.uint32)) == r["xs_bits_g%d_sha256" % grp]
