@@ -25,7 +25,12 @@ __device__ __forceinline__ uint32_t f2u(float f) { return __builtin_bit_cast(uin
 __device__ __forceinline__ float bf16_to_f(uint16_t b) { return u2f((uint32_t)b << 16); }
 __device__ __forceinline__ uint16_t f_to_bf16(float v) { return __builtin_bit_cast(uint16_t, (__bf16)v); }
 __device__ __forceinline__ float f16_to_f(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
-__device__ __forceinline__ uint16_t f_to_f16(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
+// The empty asm keeps the compiler from folding a preceding fp32 fma into v_fma_mixlo_f16, which rounds the exact
+// fma result to f16 once; the reference rounds to fp32 first and converts afterwards, and ties differ between the two.
+__device__ __forceinline__ uint16_t f_to_f16(float v) {
+    asm("" : "+v"(v));
+    return __builtin_bit_cast(uint16_t, (_Float16)v);
+}
 
 // Round a float to the precision of the dtype code and widen back (rnd<T>, csrc/common.cuh:25-28).
 template <int DT> __device__ __forceinline__ float rnd_dt(float v) {

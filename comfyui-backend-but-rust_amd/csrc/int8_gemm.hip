@@ -8,6 +8,9 @@
 // stores 8-byte (bf16/f16) or 16-byte (f32) vectors straight from the accumulators.
 #include "common.hpp"
 
+// Nothing is scheduled across this point: it pins hand-interleaved instruction orders and keeps live ranges short.
+#define SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
+
 namespace {
 
 enum { EPI_PLAIN = 0, EPI_RESID = 1, EPI_ACC = 2 };
@@ -101,6 +104,260 @@ __device__ __forceinline__ float epi_value(int acc, float xs, float ws, float b,
     const float t = __builtin_fmaf((float)acc * xs, ws, b);
     if (EPI == EPI_RESID) return __builtin_fmaf(rnd_dt<OUT_DT>(t), rs, res);
     return t;
+}
+
+// Epilogue of one wave tile whose origin is (mb, nb).  acc[in][im][4*rb + j] is the accumulator of
+// (m = mb + 32*im + lane%32, n = nb + 32*in + 8*rb + 4*(lane/32) + j): four consecutive n per lane and register group.
+template <int TM, int TN, int OUT_DT, int EPI>
+__device__ __forceinline__ void epilogue_store(const GemmArgs& p, v16i (&acc)[TN][TM], int mb, int nb, int lane, bool vec_ok) {
+    const int frow = lane & 31, fhalf = lane >> 5;
+#pragma unroll
+    for (int im = 0; im < TM; ++im) {
+        const int m = mb + im * 32 + frow;
+        if (m >= p.M) continue;
+        const float xs = EPI == EPI_ACC ? 0.f : p.xs[m];
+#pragma unroll
+        for (int in = 0; in < TN; ++in) {
+#pragma unroll
+            for (int rb = 0; rb < 4; ++rb) {
+                const int n = nb + in * 32 + rb * 8 + fhalf * 4;
+                if (n >= p.N) continue;
+                const int64_t o = (int64_t)m * p.N + n;
+                if (EPI == EPI_ACC) {
+                    int* d = (int*)p.D + o;
+                    if (vec_ok) {
+                        *reinterpret_cast<v4i*>(d) = v4i{acc[in][im][4 * rb], acc[in][im][4 * rb + 1], acc[in][im][4 * rb + 2], acc[in][im][4 * rb + 3]};
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) if (n + j < p.N) d[j] = acc[in][im][4 * rb + j];
+                    }
+                    continue;
+                }
+                float ws[4], b[4] = {0.f, 0.f, 0.f, 0.f}, rs[4] = {0.f, 0.f, 0.f, 0.f}, res[4] = {0.f, 0.f, 0.f, 0.f}, out[4];
+                if (vec_ok) {
+                    const float4 w4 = *reinterpret_cast<const float4*>(p.ws + n);
+                    ws[0] = w4.x; ws[1] = w4.y; ws[2] = w4.z; ws[3] = w4.w;
+                    if (p.bias) load4<OUT_DT>(p.bias, n, b);
+                    if (EPI == EPI_RESID) { load4<OUT_DT>(p.rscale, n, rs); load4<OUT_DT>(p.resid, o, res); }
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        if (n + j >= p.N) { ws[j] = 0.f; continue; }
+                        ws[j] = p.ws[n + j];
+                        if (p.bias) b[j] = ld_dt<OUT_DT>(p.bias, n + j);
+                        if (EPI == EPI_RESID) { rs[j] = ld_dt<OUT_DT>(p.rscale, n + j); res[j] = ld_dt<OUT_DT>(p.resid, o + j); }
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) out[j] = epi_value<OUT_DT, EPI>(acc[in][im][4 * rb + j], xs, ws[j], b[j], rs[j], res[j]);
+                if (vec_ok) {
+                    store4<OUT_DT>(p.D, o, out);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) if (n + j < p.N) st_dt<OUT_DT>(p.D, o + j, out[j]);
+                }
+            }
+        }
+    }
+}
+
+// Coalesced epilogue: the accumulator layout (lane = one m, four consecutive n per register group) would store 16-byte
+// pieces scattered over 32 rows per instruction.  Instead each wave rounds its values to the output type, passes a
+// 32-row piece of its tile through a private LDS region (XOR-swizzled 16-byte chunks, conflict-free both ways) and
+// writes whole rows: 16 bytes per lane, consecutive lanes on consecutive addresses.  For the residual form the LDS
+// holds z = Out(acc*xs*ws + bias), exactly the intermediate the reference rounds, and fma(z, rscale, resid) is applied
+// on the way out.  Needs row starts of D (and resid) 16-byte aligned; the caller falls back to epilogue_store otherwise.
+template <int TM, int TN, int OUT_DT, int EPI, int PW = TN * 32>
+__device__ __forceinline__ void epilogue_shuffle(const GemmArgs& p, v16i (&acc)[TN][TM], int mb, int nb, int lane, uint8_t* wl) {
+    // a piece is 32 rows x PW columns of the wave tile: PW*SZ bytes per LDS row, 32*PW*SZ bytes per wave
+    constexpr int SZ = (EPI == EPI_ACC || OUT_DT == DT_F32) ? 4 : 2;
+    constexpr int WTN = TN * 32, NP = WTN / PW, TNP = PW / 32;
+    constexpr int ROWB = PW * SZ, CPRW = ROWB / 16, MASK = CPRW - 1;
+    constexpr int EPC = 16 / SZ;                  // elements per 16-byte chunk
+    constexpr int RPI = 64 / CPRW, PASSES = 32 / RPI;
+    static_assert(PW % 32 == 0 && WTN % PW == 0, "piece width");
+    static_assert((CPRW & MASK) == 0 && CPRW <= 64 && CPRW >= 2, "chunks per row must be a power of two");
+    // Everything below is a function of the lane number only, so in a persistent kernel the compiler would hoist dozens
+    // of addresses out of the tile loop, keep them live across the K loop and spill them; the reloads then sit between
+    // the stores, each behind a full memory wait.  Making the lane number opaque here keeps the address arithmetic local.
+    asm volatile("" : "+v"(lane));
+    const int frow = lane & 31, fhalf = lane >> 5;
+
+    // per-lane column constants, loaded once and in one batch (no branches between the loads, so a single wait covers
+    // them): ws and the raw bias words for the 4 n of every (in, rb).  Columns past N read the last valid vector.
+    constexpr int BW = SZ == 4 ? 4 : 2;            // 32-bit words holding 4 bias values
+    float wsr[TN][4][4];
+    uint32_t braw[TN][4][BW];
+    if (EPI != EPI_ACC) {
+#pragma unroll
+        for (int in = 0; in < TN; ++in)
+#pragma unroll
+            for (int rb = 0; rb < 4; ++rb) {
+                int n = nb + in * 32 + rb * 8 + fhalf * 4;
+                n = n < p.N ? n : p.N - 4;
+                const float4 w4 = *reinterpret_cast<const float4*>(p.ws + n);
+                wsr[in][rb][0] = w4.x; wsr[in][rb][1] = w4.y; wsr[in][rb][2] = w4.z; wsr[in][rb][3] = w4.w;
+                if (p.bias) {
+                    if (SZ == 4) {
+                        const uint4 b4 = *reinterpret_cast<const uint4*>((const uint8_t*)p.bias + (int64_t)n * 4);
+                        braw[in][rb][0] = b4.x; braw[in][rb][1] = b4.y; braw[in][rb][BW - 2] = b4.z; braw[in][rb][BW - 1] = b4.w;
+                    } else {
+                        const uint2 b2 = *reinterpret_cast<const uint2*>((const uint8_t*)p.bias + (int64_t)n * 2);
+                        braw[in][rb][0] = b2.x; braw[in][rb][1] = b2.y;
+                    }
+                } else {
+#pragma unroll
+                    for (int j = 0; j < BW; ++j) braw[in][rb][j] = 0u;
+                }
+            }
+    }
+    // bias value j of (in, rb) as float: +0.0 for a null bias
+    auto bias_f = [&](int in, int rb, int j) -> float {
+        if (SZ == 4) return u2f(braw[in][rb][j]);
+        const uint32_t w = braw[in][rb][j >> 1];
+        if (OUT_DT == DT_BF16) return (j & 1) ? u2f(w & 0xffff0000u) : u2f(w << 16);
+        return f16_to_f((uint16_t)((j & 1) ? (w >> 16) : (w & 0xffffu)));
+    };
+    const int rrow = lane / CPRW, rc = lane % CPRW;   // read phase: row within a pass, chunk
+
+    // Every global load is issued ahead of the stores that precede its use: the memory counter retires in order, so a
+    // load issued after a store cannot be waited for without also waiting for that store to reach memory.
+    float xsr[TM];
+#pragma unroll
+    for (int im = 0; im < TM; ++im) {
+        const int mrow = mb + im * 32 + frow;
+        xsr[im] = (EPI == EPI_ACC || mrow >= p.M) ? 0.f : p.xs[mrow];
+    }
+    float rs[NP][EPC];
+    if (EPI == EPI_RESID) {
+#pragma unroll
+        for (int np = 0; np < NP; ++np) {
+            const int ncol = nb + np * PW + rc * EPC;
+#pragma unroll
+            for (int h = 0; h < EPC / 4; ++h) {
+                if (ncol < p.N) load4<OUT_DT>(p.rscale, ncol + 4 * h, rs[np] + 4 * h);
+                else { rs[np][4 * h] = 0.f; rs[np][4 * h + 1] = 0.f; rs[np][4 * h + 2] = 0.f; rs[np][4 * h + 3] = 0.f; }
+            }
+        }
+    }
+    // residual rows of piece (im, np), in the read phase's layout
+    auto load_resid = [&](int im, int np, uint4* rv) {
+        const int ncol = nb + np * PW + rc * EPC;
+#pragma unroll
+        for (int t = 0; t < PASSES; ++t) {
+            const int m = mb + im * 32 + t * RPI + rrow;
+            if (m < p.M && ncol < p.N) rv[t] = *reinterpret_cast<const uint4*>((const uint8_t*)p.resid + ((int64_t)m * p.N + ncol) * SZ);
+            else rv[t] = make_uint4(0, 0, 0, 0);
+        }
+    };
+    uint4 rv_next[PASSES];
+    if (EPI == EPI_RESID) load_resid(0, 0, rv_next);
+
+#pragma unroll
+    for (int im = 0; im < TM; ++im) {
+        const float xs = xsr[im];
+#pragma unroll
+        for (int np = 0; np < NP; ++np) {
+            // write phase: row frow of the piece
+#pragma unroll
+            for (int ip = 0; ip < TNP; ++ip)
+#pragma unroll
+                for (int rb = 0; rb < 4; ++rb) {
+                    const int in = np * TNP + ip;
+                    const int byte = (ip * 32 + rb * 8 + fhalf * 4) * SZ;
+                    uint8_t* dst = wl + frow * ROWB + ((((byte >> 4) ^ frow) & MASK) << 4) + (byte & 15);
+                    if (EPI == EPI_ACC) {
+                        *reinterpret_cast<v4i*>(dst) = v4i{acc[in][im][4 * rb], acc[in][im][4 * rb + 1], acc[in][im][4 * rb + 2], acc[in][im][4 * rb + 3]};
+                    } else {
+                        float o[4];
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) o[j] = __builtin_fmaf((float)acc[in][im][4 * rb + j] * xs, wsr[in][rb][j], bias_f(in, rb, j));
+                        if (OUT_DT == DT_F32) {
+                            *reinterpret_cast<float4*>(dst) = make_float4(o[0], o[1], o[2], o[3]);
+                        } else if (OUT_DT == DT_BF16) {
+                            *reinterpret_cast<uint2*>(dst) = make_uint2((uint32_t)f_to_bf16(o[0]) | ((uint32_t)f_to_bf16(o[1]) << 16),
+                                                                        (uint32_t)f_to_bf16(o[2]) | ((uint32_t)f_to_bf16(o[3]) << 16));
+                        } else {
+                            *reinterpret_cast<uint2*>(dst) = make_uint2((uint32_t)f_to_f16(o[0]) | ((uint32_t)f_to_f16(o[1]) << 16),
+                                                                        (uint32_t)f_to_f16(o[2]) | ((uint32_t)f_to_f16(o[3]) << 16));
+                        }
+                    }
+                    SCHED_FENCE();
+                }
+            asm volatile("" ::: "memory");   // the wave's own LDS writes are ordered before its reads by the LDS queue
+            // residual of this piece was requested one piece ago; request the next piece's before this piece's stores
+            uint4 rv[PASSES];
+            if (EPI == EPI_RESID) {
+#pragma unroll
+                for (int t = 0; t < PASSES; ++t) rv[t] = rv_next[t];
+                const int nxt = im * NP + np + 1;
+                if (nxt < TM * NP) load_resid(nxt / NP, nxt % NP, rv_next);
+            }
+            // read phase: whole rows out
+            const int ncol = nb + np * PW + rc * EPC;
+#pragma unroll
+            for (int t = 0; t < PASSES; ++t) {
+                const int r = t * RPI + rrow;
+                const uint4 v = *reinterpret_cast<const uint4*>(wl + r * ROWB + (((rc ^ r) & MASK) << 4));
+                const int m = mb + im * 32 + r;
+                if (m >= p.M || ncol >= p.N) continue;
+                const int64_t o = (int64_t)m * p.N + ncol;
+                if (EPI != EPI_RESID) {
+                    *reinterpret_cast<uint4*>((uint8_t*)p.D + o * SZ) = v;
+                } else {
+                    const uint32_t zw[4] = {v.x, v.y, v.z, v.w}, rw[4] = {rv[t].x, rv[t].y, rv[t].z, rv[t].w};
+                    uint32_t ow[4];
+                    if (OUT_DT == DT_F32) {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) ow[j] = f2u(__builtin_fmaf(u2f(zw[j]), rs[np][j], u2f(rw[j])));
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            float z0, z1, r0, r1;
+                            if (OUT_DT == DT_BF16) {
+                                z0 = u2f(zw[j] << 16); z1 = u2f(zw[j] & 0xffff0000u); r0 = u2f(rw[j] << 16); r1 = u2f(rw[j] & 0xffff0000u);
+                                ow[j] = (uint32_t)f_to_bf16(__builtin_fmaf(z0, rs[np][2 * j], r0)) | ((uint32_t)f_to_bf16(__builtin_fmaf(z1, rs[np][2 * j + 1], r1)) << 16);
+                            } else {
+                                z0 = f16_to_f((uint16_t)(zw[j] & 0xffffu)); z1 = f16_to_f((uint16_t)(zw[j] >> 16));
+                                r0 = f16_to_f((uint16_t)(rw[j] & 0xffffu)); r1 = f16_to_f((uint16_t)(rw[j] >> 16));
+                                ow[j] = (uint32_t)f_to_f16(__builtin_fmaf(z0, rs[np][2 * j], r0)) | ((uint32_t)f_to_f16(__builtin_fmaf(z1, rs[np][2 * j + 1], r1)) << 16);
+                            }
+                        }
+                    }
+                    *reinterpret_cast<uint4*>((uint8_t*)p.D + o * SZ) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+                }
+                SCHED_FENCE();
+            }
+            asm volatile("" ::: "memory");
+        }
+    }
+}
+
+// Chooses the coalesced epilogue when row starts are 16-byte aligned.  Must be called by all waves of the workgroup:
+// it begins with a workgroup barrier because the shuffle reuses the LDS of the K loop.
+template <int OUT_DT, int EPI>
+__host__ __device__ __forceinline__ void epilogue_alignment(const GemmArgs& p, bool& vec_ok, bool& aligned) {
+    constexpr int SZ = (EPI == EPI_ACC || OUT_DT == DT_F32) ? 4 : 2;
+    constexpr uintptr_t V4 = 4 * SZ - 1;   // mask of a 4-element vector of the output type
+    const uintptr_t ptrs = EPI == EPI_ACC ? (uintptr_t)p.D
+                                          : ((uintptr_t)p.D | (uintptr_t)p.bias | (uintptr_t)p.rscale | (uintptr_t)p.resid);
+    vec_ok = (p.N & 3) == 0 && (ptrs & V4) == 0 && (EPI == EPI_ACC || (((uintptr_t)p.ws) & 15) == 0);
+    aligned = vec_ok && (((int64_t)p.N * SZ) & 15) == 0 &&
+              (((uintptr_t)p.D | (uintptr_t)p.resid | (uintptr_t)p.rscale) & 15) == 0;
+}
+
+template <int TM, int TN, int OUT_DT, int EPI>
+__device__ __forceinline__ void epilogue(const GemmArgs& p, v16i (&acc)[TN][TM], int mb, int nb, int lane, int wave, uint8_t* smem) {
+    constexpr int SZ = (EPI == EPI_ACC || OUT_DT == DT_F32) ? 4 : 2;
+    constexpr int PIECE = 32 * TN * 32 * SZ;   // bytes of one wave's 32-row piece
+    bool vec_ok, aligned;
+    epilogue_alignment<OUT_DT, EPI>(p, vec_ok, aligned);
+    if (aligned) {
+        __syncthreads();
+        epilogue_shuffle<TM, TN, OUT_DT, EPI>(p, acc, mb, nb, lane, smem + wave * PIECE);
+    } else {
+        epilogue_store<TM, TN, OUT_DT, EPI>(p, acc, mb, nb, lane, vec_ok);
+    }
 }
 
 template <class C, int OUT_DT, int EPI>
@@ -218,56 +475,521 @@ __global__ void __launch_bounds__(C::NT, C::OCC) int8_gemm_kernel(GemmArgs p) {
         __syncthreads();
     }
 
-    // Epilogue.  acc[in][im][4*rb + j] is (n = nb + 8*rb + 4*fhalf + j, m = mb + frow).
-    const bool vec_ok = (p.N & 3) == 0;
+    static_assert(4 * 32 * C::WTN * 4 <= C::SMEM || C::NT != 256, "epilogue shuffle needs 4 pieces of LDS");
+    epilogue<C::TM, C::TN, OUT_DT, EPI>(p, acc, m0 + wm * C::WTM, n0 + wn * C::WTN, lane, wave, smem);
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// The large-shape kernel: tiles stream global -> LDS with global_load_lds_dwordx4 (no register staging) into a ring of
+// NS stages, and the MFMA loop is software-pipelined by hand: while the 16 (TN*TM) MFMAs of one 32-deep K sub-step
+// issue, the ds_read_b128 fragment loads of the next sub-step and the DMA loads of a tile NS-1 ahead are interleaved
+// between them, pinned in that order with scheduling barriers.
+//
+// One 64-lane DMA instruction fills 1 KB of LDS (lane l -> bytes 16*l..16*l+15): 16 tile rows of 64 bytes.  The XOR
+// swizzle is applied on the global side: lane l fetches chunk (l%4) ^ swizzle(row) of row l/4, so the chunk lands in its
+// swizzled slot.  Requires K % 64 == 0.
+// ---------------------------------------------------------------------------------------------------------------
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* glb_ptr_t;
+
+
+template <int N> __device__ __forceinline__ void wait_vmcnt() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+// vmcnt wait whose count is only known at run time (a multiple of a tile's DMA count): pick the immediate by switch
+__device__ __forceinline__ void wait_vmcnt_n(int n) {
+    switch (n) {
+        case 4: wait_vmcnt<4>(); break;
+        case 6: wait_vmcnt<6>(); break;
+        case 8: wait_vmcnt<8>(); break;
+        case 12: wait_vmcnt<12>(); break;
+        case 16: wait_vmcnt<16>(); break;
+        case 24: wait_vmcnt<24>(); break;
+        case 32: wait_vmcnt<32>(); break;
+        default: wait_vmcnt<0>(); break;
+    }
+}
+__device__ __forceinline__ void wg_barrier() { asm volatile("s_barrier" ::: "memory"); }
+
+template <int BM_, int BN_, int WGM_, int WGN_, int NS_>
+struct DmaCfg {
+    static constexpr int BM = BM_, BN = BN_, BK = 64, WGM = WGM_, WGN = WGN_, NS = NS_;
+    static constexpr int NT = 256;
+    static constexpr int WTM = BM / WGM, WTN = BN / WGN, TM = WTM / 32, TN = WTN / 32;
+    static constexpr int A_LD = BM / 64, W_LD = BN / 64;   // DMA instructions per wave per K tile (16 rows each, 4 waves)
+    static constexpr int LD = A_LD + W_LD;
+    static constexpr int STAGE = (BM + BN) * BK;
+    static constexpr int SMEM = NS * STAGE;
+    static_assert(WGM * WGN == 4, "four waves");
+    static_assert(BM % (32 * WGM) == 0 && BN % (32 * WGN) == 0 && BM % 64 == 0 && BN % 64 == 0, "tile shape");
+    static_assert(NS >= 3 && (NS - 1) * LD < 64, "vmcnt is a 6-bit counter");
+};
+
+template <bool V> struct flag { static constexpr bool value = V; };
+
+template <class C, int OUT_DT, int EPI>
+__device__ __forceinline__ void dma_gemm_tile(const GemmArgs& p, uint8_t* smem, int m0, int n0) {
+    constexpr int BM = C::BM, BN = C::BN, BK = C::BK, NS = C::NS, TM = C::TM, TN = C::TN, LD = C::LD;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar: LDS destinations of the DMA go through M0
+    const int wm = wave / C::WGN, wn = wave % C::WGN;
+    const int K = p.K, nk = K / BK;
+
+    // DMA sources: wave w owns 16-row blocks w, w+4, ... of the A tile and of the W tile.  Per-lane 32-bit offsets from
+    // the tile bases (the launcher guarantees M*K and N*K fit), so an instruction is scalar base + vector offset.
+    uint32_t ga[C::A_LD], gw[C::W_LD];
+    const int lrow = lane >> 2, lch = (lane & 3) ^ ((lrow >> 1) & 3);
 #pragma unroll
-    for (int im = 0; im < C::TM; ++im) {
-        const int m = m0 + wm * C::WTM + im * 32 + frow;
-        if (m >= p.M) continue;
-        const float xs = EPI == EPI_ACC ? 0.f : p.xs[m];
+    for (int i = 0; i < C::A_LD; ++i) {
+        const int row = (wave + 4 * i) * 16 + lrow;
+        const int gr = m0 + row < p.M ? m0 + row : p.M - 1;
+        ga[i] = (uint32_t)gr * (uint32_t)K + lch * 16;
+    }
 #pragma unroll
-        for (int in = 0; in < C::TN; ++in) {
+    for (int i = 0; i < C::W_LD; ++i) {
+        const int row = (wave + 4 * i) * 16 + lrow;
+        const int gr = n0 + row < p.N ? n0 + row : p.N - 1;
+        gw[i] = (uint32_t)gr * (uint32_t)K + lch * 16;
+    }
+    // One DMA instruction of ring slot t (K tile min(t, nk-1): slots past the last tile re-fetch it into a stage that
+    // nothing reads again, which keeps the loop body and its vmcnt bookkeeping free of branches).
+    auto dma = [&](int t, int j) {
+        const int kt = t < nk ? t : nk - 1;
+        uint8_t* s = smem + (t % NS) * C::STAGE;
+        if (j < C::A_LD)
+            __builtin_amdgcn_global_load_lds((glb_ptr_t)(p.A + (int64_t)kt * BK + ga[j]), (lds_ptr_t)(s + (wave + 4 * j) * 1024), 16, 0, 0);
+        else
+            __builtin_amdgcn_global_load_lds((glb_ptr_t)(p.W + (int64_t)kt * BK + gw[j - C::A_LD]),
+                                             (lds_ptr_t)(s + BM * BK + (wave + 4 * (j - C::A_LD)) * 1024), 16, 0, 0);
+    };
+
+    // fragment addresses: row r of a tile at r*64, chunk c at slot c ^ ((r>>1)&3); K sub-step kk flips address bit 5
+    const int frow = lane & 31, fhalf = lane >> 5;
+    const int fsw = (fhalf ^ ((frow >> 1) & 3)) << 4;
+    int aoff[2], woff[2];
+    aoff[0] = (wm * C::WTM + frow) * BK + fsw;
+    woff[0] = BM * BK + (wn * C::WTN + frow) * BK + fsw;
+    aoff[1] = aoff[0] ^ 32;
+    woff[1] = woff[0] ^ 32;
+    // fragment j of sub-step kk of the stage at s: j < TM are A fragments, the rest W fragments
+    auto frag = [&](const uint8_t* s, int kk, int j) -> v4i {
+        if (j < TM) return *reinterpret_cast<const v4i*>(s + aoff[kk] + j * 32 * BK);
+        return *reinterpret_cast<const v4i*>(s + woff[kk] + (j - TM) * 32 * BK);
+    };
+
+    v16i acc[TN][TM];
 #pragma unroll
-            for (int rb = 0; rb < 4; ++rb) {
-                const int n = n0 + wn * C::WTN + in * 32 + rb * 8 + fhalf * 4;
-                if (n >= p.N) continue;
-                const int64_t o = (int64_t)m * p.N + n;
-                if (EPI == EPI_ACC) {
-                    int* d = (int*)p.D + o;
-                    if (vec_ok) {
-                        *reinterpret_cast<v4i*>(d) = v4i{acc[in][im][4 * rb], acc[in][im][4 * rb + 1], acc[in][im][4 * rb + 2], acc[in][im][4 * rb + 3]};
-                    } else {
+    for (int in = 0; in < TN; ++in)
 #pragma unroll
-                        for (int j = 0; j < 4; ++j) if (n + j < p.N) d[j] = acc[in][im][4 * rb + j];
-                    }
-                    continue;
-                }
-                float ws[4], b[4] = {0.f, 0.f, 0.f, 0.f}, rs[4] = {0.f, 0.f, 0.f, 0.f}, res[4] = {0.f, 0.f, 0.f, 0.f}, out[4];
-                if (vec_ok) {
-                    const float4 w4 = *reinterpret_cast<const float4*>(p.ws + n);
-                    ws[0] = w4.x; ws[1] = w4.y; ws[2] = w4.z; ws[3] = w4.w;
-                    if (p.bias) load4<OUT_DT>(p.bias, n, b);
-                    if (EPI == EPI_RESID) { load4<OUT_DT>(p.rscale, n, rs); load4<OUT_DT>(p.resid, o, res); }
-                } else {
+        for (int im = 0; im < TM; ++im)
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        if (n + j >= p.N) { ws[j] = 0.f; continue; }
-                        ws[j] = p.ws[n + j];
-                        if (p.bias) b[j] = ld_dt<OUT_DT>(p.bias, n + j);
-                        if (EPI == EPI_RESID) { rs[j] = ld_dt<OUT_DT>(p.rscale, n + j); res[j] = ld_dt<OUT_DT>(p.resid, o + j); }
-                    }
-                }
+            for (int r = 0; r < 16; ++r) acc[in][im][r] = 0;
+
+    v4i f0[TM + TN], f1[TM + TN];   // fragments of the two sub-steps in flight
+
+    // One sub-step: TN*TM MFMAs on `cur`; between them, optionally the fragment loads of the next sub-step into `nxt`
+    // and the DMA instructions of ring slot t_dma.
+    auto substep = [&](auto LOAD, auto DMA, v4i* cur, v4i* nxt, const uint8_t* s_nxt, int kk_nxt, int t_dma) {
+        constexpr int NM = TN * TM, NF = TM + TN, EVERY = 1;   // fragment loads ride behind the first NF MFMAs
+        static_assert(NF <= NM, "more fragments than MFMAs");
 #pragma unroll
-                for (int j = 0; j < 4; ++j) out[j] = epi_value<OUT_DT, EPI>(acc[in][im][4 * rb + j], xs, ws[j], b[j], rs[j], res[j]);
-                if (vec_ok) {
-                    store4<OUT_DT>(p.D, o, out);
-                } else {
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) if (n + j < p.N) st_dt<OUT_DT>(p.D, o + j, out[j]);
-                }
+        for (int i = 0; i < NM; ++i) {
+            const int in = i / TM, im = i % TM;
+            acc[in][im] = __builtin_amdgcn_mfma_i32_32x32x32_i8(cur[TM + in], cur[im], acc[in][im], 0, 0, 0);
+            SCHED_FENCE();
+            if constexpr (decltype(DMA)::value) {
+                if (i < LD) { dma(t_dma, i); SCHED_FENCE(); }
+            }
+            if constexpr (decltype(LOAD)::value) {
+                if (i % EVERY == 0 && i / EVERY < NF) { nxt[i / EVERY] = frag(s_nxt, kk_nxt, i / EVERY); SCHED_FENCE(); }
             }
         }
+    };
+
+    // prologue: ring slots 0..NS-2 in flight, wait for slot 0
+#pragma unroll
+    for (int t = 0; t < NS - 1; ++t)
+#pragma unroll
+        for (int j = 0; j < LD; ++j) dma(t, j);
+    wait_vmcnt<(NS - 2) * LD>();
+    wg_barrier();
+#pragma unroll
+    for (int j = 0; j < TM + TN; ++j) f0[j] = frag(smem, 0, j);
+
+    for (int kt = 0; kt + 1 < nk; ++kt) {
+        const uint8_t* s_cur = smem + (kt % NS) * C::STAGE;
+        const uint8_t* s_nxt = smem + ((kt + 1) % NS) * C::STAGE;
+        // first half: MFMAs of sub-step 0; fragment loads of sub-step 1 of the same tile
+        substep(flag<true>{}, flag<false>{}, f0, f1, s_cur, 1, 0);
+        // slot kt+1 must have landed for every wave (the NS-3 slots issued after it may stay in flight), and every wave
+        // must be done reading slot kt-1 before its stage is refilled
+        wait_vmcnt<(NS - 3) * LD>();
+        wg_barrier();
+        // second half: MFMAs of sub-step 1; DMA of slot kt+NS-1; fragment loads of sub-step 0 of tile kt+1
+        substep(flag<true>{}, flag<true>{}, f1, f0, s_nxt, 0, kt + NS - 1);
     }
+    {
+        const uint8_t* s_cur = smem + ((nk - 1) % NS) * C::STAGE;
+        substep(flag<true>{}, flag<false>{}, f0, f1, s_cur, 1, 0);
+        substep(flag<false>{}, flag<false>{}, f1, f0, s_cur, 0, 0);
+    }
+    wait_vmcnt<0>();   // drain the re-fetches of the last slots before the LDS is reused
+    epilogue<TM, TN, OUT_DT, EPI>(p, acc, m0 + wm * C::WTM, n0 + wn * C::WTN, lane, wave, smem);
+}
+
+template <class C, int OUT_DT, int EPI>
+__global__ void __launch_bounds__(256, 1) int8_gemm_dma_kernel(GemmArgs p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    int tm, tn;
+    tile_of_block(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, tm, tn);
+    dma_gemm_tile<C, OUT_DT, EPI>(p, smem, tm * C::BM, tn * C::BN);
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// Variant with 128-byte tile rows (BK = 128) and two LDS stages: every DMA lane group fetches whole 128-byte cache
+// lines (8 rows per 1 KB instruction), which halves the number of L2 requests per byte compared with 64-byte rows.
+// A K tile is four 32-deep sub-steps.  Two workgroup barriers per tile: X, after which the other stage is free and the
+// DMA of the next tile is issued (it then has three sub-steps of MFMAs to land), and Y, before the last sub-step, after
+// which the next tile is visible and its first fragments are prefetched.
+// ---------------------------------------------------------------------------------------------------------------
+template <int BM_, int BN_, int WGM_, int WGN_>
+struct Dma2Cfg {
+    static constexpr int BM = BM_, BN = BN_, BK = 128, WGM = WGM_, WGN = WGN_, NS = 2;
+    static constexpr int NT = 256;
+    static constexpr int WTM = BM / WGM, WTN = BN / WGN, TM = WTM / 32, TN = WTN / 32;
+    static constexpr int A_LD = BM / 32, W_LD = BN / 32;   // DMA instructions per wave per K tile (8 rows each, 4 waves)
+    static constexpr int LD = A_LD + W_LD;
+    static constexpr int STAGE = (BM + BN) * BK;
+    static constexpr int SMEM = NS * STAGE;
+    static_assert(WGM * WGN == 4, "four waves");
+    static_assert(BM % (32 * WGM) == 0 && BN % (32 * WGN) == 0, "tile shape");
+};
+
+template <class C, int OUT_DT, int EPI>
+__device__ __forceinline__ void dma2_gemm_tile(const GemmArgs& p, uint8_t* smem, int m0, int n0) {
+    constexpr int BM = C::BM, BN = C::BN, BK = C::BK, TM = C::TM, TN = C::TN, LD = C::LD;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar: LDS destinations of the DMA go through M0
+    const int wm = wave / C::WGN, wn = wave % C::WGN;
+    const int K = p.K, nk = K / BK;
+
+    // DMA sources: wave w owns 8-row blocks w, w+4, ... of the A tile and of the W tile, as 32-bit lane offsets
+    uint32_t ga[C::A_LD], gw[C::W_LD];
+    const int lrow = lane >> 3, lch = (lane & 7) ^ lrow;
+#pragma unroll
+    for (int i = 0; i < C::A_LD; ++i) {
+        const int row = (wave + 4 * i) * 8 + lrow;
+        const int gr = m0 + row < p.M ? m0 + row : p.M - 1;
+        ga[i] = (uint32_t)gr * (uint32_t)K + lch * 16;
+    }
+#pragma unroll
+    for (int i = 0; i < C::W_LD; ++i) {
+        const int row = (wave + 4 * i) * 8 + lrow;
+        const int gr = n0 + row < p.N ? n0 + row : p.N - 1;
+        gw[i] = (uint32_t)gr * (uint32_t)K + lch * 16;
+    }
+    // One DMA instruction of K tile min(t, nk-1) into stage t&1 (a tile index past the end re-fetches the last tile
+    // into the stage nothing reads again, which keeps the loop body free of branches).
+    auto dma = [&](int t, int j) {
+        const int kt = t < nk ? t : nk - 1;
+        uint8_t* s = smem + (t & 1) * C::STAGE;
+        if (j < C::A_LD)
+            __builtin_amdgcn_global_load_lds((glb_ptr_t)(p.A + (int64_t)kt * BK + ga[j]), (lds_ptr_t)(s + (wave + 4 * j) * 1024), 16, 0, 0);
+        else
+            __builtin_amdgcn_global_load_lds((glb_ptr_t)(p.W + (int64_t)kt * BK + gw[j - C::A_LD]),
+                                             (lds_ptr_t)(s + BM * BK + (wave + 4 * (j - C::A_LD)) * 1024), 16, 0, 0);
+    };
+
+    // fragment addresses: row r at r*128, chunk c at slot c ^ (r&7); K sub-step kk flips address bits 5 and 6
+    const int frow = lane & 31, fhalf = lane >> 5;
+    const int fsw = (fhalf ^ (frow & 7)) << 4;
+    int aoff[4], woff[4];
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+        aoff[kk] = ((wm * C::WTM + frow) * BK + fsw) ^ (kk << 5);
+        woff[kk] = (BM * BK + (wn * C::WTN + frow) * BK + fsw) ^ (kk << 5);
+    }
+    auto frag = [&](const uint8_t* s, int kk, int j) -> v4i {
+        if (j < TM) return *reinterpret_cast<const v4i*>(s + aoff[kk] + j * 32 * BK);
+        return *reinterpret_cast<const v4i*>(s + woff[kk] + (j - TM) * 32 * BK);
+    };
+
+    v16i acc[TN][TM];
+#pragma unroll
+    for (int in = 0; in < TN; ++in)
+#pragma unroll
+        for (int im = 0; im < TM; ++im)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[in][im][r] = 0;
+
+    v4i f0[TM + TN], f1[TM + TN];
+
+    // One sub-step: TN*TM MFMAs on `cur`, with the fragment loads of the next sub-step into `nxt` behind the first
+    // MFMAs, and one DMA instruction of tile t_dma after every DMA_EVERY-th MFMA of the tile (this sub-step's MFMAs
+    // are numbers mfma_base .. mfma_base + TN*TM - 1 of the tile).  The
+    // texture-address unit takes about 16 cycles per 1 KB DMA instruction and serves all four waves, so the DMA of a
+    // tile is spread over three sub-steps instead of being bunched: bunched, the waves stall at issue and the MFMA
+    // pipe drains.
+    constexpr int DMA_EVERY = 3;
+    auto substep = [&](auto DMA, v4i* cur, v4i* nxt, const uint8_t* s_nxt, int kk_nxt, int t_dma, int mfma_base) {
+        constexpr int NM = TN * TM, NF = TM + TN;
+        static_assert(NF <= NM, "more fragment loads than MFMAs to hide them behind");
+#pragma unroll
+        for (int i = 0; i < NM; ++i) {
+            const int in = i / TM, im = i % TM;
+            acc[in][im] = __builtin_amdgcn_mfma_i32_32x32x32_i8(cur[TM + in], cur[im], acc[in][im], 0, 0, 0);
+            SCHED_FENCE();
+            if constexpr (decltype(DMA)::value) {
+                if ((mfma_base + i) % DMA_EVERY == 0 && (mfma_base + i) / DMA_EVERY < LD) {
+                    dma(t_dma, (mfma_base + i) / DMA_EVERY);
+                    SCHED_FENCE();
+                }
+            }
+            if (i < NF) { nxt[i] = frag(s_nxt, kk_nxt, i); SCHED_FENCE(); }
+        }
+    };
+    static_assert((LD - 1) * DMA_EVERY < 3 * TN * TM, "the DMA of a tile must fit in three sub-steps");
+
+#pragma unroll
+    for (int j = 0; j < LD; ++j) dma(0, j);
+    wait_vmcnt<0>();
+    wg_barrier();
+#pragma unroll
+    for (int j = 0; j < TM + TN; ++j) f0[j] = frag(smem, 0, j);
+
+    for (int kt = 0; kt < nk; ++kt) {
+        const uint8_t* s_cur = smem + (kt & 1) * C::STAGE;
+        const uint8_t* s_nxt = smem + ((kt + 1) & 1) * C::STAGE;
+        wg_barrier();                                              // X: every wave is done with tile kt-1
+        substep(flag<true>{}, f0, f1, s_cur, 1, kt + 1, 0);
+        substep(flag<true>{}, f1, f0, s_cur, 2, kt + 1, TN * TM);
+        substep(flag<true>{}, f0, f1, s_cur, 3, kt + 1, 2 * TN * TM);
+        wait_vmcnt<0>();
+        wg_barrier();                                              // Y: tile kt+1 has landed for every wave
+        substep(flag<false>{}, f1, f0, s_nxt, 0, 0, 0);
+    }
+    epilogue<TM, TN, OUT_DT, EPI>(p, acc, m0 + wm * C::WTM, n0 + wn * C::WTN, lane, wave, smem);
+}
+
+template <class C, int OUT_DT, int EPI>
+__global__ void __launch_bounds__(256, 1) int8_gemm_dma2_kernel(GemmArgs p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    int tm, tn;
+    tile_of_block(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, tm, tn);
+    dma2_gemm_tile<C, OUT_DT, EPI>(p, smem, tm * C::BM, tn * C::BN);
+}
+
+using Dma2L = Dma2Cfg<256, 256, 2, 2>;
+
+using DmaL = DmaCfg<256, 256, 2, 2, 4>;
+
+template <class C, int OUT_DT, int EPI>
+int launch_dma(GemmArgs a, hipStream_t st) {
+    a.tiles_m = (a.M + C::BM - 1) / C::BM;
+    a.tiles_n = (a.N + C::BN - 1) / C::BN;
+    const int64_t nblocks = (int64_t)a.tiles_m * a.tiles_n;
+    if (nblocks > 0x7fffffff) return -1;
+    auto kern = int8_gemm_dma_kernel<C, OUT_DT, EPI>;
+    static bool once = false;  // benign race: the attribute is idempotent
+    if (!once) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
+        if (e != hipSuccess) return (int)e;
+        once = true;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(C::NT), C::SMEM, st, a);
+    KCHECK();
+    return 0;
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// The persistent ring kernel: one workgroup per CU walks its share of the 256x256 output tiles and keeps ONE
+// global -> LDS pipeline running across all of them.  Tiles have 128-byte K rows (whole cache lines per DMA lane
+// group).  LDS holds two stages of A (2 x 32 KB) and three of W (3 x 32 KB) = 160 KB: in iteration g the DMA fetches
+// A of iteration g+1 (it must land before barrier Y of this iteration) and W of iteration g+2 (a full iteration of
+// slack), so the last-issued loads of an iteration are never the ones the next wait needs.  Iterations number
+// straight through tile boundaries: while the last K tiles of one output tile are multiplied, the first K tiles of
+// the next one are already in flight, and the stores of an epilogue drain under the next tile's K loop.
+//
+// Per iteration (64 MFMAs per wave = four 32-deep sub-steps): barrier X (every wave is done with iteration g-1, whose
+// stages are now free); sub-steps 0-2 with A DMA after MFMAs 0,3,..,21 and W DMA after MFMAs 24,28,..,52; vmcnt wait
+// that leaves only this iteration's W DMA in flight; barrier Y; sub-step 3, which prefetches the first fragments of
+// iteration g+1.  Requires K % 128 == 0 and M*K, N*K < 2^32.
+// ---------------------------------------------------------------------------------------------------------------
+struct RingCfg {
+    static constexpr int BM = 256, BN = 256, BK = 128, WGM = 2, WGN = 2, NT = 256;
+    static constexpr int WTM = 128, WTN = 128, TM = 4, TN = 4;
+    static constexpr int A_LD = 8, W_LD = 8;                 // DMA instructions per wave per stage (8 rows each)
+    static constexpr int A_STAGE = BM * BK, W_STAGE = BN * BK;
+    static constexpr int W_BASE = 2 * A_STAGE;
+    static constexpr int SMEM = 2 * A_STAGE + 3 * W_STAGE;   // 163840
+    static constexpr int A_EVERY = 3, W_FIRST = 24, W_EVERY = 4, W_BEFORE_Y = 6;   // DMA slots, in MFMA numbers of an iteration
+};
+
+template <int OUT_DT, int EPI>
+__global__ void __launch_bounds__(256, 1) int8_gemm_ring_kernel(GemmArgs p) {
+    using C = RingCfg;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    constexpr int BK = C::BK, TM = C::TM, TN = C::TN, NM = TM * TN, NF = TM + TN;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int K = p.K, nk = K / BK;
+    const int G = gridDim.x, ntiles = p.tiles_m * p.tiles_n;
+    const int nt_b = (ntiles - (int)blockIdx.x + G - 1) / G;   // tiles of this workgroup: blockIdx, blockIdx + G, ...
+
+    auto tile_origin = [&](int i, int& m0, int& n0) {
+        int tm, tn;
+        tile_of_block((int)blockIdx.x + i * G, ntiles, p.tiles_m, p.tiles_n, tm, tn);
+        m0 = tm * C::BM;
+        n0 = tn * C::BN;
+    };
+
+    // DMA streams.  Each walks (tile, K tile) pairs in the order the MFMAs will consume them and stops on the last one
+    // (re-fetching it into a stage nothing reads again keeps the loop free of branches around the DMA slots).
+    const int lrow = lane >> 3, lch = ((lane & 7) ^ lrow) * 16;
+    uint32_t ga[C::A_LD], gw[C::W_LD];
+    int a_tile = 0, a_kt = 0, a_stage = 0, w_tile = 0, w_kt = 0, w_stage = 0;
+    auto set_a = [&](int i) {
+        int m0, n0;
+        tile_origin(i, m0, n0);
+#pragma unroll
+        for (int j = 0; j < C::A_LD; ++j) {
+            const int row = (wave + 4 * j) * 8 + lrow;
+            const int gr = m0 + row < p.M ? m0 + row : p.M - 1;
+            ga[j] = (uint32_t)gr * (uint32_t)K + lch;
+        }
+    };
+    auto set_w = [&](int i) {
+        int m0, n0;
+        tile_origin(i, m0, n0);
+#pragma unroll
+        for (int j = 0; j < C::W_LD; ++j) {
+            const int row = (wave + 4 * j) * 8 + lrow;
+            const int gr = n0 + row < p.N ? n0 + row : p.N - 1;
+            gw[j] = (uint32_t)gr * (uint32_t)K + lch;
+        }
+    };
+    // The DMA is written as inline assembly: through the builtin the compiler, unable to prove that a fragment read and
+    // an in-flight DMA touch different stages, puts a full vmcnt(0) wait in front of the fragment reads, which serializes
+    // the whole pipeline.  Ordering is kept by hand instead (wait_vmcnt + barriers).  scalar base + 32-bit lane offset.
+    const uint32_t lds_base = (uint32_t)(uintptr_t)smem;   // LDS byte address of the dynamic segment
+    auto dma_a = [&](int j) {
+        const int8_t* base = p.A + (int64_t)a_kt * BK;
+        const uint32_t dst = lds_base + a_stage * C::A_STAGE + (wave + 4 * j) * 1024;
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(ga[j]), "s"(base) : "memory", "m0");
+    };
+    auto dma_w = [&](int j) {
+        const int8_t* base = p.W + (int64_t)w_kt * BK;
+        const uint32_t dst = lds_base + C::W_BASE + w_stage * C::W_STAGE + (wave + 4 * j) * 1024;
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(gw[j]), "s"(base) : "memory", "m0");
+    };
+    auto advance_a = [&]() {
+        a_stage ^= 1;
+        if (a_tile == nt_b - 1 && a_kt == nk - 1) return;
+        if (++a_kt == nk) { a_kt = 0; set_a(++a_tile); }
+    };
+    auto advance_w = [&]() {
+        w_stage = w_stage == 2 ? 0 : w_stage + 1;
+        if (w_tile == nt_b - 1 && w_kt == nk - 1) return;
+        if (++w_kt == nk) { w_kt = 0; set_w(++w_tile); }
+    };
+
+    // fragment addresses inside a stage: row r at r*128, chunk c at slot c ^ (r&7); K sub-step kk flips bits 5 and 6
+    const int frow = lane & 31, fhalf = lane >> 5;
+    const int fsw = (fhalf ^ (frow & 7)) << 4;
+    int aoff[4], woff[4];
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+        aoff[kk] = ((wm * C::WTM + frow) * BK + fsw) ^ (kk << 5);
+        woff[kk] = ((wn * C::WTN + frow) * BK + fsw) ^ (kk << 5);
+    }
+    auto frag = [&](const uint8_t* sa, const uint8_t* sw, int kk, int j) -> v4i {
+        if (j < TM) return *reinterpret_cast<const v4i*>(sa + aoff[kk] + j * 32 * BK);
+        return *reinterpret_cast<const v4i*>(sw + woff[kk] + (j - TM) * 32 * BK);
+    };
+
+    v16i acc[TN][TM];
+    v4i f0[NF], f1[NF];
+
+    // One sub-step: NM MFMAs on `cur`; the NF fragment loads of the next sub-step ride behind the first MFMAs; DMA
+    // instructions sit in their slots (MFMA numbers mfma_base .. mfma_base + NM - 1 of the iteration).
+    auto substep = [&](auto DMA, v4i* cur, v4i* nxt, const uint8_t* sa_n, const uint8_t* sw_n, int kk_n, int mfma_base) {
+#pragma unroll
+        for (int i = 0; i < NM; ++i) {
+            const int in = i / TM, im = i % TM;
+            acc[in][im] = __builtin_amdgcn_mfma_i32_32x32x32_i8(cur[TM + in], cur[im], acc[in][im], 0, 0, 0);
+            SCHED_FENCE();
+            if constexpr (decltype(DMA)::value) {
+                const int n = mfma_base + i;
+                if (n % C::A_EVERY == 0 && n / C::A_EVERY < C::A_LD) { dma_a(n / C::A_EVERY); SCHED_FENCE(); }
+                if (n >= C::W_FIRST && (n - C::W_FIRST) % C::W_EVERY == 0 && (n - C::W_FIRST) / C::W_EVERY < C::W_LD) {
+                    dma_w((n - C::W_FIRST) / C::W_EVERY);
+                    SCHED_FENCE();
+                }
+            }
+            if (i < NF) { nxt[i] = frag(sa_n, sw_n, kk_n, i); SCHED_FENCE(); }
+        }
+    };
+    static_assert((C::A_LD - 1) * C::A_EVERY < C::W_FIRST && C::W_FIRST + (C::W_LD - 1) * C::W_EVERY < 4 * NM, "DMA slots");
+    static_assert(C::W_FIRST + (C::W_BEFORE_Y - 1) * C::W_EVERY < 3 * NM && C::W_FIRST + C::W_BEFORE_Y * C::W_EVERY >= 3 * NM,
+                  "W_BEFORE_Y must count the W DMA slots ahead of barrier Y");
+
+    // prologue: A(0), W(0), W(1) in flight; A(0) and W(0) must land
+    set_a(0);
+    set_w(0);
+#pragma unroll
+    for (int j = 0; j < C::A_LD; ++j) dma_a(j);
+    advance_a();
+#pragma unroll
+    for (int j = 0; j < C::W_LD; ++j) dma_w(j);
+    advance_w();
+#pragma unroll
+    for (int j = 0; j < C::W_LD; ++j) dma_w(j);
+    advance_w();
+    wait_vmcnt<C::W_LD>();
+    wg_barrier();
+#pragma unroll
+    for (int j = 0; j < NF; ++j) f0[j] = frag(smem, smem + C::W_BASE, 0, j);
+
+    int ca = 0, cw = 0;   // stages of the iteration being multiplied
+    for (int ti = 0; ti < nt_b; ++ti) {
+#pragma unroll
+        for (int in = 0; in < TN; ++in)
+#pragma unroll
+            for (int im = 0; im < TM; ++im)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[in][im][r] = 0;
+        // A wait the compiler can see: without it, it assumes that loads and stores of the previous tile's epilogue may
+        // still be pending at the K loop's header and parks a vmcnt(0) inside the loop, in front of the first fragment
+        // read, which would drain the DMA pipeline every iteration.
+        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0) only
+
+        for (int kt = 0; kt < nk; ++kt) {
+            const uint8_t* sa = smem + ca * C::A_STAGE;
+            const uint8_t* sw = smem + C::W_BASE + cw * C::W_STAGE;
+            const int na = ca ^ 1, nw = cw == 2 ? 0 : cw + 1;
+            wg_barrier();                                                   // X
+            substep(flag<true>{}, f0, f1, sa, sw, 1, 0);
+            substep(flag<true>{}, f1, f0, sa, sw, 2, NM);
+            substep(flag<true>{}, f0, f1, sa, sw, 3, 2 * NM);
+            wait_vmcnt<C::W_BEFORE_Y>();
+            wg_barrier();                                                   // Y
+            substep(flag<true>{}, f1, f0, smem + na * C::A_STAGE, smem + C::W_BASE + nw * C::W_STAGE, 0, 3 * NM);
+            advance_a();
+            advance_w();
+            ca = na;
+            cw = nw;
+        }
+
+        // epilogue of tile ti; the A stage that was just multiplied (ca ^ 1 after the swap) is the shuffle scratch.
+        // (The launcher only picks this kernel when the coalesced epilogue's alignment conditions hold.)
+        int m0, n0;
+        tile_origin(ti, m0, n0);
+        __syncthreads();   // every wave is done reading that stage
+        constexpr int SZ = (EPI == EPI_ACC || OUT_DT == DT_F32) ? 4 : 2;
+        constexpr int PW = 256 / SZ;   // 256-byte LDS rows: 8 KB per wave, 32 KB in all
+        epilogue_shuffle<TM, TN, OUT_DT, EPI, PW>(p, acc, m0 + wm * C::WTM, n0 + wn * C::WTN, lane,
+                                                   smem + (ca ^ 1) * C::A_STAGE + wave * 8192);
+    }
+    wait_vmcnt<0>();   // no DMA may still be writing this workgroup's LDS when it retires
 }
 
 // Tile shapes.  L: the large-shape workhorse, one workgroup per CU, each of 4 waves owns a 128x128 accumulator tile
@@ -296,13 +1018,63 @@ int launch_cfg(GemmArgs a, hipStream_t st) {
     return 0;
 }
 
+template <int OUT_DT, int EPI>
+int launch_ring(GemmArgs a, hipStream_t st) {
+    using C = RingCfg;
+    a.tiles_m = (a.M + C::BM - 1) / C::BM;
+    a.tiles_n = (a.N + C::BN - 1) / C::BN;
+    const int64_t ntiles = (int64_t)a.tiles_m * a.tiles_n;
+    if (ntiles > 0x7fffffff) return -1;
+    static int num_cu = 0;   // benign race: every thread computes the same value
+    if (num_cu == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        num_cu = n;
+    }
+    bool vec_ok, aligned;
+    epilogue_alignment<OUT_DT, EPI>(a, vec_ok, aligned);
+    if (!aligned) return launch_cfg<CfgL, OUT_DT, EPI>(a, st);   // the ring kernel has only the coalesced epilogue
+    auto kern = int8_gemm_ring_kernel<OUT_DT, EPI>;
+    static bool once = false;
+    if (!once) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
+        if (e != hipSuccess) return (int)e;
+        once = true;
+    }
+    const unsigned grid = (unsigned)(ntiles < num_cu ? ntiles : num_cu);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(C::NT), C::SMEM, st, a);
+    KCHECK();
+    return 0;
+}
+
+template <class C, int OUT_DT, int EPI>
+int launch_dma2(GemmArgs a, hipStream_t st) {
+    a.tiles_m = (a.M + C::BM - 1) / C::BM;
+    a.tiles_n = (a.N + C::BN - 1) / C::BN;
+    const int64_t nblocks = (int64_t)a.tiles_m * a.tiles_n;
+    if (nblocks > 0x7fffffff) return -1;
+    auto kern = int8_gemm_dma2_kernel<C, OUT_DT, EPI>;
+    static bool once = false;  // benign race: the attribute is idempotent
+    if (!once) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
+        if (e != hipSuccess) return (int)e;
+        once = true;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(C::NT), C::SMEM, st, a);
+    KCHECK();
+    return 0;
+}
+
 // 0 = L, 1 = M, 2 = S; -1 = choose by shape.
 int g_force_cfg = -1;
 
-int choose_cfg(int64_t M, int64_t N) {
-    if (g_force_cfg >= 0) return g_force_cfg;
+int choose_cfg(int64_t M, int64_t N, int64_t K) {
+    const bool dma_ok = M * K < ((int64_t)1 << 32) && N * K < ((int64_t)1 << 32);   // 32-bit lane offsets
+    if (!dma_ok && g_force_cfg >= 3) return 0;
+    if (g_force_cfg == 4 || g_force_cfg == 5) return (K % 128) == 0 ? g_force_cfg : 0;
+    if (g_force_cfg >= 0) return (g_force_cfg == 3 && (K % 64) != 0) ? 0 : g_force_cfg;
     const int64_t tiles_l = ((M + 255) / 256) * ((N + 255) / 256);
-    if (M >= 512 && N >= 512 && tiles_l >= 192) return 0;
+    if (M >= 512 && N >= 512 && tiles_l >= 192) return !dma_ok ? 0 : (K % 128) == 0 ? 5 : (K % 64) == 0 ? 3 : 0;
     const int64_t tiles_m = ((M + 127) / 128) * ((N + 127) / 128);
     if (M > 64 && N > 64 && tiles_m >= 128) return 1;
     return 2;
@@ -310,7 +1082,10 @@ int choose_cfg(int64_t M, int64_t N) {
 
 template <int OUT_DT, int EPI>
 int dispatch_cfg(const GemmArgs& a, hipStream_t st) {
-    switch (choose_cfg(a.M, a.N)) {
+    switch (choose_cfg(a.M, a.N, a.K)) {
+        case 3: return launch_dma<DmaL, OUT_DT, EPI>(a, st);
+        case 4: return launch_dma2<Dma2L, OUT_DT, EPI>(a, st);
+        case 5: return launch_ring<OUT_DT, EPI>(a, st);
         case 0: return launch_cfg<CfgL, OUT_DT, EPI>(a, st);
         case 1: return launch_cfg<CfgM, OUT_DT, EPI>(a, st);
         default: return launch_cfg<CfgS, OUT_DT, EPI>(a, st);

@@ -318,7 +318,7 @@ def test_epilogue_forms(synth):
         a = tof(oracle.epilogue(acc, xs, ws, bias, out_dt, fma=0)).astype(np.float64)
         b = tof(got).astype(np.float64)
         ulp = {BF16: 2.0 ** -7, F16: 2.0 ** -10, F32: 2.0 ** -23}[out_dt]
-        assert (np.abs(a - b) <= ulp * np.maximum(np.abs(a), np.abs(b)) + 1e-30).all()
+        assert (np.abs(a - b) <= ulp * (np.maximum(np.abs(a), np.abs(b)) + np.abs(bf)[None, :]) + 1e-30).all()
 
 
 def test_epilogue_residual(synth):
