@@ -34,6 +34,9 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-skinny", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run a plain 256 MiB device copy a few times: under rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE its "
+                         "known size calibrates the counters that roofline.traffic is derived from")
     return ap.parse_args()
 
 
@@ -119,6 +122,13 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(1)
     M, K, N = (int(v) for v in a.shape.split(","))
+    if a.copy_probe:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda:0").random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     host, d = make_inputs(torch, synth, M, K, N)
     gpu_ms, wall_ms, tq, tg = time_linear(torch, ffi, d, M, K, N, a.rotate, a.steps, a.warmup)
     ops = 2.0 * M * N * K
