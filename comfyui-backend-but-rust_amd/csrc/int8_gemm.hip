@@ -26,6 +26,7 @@ struct GemmArgs {
     void* D;
     int M, N, K;
     int tiles_m, tiles_n;
+    int kslice;   // ring kernel only: K elements per split-K slice (a multiple of 128), 0 = no split
 };
 
 template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int OCC_>
@@ -813,25 +814,64 @@ int launch_dma(GemmArgs a, hipStream_t st) {
 // that leaves only this iteration's W DMA in flight; barrier Y; sub-step 3, which prefetches the first fragments of
 // iteration g+1.  Requires K % 128 == 0 and M*K, N*K < 2^32.
 // ---------------------------------------------------------------------------------------------------------------
+template <int V> struct ic { static constexpr int value = V; };
+
+// BN: tile width; WGM x WGN: wave grid (four waves); NSA: LDS stages of A (2 for the 256-wide tile, where 160 KB of LDS
+// leave no room for a third; 3 for the narrow tiles of the skinny shapes).  W always has three stages.
+template <int BN_, int WGM_, int WGN_, int NSA_>
 struct RingCfg {
-    static constexpr int BM = 256, BN = 256, BK = 128, WGM = 2, WGN = 2, NT = 256;
-    static constexpr int WTM = 128, WTN = 128, TM = 4, TN = 4;
-    static constexpr int A_LD = 8, W_LD = 8;                 // DMA instructions per wave per stage (8 rows each)
+    static constexpr int BM = 256, BN = BN_, BK = 128, WGM = WGM_, WGN = WGN_, NT = 256, NSA = NSA_, NSW = 3;
+    static constexpr int WTM = BM / WGM, WTN = BN / WGN, TM = WTM / 32, TN = WTN / 32;
+    static constexpr int A_LD = BM / 32, W_LD = BN / 32;     // DMA instructions per wave per stage (8 rows each)
+    static constexpr int NDMA = A_LD + W_LD, NM = TM * TN, NF = TM + TN;
     static constexpr int A_STAGE = BM * BK, W_STAGE = BN * BK;
-    static constexpr int W_BASE = 2 * A_STAGE;
-    static constexpr int SMEM = 2 * A_STAGE + 3 * W_STAGE;   // 163840
-    static constexpr int A_EVERY = 3, W_FIRST = 24, W_EVERY = 4, W_BEFORE_Y = 6;   // DMA slots, in MFMA numbers of an iteration
+    static constexpr int W_BASE = NSA * A_STAGE;
+    static constexpr int SMEM = NSA * A_STAGE + NSW * W_STAGE;
+    static_assert(WGM * WGN == 4 && BM % (32 * WGM) == 0 && BN % (32 * WGN) == 0 && BN % 32 == 0, "tile shape");
+    static_assert(NF <= NM && SMEM <= 160 * 1024, "fragment loads hide behind MFMAs; LDS fits");
+    // Slot of the d-th DMA instruction of an iteration (A first, then W), as the number of the MFMA it follows; an
+    // iteration has 4*NM MFMAs and barrier Y sits after MFMA 3*NM - 1.  With two A stages the A DMA is needed by this
+    // iteration's barrier Y, so it goes first and dense; with three, everything has an iteration of slack and is
+    // spread evenly.
+    static constexpr int slot(int d) {
+        return NSA == 2 ? (d < A_LD ? d * 3 : 24 + (d - A_LD) * 4) : (d * 4 * NM) / NDMA;
+    }
+    // DMA instructions of this iteration that may still be in flight at barrier Y
+    static constexpr int in_flight_at_y() {
+        int n = 0;
+        for (int d = (NSA == 2 ? A_LD : 0); d < NDMA; ++d) n += slot(d) < 3 * NM ? 1 : 0;
+        return n;
+    }
+    static constexpr bool slots_ok() {
+        for (int d = 0; d < NDMA; ++d) {
+            if (slot(d) >= 4 * NM) return false;
+            if (d > 0 && slot(d) <= slot(d - 1)) return false;
+            if (NSA == 2 && d < A_LD && slot(d) >= 2 * NM) return false;
+        }
+        return true;
+    }
+    static_assert(slots_ok(), "DMA slots must be distinct, inside the iteration, and early for a two-stage A");
+    // columns of one epilogue shuffle piece for an output element of SZ bytes: 64..256-byte LDS rows
+    static constexpr int piece_cols(int sz) {
+        return sz == 2 ? (WTN % 128 == 0 ? 128 : WTN % 64 == 0 ? 64 : 32) : (WTN % 64 == 0 ? 64 : 32);
+    }
 };
 
-template <int OUT_DT, int EPI>
+template <class C, int OUT_DT, int EPI>
 __global__ void __launch_bounds__(256, 1) int8_gemm_ring_kernel(GemmArgs p) {
-    using C = RingCfg;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    constexpr int BK = C::BK, TM = C::TM, TN = C::TN, NM = TM * TN, NF = TM + TN;
+    constexpr int BK = C::BK, TM = C::TM, TN = C::TN, NM = C::NM, NF = C::NF, NSA = C::NSA;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave >> 1, wn = wave & 1;
-    const int K = p.K, nk = K / BK;
+    const int wm = wave / C::WGN, wn = wave % C::WGN;
+    const int ld = p.K;                                  // row stride of A and W
+    // split K: workgroup row blockIdx.y multiplies K slice [k_lo, k_lo + nk*128) and writes its own int32 plane
+    const int k_lo = p.kslice ? (int)blockIdx.y * p.kslice : 0;
+    const int k_len = p.kslice ? (p.K - k_lo < p.kslice ? p.K - k_lo : p.kslice) : p.K;
+    const int nk = k_len / BK;
+    if (p.kslice) p.D = (uint8_t*)p.D + (int64_t)blockIdx.y * p.M * p.N * 4;
+    const int8_t* Ab = p.A + k_lo;
+    const int8_t* Wb = p.W + k_lo;
     const int G = gridDim.x, ntiles = p.tiles_m * p.tiles_n;
     const int nt_b = (ntiles - (int)blockIdx.x + G - 1) / G;   // tiles of this workgroup: blockIdx, blockIdx + G, ...
 
@@ -854,7 +894,7 @@ __global__ void __launch_bounds__(256, 1) int8_gemm_ring_kernel(GemmArgs p) {
         for (int j = 0; j < C::A_LD; ++j) {
             const int row = (wave + 4 * j) * 8 + lrow;
             const int gr = m0 + row < p.M ? m0 + row : p.M - 1;
-            ga[j] = (uint32_t)gr * (uint32_t)K + lch;
+            ga[j] = (uint32_t)gr * (uint32_t)ld + lch;
         }
     };
     auto set_w = [&](int i) {
@@ -864,7 +904,7 @@ __global__ void __launch_bounds__(256, 1) int8_gemm_ring_kernel(GemmArgs p) {
         for (int j = 0; j < C::W_LD; ++j) {
             const int row = (wave + 4 * j) * 8 + lrow;
             const int gr = n0 + row < p.N ? n0 + row : p.N - 1;
-            gw[j] = (uint32_t)gr * (uint32_t)K + lch;
+            gw[j] = (uint32_t)gr * (uint32_t)ld + lch;
         }
     };
     // The DMA is written as inline assembly: through the builtin the compiler, unable to prove that a fragment read and
@@ -872,22 +912,22 @@ __global__ void __launch_bounds__(256, 1) int8_gemm_ring_kernel(GemmArgs p) {
     // the whole pipeline.  Ordering is kept by hand instead (wait_vmcnt + barriers).  scalar base + 32-bit lane offset.
     const uint32_t lds_base = (uint32_t)(uintptr_t)smem;   // LDS byte address of the dynamic segment
     auto dma_a = [&](int j) {
-        const int8_t* base = p.A + (int64_t)a_kt * BK;
+        const int8_t* base = Ab + (int64_t)a_kt * BK;
         const uint32_t dst = lds_base + a_stage * C::A_STAGE + (wave + 4 * j) * 1024;
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(ga[j]), "s"(base) : "memory", "m0");
     };
     auto dma_w = [&](int j) {
-        const int8_t* base = p.W + (int64_t)w_kt * BK;
+        const int8_t* base = Wb + (int64_t)w_kt * BK;
         const uint32_t dst = lds_base + C::W_BASE + w_stage * C::W_STAGE + (wave + 4 * j) * 1024;
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(gw[j]), "s"(base) : "memory", "m0");
     };
     auto advance_a = [&]() {
-        a_stage ^= 1;
+        a_stage = a_stage == NSA - 1 ? 0 : a_stage + 1;
         if (a_tile == nt_b - 1 && a_kt == nk - 1) return;
         if (++a_kt == nk) { a_kt = 0; set_a(++a_tile); }
     };
     auto advance_w = [&]() {
-        w_stage = w_stage == 2 ? 0 : w_stage + 1;
+        w_stage = w_stage == C::NSW - 1 ? 0 : w_stage + 1;
         if (w_tile == nt_b - 1 && w_kt == nk - 1) return;
         if (++w_kt == nk) { w_kt = 0; set_w(++w_tile); }
     };
@@ -910,29 +950,26 @@ __global__ void __launch_bounds__(256, 1) int8_gemm_ring_kernel(GemmArgs p) {
     v4i f0[NF], f1[NF];
 
     // One sub-step: NM MFMAs on `cur`; the NF fragment loads of the next sub-step ride behind the first MFMAs; DMA
-    // instructions sit in their slots (MFMA numbers mfma_base .. mfma_base + NM - 1 of the iteration).
-    auto substep = [&](auto DMA, v4i* cur, v4i* nxt, const uint8_t* sa_n, const uint8_t* sw_n, int kk_n, int mfma_base) {
+    // instructions sit in their slots (this sub-step's MFMAs are numbers BASE .. BASE + NM - 1 of the iteration).
+    auto substep = [&](auto BASE, v4i* cur, v4i* nxt, const uint8_t* sa_n, const uint8_t* sw_n, int kk_n) {
 #pragma unroll
         for (int i = 0; i < NM; ++i) {
             const int in = i / TM, im = i % TM;
             acc[in][im] = __builtin_amdgcn_mfma_i32_32x32x32_i8(cur[TM + in], cur[im], acc[in][im], 0, 0, 0);
             SCHED_FENCE();
-            if constexpr (decltype(DMA)::value) {
-                const int n = mfma_base + i;
-                if (n % C::A_EVERY == 0 && n / C::A_EVERY < C::A_LD) { dma_a(n / C::A_EVERY); SCHED_FENCE(); }
-                if (n >= C::W_FIRST && (n - C::W_FIRST) % C::W_EVERY == 0 && (n - C::W_FIRST) / C::W_EVERY < C::W_LD) {
-                    dma_w((n - C::W_FIRST) / C::W_EVERY);
+#pragma unroll
+            for (int d = 0; d < C::NDMA; ++d) {
+                if (C::slot(d) == decltype(BASE)::value + i) {
+                    if (d < C::A_LD) dma_a(d);
+                    else dma_w(d - C::A_LD);
                     SCHED_FENCE();
                 }
             }
             if (i < NF) { nxt[i] = frag(sa_n, sw_n, kk_n, i); SCHED_FENCE(); }
         }
     };
-    static_assert((C::A_LD - 1) * C::A_EVERY < C::W_FIRST && C::W_FIRST + (C::W_LD - 1) * C::W_EVERY < 4 * NM, "DMA slots");
-    static_assert(C::W_FIRST + (C::W_BEFORE_Y - 1) * C::W_EVERY < 3 * NM && C::W_FIRST + C::W_BEFORE_Y * C::W_EVERY >= 3 * NM,
-                  "W_BEFORE_Y must count the W DMA slots ahead of barrier Y");
 
-    // prologue: A(0), W(0), W(1) in flight; A(0) and W(0) must land
+    // prologue: A(0), W(0), [A(1),] W(1) in flight; A(0) and W(0) must land
     set_a(0);
     set_w(0);
 #pragma unroll
@@ -941,10 +978,15 @@ __global__ void __launch_bounds__(256, 1) int8_gemm_ring_kernel(GemmArgs p) {
 #pragma unroll
     for (int j = 0; j < C::W_LD; ++j) dma_w(j);
     advance_w();
+    if (NSA == 3) {
+#pragma unroll
+        for (int j = 0; j < C::A_LD; ++j) dma_a(j);
+        advance_a();
+    }
 #pragma unroll
     for (int j = 0; j < C::W_LD; ++j) dma_w(j);
     advance_w();
-    wait_vmcnt<C::W_LD>();
+    wait_vmcnt<(NSA == 3 ? C::A_LD : 0) + C::W_LD>();
     wg_barrier();
 #pragma unroll
     for (int j = 0; j < NF; ++j) f0[j] = frag(smem, smem + C::W_BASE, 0, j);
@@ -962,34 +1004,62 @@ __global__ void __launch_bounds__(256, 1) int8_gemm_ring_kernel(GemmArgs p) {
         // read, which would drain the DMA pipeline every iteration.
         __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0) only
 
+        int pa = 0;
         for (int kt = 0; kt < nk; ++kt) {
             const uint8_t* sa = smem + ca * C::A_STAGE;
             const uint8_t* sw = smem + C::W_BASE + cw * C::W_STAGE;
-            const int na = ca ^ 1, nw = cw == 2 ? 0 : cw + 1;
+            const int na = ca == NSA - 1 ? 0 : ca + 1, nw = cw == C::NSW - 1 ? 0 : cw + 1;
             wg_barrier();                                                   // X
-            substep(flag<true>{}, f0, f1, sa, sw, 1, 0);
-            substep(flag<true>{}, f1, f0, sa, sw, 2, NM);
-            substep(flag<true>{}, f0, f1, sa, sw, 3, 2 * NM);
-            wait_vmcnt<C::W_BEFORE_Y>();
+            substep(ic<0>{}, f0, f1, sa, sw, 1);
+            substep(ic<NM>{}, f1, f0, sa, sw, 2);
+            substep(ic<2 * NM>{}, f0, f1, sa, sw, 3);
+            wait_vmcnt<C::in_flight_at_y()>();
             wg_barrier();                                                   // Y
-            substep(flag<true>{}, f1, f0, smem + na * C::A_STAGE, smem + C::W_BASE + nw * C::W_STAGE, 0, 3 * NM);
+            substep(ic<3 * NM>{}, f1, f0, smem + na * C::A_STAGE, smem + C::W_BASE + nw * C::W_STAGE, 0);
             advance_a();
             advance_w();
+            pa = ca;
             ca = na;
             cw = nw;
         }
 
-        // epilogue of tile ti; the A stage that was just multiplied (ca ^ 1 after the swap) is the shuffle scratch.
+        // epilogue of tile ti; the A stage that was just multiplied is the shuffle scratch (8 KB per wave).
         // (The launcher only picks this kernel when the coalesced epilogue's alignment conditions hold.)
         int m0, n0;
         tile_origin(ti, m0, n0);
         __syncthreads();   // every wave is done reading that stage
         constexpr int SZ = (EPI == EPI_ACC || OUT_DT == DT_F32) ? 4 : 2;
-        constexpr int PW = 256 / SZ;   // 256-byte LDS rows: 8 KB per wave, 32 KB in all
+        constexpr int PW = C::piece_cols(SZ);
+        static_assert(32 * PW * SZ <= 8192, "shuffle piece");
         epilogue_shuffle<TM, TN, OUT_DT, EPI, PW>(p, acc, m0 + wm * C::WTM, n0 + wn * C::WTN, lane,
-                                                   smem + (ca ^ 1) * C::A_STAGE + wave * 8192);
+                                                   smem + pa * C::A_STAGE + wave * 8192);
     }
     wait_vmcnt<0>();   // no DMA may still be writing this workgroup's LDS when it retires
+}
+
+// Sum of the int32 planes of a split-K run, then the epilogue.  planes[s][M][N]; four consecutive n per thread.
+template <int OUT_DT, int EPI>
+__global__ void __launch_bounds__(256) splitk_epilogue_kernel(GemmArgs p, const int* planes, int slices) {
+    const int64_t nvec = (int64_t)p.M * p.N / 4, plane = (int64_t)p.M * p.N;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * 256) {
+        const int64_t o = i * 4;
+        const int m = (int)(o / p.N), n = (int)(o - (int64_t)m * p.N);
+        v4i acc = *reinterpret_cast<const v4i*>(planes + o);
+        for (int s = 1; s < slices; ++s) acc += *reinterpret_cast<const v4i*>(planes + s * plane + o);
+        if (EPI == EPI_ACC) {   // the caller asked for the accumulators themselves: no scales to apply
+            *reinterpret_cast<v4i*>((int*)p.D + o) = acc;
+            continue;
+        }
+        const float xs = p.xs[m];
+        const float4 w4 = *reinterpret_cast<const float4*>(p.ws + n);
+        const float ws[4] = {w4.x, w4.y, w4.z, w4.w};
+        float b[4] = {0.f, 0.f, 0.f, 0.f}, rs[4] = {0.f, 0.f, 0.f, 0.f}, res[4] = {0.f, 0.f, 0.f, 0.f}, out[4];
+        if (p.bias) load4<OUT_DT>(p.bias, n, b);
+        if (EPI == EPI_RESID) { load4<OUT_DT>(p.rscale, n, rs); load4<OUT_DT>(p.resid, o, res); }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) out[j] = epi_value<OUT_DT, EPI>(acc[j], xs, ws[j], b[j], rs[j], res[j]);
+        store4<OUT_DT>(p.D, o, out);
+    }
 }
 
 // Tile shapes.  L: the large-shape workhorse, one workgroup per CU, each of 4 waves owns a 128x128 accumulator tile
@@ -1018,33 +1088,86 @@ int launch_cfg(GemmArgs a, hipStream_t st) {
     return 0;
 }
 
-template <int OUT_DT, int EPI>
-int launch_ring(GemmArgs a, hipStream_t st) {
-    using C = RingCfg;
-    a.tiles_m = (a.M + C::BM - 1) / C::BM;
-    a.tiles_n = (a.N + C::BN - 1) / C::BN;
-    const int64_t ntiles = (int64_t)a.tiles_m * a.tiles_n;
-    if (ntiles > 0x7fffffff) return -1;
+int device_cu_count() {
     static int num_cu = 0;   // benign race: every thread computes the same value
     if (num_cu == 0) {
         int dev = 0, n = 0;
         if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
         num_cu = n;
     }
-    bool vec_ok, aligned;
-    epilogue_alignment<OUT_DT, EPI>(a, vec_ok, aligned);
-    if (!aligned) return launch_cfg<CfgL, OUT_DT, EPI>(a, st);   // the ring kernel has only the coalesced epilogue
-    auto kern = int8_gemm_ring_kernel<OUT_DT, EPI>;
-    static bool once = false;
+    return num_cu;
+}
+
+// Launches the persistent ring kernel on `slices` K slices (1 = whole K).  With slices > 1, EPI must be EPI_ACC and
+// a.D the int32 planes.
+template <class C, int OUT_DT, int EPI>
+int launch_ring_cfg(GemmArgs a, int slices, hipStream_t st) {
+    a.tiles_m = (a.M + C::BM - 1) / C::BM;
+    a.tiles_n = (a.N + C::BN - 1) / C::BN;
+    const int64_t ntiles = (int64_t)a.tiles_m * a.tiles_n;
+    if (ntiles > 0x7fffffff) return -1;
+    auto kern = int8_gemm_ring_kernel<C, OUT_DT, EPI>;
+    static bool once = false;  // benign race: the attribute is idempotent
     if (!once) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
         if (e != hipSuccess) return (int)e;
         once = true;
     }
-    const unsigned grid = (unsigned)(ntiles < num_cu ? ntiles : num_cu);
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(C::NT), C::SMEM, st, a);
+    const int num_cu = device_cu_count();
+    const int64_t per_slice = slices > 1 ? (num_cu / slices > 0 ? num_cu / slices : 1) : num_cu;
+    const unsigned grid = (unsigned)(ntiles < per_slice ? ntiles : per_slice);
+    hipLaunchKernelGGL(kern, dim3(grid, (unsigned)slices), dim3(C::NT), C::SMEM, st, a);
     KCHECK();
     return 0;
+}
+
+using RingL = RingCfg<256, 2, 2, 2>;    // 256x256, waves 2x2 of 128x128: the compute-bound workhorse
+using RingN96 = RingCfg<96, 4, 1, 3>;   // 256x96, waves 4x1 of 64x96: skinny M with enough columns for every CU
+using RingN128 = RingCfg<128, 4, 1, 3>; // 256x128, waves 4x1 of 64x128: skinny M, split K
+
+template <int OUT_DT, int EPI>
+int launch_ring(GemmArgs a, hipStream_t st) {
+    bool vec_ok, aligned;
+    epilogue_alignment<OUT_DT, EPI>(a, vec_ok, aligned);
+    if (!aligned) return launch_cfg<CfgL, OUT_DT, EPI>(a, st);   // the ring kernel has only the coalesced epilogue
+    return launch_ring_cfg<RingL, OUT_DT, EPI>(a, 1, st);
+}
+
+// M <= 256: one row of tiles, the weights are read once and the run is bound by how fast they stream.  Narrow tiles
+// give every CU a column slab; when N is too small for that, K is split as well: each slice writes an int32 plane
+// (exact, so the order of the sum does not matter) into a stream-ordered scratch allocation and a second kernel adds
+// the planes and applies the epilogue.
+template <int OUT_DT, int EPI>
+int launch_skinny(GemmArgs a, hipStream_t st) {
+    bool vec_ok, aligned;
+    epilogue_alignment<OUT_DT, EPI>(a, vec_ok, aligned);
+    if (!aligned) return launch_cfg<CfgM, OUT_DT, EPI>(a, st);
+    const int num_cu = device_cu_count();
+    const int t96 = (a.N + 95) / 96, t128 = (a.N + 127) / 128, nk = a.K / 128;
+    if (t96 * 4 >= num_cu * 3) return launch_ring_cfg<RingN96, OUT_DT, EPI>(a, 1, st);
+    int slices = num_cu / t128;
+    if (slices > nk) slices = nk;
+    if (slices <= 1) return launch_ring_cfg<RingN128, OUT_DT, EPI>(a, 1, st);
+    const int per = (nk + slices - 1) / slices;       // K tiles per slice
+    slices = (nk + per - 1) / per;                    // no empty slice
+    if (slices <= 1) return launch_ring_cfg<RingN128, OUT_DT, EPI>(a, 1, st);
+    int* planes = nullptr;
+    hipError_t e = hipMallocAsync((void**)&planes, (size_t)slices * a.M * a.N * sizeof(int), st);
+    if (e != hipSuccess) return (int)e;
+    GemmArgs pa = a;
+    pa.D = planes;
+    pa.kslice = per * 128;
+    int rc = launch_ring_cfg<RingN128, DT_F32, EPI_ACC>(pa, slices, st);
+    if (rc == 0) {
+        const int64_t nvec = (int64_t)a.M * a.N / 4;
+        const unsigned grid = (unsigned)((nvec + 255) / 256 < 4096 ? (nvec + 255) / 256 : 4096);
+        hipLaunchKernelGGL((splitk_epilogue_kernel<OUT_DT, EPI>), dim3(grid), dim3(256), 0, st, a, (const int*)planes, slices);
+        hipError_t le = hipGetLastError();
+        if (le != hipSuccess) rc = (int)le;
+    }
+    e = hipFreeAsync(planes, st);
+    if (rc == 0 && e != hipSuccess) rc = (int)e;
+    return rc;
 }
 
 template <class C, int OUT_DT, int EPI>
@@ -1071,8 +1194,9 @@ int g_force_cfg = -1;
 int choose_cfg(int64_t M, int64_t N, int64_t K) {
     const bool dma_ok = M * K < ((int64_t)1 << 32) && N * K < ((int64_t)1 << 32);   // 32-bit lane offsets
     if (!dma_ok && g_force_cfg >= 3) return 0;
-    if (g_force_cfg == 4 || g_force_cfg == 5) return (K % 128) == 0 ? g_force_cfg : 0;
+    if (g_force_cfg >= 4) return (K % 128) == 0 ? g_force_cfg : 0;
     if (g_force_cfg >= 0) return (g_force_cfg == 3 && (K % 64) != 0) ? 0 : g_force_cfg;
+    if (M <= 256 && N >= 1024 && (K % 128) == 0 && K >= 512 && dma_ok) return 6;
     const int64_t tiles_l = ((M + 255) / 256) * ((N + 255) / 256);
     if (M >= 512 && N >= 512 && tiles_l >= 192) return !dma_ok ? 0 : (K % 128) == 0 ? 5 : (K % 64) == 0 ? 3 : 0;
     const int64_t tiles_m = ((M + 127) / 128) * ((N + 127) / 128);
@@ -1086,6 +1210,7 @@ int dispatch_cfg(const GemmArgs& a, hipStream_t st) {
         case 3: return launch_dma<DmaL, OUT_DT, EPI>(a, st);
         case 4: return launch_dma2<Dma2L, OUT_DT, EPI>(a, st);
         case 5: return launch_ring<OUT_DT, EPI>(a, st);
+        case 6: return launch_skinny<OUT_DT, EPI>(a, st);
         case 0: return launch_cfg<CfgL, OUT_DT, EPI>(a, st);
         case 1: return launch_cfg<CfgM, OUT_DT, EPI>(a, st);
         default: return launch_cfg<CfgS, OUT_DT, EPI>(a, st);
@@ -1126,7 +1251,7 @@ GPU_API int gpu_int8_gemm(const int8_t* A, const int8_t* W, const float* xs, con
                           int64_t M, int64_t N, int64_t K, int out_dt, void* stream) {
     if (M == 0 || N == 0 || K == 0) return 0;  // csrc/vendor/cutlass_gemm_int8.cu:377
     if (out_dt < DT_F32 || out_dt > DT_BF16 || M < 0 || N < 0 || K < 0 || !shape_ok(M, N, K)) return -200;
-    GemmArgs a{A, W, xs, ws, bias, nullptr, nullptr, D, (int)M, (int)N, (int)K, 0, 0};
+    GemmArgs a{A, W, xs, ws, bias, nullptr, nullptr, D, (int)M, (int)N, (int)K, 0, 0, 0};
     const int rc = dispatch_dt<EPI_PLAIN>(a, out_dt, (hipStream_t)stream);
     return rc < 0 ? -200 : rc;
 }
@@ -1137,7 +1262,7 @@ GPU_API int gpu_int8_gemm_residual(const int8_t* A, const int8_t* W, const float
     if (M == 0 || N == 0) return 0;                       // csrc/vendor/cutlass_gemm_int8.cu:353
     if (K == 0 || !rscale || !resid) return -201;         // :355-357
     if (out_dt < DT_F32 || out_dt > DT_BF16 || M < 0 || N < 0 || K < 0 || !shape_ok(M, N, K)) return -201;
-    GemmArgs a{A, W, xs, ws, bias, rscale, resid, D, (int)M, (int)N, (int)K, 0, 0};
+    GemmArgs a{A, W, xs, ws, bias, rscale, resid, D, (int)M, (int)N, (int)K, 0, 0, 0};
     const int rc = dispatch_dt<EPI_RESID>(a, out_dt, (hipStream_t)stream);
     return rc < 0 ? -201 : rc;
 }
@@ -1145,7 +1270,7 @@ GPU_API int gpu_int8_gemm_residual(const int8_t* A, const int8_t* W, const float
 GPU_API int gpu_int8_gemm_acc(const int8_t* A, const int8_t* W, int32_t* acc, int64_t M, int64_t N, int64_t K, void* stream) {
     if (M == 0 || N == 0 || K == 0) return 0;
     if (M < 0 || N < 0 || K < 0 || !shape_ok(M, N, K)) return -200;
-    GemmArgs a{A, W, nullptr, nullptr, nullptr, nullptr, nullptr, acc, (int)M, (int)N, (int)K, 0, 0};
+    GemmArgs a{A, W, nullptr, nullptr, nullptr, nullptr, nullptr, acc, (int)M, (int)N, (int)K, 0, 0, 0};
     const int rc = dispatch_cfg<DT_F32, EPI_ACC>(a, (hipStream_t)stream);
     return rc < 0 ? -200 : rc;
 }

@@ -82,8 +82,9 @@ int gpu_w6_decode(const void* q, const void* s_rel, void* out, int64_t N, int K,
 /* The int32 accumulators of gpu_int8_gemm, before the epilogue: acc[M,N] = A . W^T.  For bit-exact checks. */
 int gpu_int8_gemm_acc(const int8_t* A, const int8_t* W, int32_t* acc, int64_t M, int64_t N, int64_t K, void* stream);
 
-/* Test and tuning hook: force the GEMM tile configuration (0 = 256x256, 1 = 128x128, 2 = 64x64 register-staged; 3 = 256x256
- * direct-to-LDS pipelined; -1 = automatic). */
+/* Test and tuning hook: force the GEMM kernel family.  0, 1, 2 = 256x256, 128x128, 64x64 register-staged tiles;
+ * 3, 4 = 256x256 direct-to-LDS with 64- and 128-byte rows; 5 = persistent ring kernel; 6 = narrow-tile / split-K
+ * ring kernel for M <= 256; -1 = automatic.  Shapes a family cannot run fall back to 0. */
 int gpu_int8_gemm_force_config(int cfg);
 
 /* Writes, for each of the 64 lanes and 16 accumulator registers of one v_mfma_i32_32x32x32_i8, the (row of src0,

@@ -182,10 +182,11 @@ def rand_i8(seed, stream, M, K, lo=-128, hi=127):
 
 
 ACC_CASES = [(1, 96, 256), (3, 32, 16), (64, 64, 64), (65, 72, 48), (100, 104, 320), (130, 260, 80), (257, 96, 3072),
-             (300, 520, 192), (33, 8, 1024), (260, 300, 64), (512, 256, 128), (777, 1000, 448), (300, 260, 384), (1100, 1500, 256)]
+             (300, 520, 192), (33, 8, 1024), (260, 300, 64), (512, 256, 128), (777, 1000, 448), (300, 260, 384), (1100, 1500, 256), (200, 1056, 256), (256, 2048, 1536), (1, 1024, 512),
+             (77, 4096, 1280), (250, 25000, 128)]
 
 
-@pytest.mark.parametrize("cfg", [2, 1, 0, 3, 4, 5])
+@pytest.mark.parametrize("cfg", [2, 1, 0, 3, 4, 5, 6])
 @pytest.mark.parametrize("M,N,K", ACC_CASES)
 def test_int8_gemm_acc_bit_exact(M, N, K, cfg):
     say("gemm_acc", M, N, K, "cfg", cfg)
@@ -204,7 +205,7 @@ def test_int8_gemm_acc_bit_exact(M, N, K, cfg):
 
 
 @pytest.mark.parametrize("out_dt", [BF16, F16, F32])
-@pytest.mark.parametrize("M,N,K,with_bias", [(37, 96, 256, True), (130, 264, 192, False), (256, 1024, 1024, True)])
+@pytest.mark.parametrize("M,N,K,with_bias", [(37, 96, 256, True), (130, 264, 192, False), (256, 1024, 1024, True), (100, 2048, 1024, True)])
 def test_int8_gemm_epilogue(M, N, K, with_bias, out_dt):
     say("gemm", M, N, K, with_bias, out_dt)
     A = rand_i8(2, 1, M, K, -127, 127)
@@ -215,7 +216,7 @@ def test_int8_gemm_epilogue(M, N, K, with_bias, out_dt):
     bias = tob(synth.normal(2, 5, N) * np.float32(0.02)) if with_bias else None
     want = oracle.int8_gemm(A, W, xs, ws, bias, out_dt, fma=1)
     loose = oracle.int8_gemm(A, W, xs, ws, bias, out_dt, fma=0)
-    for cfg in (-1, 0, 1, 2, 3, 4, 5):
+    for cfg in (-1, 0, 1, 2, 3, 4, 5, 6):
         ffi.raw("gpu_int8_gemm_force_config", cfg)
         try:
             got = ql.int8_gemm(dev(A), dev(W), dev(xs), dev(ws), None if bias is None else dev_bits(bias, out_dt), TDT[out_dt])
