@@ -1151,6 +1151,17 @@ int launch_skinny(GemmArgs a, hipStream_t st) {
     const int per = (nk + slices - 1) / slices;       // K tiles per slice
     slices = (nk + per - 1) / per;                    // no empty slice
     if (slices <= 1) return launch_ring_cfg<RingN128, OUT_DT, EPI>(a, 1, st);
+    // Keep freed scratch in the device's default pool instead of returning it to the driver at every synchronization,
+    // as the reference's runtime layer does at start-up (src/cuda.rs:88-97): otherwise each call pays a fresh allocation.
+    static bool pool_set = false;   // benign race: the attribute is idempotent
+    if (!pool_set) {
+        int dev = 0;
+        hipMemPool_t pool;
+        uint64_t keep = ~(uint64_t)0;
+        if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetDefaultMemPool(&pool, dev) == hipSuccess)
+            (void)hipMemPoolSetAttribute(pool, hipMemPoolAttrReleaseThreshold, &keep);
+        pool_set = true;
+    }
     int* planes = nullptr;
     hipError_t e = hipMallocAsync((void**)&planes, (size_t)slices * a.M * a.N * sizeof(int), st);
     if (e != hipSuccess) return (int)e;

@@ -72,7 +72,11 @@ template <int MODE> __device__ __forceinline__ void load16(const void* x, int64_
     }
 }
 
-// Rotate one chunk held as v[16] per lane (element 16*lane + i).  wl is the wave's LDS tile.  Uniform over the block.
+// Rotate one chunk held as v[16] per lane (element 16*lane + i).  wl is the wave's LDS tile.
+// The LDS tile is private to the wave and the LDS unit executes one wave's accesses in program order, so between the
+// phases of rotate_chunk it is enough to stop the compiler from reordering them: no workgroup barrier is needed.
+#define LDS_WAVE_ORDER() asm volatile("" ::: "memory")
+
 template <int G> __device__ __forceinline__ void rotate_chunk(float* v, float* wl, int lane) {
     // strides 1 and 4: inside the lane
 #pragma unroll
@@ -83,7 +87,7 @@ template <int G> __device__ __forceinline__ void rotate_chunk(float* v, float* w
 #pragma unroll
     for (int i = 0; i < 4; ++i)
         *reinterpret_cast<float4*>(wl + lds_pos(16 * lane + 4 * i)) = make_float4(v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]);
-    __syncthreads();
+    LDS_WAVE_ORDER();
     if (G == 256) {
         // lane (R = lane/16, b = lane%16) takes elements R*256 + a*16 + b, a = 0..15: strides 16 and 64 are lane-local
         const int base = (lane >> 4) * 256 + (lane & 15);
@@ -134,13 +138,13 @@ template <int G> __device__ __forceinline__ void rotate_chunk(float* v, float* w
 #pragma unroll
             for (int d = 0; d < 4; ++d) *reinterpret_cast<float2*>(wl + lds_pos(base + t * 64 + d * 16)) = w[t][d];
     }
-    __syncthreads();
+    LDS_WAVE_ORDER();
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const float4 f = *reinterpret_cast<float4*>(wl + lds_pos(16 * lane + 4 * i));
         v[4 * i] = f.x; v[4 * i + 1] = f.y; v[4 * i + 2] = f.z; v[4 * i + 3] = f.w;
     }
-    __syncthreads();
+    LDS_WAVE_ORDER();
 }
 
 __device__ __forceinline__ float wave_max(float v) {

@@ -55,4 +55,22 @@ GPU_API int gpu_w6_decode(const void* q, const void* s_rel, void* out, int64_t N
     return 0;
 }
 
+// The W6A8 linear as the reference's model code issues it (src/h3.rs:1208-1216,1251): expand the packed weights to the
+// int8 grid, then the ordinary int8 GEMM with the per-row s_channel as the weight scale.  The expanded weights live in
+// a stream-ordered scratch allocation that is released on the same stream.
+GPU_API int gpu_w6a8_gemm(const int8_t* A, const void* wq, const void* s_rel, int G, const float* xs, const float* s_channel,
+                          const void* bias, void* D, int64_t M, int64_t N, int64_t K, int out_dt, void* stream) {
+    if (K % 32 || G % 16 || K > 0x7fffffff) return -1;
+    if (M == 0 || N == 0 || K == 0) return 0;
+    hipStream_t st = (hipStream_t)stream;
+    int8_t* w8 = nullptr;
+    hipError_t e = hipMallocAsync((void**)&w8, (size_t)N * (size_t)K, st);
+    if (e != hipSuccess) return (int)e;
+    int rc = gpu_w6_decode(wq, s_rel, w8, N, (int)K, G, stream);
+    if (rc == 0) rc = gpu_int8_gemm(A, w8, xs, s_channel, bias, D, M, N, K, out_dt, stream);
+    e = hipFreeAsync(w8, st);
+    if (rc == 0 && e != hipSuccess) rc = (int)e;
+    return rc;
+}
+
 GPU_API const char* gpu_kernels_build_info(void) { return "gpu_kernels gfx950 quantized-linear " __DATE__; }

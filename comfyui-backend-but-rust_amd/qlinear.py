@@ -79,6 +79,16 @@ def w6_decode(wq, s_rel, N, K, G):
     return out
 
 
+def w6a8_gemm(A, wq, s_rel, G, xs, s_channel, bias=None, out_dtype=torch.bfloat16):
+    """W6A8 linear on already-quantized rows: packed two-plane weights wq [N, 3K/4], e4m3 s_rel [N, K/G], f32 s_channel."""
+    M, K = A.shape
+    N = wq.shape[0]
+    D = torch.empty((M, N), dtype=out_dtype, device=A.device)
+    ffi.k("gpu_w6a8_gemm", _ptr(A), _ptr(wq), _ptr(s_rel), G, _ptr(xs), _ptr(s_channel), _ptr(bias), _ptr(D), M, N, K,
+          _TORCH_DT[out_dtype], _stream())
+    return D
+
+
 def linear_w8a8(x, W, ws, bias=None, rotate=0, out_dtype=None):
     """One W8A8 linear: y = dequant(quant(x) . W^T)."""
     q, xs = quant_rows(x, rotate)

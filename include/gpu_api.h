@@ -82,6 +82,12 @@ int gpu_w6_decode(const void* q, const void* s_rel, void* out, int64_t N, int K,
 /* The int32 accumulators of gpu_int8_gemm, before the epilogue: acc[M,N] = A . W^T.  For bit-exact checks. */
 int gpu_int8_gemm_acc(const int8_t* A, const int8_t* W, int32_t* acc, int64_t M, int64_t N, int64_t K, void* stream);
 
+/* One W6A8 linear in a single call: gpu_w6_decode into a stream-ordered scratch buffer, then gpu_int8_gemm with
+ * ws = s_channel (the call pattern of src/h3.rs:1208-1216,1251).  Returns -1 for K % 32 or G % 16, otherwise as
+ * gpu_int8_gemm. */
+int gpu_w6a8_gemm(const int8_t* A, const void* wq, const void* s_rel, int G, const float* xs, const float* s_channel,
+                  const void* bias, void* D, int64_t M, int64_t N, int64_t K, int out_dt, void* stream);
+
 /* Test and tuning hook: force the GEMM kernel family.  0, 1, 2 = 256x256, 128x128, 64x64 register-staged tiles;
  * 3, 4 = 256x256 direct-to-LDS with 64- and 128-byte rows; 5 = persistent ring kernel; 6 = narrow-tile / split-K
  * ring kernel for M <= 256; -1 = automatic.  Shapes a family cannot run fall back to 0. */

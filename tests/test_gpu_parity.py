@@ -302,6 +302,27 @@ def test_w6_decode_exhaustive_and_random():
     assert np.array_equal(got.cpu().numpy(), want)
 
 
+def test_w6a8_linear_matches_decode_then_gemm():
+    """The H3-style W6A8 linear (src/h3.rs:1208-1251): rows quantized with the 256-wide rotation, weights decoded from
+    the packed planes, per-row s_channel as the weight scale."""
+    M, K, N, G = 300, 1536, 640, 32
+    xb = synth.bf16_bits(synth.activations(8, M, K, "t3"))
+    codes = (synth.w6_codes(8, N, K).astype(np.int16) + 32).astype(np.uint8)
+    wq = oracle.w6_pack_planes(codes)
+    s_rel = synth.w6_srel_bytes(8, N, K, G)
+    s_ch = synth.uniform(8, 30, N, 1e-3, 1e-2)
+    bias = synth.bf16_bits(synth.normal(8, 31, N) * np.float32(0.02))
+    rc, q, xs = oracle.quant_rows(BF16, xb, K, 1)
+    rc2, w8 = oracle.w6_decode(wq, s_rel, N, K, G)
+    assert rc == 0 and rc2 == 0
+    want = oracle.int8_gemm(q, w8, xs, s_ch, bias, BF16, fma=1)
+    qd, xsd = ql.quant_rows(dev_bits(xb, BF16), 1)
+    got = ql.w6a8_gemm(qd, dev(wq), dev(s_rel), G, xsd, dev(s_ch), dev_bits(bias, BF16))
+    torch.cuda.synchronize()
+    assert np.array_equal(host_bits(got), want)
+    assert ffi.raw("gpu_w6a8_gemm", 0, 0, 0, 32, 0, 0, 0, 0, 4, 8, 48, 2, 0) == -1
+
+
 # ------------------------------------------------------------------------------------------------ full-size shapes
 FULL = [  # (name, M, K, N, rotate, kind)
     ("dit mlp up", 4608, 3072, 12288, 128, "t3"),
