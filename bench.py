@@ -136,6 +136,13 @@ def main():
     value = ops / (ms_per_step * 1e-3) / 1e12
     gemm_tops = ops / (tg * 1e-3) / 1e12
     quant_bytes = M * K * 2 + M * K + M * 4
+    traffic = None   # HBM bytes per GEMM launch, measured off-line with rocprofv3 counters (profiles/hbm_traffic.json)
+    try:
+        with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
+            rec = json.load(f).get("int8_gemm M%d K%d N%d bf16" % (M, K, N))
+        traffic = rec["bytes"] if rec else None
+    except (OSError, ValueError):
+        pass
     out = {
         "metric": "W8A8 linear TOPS @M%d K%d N%d (quantize + int8 GEMM + dequant epilogue)" % (M, K, N),
         "value": round(value, 2), "unit": "TOPS", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
@@ -144,9 +151,10 @@ def main():
         "config": {"workload": "image-DiT MLP up-projection W8A8 linear, bf16 activations M=%d K=%d -> N=%d, Hadamard "
                                "block %d, per-channel scales, bf16 bias and output" % (M, K, N, a.rotate),
                    "M": M, "K": K, "N": N, "rotate": a.rotate},
-        "roofline": {"bound": "mfma", "kernel": "int8_gemm_kernel (gpu_int8_gemm)", "achieved": round(gemm_tops, 2),
+        "roofline": {"bound": "mfma", "kernel": "int8_gemm_ring_kernel (gpu_int8_gemm)", "achieved": round(gemm_tops, 2),
                      "peak": PEAK_INT8_TOPS, "unit": "TFLOP/s", "frac": round(gemm_tops / PEAK_INT8_TOPS, 4),
-                     "traffic": None, "avg_launch_us": round(tg * 1e3, 2)},
+                     "traffic": traffic, "avg_launch_us": round(tg * 1e3, 2),
+                     "algorithmic_ops": ops, "algorithmic_bytes": M * K + M * 4 + N * K + N * 4 + N * 2 + M * N * 2},
         "kernels": {"quant_rows_us": round(tq * 1e3, 2), "quant_rows_GBs": round(quant_bytes / (tq * 1e-3) / 1e9, 1),
                     "int8_gemm_us": round(tg * 1e3, 2), "gpu_ms_total": round(gpu_ms, 4)},
     }
