@@ -32,6 +32,13 @@ __device__ __forceinline__ uint16_t f_to_f16(float v) {
     return __builtin_bit_cast(uint16_t, (_Float16)v);
 }
 
+// Two floats -> packed bf16 pair (a in the low half), one v_cvt_pk_bf16_f32.
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, bf16x2));
+}
+
 // Round a float to the precision of the dtype code and widen back (rnd<T>, csrc/common.cuh:25-28).
 template <int DT> __device__ __forceinline__ float rnd_dt(float v) {
     if (DT == DT_BF16) return bf16_to_f(f_to_bf16(v));

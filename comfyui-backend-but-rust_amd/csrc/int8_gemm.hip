@@ -13,6 +13,8 @@
 
 namespace {
 
+__device__ __forceinline__ void store16_untracked(void* ptr, uint4 v);
+
 enum { EPI_PLAIN = 0, EPI_RESID = 1, EPI_ACC = 2 };
 
 struct GemmArgs {
@@ -86,8 +88,8 @@ template <int OUT_DT> __device__ __forceinline__ void store4(void* p, int64_t i,
         *reinterpret_cast<float4*>((float*)p + i) = make_float4(v[0], v[1], v[2], v[3]);
     } else if (OUT_DT == DT_BF16) {
         uint2 u;
-        u.x = (uint32_t)f_to_bf16(v[0]) | ((uint32_t)f_to_bf16(v[1]) << 16);
-        u.y = (uint32_t)f_to_bf16(v[2]) | ((uint32_t)f_to_bf16(v[3]) << 16);
+        u.x = pack_bf16x2(v[0], v[1]);
+        u.y = pack_bf16x2(v[2], v[3]);
         *reinterpret_cast<uint2*>((uint16_t*)p + i) = u;
     } else {
         uint2 u;
@@ -168,7 +170,7 @@ __device__ __forceinline__ void epilogue_store(const GemmArgs& p, v16i (&acc)[TN
 // writes whole rows: 16 bytes per lane, consecutive lanes on consecutive addresses.  For the residual form the LDS
 // holds z = Out(acc*xs*ws + bias), exactly the intermediate the reference rounds, and fma(z, rscale, resid) is applied
 // on the way out.  Needs row starts of D (and resid) 16-byte aligned; the caller falls back to epilogue_store otherwise.
-template <int TM, int TN, int OUT_DT, int EPI, int PW = TN * 32>
+template <int TM, int TN, int OUT_DT, int EPI, int PW = TN * 32, bool UNTRACKED = false>
 __device__ __forceinline__ void epilogue_shuffle(const GemmArgs& p, v16i (&acc)[TN][TM], int mb, int nb, int lane, uint8_t* wl) {
     // a piece is 32 rows x PW columns of the wave tile: PW*SZ bytes per LDS row, 32*PW*SZ bytes per wave
     constexpr int SZ = (EPI == EPI_ACC || OUT_DT == DT_F32) ? 4 : 2;
@@ -251,14 +253,16 @@ __device__ __forceinline__ void epilogue_shuffle(const GemmArgs& p, v16i (&acc)[
             else rv[t] = make_uint4(0, 0, 0, 0);
         }
     };
-    uint4 rv_next[PASSES];
-    if (EPI == EPI_RESID) load_resid(0, 0, rv_next);
 
 #pragma unroll
     for (int im = 0; im < TM; ++im) {
         const float xs = xsr[im];
 #pragma unroll
         for (int np = 0; np < NP; ++np) {
+            // The residual rows of this piece are requested before its write phase, whose arithmetic covers their latency
+            // (and that of the previous piece's stores, which retire ahead of them).
+            uint4 rv[PASSES];
+            if (EPI == EPI_RESID) load_resid(im, np, rv);
             // write phase: row frow of the piece
 #pragma unroll
             for (int ip = 0; ip < TNP; ++ip)
@@ -276,24 +280,14 @@ __device__ __forceinline__ void epilogue_shuffle(const GemmArgs& p, v16i (&acc)[
                         if (OUT_DT == DT_F32) {
                             *reinterpret_cast<float4*>(dst) = make_float4(o[0], o[1], o[2], o[3]);
                         } else if (OUT_DT == DT_BF16) {
-                            *reinterpret_cast<uint2*>(dst) = make_uint2((uint32_t)f_to_bf16(o[0]) | ((uint32_t)f_to_bf16(o[1]) << 16),
-                                                                        (uint32_t)f_to_bf16(o[2]) | ((uint32_t)f_to_bf16(o[3]) << 16));
+                            *reinterpret_cast<uint2*>(dst) = make_uint2(pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]));
                         } else {
                             *reinterpret_cast<uint2*>(dst) = make_uint2((uint32_t)f_to_f16(o[0]) | ((uint32_t)f_to_f16(o[1]) << 16),
                                                                         (uint32_t)f_to_f16(o[2]) | ((uint32_t)f_to_f16(o[3]) << 16));
                         }
                     }
-                    SCHED_FENCE();
                 }
             asm volatile("" ::: "memory");   // the wave's own LDS writes are ordered before its reads by the LDS queue
-            // residual of this piece was requested one piece ago; request the next piece's before this piece's stores
-            uint4 rv[PASSES];
-            if (EPI == EPI_RESID) {
-#pragma unroll
-                for (int t = 0; t < PASSES; ++t) rv[t] = rv_next[t];
-                const int nxt = im * NP + np + 1;
-                if (nxt < TM * NP) load_resid(nxt / NP, nxt % NP, rv_next);
-            }
             // read phase: whole rows out
             const int ncol = nb + np * PW + rc * EPC;
 #pragma unroll
@@ -304,7 +298,8 @@ __device__ __forceinline__ void epilogue_shuffle(const GemmArgs& p, v16i (&acc)[
                 if (m >= p.M || ncol >= p.N) continue;
                 const int64_t o = (int64_t)m * p.N + ncol;
                 if (EPI != EPI_RESID) {
-                    *reinterpret_cast<uint4*>((uint8_t*)p.D + o * SZ) = v;
+                    if (UNTRACKED) store16_untracked((uint8_t*)p.D + o * SZ, v);
+                    else *reinterpret_cast<uint4*>((uint8_t*)p.D + o * SZ) = v;
                 } else {
                     const uint32_t zw[4] = {v.x, v.y, v.z, v.w}, rw[4] = {rv[t].x, rv[t].y, rv[t].z, rv[t].w};
                     uint32_t ow[4];
@@ -317,7 +312,7 @@ __device__ __forceinline__ void epilogue_shuffle(const GemmArgs& p, v16i (&acc)[
                             float z0, z1, r0, r1;
                             if (OUT_DT == DT_BF16) {
                                 z0 = u2f(zw[j] << 16); z1 = u2f(zw[j] & 0xffff0000u); r0 = u2f(rw[j] << 16); r1 = u2f(rw[j] & 0xffff0000u);
-                                ow[j] = (uint32_t)f_to_bf16(__builtin_fmaf(z0, rs[np][2 * j], r0)) | ((uint32_t)f_to_bf16(__builtin_fmaf(z1, rs[np][2 * j + 1], r1)) << 16);
+                                ow[j] = pack_bf16x2(__builtin_fmaf(z0, rs[np][2 * j], r0), __builtin_fmaf(z1, rs[np][2 * j + 1], r1));
                             } else {
                                 z0 = f16_to_f((uint16_t)(zw[j] & 0xffffu)); z1 = f16_to_f((uint16_t)(zw[j] >> 16));
                                 r0 = f16_to_f((uint16_t)(rw[j] & 0xffffu)); r1 = f16_to_f((uint16_t)(rw[j] >> 16));
@@ -325,7 +320,8 @@ __device__ __forceinline__ void epilogue_shuffle(const GemmArgs& p, v16i (&acc)[
                             }
                         }
                     }
-                    *reinterpret_cast<uint4*>((uint8_t*)p.D + o * SZ) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+                    if (UNTRACKED) store16_untracked((uint8_t*)p.D + o * SZ, make_uint4(ow[0], ow[1], ow[2], ow[3]));
+                    else *reinterpret_cast<uint4*>((uint8_t*)p.D + o * SZ) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
                 }
                 SCHED_FENCE();
             }
@@ -493,6 +489,12 @@ __global__ void __launch_bounds__(C::NT, C::OCC) int8_gemm_kernel(GemmArgs p) {
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef const __attribute__((address_space(1))) void* glb_ptr_t;
 
+
+// 16-byte global store the compiler's wait-count bookkeeping does not see (see the ring kernel's epilogue)
+__device__ __forceinline__ void store16_untracked(void* ptr, uint4 v) {
+    const v4i d = v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+    asm volatile("global_store_dwordx4 %0, %1, off" ::"v"(ptr), "v"(d) : "memory");
+}
 
 template <int N> __device__ __forceinline__ void wait_vmcnt() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
 // vmcnt wait whose count is only known at run time (a multiple of a tile's DMA count): pick the immediate by switch
@@ -999,10 +1001,10 @@ __global__ void __launch_bounds__(256, 1) int8_gemm_ring_kernel(GemmArgs p) {
             for (int im = 0; im < TM; ++im)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc[in][im][r] = 0;
-        // A wait the compiler can see: without it, it assumes that loads and stores of the previous tile's epilogue may
-        // still be pending at the K loop's header and parks a vmcnt(0) inside the loop, in front of the first fragment
-        // read, which would drain the DMA pipeline every iteration.
-        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0) only
+        // The epilogue's stores are issued from inline assembly: were they visible to the compiler, it would assume
+        // them pending at the K loop's header and park a vmcnt(0) inside the loop, in front of the first fragment read,
+        // draining the DMA pipeline every iteration.  (Waits it derives for its own loads stay correct: the memory
+        // counter retires in order, so instructions it does not know about only make those waits stricter.)
 
         int pa = 0;
         for (int kt = 0; kt < nk; ++kt) {
@@ -1031,8 +1033,12 @@ __global__ void __launch_bounds__(256, 1) int8_gemm_ring_kernel(GemmArgs p) {
         constexpr int SZ = (EPI == EPI_ACC || OUT_DT == DT_F32) ? 4 : 2;
         constexpr int PW = C::piece_cols(SZ);
         static_assert(32 * PW * SZ <= 8192, "shuffle piece");
-        epilogue_shuffle<TM, TN, OUT_DT, EPI, PW>(p, acc, m0 + wm * C::WTM, n0 + wn * C::WTN, lane,
-                                                   smem + pa * C::A_STAGE + wave * 8192);
+        epilogue_shuffle<TM, TN, OUT_DT, EPI, PW, true>(p, acc, m0 + wm * C::WTM, n0 + wn * C::WTN, lane,
+                                                         smem + pa * C::A_STAGE + wave * 8192);
+        // The first fragments of the next tile were prefetched by the last sub-step; fetching them again here instead of
+        // carrying 32 registers across the epilogue keeps the epilogue free of spills.
+#pragma unroll
+        for (int j = 0; j < NF; ++j) f0[j] = frag(smem + ca * C::A_STAGE, smem + C::W_BASE + cw * C::W_STAGE, 0, j);
     }
     wait_vmcnt<0>();   // no DMA may still be writing this workgroup's LDS when it retires
 }
