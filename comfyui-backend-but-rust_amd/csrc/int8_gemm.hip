@@ -493,7 +493,9 @@ typedef const __attribute__((address_space(1))) void* glb_ptr_t;
 // 16-byte global store the compiler's wait-count bookkeeping does not see (see the ring kernel's epilogue)
 __device__ __forceinline__ void store16_untracked(void* ptr, uint4 v) {
     const v4i d = v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w};
-    asm volatile("global_store_dwordx4 %0, %1, off" ::"v"(ptr), "v"(d) : "memory");
+    // The trailing s_nop is the wait state the hardware needs between a store of more than 8 bytes and a write to its
+    // data registers; the compiler inserts it for its own stores but cannot see into this one.
+    asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 0" ::"v"(ptr), "v"(d) : "memory");
 }
 
 template <int N> __device__ __forceinline__ void wait_vmcnt() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }

@@ -204,6 +204,34 @@ def test_int8_gemm_acc_bit_exact(M, N, K, cfg):
     assert np.array_equal(got.cpu().numpy(), want)
 
 
+# More 256x256 tiles than CUs, and not a multiple of the CU count: the persistent kernel's workgroups then own unequal
+# numbers of tiles, and every output form runs through its coalesced epilogue.
+MANY_TILE_CASES = [(4352, 4096, 256), (4100, 4400, 384), (2304, 8200, 640)]
+
+
+@pytest.mark.parametrize("M,N,K", MANY_TILE_CASES)
+def test_int8_gemm_many_tiles_bit_exact(M, N, K):
+    say("gemm_many_tiles", M, N, K)
+    A = rand_i8(4, 500 + M, M, K)
+    W = rand_i8(4, 600 + N, N, K)
+    want = oracle.int8_gemm_acc(A, W)
+    xs = synth.uniform(4, 3, M, 0.005, 0.2)
+    ws = synth.uniform(4, 4, N, 1e-3, 1e-2)
+    bias = oracle.bf16_bits(synth.normal(4, 5, N) * np.float32(0.02))
+    rscale = oracle.bf16_bits(synth.normal(4, 6, N))
+    resid = oracle.bf16_bits(synth.normal(4, 7, M * N).reshape(M, N))
+    want_d = oracle.epilogue(want, xs, ws, bias, BF16, fma=1)
+    want_r = oracle.epilogue_residual(want, xs, ws, bias, rscale, resid, BF16, fma=1)
+    Ad, Wd = dev(A), dev(W)
+    got = ql.int8_gemm_acc(Ad, Wd)
+    d = ql.int8_gemm(Ad, Wd, dev(xs), dev(ws), dev_bits(bias, BF16), torch.bfloat16)
+    r = ql.int8_gemm_residual(Ad, Wd, dev(xs), dev(ws), dev_bits(bias, BF16), dev_bits(rscale, BF16), dev_bits(resid, BF16))
+    torch.cuda.synchronize()
+    assert np.array_equal(got.cpu().numpy(), want)
+    assert np.array_equal(host_bits(d), want_d)
+    assert np.array_equal(host_bits(r), want_r)
+
+
 @pytest.mark.parametrize("out_dt", [BF16, F16, F32])
 @pytest.mark.parametrize("M,N,K,with_bias", [(37, 96, 256, True), (130, 264, 192, False), (256, 1024, 1024, True), (100, 2048, 1024, True)])
 def test_int8_gemm_epilogue(M, N, K, with_bias, out_dt):
@@ -350,7 +378,7 @@ def test_full_size_linear_rows_against_oracle(name, M, K, N, rotate, kind):
     acc = ql.int8_gemm_acc(qd, Wd)
     torch.cuda.synchronize()
     assert np.array_equal(qd.cpu().numpy(), q) and np.array_equal(xsd.cpu().numpy(), xs)
-    rows = sorted(set([0, 1, 31, 32, 127, 128, 255, M // 2, M - 129, M - 2, M - 1]))
+    rows = sorted(set([0, 1, 31, 32, 127, 128, 255, M // 2, M - 129, M - 2, M - 1] + list(range(5, M, 256))))   # every tile row
     want = oracle.int8_gemm(q[rows], W, xs[rows], ws, bias, BF16, fma=1)
     got = host_bits(d[torch.tensor(rows, device=DEV)])
     assert np.array_equal(got, want)
@@ -358,3 +386,12 @@ def test_full_size_linear_rows_against_oracle(name, M, K, N, rotate, kind):
     want_rowsum = q.astype(np.int64) @ colsum
     got_rowsum = acc.to(torch.int64).sum(dim=1).cpu().numpy()
     assert np.array_equal(got_rowsum, want_rowsum)
+    # every kernel family that can run the shape gives the same bits
+    for cfg in (0, 3, 5) if M > 256 else (6, 1):
+        ffi.raw("gpu_int8_gemm_force_config", cfg)
+        try:
+            d2 = ql.int8_gemm(qd, Wd, xsd, wsd, bd, torch.bfloat16)
+            torch.cuda.synchronize()
+        finally:
+            ffi.raw("gpu_int8_gemm_force_config", -1)
+        assert torch.equal(d2.view(torch.int16), d.view(torch.int16)), cfg
