@@ -56,3 +56,53 @@ template <int DT> __device__ __forceinline__ void st_dt(void* p, int64_t i, floa
     else ((float*)p)[i] = v;
 }
 template <int DT> struct dt_size { static constexpr int value = DT == DT_F32 ? 4 : 2; };
+
+// Workgroup -> tile.  Workgroups are dealt round-robin to the 8 XCDs (each with its own L2), so first renumber them
+// XCD-contiguously, then walk tiles in panels of 4 tile rows so that the 32 workgroups an XCD runs at once cover a
+// 4 x 8 patch of tiles and share A rows / W rows in that XCD's L2.
+__device__ __forceinline__ void tile_of_block(int b, int nblocks, int tiles_m, int tiles_n, int& tm, int& tn) {
+    const int base = nblocks >> 3, rem = nblocks & 7;
+    const int xcd = b & 7, idx = b >> 3;
+    const int lin = xcd * base + (xcd < rem ? xcd : rem) + idx;
+    constexpr int GM = 4;
+    const int per_panel = GM * tiles_n;
+    const int panel = lin / per_panel;
+    const int first_m = panel * GM;
+    const int rows = tiles_m - first_m < GM ? tiles_m - first_m : GM;
+    const int in_panel = lin - panel * per_panel;
+    tm = first_m + in_panel % rows;
+    tn = in_panel / rows;
+}
+
+
+// Four consecutive elements of a dtype-coded array <-> four floats (8- or 16-byte vector access).
+template <int OUT_DT> __device__ __forceinline__ void load4(const void* p, int64_t i, float* v) {
+    if (OUT_DT == DT_F32) {
+        const float4 f = *reinterpret_cast<const float4*>((const float*)p + i);
+        v[0] = f.x; v[1] = f.y; v[2] = f.z; v[3] = f.w;
+    } else {
+        const uint2 u = *reinterpret_cast<const uint2*>((const uint16_t*)p + i);
+        if (OUT_DT == DT_BF16) {
+            v[0] = u2f(u.x << 16); v[1] = u2f(u.x & 0xffff0000u); v[2] = u2f(u.y << 16); v[3] = u2f(u.y & 0xffff0000u);
+        } else {
+            v[0] = f16_to_f((uint16_t)(u.x & 0xffffu)); v[1] = f16_to_f((uint16_t)(u.x >> 16));
+            v[2] = f16_to_f((uint16_t)(u.y & 0xffffu)); v[3] = f16_to_f((uint16_t)(u.y >> 16));
+        }
+    }
+}
+template <int OUT_DT> __device__ __forceinline__ void store4(void* p, int64_t i, const float* v) {
+    if (OUT_DT == DT_F32) {
+        *reinterpret_cast<float4*>((float*)p + i) = make_float4(v[0], v[1], v[2], v[3]);
+    } else if (OUT_DT == DT_BF16) {
+        uint2 u;
+        u.x = pack_bf16x2(v[0], v[1]);
+        u.y = pack_bf16x2(v[2], v[3]);
+        *reinterpret_cast<uint2*>((uint16_t*)p + i) = u;
+    } else {
+        uint2 u;
+        u.x = (uint32_t)f_to_f16(v[0]) | ((uint32_t)f_to_f16(v[1]) << 16);
+        u.y = (uint32_t)f_to_f16(v[2]) | ((uint32_t)f_to_f16(v[3]) << 16);
+        *reinterpret_cast<uint2*>((uint16_t*)p + i) = u;
+    }
+}
+

@@ -27,6 +27,7 @@ SIGNATURES = {
     "gpu_w6_decode": [_P, _P, _P, _I64, _I32, _I32, _P],
     "gpu_int8_gemm_acc": [_P, _P, _P, _I64, _I64, _I64, _P],
     "gpu_w6a8_gemm": [_P, _P, _P, _I32, _P, _P, _P, _P, _I64, _I64, _I64, _I32, _P],
+    "gpu_w6a8_group_gemm": [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I32, _P],
     "gpu_int8_gemm_force_config": [_I32],
     "gpu_mfma_layout_probe": [_P, _P],
 }

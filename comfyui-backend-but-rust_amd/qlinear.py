@@ -89,6 +89,18 @@ def w6a8_gemm(A, wq, s_rel, G, xs, s_channel, bias=None, out_dtype=torch.bfloat1
     return D
 
 
+def w6a8_group_gemm(A, packed, xs, sw, bias=None, out_dtype=torch.bfloat16, want_partials=False):
+    """W6A8 linear on already-quantized rows with the library's own weight format: 24-bit words of four 6-bit codes,
+    packed [N, 3K/4], and f32 group scales sw [N, K/128].  Returns D, or (D, partials [M, N, K/128]) on request."""
+    M, K = A.shape
+    N = packed.shape[0]
+    D = torch.empty((M, N), dtype=out_dtype, device=A.device)
+    part = torch.empty((M, N, K // 128), dtype=torch.int32, device=A.device) if want_partials else None
+    ffi.k("gpu_w6a8_group_gemm", _ptr(A), _ptr(packed), _ptr(xs), _ptr(sw), _ptr(bias), _ptr(D), _ptr(part), M, N, K,
+          _TORCH_DT[out_dtype], _stream())
+    return (D, part) if want_partials else D
+
+
 def linear_w8a8(x, W, ws, bias=None, rotate=0, out_dtype=None):
     """One W8A8 linear: y = dequant(quant(x) . W^T)."""
     q, xs = quant_rows(x, rotate)

@@ -88,6 +88,19 @@ int gpu_int8_gemm_acc(const int8_t* A, const int8_t* W, int32_t* acc, int64_t M,
 int gpu_w6a8_gemm(const int8_t* A, const void* wq, const void* s_rel, int G, const float* xs, const float* s_channel,
                   const void* bias, void* D, int64_t M, int64_t N, int64_t K, int out_dt, void* stream);
 
+/* W6A8 linear with the unpack fused ahead of the MFMA, for this library's own packed format (no counterpart in the
+ * reference, whose W6 weights are two-plane with e4m3 group factors: gpu_w6_decode / gpu_w6a8_gemm above).
+ *   Wp  uint8 [N, 3K/4]: codes u = q + 32 with q in [-32, 31]; every three bytes are the little-endian 24-bit word
+ *       u0 | u1 << 6 | u2 << 12 | u3 << 18 of four consecutive k.
+ *   sw  f32 [N, K/128]: one scale per output channel and group of 128 along K.
+ *   D[m,n] = Out(fma(accf, xs[m], bias[n])), where accf starts at 0 and takes accf = fma(float(p_g), sw[n,g], accf) for
+ *       g = 0, 1, ..., with p_g the exact int32 dot product of A[m, 128g .. 128g+127] and the codes q[n, same].
+ *   partials: null, or int32 [M, N, K/128] that receives every p_g (a check hook; slow).
+ * A rows, Wp rows and D are 16-byte aligned (K % 128 == 0 gives that for rows of contiguous tensors).
+ * Returns -1 for K % 128 != 0; -200 for an unknown out_dt, K == 0, or sizes beyond 32-bit byte offsets. */
+int gpu_w6a8_group_gemm(const int8_t* A, const void* Wp, const float* xs, const float* sw, const void* bias, void* D,
+                        int32_t* partials, int64_t M, int64_t N, int64_t K, int out_dt, void* stream);
+
 /* Test and tuning hook: force the GEMM kernel family.  0, 1, 2 = 256x256, 128x128, 64x64 register-staged tiles;
  * 3, 4 = 256x256 direct-to-LDS with 64- and 128-byte rows; 5 = persistent ring kernel; 6 = narrow-tile / split-K
  * ring kernel for M <= 256; -1 = automatic.  Shapes a family cannot run fall back to 0. */

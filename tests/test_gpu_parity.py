@@ -351,6 +351,45 @@ def test_w6a8_linear_matches_decode_then_gemm():
     assert ffi.raw("gpu_w6a8_gemm", 0, 0, 0, 32, 0, 0, 0, 0, 4, 8, 48, 2, 0) == -1
 
 
+# ------------------------------------------------------------------------- W6A8, packed words + fp32 group scales
+W6G_CASES = [  # (M, N, K, out_dt, with_bias)
+    (256, 128, 128, BF16, True), (100, 200, 256, BF16, False), (300, 136, 640, F32, True), (513, 260, 384, F16, True),
+    (1, 8, 128, BF16, True), (777, 1000, 1280, BF16, True),
+]
+
+
+@pytest.mark.parametrize("M,N,K,out_dt,with_bias", W6G_CASES)
+def test_w6a8_group_gemm_matches_oracle(M, N, K, out_dt, with_bias):
+    """The fused-unpack kernel against the oracle: every int32 group partial and every output bit."""
+    say("w6a8_group", M, N, K, out_dt, with_bias)
+    A = rand_i8(9, 1, M, K, -127, 127)
+    A[0, :] = -128
+    qv = synth.w6_codes(9, N, K)
+    qv[0, :] = -32                                           # extreme partial: 128 * 128 * 32
+    qv[N - 1, :] = 31
+    packed = oracle.w6_pack_words(qv)
+    xs = synth.uniform(9, 3, M, 0.005, 0.2)
+    sw = synth.w6_group_scales(9, N, K)
+    tob = {BF16: oracle.bf16_bits, F16: oracle.f16_bits, F32: lambda a: a.astype(np.float32)}[out_dt]
+    bias = tob(synth.normal(9, 5, N) * np.float32(0.02)) if with_bias else None
+    rc, want, want_part = oracle.w6a8_group_gemm(A, packed, xs, sw, bias, out_dt, want_partials=True)
+    assert rc == 0
+    bd = None if bias is None else dev_bits(bias, out_dt)
+    got, part = ql.w6a8_group_gemm(dev(A), dev(packed), dev(xs), dev(sw), bd, TDT[out_dt], want_partials=True)
+    got2 = ql.w6a8_group_gemm(dev(A), dev(packed), dev(xs), dev(sw), bd, TDT[out_dt])
+    torch.cuda.synchronize()
+    assert np.array_equal(part.cpu().numpy(), want_part)
+    view = np.uint32 if out_dt == F32 else np.uint16
+    assert np.array_equal(host_bits(got).view(view), want.view(view))
+    assert np.array_equal(host_bits(got2).view(view), want.view(view))
+
+
+def test_w6a8_group_gemm_argument_checks():
+    assert ffi.raw("gpu_w6a8_group_gemm", 0, 0, 0, 0, 0, 0, 0, 4, 8, 64, 2, 0) == -1      # K % 128
+    assert ffi.raw("gpu_w6a8_group_gemm", 0, 0, 0, 0, 0, 0, 0, 4, 8, 128, 7, 0) == -200   # out_dt
+    assert ffi.raw("gpu_w6a8_group_gemm", 0, 0, 0, 0, 0, 0, 0, 0, 8, 128, 2, 0) == 0      # empty
+
+
 # ------------------------------------------------------------------------------------------------ full-size shapes
 FULL = [  # (name, M, K, N, rotate, kind)
     ("dit mlp up", 4608, 3072, 12288, 128, "t3"),
