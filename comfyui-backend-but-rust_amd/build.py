@@ -19,11 +19,14 @@ FLAGS = [
     # keep the compiler from forming packed-fp32 instructions
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
+# Per-file additions.  The grouped W6A8 kernel reads every MFMA result with VALU instructions (int32 partial -> fp32),
+# which cannot take accumulator registers as operands: keep its MFMA destinations in ordinary vector registers.
+EXTRA = {"w6a8_group_gemm.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 
 
 def _compile(src):
     obj = os.path.join(CSRC, os.path.splitext(src)[0] + ".o")
-    cmd = ["hipcc", *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = ["hipcc", *FLAGS, *EXTRA.get(src, []), "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
     if r.returncode != 0:

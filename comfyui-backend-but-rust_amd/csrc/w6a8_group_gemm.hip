@@ -9,15 +9,17 @@
 //   p_g = sum over the 128 k of group g of A[m,k] * q[n,k], an exact int32.
 //
 // One K tile of the kernel is one group, so every group's int32 partial is a fresh MFMA accumulation (first MFMA with
-// C = 0) that is folded into the fp32 accumulators while the next partials are being multiplied.  Per iteration:
+// C = 0) that is folded into the fp32 accumulators.  A workgroup of eight waves owns a 256 x 128 tile; per iteration:
 //   * LDS-DMA brings A(g+1) (256 x 128 int8), the packed weights of group g+2 (128 rows x 96 bytes) and the 128 scales
 //     of group g+1 straight into LDS;
-//   * every thread expands four 12-byte pieces of the packed weights of group g+1 into 16 int8 each and writes them
+//   * every thread expands two 12-byte pieces of the packed weights of group g+1 into 16 int8 each and writes them
 //     in the swizzled fragment layout (conflict-free both ways);
-//   * each wave (2 x 2 grid, 128 x 64 outputs, 8 MFMA tiles) multiplies group g in four pairs of tiles; the
-//     fp32 scaling of a pair rides between the MFMAs of the next pair.
-// The scaling costs two VALU operations per output and group and the unpack about ten per four codes, together more
-// issue slots than the MFMAs themselves: the kernel is bound by VALU issue, not by the matrix pipe.
+//   * each wave (2 x 4 grid, 128 x 32 outputs, four MFMA tiles) multiplies group g in two pairs of tiles; the fp32
+//     fold of the first pair rides between the MFMAs of the second.
+// The fold costs two VALU operations per output and group (plus the read of the accumulation register) and the unpack
+// about six per code word: together more issue slots than the MFMAs, so the kernel is bound by VALU issue, not by the
+// matrix pipe.  Two waves share a SIMD; the upper four waves fold their second pair at the end of an iteration, the
+// lower four at the start of the next, so that on every SIMD one wave's VALU-only stretch meets the other's MFMAs.
 #include "common.hpp"
 
 #define SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
@@ -39,8 +41,9 @@ struct W6Args {
 constexpr int BM = 256, BN = 128, BK = 128, RAW_ROW = 96;
 constexpr int A_STAGE = BM * BK, U_STAGE = BN * BK, R_STAGE = BN * RAW_ROW, S_STAGE = BN * 4;
 constexpr int U_BASE = 2 * A_STAGE, R_BASE = U_BASE + 2 * U_STAGE, S_BASE = R_BASE + 2 * R_STAGE;
-constexpr int SMEM = S_BASE + 2 * S_STAGE;
-constexpr int TM = 4, TN = 2;   // 32x32 MFMA tiles of one wave: 128 rows (m) x 64 columns (n)
+constexpr int SMEM = S_BASE + 3 * S_STAGE;   // three stages of scales: the deferred fold reads those of the group before
+constexpr int TM = 4, TN = 1;   // 32x32 MFMA tiles of one wave: 128 rows (m) x 32 columns (n)
+constexpr int NT = 512;         // eight waves, 2 (m) x 4 (n)
 
 // Four 6-bit fields of a 24-bit word (bits above 23 are ignored) -> four int8 q = u - 32, one per byte.
 __device__ __forceinline__ int spread6(uint32_t w) {
@@ -58,11 +61,11 @@ __device__ __forceinline__ void dma4(uint32_t lds_dst, uint32_t lane_off, const 
 }
 
 template <int OUT_DT, bool DUMP>
-__global__ void __launch_bounds__(256, 1) w6a8_group_gemm_kernel(W6Args p) {
+__global__ void __launch_bounds__(NT, 1) w6a8_group_gemm_kernel(W6Args p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave >> 2, wn = wave & 3;
     int tm, tn;
     tile_of_block((int)blockIdx.x, (int)gridDim.x, p.tiles_m, p.tiles_n, tm, tn);
     const int m0 = tm * BM, n0 = tn * BN, ng = p.ng;
@@ -71,47 +74,50 @@ __global__ void __launch_bounds__(256, 1) w6a8_group_gemm_kernel(W6Args p) {
     // DMA sources: 32-bit lane offsets from a per-group scalar base.  Rows past the edge re-read the last valid row;
     // what they produce is never stored.
     const int lrow = lane >> 3, lch = ((lane & 7) ^ lrow) * 16;   // swizzle applied on the global side
-    uint32_t ga[8], gr[3], gs;
+    uint32_t ga[4], gr[2], gs;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        const int row = (wave + 4 * j) * 8 + lrow;
+    for (int j = 0; j < 4; ++j) {
+        const int row = (wave + 8 * j) * 8 + lrow;
         const int r = m0 + row < p.M ? m0 + row : p.M - 1;
         ga[j] = (uint32_t)r * (uint32_t)p.K + lch;
     }
     const uint32_t wrow = (uint32_t)p.K / 4 * 3;                   // bytes per packed weight row
 #pragma unroll
-    for (int j = 0; j < 3; ++j) {
-        const int c = (wave + 4 * j) * 64 + lane;                  // 16-byte chunk of the raw tile: row c/6, part c%6
-        const int row = c / 6, part = c - row * 6;
+    for (int j = 0; j < 2; ++j) {                                  // 12 instructions cover the raw tile: waves 0-3 issue two
+        const int c = (wave + 8 * j) * 64 + lane;                  // 16-byte chunk of the raw tile: row c/6, part c%6
+        const int row = (c / 6) & 127, part = c % 6;
         const int r = n0 + row < p.N ? n0 + row : p.N - 1;
         gr[j] = (uint32_t)r * wrow + part * 16;
     }
     {
-        const int row = 32 * wave + (lane & 31);
+        const int row = 32 * (wave & 3) + (lane & 31);
         const int r = n0 + row < p.N ? n0 + row : p.N - 1;
         gs = (uint32_t)r * (uint32_t)ng * 4u;
     }
     auto fetch_a = [&](int g, int stage) {
         const int8_t* base = p.A + (int64_t)(g < ng ? g : ng - 1) * BK;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) dma16(lds_base + stage * A_STAGE + (wave + 4 * j) * 1024, ga[j], base);
+        for (int j = 0; j < 4; ++j) dma16(lds_base + stage * A_STAGE + (wave + 8 * j) * 1024, ga[j], base);
     };
     auto fetch_raw = [&](int g, int stage) {
         const uint8_t* base = p.Wp + (int64_t)(g < ng ? g : ng - 1) * RAW_ROW;
-#pragma unroll
-        for (int j = 0; j < 3; ++j) dma16(lds_base + R_BASE + stage * R_STAGE + (wave + 4 * j) * 1024, gr[j], base);
+        dma16(lds_base + R_BASE + stage * R_STAGE + wave * 1024, gr[0], base);
+        if (wave < 4) dma16(lds_base + R_BASE + stage * R_STAGE + (wave + 8) * 1024, gr[1], base);
     };
     auto fetch_scales = [&](int g, int stage) {
         const float* base = p.sw + (g < ng ? g : ng - 1);
-        if (lane < 32) dma4(lds_base + S_BASE + stage * S_STAGE + wave * 128, gs, base);
+        if (wave < 4 && lane < 32) dma4(lds_base + S_BASE + stage * S_STAGE + wave * 128, gs, base);
     };
-    // Piece e of the raw tile is bytes [12e, 12e+12): row e/8, codes 16*(e%8) .. +15 -> one 16-byte chunk.
-    auto unpack = [&](int rstage, int ustage, int i) {
-        const int e = tid + 256 * i;
-        const uint32_t* src = reinterpret_cast<const uint32_t*>(smem + R_BASE + rstage * R_STAGE + 12 * e);
-        const uint32_t d0 = src[0], d1 = src[1], d2 = src[2];
-        const v4i out = v4i{spread6(d0), spread6(__builtin_amdgcn_alignbit(d1, d0, 24)),
-                            spread6(__builtin_amdgcn_alignbit(d2, d1, 16)), spread6(d2 >> 8)};
+    // Piece e of the raw tile is bytes [12e, 12e+12): row e/8, codes 16*(e%8) .. +15 -> one 16-byte chunk.  Reading
+    // the three words and expanding them are separate steps so that the LDS latency hides behind other work.
+    auto raw_read = [&](int rstage, int i, uint32_t (&d)[3]) {
+        const uint32_t* src = reinterpret_cast<const uint32_t*>(smem + R_BASE + rstage * R_STAGE + 12 * (tid + NT * i));
+        d[0] = src[0]; d[1] = src[1]; d[2] = src[2];
+    };
+    auto unpack_write = [&](int ustage, int i, const uint32_t (&d)[3]) {
+        const int e = tid + NT * i;
+        const v4i out = v4i{spread6(d[0]), spread6(__builtin_amdgcn_alignbit(d[1], d[0], 24)),
+                            spread6(__builtin_amdgcn_alignbit(d[2], d[1], 16)), spread6(d[2] >> 8)};
         const int r = e >> 3, pc = e & 7;
         *reinterpret_cast<v4i*>(smem + U_BASE + ustage * U_STAGE + r * BK + ((pc ^ (r & 7)) << 4)) = out;
     };
@@ -123,7 +129,7 @@ __global__ void __launch_bounds__(256, 1) w6a8_group_gemm_kernel(W6Args p) {
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {
         aoff[kk] = ((wm * 128 + frow) * BK + fsw) ^ (kk << 5);
-        woff[kk] = ((wn * 64 + frow) * BK + fsw) ^ (kk << 5);
+        woff[kk] = ((wn * 32 + frow) * BK + fsw) ^ (kk << 5);
     }
 
     v16i part[TN][TM];      // int32 partial of the current group
@@ -143,44 +149,53 @@ __global__ void __launch_bounds__(256, 1) w6a8_group_gemm_kernel(W6Args p) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 #pragma unroll
-    for (int i = 0; i < 4; ++i) unpack(0, 0, i);
+    for (int i = 0; i < 2; ++i) {
+        uint32_t d[3];
+        raw_read(0, i, d);
+        unpack_write(0, i, d);
+    }
     __syncthreads();
 
+    const bool defer = wm == 0;   // these waves fold their second pair at the start of the next iteration
+#pragma unroll
+    for (int im = 0; im < TM; ++im)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) part[0][im][r] = 0;
+
+    // fp32 fold of four values: register group q of tile im.  accf += float(part) * sw[n, g]
+    auto fold = [&](int im, int q, const float4& s4) {
+        const float sv[4] = {s4.x, s4.y, s4.z, s4.w};
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+            accf[0][im][4 * q + c] = __builtin_fmaf((float)part[0][im][4 * q + c], sv[c], accf[0][im][4 * q + c]);
+    };
+
+    int ss = 0;   // scale stage of group g = g mod 3
     for (int g = 0; g < ng; ++g) {
         const int s = g & 1;
         const uint8_t* sa = smem + s * A_STAGE;
         const uint8_t* su = smem + U_BASE + s * U_STAGE;
-        const float* sc = reinterpret_cast<const float*>(smem + S_BASE + s * S_STAGE);
-        // All of these targets were last read during iteration g-1, which every wave has left.
+        const float* sc = reinterpret_cast<const float*>(smem + S_BASE + ss * S_STAGE);
+        const float* sc_prev = reinterpret_cast<const float*>(smem + S_BASE + (ss == 0 ? 2 : ss - 1) * S_STAGE);
+        const int ss_next = ss == 2 ? 0 : ss + 1;
+        // All of these targets were last read during iteration g-1 (the scale stage: g-2), which every wave has left.
         fetch_a(g + 1, s ^ 1);
         fetch_raw(g + 2, s);
-        fetch_scales(g + 1, s ^ 1);
+        fetch_scales(g + 1, ss_next);
         SCHED_FENCE();
 
-        v4i fa[2][4], fw[4], na[2][4], nw[4];
+        v4i fa[2][4], fw[4], na[2][4];
+        float4 sv[4];
+        uint32_t raw[2][3];
         auto load_a = [&](v4i (&dst)[2][4], int imb) {
 #pragma unroll
             for (int t = 0; t < 2; ++t)
 #pragma unroll
                 for (int kk = 0; kk < 4; ++kk) dst[t][kk] = *reinterpret_cast<const v4i*>(sa + aoff[kk] + (imb + t) * 32 * BK);
         };
-        auto load_w = [&](v4i (&dst)[4], int in) {
-#pragma unroll
-            for (int kk = 0; kk < 4; ++kk) dst[kk] = *reinterpret_cast<const v4i*>(su + woff[kk] + in * 32 * BK);
-        };
-        // fp32 fold of register group q of both tiles of a pair: accf += float(part) * sw[n, g]
-        auto fold = [&](int in, int imb, int q) {
-            const float4 s4 = *reinterpret_cast<const float4*>(sc + wn * 64 + in * 32 + 8 * q + 4 * fhalf);
-            const float sv[4] = {s4.x, s4.y, s4.z, s4.w};
-#pragma unroll
-            for (int t = 0; t < 2; ++t)
-#pragma unroll
-                for (int c = 0; c < 4; ++c)
-                    accf[in][imb + t][4 * q + c] = __builtin_fmaf((float)part[in][imb + t][4 * q + c], sv[c], accf[in][imb + t][4 * q + c]);
-        };
-        // Eight MFMAs of the pair (in; imb, imb+1), the two accumulation chains interleaved; between(i) is issued
-        // after the i-th of them.
-        auto mma_pair = [&](int in, int imb, v4i (&a)[2][4], v4i (&w)[4], auto&& between) {
+        // Eight MFMAs of the pair (imb, imb+1), the two accumulation chains interleaved; between(i) is issued after the
+        // i-th of them.
+        auto mma_pair = [&](int imb, v4i (&a)[2][4], auto&& between) {
 #pragma unroll
             for (int kk = 0; kk < 4; ++kk)
 #pragma unroll
@@ -189,9 +204,9 @@ __global__ void __launch_bounds__(256, 1) w6a8_group_gemm_kernel(W6Args p) {
                         v16i zero;
 #pragma unroll
                         for (int r = 0; r < 16; ++r) zero[r] = 0;
-                        part[in][imb + t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(w[kk], a[t][kk], zero, 0, 0, 0);
+                        part[0][imb + t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fw[kk], a[t][kk], zero, 0, 0, 0);
                     } else {
-                        part[in][imb + t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(w[kk], a[t][kk], part[in][imb + t], 0, 0, 0);
+                        part[0][imb + t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fw[kk], a[t][kk], part[0][imb + t], 0, 0, 0);
                     }
                     SCHED_FENCE();
                     between(kk * 2 + t);
@@ -199,76 +214,140 @@ __global__ void __launch_bounds__(256, 1) w6a8_group_gemm_kernel(W6Args p) {
                 }
         };
 
-        load_w(fw, 0);
-        load_a(fa, 0);
-        mma_pair(0, 0, fa, fw, [&](int i) {
-            if (i == 0) load_a(na, 2);
-            if (i == 4) unpack(s ^ 1, s ^ 1, 0);
-        });
-        mma_pair(0, 2, na, fw, [&](int i) {
-            if (i < 4) fold(0, 0, i);
-            if (i == 4) { load_w(nw, 1); load_a(fa, 0); }
-            if (i == 6) unpack(s ^ 1, s ^ 1, 1);
-        });
-        mma_pair(1, 0, fa, nw, [&](int i) {
-            if (i < 4) fold(0, 2, i);
-            if (i == 4) load_a(na, 2);
-            if (i == 6) unpack(s ^ 1, s ^ 1, 2);
-        });
-        mma_pair(1, 2, na, nw, [&](int i) {
-            if (i < 4) fold(1, 0, i);
-            if (i == 5) unpack(s ^ 1, s ^ 1, 3);
-        });
+        // everything this iteration reads from LDS early: fragments of the first pair, the group's scales, packed words
 #pragma unroll
-        for (int q = 0; q < 4; ++q) fold(1, 2, q);
+        for (int kk = 0; kk < 4; ++kk) fw[kk] = *reinterpret_cast<const v4i*>(su + woff[kk]);
+        load_a(fa, 0);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) sv[q] = *reinterpret_cast<const float4*>(sc + wn * 32 + 8 * q + 4 * fhalf);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) raw_read(s ^ 1, i, raw[i]);
+        SCHED_FENCE();
+        if (defer && g > 0) {   // the fold the previous iteration left over
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const float4 sp = *reinterpret_cast<const float4*>(sc_prev + wn * 32 + 8 * q + 4 * fhalf);
+                fold(2, q, sp);
+                fold(3, q, sp);
+            }
+            SCHED_FENCE();
+        }
+        // the second pair's A fragments take over the registers of the first pair's as those are consumed
+        mma_pair(0, fa, [&](int i) {
+            na[i & 1][i >> 1] = *reinterpret_cast<const v4i*>(sa + aoff[i >> 1] + (2 + (i & 1)) * 32 * BK);
+            if (i == 2) unpack_write(s ^ 1, 0, raw[0]);
+            if (i == 4) unpack_write(s ^ 1, 1, raw[1]);
+        });
+        mma_pair(2, na, [&](int i) { fold(i & 1, i >> 1, sv[i >> 1]); });
+        if (!defer) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) fold(2 + (i & 1), i >> 1, sv[i >> 1]);
+        }
 
         if (DUMP) {   // test hook: the exact int32 partials, [M, N, ng]
 #pragma unroll
-            for (int in = 0; in < TN; ++in)
+            for (int im = 0; im < TM; ++im)
 #pragma unroll
-                for (int im = 0; im < TM; ++im)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const int m = m0 + wm * 128 + im * 32 + frow;
-                        const int n = n0 + wn * 64 + in * 32 + 8 * (r >> 2) + 4 * fhalf + (r & 3);
-                        if (m < p.M && n < p.N) p.partials[((int64_t)m * p.N + n) * ng + g] = part[in][im][r];
-                    }
+                for (int r = 0; r < 16; ++r) {
+                    const int m = m0 + wm * 128 + im * 32 + frow;
+                    const int n = n0 + wn * 32 + 8 * (r >> 2) + 4 * fhalf + (r & 3);
+                    if (m < p.M && n < p.N) p.partials[((int64_t)m * p.N + n) * ng + g] = part[0][im][r];
+                }
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the DMA of this iteration has landed
         __syncthreads();                                    // ... for every wave, and the unpacked tile is written
+        ss = ss_next;
+    }
+    if (defer) {   // ss now names the stage after the last group's
+        const float* sc_last = reinterpret_cast<const float*>(smem + S_BASE + (ss == 0 ? 2 : ss - 1) * S_STAGE);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const float4 sp = *reinterpret_cast<const float4*>(sc_last + wn * 32 + 8 * q + 4 * fhalf);
+            fold(2, q, sp);
+            fold(3, q, sp);
+        }
     }
 
-    // epilogue: four consecutive n per lane and register group, straight from the accumulators
-    const bool vec_ok = (p.N & 3) == 0 && ((uintptr_t)p.D & (4 * dt_size<OUT_DT>::value - 1)) == 0 &&
-                        ((uintptr_t)p.bias & (4 * dt_size<OUT_DT>::value - 1)) == 0;
+    // Epilogue.  A lane holds one m and runs of four consecutive n, so storing straight from the registers would touch
+    // 32 rows per instruction.  When the rows of D are 16-byte aligned each wave instead passes its tile, 32 rows at a
+    // time, through a private 4 KB of LDS (16-byte chunks XOR-swizzled by row, conflict-free both ways) and writes whole
+    // row segments, 16 bytes per lane.
+    constexpr int SZ = dt_size<OUT_DT>::value;
+    const bool vec_ok = (p.N & 3) == 0 && ((uintptr_t)p.D & (4 * SZ - 1)) == 0 && ((uintptr_t)p.bias & (4 * SZ - 1)) == 0;
+    const bool rows_ok = vec_ok && (((int64_t)p.N * SZ) & 15) == 0 && ((uintptr_t)p.D & 15) == 0;
+    const int nb = n0 + wn * 32;
+    float bv[4][4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const int n = nb + 8 * q + 4 * fhalf;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) bv[q][c] = 0.f;
+        if (p.bias && n < p.N) {
+            if (vec_ok) {
+                load4<OUT_DT>(p.bias, n, bv[q]);
+            } else {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) if (n + c < p.N) bv[q][c] = ld_dt<OUT_DT>(p.bias, n + c);
+            }
+        }
+    }
+    if (rows_ok) {
+        constexpr int ROWB = 32 * SZ, CPR = ROWB / 16;          // bytes and 16-byte chunks per LDS row (32 columns)
+        constexpr int RPI = 64 / CPR, NI = 32 / RPI;            // rows per store instruction, instructions per piece
+        uint8_t* wl = smem + wave * 4096;                        // the stages are idle: the loop ended with a barrier
+#pragma unroll
+        for (int im = 0; im < TM; ++im) {
+            const int mb = m0 + wm * 128 + im * 32;
+            const float xs = p.xs[mb + frow < p.M ? mb + frow : p.M - 1];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                float out[4];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) out[c] = __builtin_fmaf(accf[0][im][4 * q + c], xs, bv[q][c]);
+                const int byte = (8 * q + 4 * fhalf) * SZ;       // columns 8q + 4*fhalf .. +3 of row frow
+                uint8_t* dst = wl + frow * ROWB + ((((byte >> 4) ^ (frow & (CPR - 1))) << 4) | (byte & 15));
+                if (OUT_DT == DT_F32) {
+                    *reinterpret_cast<float4*>(dst) = make_float4(out[0], out[1], out[2], out[3]);
+                } else if (OUT_DT == DT_BF16) {
+                    *reinterpret_cast<uint2*>(dst) = make_uint2(pack_bf16x2(out[0], out[1]), pack_bf16x2(out[2], out[3]));
+                } else {
+                    *reinterpret_cast<uint2*>(dst) = make_uint2((uint32_t)f_to_f16(out[0]) | ((uint32_t)f_to_f16(out[1]) << 16),
+                                                                (uint32_t)f_to_f16(out[2]) | ((uint32_t)f_to_f16(out[3]) << 16));
+                }
+            }
+            asm volatile("" ::: "memory");   // the wave's own LDS writes are ordered before its reads
+#pragma unroll
+            for (int t = 0; t < NI; ++t) {
+                const int row = t * RPI + lane / CPR, ch = lane % CPR;
+                const uint4 v = *reinterpret_cast<const uint4*>(wl + row * ROWB + ((ch ^ (row & (CPR - 1))) << 4));
+                const int m = mb + row, n = nb + ch * (16 / SZ);
+                if (m < p.M && n < p.N) *reinterpret_cast<uint4*>((uint8_t*)p.D + ((int64_t)m * p.N + n) * SZ) = v;
+            }
+            asm volatile("" ::: "memory");   // ... and the reads before the next piece's writes
+        }
+        return;
+    }
+    // fallback for unaligned rows: four consecutive n per lane and register group, straight from the accumulators
 #pragma unroll
     for (int im = 0; im < TM; ++im) {
         const int m = m0 + wm * 128 + im * 32 + frow;
         if (m >= p.M) continue;
         const float xs = p.xs[m];
 #pragma unroll
-        for (int in = 0; in < TN; ++in)
+        for (int q = 0; q < 4; ++q) {
+            const int n = nb + 8 * q + 4 * fhalf;
+            if (n >= p.N) continue;
+            const int64_t o = (int64_t)m * p.N + n;
+            float out[4];
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int n = n0 + wn * 64 + in * 32 + 8 * q + 4 * fhalf;
-                if (n >= p.N) continue;
-                const int64_t o = (int64_t)m * p.N + n;
-                float b[4] = {0.f, 0.f, 0.f, 0.f}, out[4];
-                if (vec_ok) {
-                    if (p.bias) load4<OUT_DT>(p.bias, n, b);
-                } else {
+            for (int c = 0; c < 4; ++c) out[c] = __builtin_fmaf(accf[0][im][4 * q + c], xs, bv[q][c]);
+            if (vec_ok) {
+                store4<OUT_DT>(p.D, o, out);
+            } else {
 #pragma unroll
-                    for (int c = 0; c < 4; ++c) if (p.bias && n + c < p.N) b[c] = ld_dt<OUT_DT>(p.bias, n + c);
-                }
-#pragma unroll
-                for (int c = 0; c < 4; ++c) out[c] = __builtin_fmaf(accf[in][im][4 * q + c], xs, b[c]);
-                if (vec_ok) {
-                    store4<OUT_DT>(p.D, o, out);
-                } else {
-#pragma unroll
-                    for (int c = 0; c < 4; ++c) if (n + c < p.N) st_dt<OUT_DT>(p.D, o + c, out[c]);
-                }
+                for (int c = 0; c < 4; ++c) if (n + c < p.N) st_dt<OUT_DT>(p.D, o + c, out[c]);
             }
+        }
     }
 }
 
@@ -281,7 +360,7 @@ int launch(W6Args a, hipStream_t st) {
         if (e != hipSuccess) return (int)e;
         once = true;
     }
-    hipLaunchKernelGGL(kern, dim3((unsigned)(a.tiles_m * a.tiles_n)), dim3(256), SMEM, st, a);
+    hipLaunchKernelGGL(kern, dim3((unsigned)(a.tiles_m * a.tiles_n)), dim3(NT), SMEM, st, a);
     KCHECK();
     return 0;
 }
