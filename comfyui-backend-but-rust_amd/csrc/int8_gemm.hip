@@ -46,10 +46,13 @@ struct Cfg {
     static_assert(BK == 64 || BK == 128, "swizzle is written for 64- and 128-byte rows");
 };
 
-// Chunk swizzle: rows are BK bytes apart, so 8 consecutive rows of one chunk column would share banks; XOR the chunk
-// index with row bits so that any 8 consecutive rows land on 8 distinct 16-byte bank groups.
+// Chunk swizzle.  The LDS of gfx950 has 64 banks of 4 bytes, and a ds_read_b128 is served 16 lanes (256 bytes) at a
+// time: a fragment read takes 16 consecutive rows at one chunk column, so those 16 rows must land on 16 distinct
+// 16-byte bank groups.  Rows are BK bytes apart: with 128-byte rows an even/odd row pair already covers the two halves
+// of the bank space, so the chunk index is XORed with bits 1..3 of the row; with 64-byte rows four rows span the banks
+// and bits 2..3 are used.  (Measured: XOR with the low row bits instead costs 25 % of the read bandwidth.)
 template <int BK> __device__ __forceinline__ int swz(int row, int chunk) {
-    return BK == 64 ? (chunk ^ ((row >> 1) & 3)) : (chunk ^ (row & 7));
+    return BK == 64 ? (chunk ^ ((row >> 2) & 3)) : (chunk ^ ((row >> 1) & 7));
 }
 
 // The epilogue arithmetic for one value.  t0 = float(acc)*xs; then fma(t0, ws, bias): the reference composes a
@@ -494,7 +497,7 @@ __device__ __forceinline__ void dma_gemm_tile(const GemmArgs& p, uint8_t* smem, 
     // DMA sources: wave w owns 16-row blocks w, w+4, ... of the A tile and of the W tile.  Per-lane 32-bit offsets from
     // the tile bases (the launcher guarantees M*K and N*K fit), so an instruction is scalar base + vector offset.
     uint32_t ga[C::A_LD], gw[C::W_LD];
-    const int lrow = lane >> 2, lch = (lane & 3) ^ ((lrow >> 1) & 3);
+    const int lrow = lane >> 2, lch = (lane & 3) ^ ((lrow >> 2) & 3);   // rows come in blocks of 16: swz<64> of the row
 #pragma unroll
     for (int i = 0; i < C::A_LD; ++i) {
         const int row = (wave + 4 * i) * 16 + lrow;
@@ -521,7 +524,7 @@ __device__ __forceinline__ void dma_gemm_tile(const GemmArgs& p, uint8_t* smem, 
 
     // fragment addresses: row r of a tile at r*64, chunk c at slot c ^ ((r>>1)&3); K sub-step kk flips address bit 5
     const int frow = lane & 31, fhalf = lane >> 5;
-    const int fsw = (fhalf ^ ((frow >> 1) & 3)) << 4;
+    const int fsw = (fhalf ^ ((frow >> 2) & 3)) << 4;
     int aoff[2], woff[2];
     aoff[0] = (wm * C::WTM + frow) * BK + fsw;
     woff[0] = BM * BK + (wn * C::WTN + frow) * BK + fsw;
@@ -631,7 +634,8 @@ __device__ __forceinline__ void dma2_gemm_tile(const GemmArgs& p, uint8_t* smem,
 
     // DMA sources: wave w owns 8-row blocks w, w+4, ... of the A tile and of the W tile, as 32-bit lane offsets
     uint32_t ga[C::A_LD], gw[C::W_LD];
-    const int lrow = lane >> 3, lch = (lane & 7) ^ lrow;
+    // rows come in blocks of 8 (block index wave + 4i has the parity of wave): swz<128> of the row
+    const int lrow = lane >> 3, lch = (lane & 7) ^ (((wave & 1) << 2) | (lrow >> 1));
 #pragma unroll
     for (int i = 0; i < C::A_LD; ++i) {
         const int row = (wave + 4 * i) * 8 + lrow;
@@ -656,9 +660,9 @@ __device__ __forceinline__ void dma2_gemm_tile(const GemmArgs& p, uint8_t* smem,
                                              (lds_ptr_t)(s + BM * BK + (wave + 4 * (j - C::A_LD)) * 1024), 16, 0, 0);
     };
 
-    // fragment addresses: row r at r*128, chunk c at slot c ^ (r&7); K sub-step kk flips address bits 5 and 6
+    // fragment addresses: row r at r*128, chunk c at slot c ^ ((r>>1)&7); K sub-step kk flips address bits 5 and 6
     const int frow = lane & 31, fhalf = lane >> 5;
-    const int fsw = (fhalf ^ (frow & 7)) << 4;
+    const int fsw = (fhalf ^ ((frow >> 1) & 7)) << 4;
     int aoff[4], woff[4];
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {
@@ -841,7 +845,8 @@ __global__ void __launch_bounds__(256, 1) int8_gemm_ring_kernel(GemmArgs p) {
 
     // DMA streams.  Each walks (tile, K tile) pairs in the order the MFMAs will consume them and stops on the last one
     // (re-fetching it into a stage nothing reads again keeps the loop free of branches around the DMA slots).
-    const int lrow = lane >> 3, lch = ((lane & 7) ^ lrow) * 16;
+    // rows come in blocks of 8 (block index wave + 4j has the parity of wave): swz<128> of the row
+    const int lrow = lane >> 3, lch = ((lane & 7) ^ (((wave & 1) << 2) | (lrow >> 1))) * 16;
     uint32_t ga[C::A_LD], gw[C::W_LD];
     int a_tile = 0, a_kt = 0, a_stage = 0, w_tile = 0, w_kt = 0, w_stage = 0;
     auto set_a = [&](int i) {
@@ -889,9 +894,9 @@ __global__ void __launch_bounds__(256, 1) int8_gemm_ring_kernel(GemmArgs p) {
         if (++w_kt == nk) { w_kt = 0; set_w(++w_tile); }
     };
 
-    // fragment addresses inside a stage: row r at r*128, chunk c at slot c ^ (r&7); K sub-step kk flips bits 5 and 6
+    // fragment addresses inside a stage: row r at r*128, chunk c at slot c ^ ((r>>1)&7); K sub-step kk flips bits 5 and 6
     const int frow = lane & 31, fhalf = lane >> 5;
-    const int fsw = (fhalf ^ (frow & 7)) << 4;
+    const int fsw = (fhalf ^ ((frow >> 1) & 7)) << 4;
     int aoff[4], woff[4];
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {

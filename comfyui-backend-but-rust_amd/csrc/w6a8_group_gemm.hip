@@ -9,17 +9,19 @@
 //   p_g = sum over the 128 k of group g of A[m,k] * q[n,k], an exact int32.
 //
 // One K tile of the kernel is one group, so every group's int32 partial is a fresh MFMA accumulation (first MFMA with
-// C = 0) that is folded into the fp32 accumulators.  A workgroup of eight waves owns a 256 x 128 tile; per iteration:
-//   * LDS-DMA brings A(g+1) (256 x 128 int8), the packed weights of group g+2 (128 rows x 96 bytes) and the 128 scales
-//     of group g+1 straight into LDS;
-//   * every thread expands two 12-byte pieces of the packed weights of group g+1 into 16 int8 each and writes them
-//     in the swizzled fragment layout (conflict-free both ways);
+// C = 0) that is folded into the fp32 accumulators.  A workgroup of eight waves owns a 256 x 128 tile; per iteration g:
+//   * LDS-DMA brings A(g+2) (256 x 128 int8, three stages), the packed weights of group g+2 (128 rows x 96 bytes, two
+//     stages) and the 128 scales of group g+2 (four stages) straight into LDS.  Every wave issues the same seven
+//     instructions, one after every other MFMA, so one counted wait serves all waves;
+//   * the packed weights are wave-local: wave w fetches rows 16w..16w+15 itself (1.5 KB), waits for its own fetch, and
+//     expands its 128 twelve-byte pieces (two per lane) of group g+1 into 16 int8 each, written in the swizzled
+//     fragment layout (conflict-free both ways).  Only the expanded tile crosses waves, behind the iteration's barrier;
 //   * each wave (2 x 4 grid, 128 x 32 outputs, four MFMA tiles) multiplies group g in two pairs of tiles; the fp32
 //     fold of the first pair rides between the MFMAs of the second.
-// The fold costs two VALU operations per output and group (plus the read of the accumulation register) and the unpack
-// about six per code word: together more issue slots than the MFMAs, so the kernel is bound by VALU issue, not by the
-// matrix pipe.  Two waves share a SIMD; the upper four waves fold their second pair at the end of an iteration, the
-// lower four at the start of the next, so that on every SIMD one wave's VALU-only stretch meets the other's MFMAs.
+// The fold costs two VALU operations per output and group and the unpack about six per code word: together more issue
+// slots than the MFMAs, so the kernel is bound by VALU issue, not by the matrix pipe.  Two waves share a SIMD; the upper
+// four waves fold their second pair at the end of an iteration, the lower four at the start of the next, so that on
+// every SIMD one wave's VALU-only stretch meets the other's MFMAs.
 #include "common.hpp"
 
 #define SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
@@ -40,8 +42,11 @@ struct W6Args {
 
 constexpr int BM = 256, BN = 128, BK = 128, RAW_ROW = 96;
 constexpr int A_STAGE = BM * BK, U_STAGE = BN * BK, R_STAGE = BN * RAW_ROW, S_STAGE = BN * 4;
-constexpr int U_BASE = 2 * A_STAGE, R_BASE = U_BASE + 2 * U_STAGE, S_BASE = R_BASE + 2 * R_STAGE;
-constexpr int SMEM = S_BASE + 3 * S_STAGE;   // three stages of scales: the deferred fold reads those of the group before
+constexpr int NSA = 3, NSS = 4;   // stages of A and of the scales (the deferred fold still reads group g-1 in iteration g)
+constexpr int U_BASE = NSA * A_STAGE, R_BASE = U_BASE + 2 * U_STAGE, S_BASE = R_BASE + 2 * R_STAGE;
+constexpr int SMEM = S_BASE + NSS * S_STAGE;
+constexpr int RAW_WAVE = 16 * RAW_ROW;   // bytes of packed weights a wave owns per group: 16 rows
+static_assert(SMEM <= 160 * 1024, "LDS budget");
 constexpr int TM = 4, TN = 1;   // 32x32 MFMA tiles of one wave: 128 rows (m) x 32 columns (n)
 constexpr int NT = 512;         // eight waves, 2 (m) x 4 (n)
 
@@ -56,6 +61,8 @@ __device__ __forceinline__ int spread6(uint32_t w) {
 __device__ __forceinline__ void dma16(uint32_t lds_dst, uint32_t lane_off, const void* base) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_dst), "v"(lane_off), "s"(base) : "memory", "m0");
 }
+template <int N> __device__ __forceinline__ void wait_vmcnt_n() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+__device__ __forceinline__ void wait_all_dma() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 __device__ __forceinline__ void dma4(uint32_t lds_dst, uint32_t lane_off, const void* base) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds_dst), "v"(lane_off), "s"(base) : "memory", "m0");
 }
@@ -73,7 +80,9 @@ __global__ void __launch_bounds__(NT, 1) w6a8_group_gemm_kernel(W6Args p) {
 
     // DMA sources: 32-bit lane offsets from a per-group scalar base.  Rows past the edge re-read the last valid row;
     // what they produce is never stored.
-    const int lrow = lane >> 3, lch = ((lane & 7) ^ lrow) * 16;   // swizzle applied on the global side
+    // The swizzle (chunk ^ bits 1..3 of the row: 16 consecutive rows of a chunk column then cover all 64 LDS banks) is
+    // applied on the global side; rows come in blocks of 8 whose index wave + 8j has the parity of wave.
+    const int lrow = lane >> 3, lch = ((lane & 7) ^ (((wave & 1) << 2) | (lrow >> 1))) * 16;
     uint32_t ga[4], gr[2], gs;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -83,48 +92,49 @@ __global__ void __launch_bounds__(NT, 1) w6a8_group_gemm_kernel(W6Args p) {
     }
     const uint32_t wrow = (uint32_t)p.K / 4 * 3;                   // bytes per packed weight row
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {                                  // 12 instructions cover the raw tile: waves 0-3 issue two
-        const int c = (wave + 8 * j) * 64 + lane;                  // 16-byte chunk of the raw tile: row c/6, part c%6
-        const int row = (c / 6) & 127, part = c % 6;
+    for (int j = 0; j < 2; ++j) {                                  // the wave's own 1.5 KB: one full and one half instruction
+        const int b = (64 * j + (j ? (lane & 31) : lane)) * 16;    // byte inside the wave's block of 16 rows x 96 bytes
+        const int row = 16 * wave + b / RAW_ROW, col = b % RAW_ROW;
         const int r = n0 + row < p.N ? n0 + row : p.N - 1;
-        gr[j] = (uint32_t)r * wrow + part * 16;
+        gr[j] = (uint32_t)r * wrow + col;
     }
     {
-        const int row = 32 * (wave & 3) + (lane & 31);
+        const int row = 16 * wave + (lane & 15);
         const int r = n0 + row < p.N ? n0 + row : p.N - 1;
         gs = (uint32_t)r * (uint32_t)ng * 4u;
     }
-    auto fetch_a = [&](int g, int stage) {
-        const int8_t* base = p.A + (int64_t)(g < ng ? g : ng - 1) * BK;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) dma16(lds_base + stage * A_STAGE + (wave + 8 * j) * 1024, ga[j], base);
+    // The seven DMA instructions a wave issues per group.  Groups past the end re-fetch the last one (into stages that
+    // nothing reads again), which keeps the loop free of branches and the count per iteration fixed.
+    auto dma_a = [&](int g, int stage, int j) {
+        dma16(lds_base + stage * A_STAGE + (wave + 8 * j) * 1024, ga[j], p.A + (int64_t)(g < ng ? g : ng - 1) * BK);
     };
-    auto fetch_raw = [&](int g, int stage) {
+    auto dma_raw = [&](int g, int stage, int j) {
         const uint8_t* base = p.Wp + (int64_t)(g < ng ? g : ng - 1) * RAW_ROW;
-        dma16(lds_base + R_BASE + stage * R_STAGE + wave * 1024, gr[0], base);
-        if (wave < 4) dma16(lds_base + R_BASE + stage * R_STAGE + (wave + 8) * 1024, gr[1], base);
+        const uint32_t dst = lds_base + R_BASE + stage * R_STAGE + wave * RAW_WAVE + j * 1024;
+        if (j == 0) dma16(dst, gr[0], base);
+        else if (lane < 32) dma16(dst, gr[1], base);
     };
-    auto fetch_scales = [&](int g, int stage) {
-        const float* base = p.sw + (g < ng ? g : ng - 1);
-        if (wave < 4 && lane < 32) dma4(lds_base + S_BASE + stage * S_STAGE + wave * 128, gs, base);
+    auto dma_scales = [&](int g, int stage) {
+        if (lane < 16) dma4(lds_base + S_BASE + stage * S_STAGE + wave * 64, gs, p.sw + (g < ng ? g : ng - 1));
     };
-    // Piece e of the raw tile is bytes [12e, 12e+12): row e/8, codes 16*(e%8) .. +15 -> one 16-byte chunk.  Reading
-    // the three words and expanding them are separate steps so that the LDS latency hides behind other work.
+    // Piece e of the wave's block is bytes [12e, 12e+12): row 16*wave + e/8, codes 16*(e%8) .. +15 -> one 16-byte
+    // chunk.  Reading the three words and expanding them are separate steps so that the LDS latency hides behind
+    // other work.
     auto raw_read = [&](int rstage, int i, uint32_t (&d)[3]) {
-        const uint32_t* src = reinterpret_cast<const uint32_t*>(smem + R_BASE + rstage * R_STAGE + 12 * (tid + NT * i));
+        const uint32_t* src = reinterpret_cast<const uint32_t*>(smem + R_BASE + rstage * R_STAGE + wave * RAW_WAVE + 12 * (lane + 64 * i));
         d[0] = src[0]; d[1] = src[1]; d[2] = src[2];
     };
     auto unpack_write = [&](int ustage, int i, const uint32_t (&d)[3]) {
-        const int e = tid + NT * i;
+        const int e = lane + 64 * i;
         const v4i out = v4i{spread6(d[0]), spread6(__builtin_amdgcn_alignbit(d[1], d[0], 24)),
                             spread6(__builtin_amdgcn_alignbit(d[2], d[1], 16)), spread6(d[2] >> 8)};
-        const int r = e >> 3, pc = e & 7;
-        *reinterpret_cast<v4i*>(smem + U_BASE + ustage * U_STAGE + r * BK + ((pc ^ (r & 7)) << 4)) = out;
+        const int r = 16 * wave + (e >> 3), pc = e & 7;
+        *reinterpret_cast<v4i*>(smem + U_BASE + ustage * U_STAGE + r * BK + ((pc ^ ((r >> 1) & 7)) << 4)) = out;
     };
 
-    // fragment addresses inside a stage: row r at r*128, chunk c at slot c ^ (r&7); K sub-step kk flips bits 5 and 6
+    // fragment addresses inside a stage: row r at r*128, chunk c at slot c ^ ((r>>1)&7); K sub-step kk flips bits 5 and 6
     const int frow = lane & 31, fhalf = lane >> 5;
-    const int fsw = (fhalf ^ (frow & 7)) << 4;
+    const int fsw = (fhalf ^ ((frow >> 1) & 7)) << 4;
     int aoff[4], woff[4];
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {
@@ -141,13 +151,16 @@ __global__ void __launch_bounds__(NT, 1) w6a8_group_gemm_kernel(W6Args p) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) accf[in][im][r] = 0.f;
 
-    // prologue: A(0), raw(0), raw(1), scales(0) land; raw(0) is unpacked
-    fetch_a(0, 0);
-    fetch_raw(0, 0);
-    fetch_raw(1, 1);
-    fetch_scales(0, 0);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
+    // prologue: groups 0 and 1 of everything land; the wave's rows of group 0 are unpacked
+#pragma unroll
+    for (int g = 0; g < 2; ++g) {
+        dma_raw(g, g, 0);
+        dma_raw(g, g, 1);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) dma_a(g, g, j);
+        dma_scales(g, g);
+    }
+    wait_all_dma();
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
         uint32_t d[3];
@@ -170,29 +183,19 @@ __global__ void __launch_bounds__(NT, 1) w6a8_group_gemm_kernel(W6Args p) {
             accf[0][im][4 * q + c] = __builtin_fmaf((float)part[0][im][4 * q + c], sv[c], accf[0][im][4 * q + c]);
     };
 
-    int ss = 0;   // scale stage of group g = g mod 3
+    int a_cur = 0, s_cur = 0;   // stages of group g: g mod 3 (A), g mod 4 (scales)
     for (int g = 0; g < ng; ++g) {
         const int s = g & 1;
-        const uint8_t* sa = smem + s * A_STAGE;
+        const int a_new = a_cur == 0 ? 2 : a_cur - 1;                  // (g + 2) mod 3
+        const int s_new = (s_cur + 2) & 3, s_prev = (s_cur + 3) & 3;   // (g + 2) mod 4, (g - 1) mod 4
+        const uint8_t* sa = smem + a_cur * A_STAGE;
         const uint8_t* su = smem + U_BASE + s * U_STAGE;
-        const float* sc = reinterpret_cast<const float*>(smem + S_BASE + ss * S_STAGE);
-        const float* sc_prev = reinterpret_cast<const float*>(smem + S_BASE + (ss == 0 ? 2 : ss - 1) * S_STAGE);
-        const int ss_next = ss == 2 ? 0 : ss + 1;
-        // All of these targets were last read during iteration g-1 (the scale stage: g-2), which every wave has left.
-        fetch_a(g + 1, s ^ 1);
-        fetch_raw(g + 2, s);
-        fetch_scales(g + 1, ss_next);
-        SCHED_FENCE();
+        const float* sc = reinterpret_cast<const float*>(smem + S_BASE + s_cur * S_STAGE);
+        const float* sc_prev = reinterpret_cast<const float*>(smem + S_BASE + s_prev * S_STAGE);
 
         v4i fa[2][4], fw[4], na[2][4];
         float4 sv[4];
         uint32_t raw[2][3];
-        auto load_a = [&](v4i (&dst)[2][4], int imb) {
-#pragma unroll
-            for (int t = 0; t < 2; ++t)
-#pragma unroll
-                for (int kk = 0; kk < 4; ++kk) dst[t][kk] = *reinterpret_cast<const v4i*>(sa + aoff[kk] + (imb + t) * 32 * BK);
-        };
         // Eight MFMAs of the pair (imb, imb+1), the two accumulation chains interleaved; between(i) is issued after the
         // i-th of them.
         auto mma_pair = [&](int imb, v4i (&a)[2][4], auto&& between) {
@@ -214,10 +217,16 @@ __global__ void __launch_bounds__(NT, 1) w6a8_group_gemm_kernel(W6Args p) {
                 }
         };
 
+        // The wave's own packed rows of group g+1 were the first two DMA instructions of the previous iteration; the
+        // five issued after them may still be in flight.
+        wait_vmcnt_n<5>();
         // everything this iteration reads from LDS early: fragments of the first pair, the group's scales, packed words
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk) fw[kk] = *reinterpret_cast<const v4i*>(su + woff[kk]);
-        load_a(fa, 0);
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) fa[t][kk] = *reinterpret_cast<const v4i*>(sa + aoff[kk] + t * 32 * BK);
 #pragma unroll
         for (int q = 0; q < 4; ++q) sv[q] = *reinterpret_cast<const float4*>(sc + wn * 32 + 8 * q + 4 * fhalf);
 #pragma unroll
@@ -232,13 +241,24 @@ __global__ void __launch_bounds__(NT, 1) w6a8_group_gemm_kernel(W6Args p) {
             }
             SCHED_FENCE();
         }
-        // the second pair's A fragments take over the registers of the first pair's as those are consumed
+        // The second pair's A fragments take over the registers of the first pair's as those are consumed.  DMA targets:
+        // the packed stage of group g (expanded during iteration g-1), the A stage of group g-1 and the scale stage of
+        // group g-2, all of them last read before the barrier that ended iteration g-1.
         mma_pair(0, fa, [&](int i) {
             na[i & 1][i >> 1] = *reinterpret_cast<const v4i*>(sa + aoff[i >> 1] + (2 + (i & 1)) * 32 * BK);
+            if (i == 1) dma_raw(g + 2, s, 0);
+            if (i == 3) dma_raw(g + 2, s, 1);
+            if (i == 5) dma_a(g + 2, a_new, 0);
+            if (i == 7) dma_a(g + 2, a_new, 1);
             if (i == 2) unpack_write(s ^ 1, 0, raw[0]);
             if (i == 4) unpack_write(s ^ 1, 1, raw[1]);
         });
-        mma_pair(2, na, [&](int i) { fold(i & 1, i >> 1, sv[i >> 1]); });
+        mma_pair(2, na, [&](int i) {
+            fold(i & 1, i >> 1, sv[i >> 1]);
+            if (i == 1) dma_a(g + 2, a_new, 2);
+            if (i == 3) dma_a(g + 2, a_new, 3);
+            if (i == 5) dma_scales(g + 2, s_new);
+        });
         if (!defer) {
 #pragma unroll
             for (int i = 0; i < 8; ++i) fold(2 + (i & 1), i >> 1, sv[i >> 1]);
@@ -253,13 +273,16 @@ __global__ void __launch_bounds__(NT, 1) w6a8_group_gemm_kernel(W6Args p) {
                     const int n = n0 + wn * 32 + 8 * (r >> 2) + 4 * fhalf + (r & 3);
                     if (m < p.M && n < p.N) p.partials[((int64_t)m * p.N + n) * ng + g] = part[0][im][r];
                 }
+            wait_all_dma();   // the dump's stores share the counter: drain it rather than count them
         }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the DMA of this iteration has landed
-        __syncthreads();                                    // ... for every wave, and the unpacked tile is written
-        ss = ss_next;
+        wait_vmcnt_n<7>();   // everything older than this iteration's seven has landed: A and scales of group g+1
+        __syncthreads();     // ... for every wave, and the expanded weights of group g+1 are written
+        a_cur = a_cur == 2 ? 0 : a_cur + 1;
+        s_cur = (s_cur + 1) & 3;
     }
-    if (defer) {   // ss now names the stage after the last group's
-        const float* sc_last = reinterpret_cast<const float*>(smem + S_BASE + (ss == 0 ? 2 : ss - 1) * S_STAGE);
+    wait_all_dma();   // nothing may still be writing this workgroup's LDS when it retires or reuses it
+    if (defer) {
+        const float* sc_last = reinterpret_cast<const float*>(smem + S_BASE + ((s_cur + 3) & 3) * S_STAGE);
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const float4 sp = *reinterpret_cast<const float4*>(sc_last + wn * 32 + 8 * q + 4 * fhalf);
@@ -267,6 +290,7 @@ __global__ void __launch_bounds__(NT, 1) w6a8_group_gemm_kernel(W6Args p) {
             fold(3, q, sp);
         }
     }
+    __syncthreads();   // every wave's DMA is drained before the epilogue reuses the stages
 
     // Epilogue.  A lane holds one m and runs of four consecutive n, so storing straight from the registers would touch
     // 32 rows per instruction.  When the rows of D are 16-byte aligned each wave instead passes its tile, 32 rows at a
