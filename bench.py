@@ -8,7 +8,8 @@ M=4608 tokens, K=3072, N=12288, bf16 in and out, Hadamard block 128.
 
 Prints ONE JSON line: whole-step throughput in TOPS (2*M*N*K per step), the roofline of the dominant kernel (the int8
 GEMM against the dense int8 MFMA peak) from HIP events recorded inside the timed region, the CPU oracle timed on a
-bounded row sample, and the memory-bound skinny (M=256) linears as HBM GB/s.
+bounded row sample, the memory-bound skinny (M=256) linears as HBM GB/s, the other linears of the model configurations
+and the W6A8 (packed 6-bit weights, unpack fused into the GEMM) pair.
 """
 import argparse
 import importlib
@@ -33,6 +34,7 @@ def parse():
     ap.add_argument("--rotate", type=int, default=128, help="Hadamard block (0 = none, 64, 128, 256)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-skinny", action="store_true")
+    ap.add_argument("--no-extra", action="store_true", help="skip the other linears of the model configurations and the W6A8 shapes")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 256 MiB device copy a few times: under rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE its "
@@ -85,6 +87,37 @@ def time_linear(torch, ffi, d, M, K, N, rotate, steps, warmup, nbuf=1):
     tq = sum(e[0].elapsed_time(e[1]) for e in evs) / steps
     tg = sum(e[1].elapsed_time(e[2]) for e in evs) / steps
     return max(gpu_ms, 0.0), wall_ms, tq, tg
+
+
+def time_w6a8(torch, ffi, M, K, N, steps, warmup):
+    """The fused-unpack W6A8 GEMM (24-bit words of four 6-bit codes, fp32 scales per 128 along K) on synthetic weights
+    with codes uniform in [-31, 31]; returns the average microseconds of gpu_w6a8_group_gemm."""
+    g = torch.Generator(device="cuda:0").manual_seed(4)
+    u = torch.randint(1, 64, (N, K // 4, 4), dtype=torch.int32, device="cuda:0", generator=g)   # u = q + 32
+    w = u[..., 0] | (u[..., 1] << 6) | (u[..., 2] << 12) | (u[..., 3] << 18)
+    packed = torch.stack((w & 255, (w >> 8) & 255, w >> 16), dim=-1).to(torch.uint8).reshape(N, K // 4 * 3).contiguous()
+    del u, w
+    A = torch.randint(-127, 128, (M, K), dtype=torch.int8, device="cuda:0", generator=g)
+    xs = torch.rand(M, device="cuda:0", generator=g) * 0.1 + 0.01
+    sw = torch.rand(N, K // 128, device="cuda:0", generator=g) * 9e-3 + 1e-3
+    bias = (torch.randn(N, device="cuda:0", generator=g) * 0.02).to(torch.bfloat16)
+    D = torch.empty((M, N), dtype=torch.bfloat16, device="cuda:0")
+    st = torch.cuda.current_stream()
+
+    def run():
+        ffi.k("gpu_w6a8_group_gemm", A.data_ptr(), packed.data_ptr(), xs.data_ptr(), sw.data_ptr(), bias.data_ptr(), D.data_ptr(),
+              0, M, N, K, ffi.DT_BF16, st.cuda_stream)
+
+    for _ in range(warmup):
+        run()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record(st)
+    for _ in range(steps):
+        run()
+    e1.record(st)
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps * 1e3
 
 
 def cpu_baseline(host, M, K, N, rotate, target_s):
@@ -171,6 +204,25 @@ def main():
                        "quant_rows_us": round(tq2 * 1e3, 2), "weight_copies_rotated": nbuf})
             del h2, d2
         out["skinny"] = sk
+    if not a.no_extra:
+        # the other linears of the image-DiT block and the SDXL-UNet level, then the video-DiT W6A8 pair
+        extra = []
+        few = max(5, a.steps // 3)
+        for (name, m, k, n, rot) in (("dit qkv", 4608, 3072, 9216, a.rotate), ("dit out-proj", 4608, 3072, 3072, a.rotate),
+                                     ("dit mlp down", 4608, 12288, 3072, a.rotate), ("sdxl attn proj", 8192, 640, 640, 0),
+                                     ("sdxl geglu up", 8192, 640, 5120, 0), ("sdxl down", 8192, 2560, 640, 0)):
+            h2, d2 = make_inputs(torch, synth, m, k, n, seed=2, kind="t3" if rot else "normal")
+            _, wall2, tq2, tg2 = time_linear(torch, ffi, d2, m, k, n, rot, few, 3)
+            extra.append({"name": name, "M": m, "K": k, "N": n, "rotate": rot, "quant_rows_us": round(tq2 * 1e3, 2),
+                          "int8_gemm_us": round(tg2 * 1e3, 2), "gemm_TOPS": round(2.0 * m * n * k / (tg2 * 1e-3) / 1e12, 1)})
+            del h2, d2
+        out["linears"] = extra
+        w6 = []
+        for (name, m, k, n) in (("video-dit ffn up", 8192, 5120, 13824), ("video-dit ffn down", 8192, 13824, 5120)):
+            us = time_w6a8(torch, ffi, m, k, n, few, 2)
+            w6.append({"name": name, "M": m, "K": k, "N": n, "kernel": "gpu_w6a8_group_gemm", "us": round(us, 1),
+                       "TOPS": round(2.0 * m * n * k / us / 1e6, 1), "frac_int8_peak": round(2.0 * m * n * k / us / 1e6 / PEAK_INT8_TOPS, 4)})
+        out["w6a8"] = w6
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(host, M, K, N, a.rotate, a.cpu_seconds)
     print(json.dumps(out))
