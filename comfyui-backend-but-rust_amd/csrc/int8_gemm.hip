@@ -1003,6 +1003,214 @@ __global__ void __launch_bounds__(256, 1) int8_gemm_ring_kernel(GemmArgs p) {
     wait_vmcnt<0>();   // no DMA may still be writing this workgroup's LDS when it retires
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// Weight-streaming kernel for skinny M (M <= 256): one row of 256 x 96 tiles, every weight read from HBM exactly once.
+// An iteration of such a tile is short (24 MFMAs per wave) against the 44 DMA instructions that feed it, and a DMA
+// instruction holds its wave's issue port for about 70 cycles: in the ring kernel above, where the MFMA waves issue
+// their own DMA, a skinny launch spends as long issuing loads as multiplying.  Here the roles are split over eight waves:
+//   waves 0-3  multiply (64 x 96 each, MFMA + fragment reads only, no memory instruction in their K loop);
+//   wave  4    streams W: 12 DMA instructions per K tile into a ring of 5 stages, three K tiles ahead;
+//   waves 5-7  stream A (from L2: all CUs read the same 256 rows) into three stages, 10-11 instructions per K tile each.
+// Everybody meets at the ring kernel's two barriers per iteration, X (the stage of iteration g-1 is free) and Y (what
+// iteration g+1 needs has landed; the MFMA waves run three sub-steps before it and one after).  So that no wave makes
+// the others wait at a barrier, each producer splits its instructions between the two phases in the proportion of the
+// MFMA waves' work, three quarters before Y and one quarter after.  The counter a producer waits on retires in
+// order, which is why W has a wave to itself: its wait lets two and three quarter K tiles stay in flight.
+// Requires K % 128 == 0 and M*K, N*K < 2^32.
+// ---------------------------------------------------------------------------------------------------------------
+struct StreamCfg {
+    static constexpr int BM = 256, BN = 96, BK = 128, NT = 512, NSA = 3, NSW = 5;
+    static constexpr int WTM = 64, WTN = 96, TM = 2, TN = 3, NM = TM * TN, NF = TM + TN;
+    static constexpr int A_STAGE = BM * BK, W_STAGE = BN * BK, W_BASE = NSA * A_STAGE, SMEM = W_BASE + NSW * W_STAGE;
+    static constexpr int A_BLK = BM / 8, W_BLK = BN / 8;    // 1 KB DMA blocks (8 rows) per stage
+    static constexpr int A_PER = (A_BLK + 2) / 3;           // per A wave: blocks ap, ap+3, ...
+    static constexpr int A_EARLY = 8, W_EARLY = 9;          // instructions a producer issues before barrier Y
+    static_assert(SMEM <= 160 * 1024 && (NSW - 3) * W_BLK + W_EARLY <= 63, "LDS budget; wait counts are 6-bit fields");
+};
+
+template <int OUT_DT, int EPI>
+__global__ void __launch_bounds__(StreamCfg::NT, 1) int8_gemm_stream_kernel(GemmArgs p) {
+    using C = StreamCfg;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    constexpr int BK = C::BK, TM = C::TM, TN = C::TN, NM = C::NM, NF = C::NF;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int ld = p.K;
+    // split K: workgroup row blockIdx.y multiplies K slice [k_lo, k_lo + nk*128) and writes its own int32 plane
+    const int k_lo = p.kslice ? (int)blockIdx.y * p.kslice : 0;
+    const int k_len = p.kslice ? (p.K - k_lo < p.kslice ? p.K - k_lo : p.kslice) : p.K;
+    const int nk = k_len / BK;
+    if (p.kslice) p.D = (uint8_t*)p.D + (int64_t)blockIdx.y * p.M * p.N * 4;
+    const int G = gridDim.x, ntiles = p.tiles_m * p.tiles_n;
+    const int nt_b = (ntiles - (int)blockIdx.x + G - 1) / G;   // tiles of this workgroup: blockIdx, blockIdx + G, ...
+    auto tile_origin = [&](int i, int& m0, int& n0) {
+        int tm, tn;
+        tile_of_block((int)blockIdx.x + i * G, ntiles, p.tiles_m, p.tiles_n, tm, tn);
+        m0 = tm * C::BM;
+        n0 = tn * C::BN;
+    };
+    const uint32_t lds_base = (uint32_t)(uintptr_t)smem;
+    const int lrow = lane >> 3;
+    auto dma = [&](uint32_t dst, uint32_t off, const int8_t* base) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(off), "s"(base) : "memory", "m0");
+    };
+
+    if (wave == 4) {
+        // ---- the W stream.  Block j is rows 8j..8j+7 of the tile; chunk swizzle (bits 1..3 of the row) on the global side.
+        uint32_t gw[C::W_BLK];
+        int w_tile = 0, w_kt = 0, w_stage = 0;
+        auto set_w = [&](int i) {
+            int m0, n0;
+            tile_origin(i, m0, n0);
+#pragma unroll
+            for (int j = 0; j < C::W_BLK; ++j) {
+                const int row = j * 8 + lrow;
+                const int gr = n0 + row < p.N ? n0 + row : p.N - 1;
+                gw[j] = (uint32_t)gr * (uint32_t)ld + (((lane & 7) ^ (((j & 1) << 2) | (lrow >> 1))) << 4);
+            }
+        };
+        // blocks [j0, j1) of the stream's current K tile into the current stage
+        auto fetch_w = [&](int j0, int j1) {
+            const int8_t* base = p.W + k_lo + (int64_t)w_kt * BK;
+#pragma unroll
+            for (int j = 0; j < C::W_BLK; ++j)
+                if (j >= j0 && j < j1) dma(lds_base + C::W_BASE + w_stage * C::W_STAGE + j * 1024, gw[j], base);
+        };
+        auto next_w = [&]() {   // the stream stops on its last K tile and keeps re-fetching it
+            w_stage = w_stage == C::NSW - 1 ? 0 : w_stage + 1;
+            if (w_tile == nt_b - 1 && w_kt == nk - 1) return;
+            if (++w_kt == nk) { w_kt = 0; set_w(++w_tile); }
+        };
+        set_w(0);
+#pragma unroll
+        for (int i = 0; i < C::NSW - 1; ++i) { fetch_w(0, C::W_BLK); next_w(); }   // W(0) .. W(NSW-2)
+        wait_vmcnt<(C::NSW - 2) * C::W_BLK>();                                     // W(0) has landed
+        wg_barrier();
+        for (int ti = 0; ti < nt_b; ++ti) {
+            for (int kt = 0; kt < nk; ++kt) {
+                wg_barrier();                                     // X: the stage of iteration g-1 is free
+                fetch_w(0, C::W_EARLY);                           // W(g + NSW - 1), first part
+                wait_vmcnt<(C::NSW - 3) * C::W_BLK + C::W_EARLY>();   // W(g + 1) has landed
+                wg_barrier();                                     // Y
+                fetch_w(C::W_EARLY, C::W_BLK);
+                next_w();
+            }
+            wg_barrier();                                         // in front of the epilogue
+        }
+        wait_vmcnt<0>();   // no DMA may still be writing this workgroup's LDS when it retires
+        return;
+    }
+    if (wave > 4) {
+        // ---- the A stream: wave 5 + ap takes blocks ap, ap + 3, ...
+        const int ap = wave - 5;
+        uint32_t ga[C::A_PER];
+        int a_tile = 0, a_kt = 0, a_stage = 0;
+        auto set_a = [&](int i) {
+            int m0, n0;
+            tile_origin(i, m0, n0);
+#pragma unroll
+            for (int j = 0; j < C::A_PER; ++j) {
+                const int b = ap + 3 * j;
+                const int row = (b < C::A_BLK ? b : C::A_BLK - 1) * 8 + lrow;
+                const int gr = m0 + row < p.M ? m0 + row : p.M - 1;
+                ga[j] = (uint32_t)gr * (uint32_t)ld + (((lane & 7) ^ (((b & 1) << 2) | (lrow >> 1))) << 4);
+            }
+        };
+        auto fetch_a = [&](int j0, int j1) {
+            const int8_t* base = p.A + k_lo + (int64_t)a_kt * BK;
+#pragma unroll
+            for (int j = 0; j < C::A_PER; ++j)
+                if (j >= j0 && j < j1 && ap + 3 * j < C::A_BLK) dma(lds_base + a_stage * C::A_STAGE + (ap + 3 * j) * 1024, ga[j], base);
+        };
+        auto next_a = [&]() {
+            a_stage = a_stage == C::NSA - 1 ? 0 : a_stage + 1;
+            if (a_tile == nt_b - 1 && a_kt == nk - 1) return;
+            if (++a_kt == nk) { a_kt = 0; set_a(++a_tile); }
+        };
+        set_a(0);
+        fetch_a(0, C::A_PER);                                     // A(0)
+        next_a();
+        wait_vmcnt<0>();
+        fetch_a(0, C::A_PER);                                     // A(1)
+        next_a();
+        wg_barrier();
+        for (int ti = 0; ti < nt_b; ++ti) {
+            for (int kt = 0; kt < nk; ++kt) {
+                wg_barrier();                                     // X: the stage of iteration g-1 is free
+                fetch_a(0, C::A_EARLY);                           // A(g + 2), first part
+                wait_vmcnt<C::A_EARLY>();                         // A(g + 1) has landed
+                wg_barrier();                                     // Y
+                fetch_a(C::A_EARLY, C::A_PER);
+                next_a();
+            }
+            wg_barrier();                                         // in front of the epilogue
+        }
+        wait_vmcnt<0>();
+        return;
+    }
+
+    // ---- the four MFMA waves: wave w multiplies rows 64w..64w+63 of the tile by all 96 columns
+    const int wm = wave;
+    const int frow = lane & 31, fhalf = lane >> 5;
+    const int fsw = (fhalf ^ ((frow >> 1) & 7)) << 4;
+    int aoff[4], woff[4];
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+        aoff[kk] = ((wm * C::WTM + frow) * BK + fsw) ^ (kk << 5);
+        woff[kk] = (frow * BK + fsw) ^ (kk << 5);
+    }
+    auto frag = [&](const uint8_t* sa, const uint8_t* sw, int kk, int j) -> v4i {
+        if (j < TM) return *reinterpret_cast<const v4i*>(sa + aoff[kk] + j * 32 * BK);
+        return *reinterpret_cast<const v4i*>(sw + woff[kk] + (j - TM) * 32 * BK);
+    };
+    v16i acc[TN][TM];
+    v4i f0[NF], f1[NF];
+    auto substep = [&](v4i* cur, v4i* nxt, const uint8_t* sa_n, const uint8_t* sw_n, int kk_n) {
+#pragma unroll
+        for (int i = 0; i < NM; ++i) {
+            const int in = i / TM, im = i % TM;
+            acc[in][im] = __builtin_amdgcn_mfma_i32_32x32x32_i8(cur[TM + in], cur[im], acc[in][im], 0, 0, 0);
+            SCHED_FENCE();
+            if (i < NF) { nxt[i] = frag(sa_n, sw_n, kk_n, i); SCHED_FENCE(); }
+        }
+    };
+    wg_barrier();   // A(0) and W(0) have landed
+#pragma unroll
+    for (int j = 0; j < NF; ++j) f0[j] = frag(smem, smem + C::W_BASE, 0, j);
+    int ca = 0, cw = 0;   // stages of the iteration being multiplied
+    for (int ti = 0; ti < nt_b; ++ti) {
+#pragma unroll
+        for (int in = 0; in < TN; ++in)
+#pragma unroll
+            for (int im = 0; im < TM; ++im)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[in][im][r] = 0;
+        int pa = 0;
+        for (int kt = 0; kt < nk; ++kt) {
+            const uint8_t* sa = smem + ca * C::A_STAGE;
+            const uint8_t* sw = smem + C::W_BASE + cw * C::W_STAGE;
+            const int na = ca == C::NSA - 1 ? 0 : ca + 1, nw = cw == C::NSW - 1 ? 0 : cw + 1;
+            wg_barrier();                                                   // X
+            substep(f0, f1, sa, sw, 1);
+            substep(f1, f0, sa, sw, 2);
+            substep(f0, f1, sa, sw, 3);
+            wg_barrier();                                                   // Y
+            substep(f1, f0, smem + na * C::A_STAGE, smem + C::W_BASE + nw * C::W_STAGE, 0);
+            pa = ca;
+            ca = na;
+            cw = nw;
+        }
+        int m0, n0;
+        tile_origin(ti, m0, n0);
+        __syncthreads();   // every wave is done with the stage that becomes the shuffle scratch (8 KB per wave)
+        constexpr int SZ = (EPI == EPI_ACC || OUT_DT == DT_F32) ? 4 : 2;
+        // (The stage of A(g) is refilled with A(g+3), issued after barrier X of the next iteration: behind this epilogue.)
+        epilogue_shuffle<TM, TN, OUT_DT, EPI, 32, true>(p, acc, m0 + wm * C::WTM, n0, lane, smem + pa * C::A_STAGE + wave * 8192);
+#pragma unroll
+        for (int j = 0; j < NF; ++j) f0[j] = frag(smem + ca * C::A_STAGE, smem + C::W_BASE + cw * C::W_STAGE, 0, j);
+    }
+}
+
 // Sum of the int32 planes of a split-K run, then the epilogue.  planes[s][M][N]; four consecutive n per thread.
 template <int OUT_DT, int EPI>
 __global__ void __launch_bounds__(256) splitk_epilogue_kernel(GemmArgs p, const int* planes, int slices) {
@@ -1099,42 +1307,71 @@ int launch_ring(GemmArgs a, hipStream_t st) {
     return launch_ring_cfg<RingL, OUT_DT, EPI>(a, 1, st);
 }
 
-// M <= 256: one row of tiles, the weights are read once and the run is bound by how fast they stream.  Narrow tiles
-// give every CU a column slab; when N is too small for that, K is split as well: each slice writes an int32 plane
-// (exact, so the order of the sum does not matter) into a stream-ordered scratch allocation and a second kernel adds
-// the planes and applies the epilogue.
+// Keep freed scratch in the device's default pool instead of returning it to the driver at every synchronization, as
+// the reference's runtime layer does at start-up (src/cuda.rs:88-97): otherwise each call that needs scratch pays a
+// fresh allocation.
+void retain_pool_memory() {
+    static bool pool_set = false;   // benign race: the attribute is idempotent
+    if (pool_set) return;
+    int dev = 0;
+    hipMemPool_t pool;
+    uint64_t keep = ~(uint64_t)0;
+    if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetDefaultMemPool(&pool, dev) == hipSuccess)
+        (void)hipMemPoolSetAttribute(pool, hipMemPoolAttrReleaseThreshold, &keep);
+    pool_set = true;
+}
+
+// Launches the weight-streaming kernel on `slices` K slices (1 = whole K).  With slices > 1, EPI must be EPI_ACC and a.D
+// the int32 planes.
+template <int OUT_DT, int EPI>
+int launch_stream(GemmArgs a, int slices, hipStream_t st) {
+    using C = StreamCfg;
+    a.tiles_m = (a.M + C::BM - 1) / C::BM;
+    a.tiles_n = (a.N + C::BN - 1) / C::BN;
+    const int64_t ntiles = (int64_t)a.tiles_m * a.tiles_n;
+    if (ntiles > 0x7fffffff) return -1;
+    auto kern = int8_gemm_stream_kernel<OUT_DT, EPI>;
+    static bool once = false;  // benign race: the attribute is idempotent
+    if (!once) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
+        if (e != hipSuccess) return (int)e;
+        once = true;
+    }
+    const int num_cu = device_cu_count();
+    const int64_t per_slice = slices > 1 ? (num_cu / slices > 0 ? num_cu / slices : 1) : num_cu;
+    const unsigned grid = (unsigned)(ntiles < per_slice ? ntiles : per_slice);
+    hipLaunchKernelGGL(kern, dim3(grid, (unsigned)slices), dim3(C::NT), C::SMEM, st, a);
+    KCHECK();
+    return 0;
+}
+
+// M <= 256: one row of 256 x 96 tiles, the weights are read once and the run is bound by how fast they stream.  When N
+// is too small to give every CU a column slab, K is split as well: each slice writes an int32 plane (exact, so the
+// order of the sum does not matter) into a stream-ordered scratch allocation and a second kernel adds the planes and
+// applies the epilogue.
 template <int OUT_DT, int EPI>
 int launch_skinny(GemmArgs a, hipStream_t st) {
     bool vec_ok, aligned;
     epilogue_alignment<OUT_DT, EPI>(a, vec_ok, aligned);
     if (!aligned) return launch_cfg<CfgM, OUT_DT, EPI>(a, st);
     const int num_cu = device_cu_count();
-    const int t96 = (a.N + 95) / 96, t128 = (a.N + 127) / 128, nk = a.K / 128;
-    if (t96 * 4 >= num_cu * 3) return launch_ring_cfg<RingN96, OUT_DT, EPI>(a, 1, st);
-    int slices = num_cu / t128;
+    const int t96 = (a.N + 95) / 96, nk = a.K / 128;
+    int slices = t96 * 4 >= num_cu * 3 ? 1 : num_cu / t96;
     if (slices > nk) slices = nk;
-    if (slices <= 1) return launch_ring_cfg<RingN128, OUT_DT, EPI>(a, 1, st);
-    const int per = (nk + slices - 1) / slices;       // K tiles per slice
-    slices = (nk + per - 1) / per;                    // no empty slice
-    if (slices <= 1) return launch_ring_cfg<RingN128, OUT_DT, EPI>(a, 1, st);
-    // Keep freed scratch in the device's default pool instead of returning it to the driver at every synchronization,
-    // as the reference's runtime layer does at start-up (src/cuda.rs:88-97): otherwise each call pays a fresh allocation.
-    static bool pool_set = false;   // benign race: the attribute is idempotent
-    if (!pool_set) {
-        int dev = 0;
-        hipMemPool_t pool;
-        uint64_t keep = ~(uint64_t)0;
-        if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetDefaultMemPool(&pool, dev) == hipSuccess)
-            (void)hipMemPoolSetAttribute(pool, hipMemPoolAttrReleaseThreshold, &keep);
-        pool_set = true;
+    if (slices > 1) {
+        const int per = (nk + slices - 1) / slices;   // K tiles per slice
+        slices = (nk + per - 1) / per;                // no empty slice
     }
+    if (slices <= 1) return launch_stream<OUT_DT, EPI>(a, 1, st);
+    const int per = (nk + slices - 1) / slices;
+    retain_pool_memory();
     int* planes = nullptr;
     hipError_t e = hipMallocAsync((void**)&planes, (size_t)slices * a.M * a.N * sizeof(int), st);
     if (e != hipSuccess) return (int)e;
     GemmArgs pa = a;
     pa.D = planes;
     pa.kslice = per * 128;
-    int rc = launch_ring_cfg<RingN128, DT_F32, EPI_ACC>(pa, slices, st);
+    int rc = launch_stream<DT_F32, EPI_ACC>(pa, slices, st);
     if (rc == 0) {
         const int64_t nvec = (int64_t)a.M * a.N / 4;
         const unsigned grid = (unsigned)((nvec + 255) / 256 < 4096 ? (nvec + 255) / 256 : 4096);
