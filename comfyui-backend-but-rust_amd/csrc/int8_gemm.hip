@@ -778,7 +778,7 @@ int launch_dma(GemmArgs a, hipStream_t st) {
 template <int V> struct ic { static constexpr int value = V; };
 
 // BN: tile width; WGM x WGN: wave grid (four waves); NSA: LDS stages of A (2 for the 256-wide tile, where 160 KB of LDS
-// leave no room for a third; 3 for the narrow tiles of the skinny shapes).  W always has three stages.
+// leave no room for a third; 3 where a narrower tile leaves room).  W always has three stages.
 template <int BN_, int WGM_, int WGN_, int NSA_>
 struct RingCfg {
     static constexpr int BM = 256, BN = BN_, BK = 128, WGM = WGM_, WGN = WGN_, NT = 256, NSA = NSA_, NSW = 3;
@@ -1296,8 +1296,6 @@ int launch_ring_cfg(GemmArgs a, int slices, hipStream_t st) {
 }
 
 using RingL = RingCfg<256, 2, 2, 2>;    // 256x256, waves 2x2 of 128x128: the compute-bound workhorse
-using RingN96 = RingCfg<96, 4, 1, 3>;   // 256x96, waves 4x1 of 64x96: skinny M with enough columns for every CU
-using RingN128 = RingCfg<128, 4, 1, 3>; // 256x128, waves 4x1 of 64x128: skinny M, split K
 
 template <int OUT_DT, int EPI>
 int launch_ring(GemmArgs a, hipStream_t st) {
