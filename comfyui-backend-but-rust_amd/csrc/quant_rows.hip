@@ -10,7 +10,8 @@
 
 namespace {
 
-enum { MODE_BF16 = 0, MODE_F32 = 1, MODE_SD_F16 = 2, MODE_ROT_F32 = 3 };
+// MODE_BF16_WIDE: fp32 values quantized with bf16 rounding (a bf16 row whose prologue leaves unrounded fp32 values).
+enum { MODE_BF16 = 0, MODE_F32 = 1, MODE_SD_F16 = 2, MODE_ROT_F32 = 3, MODE_BF16_WIDE = 4 };
 
 struct QuantArgs {
     const void* x;
@@ -206,7 +207,7 @@ __global__ void __launch_bounds__(512) quant_rows_kernel(QuantArgs p) {
         scale = fmaxf(amax, 1e-30f) / 127.f;                       // csrc/sd.cu:589
         const float sh = rnd_dt<DT_F16>(scale);
         st = sh > 0.f ? sh : scale;                                // :593
-    } else if (MODE == MODE_BF16) {
+    } else if (MODE == MODE_BF16 || MODE == MODE_BF16_WIDE) {
         scale = fmaxf(fminf(amax, 3.38953139e38f) * (1.f / 127.f), 1.0e-30f);  // csrc/kernels.cu:241
         st = rnd_dt<DT_BF16>(scale);
         rinv = __builtin_amdgcn_rcpf(st);
@@ -228,7 +229,7 @@ __global__ void __launch_bounds__(512) quant_rows_kernel(QuantArgs p) {
             for (int j = 0; j < 4; ++j) {
                 const float x = v[c][4 * i + j];
                 float t;
-                if (MODE == MODE_BF16) {
+                if (MODE == MODE_BF16 || MODE == MODE_BF16_WIDE) {
                     // Both operands carry 8 significant bits, so their exact quotient is never closer than 2^-17
                     // (relative) to a bf16 rounding boundary: a 1-ulp reciprocal times the numerator rounds to the
                     // same bf16 value as the IEEE quotient does.
@@ -281,7 +282,7 @@ int run_quant(QuantArgs a, int g, hipStream_t st) {
     switch (g) {
         case 0: return launch_c<MODE, 0>(a, nw, C, st);
         case 64: return launch_c<MODE, 64>(a, nw, C, st);
-        case 128: if (MODE == MODE_SD_F16 || MODE == MODE_ROT_F32) return -1; return launch_c<MODE == MODE_F32 || MODE == MODE_BF16 ? MODE : MODE_BF16, 128>(a, nw, C, st);
+        case 128: if (MODE == MODE_SD_F16 || MODE == MODE_ROT_F32) return -1; return launch_c<MODE == MODE_F32 || MODE == MODE_BF16 || MODE == MODE_BF16_WIDE ? MODE : MODE_BF16, 128>(a, nw, C, st);
         default: return launch_c<MODE, 256>(a, nw, C, st);
     }
 }
@@ -292,42 +293,87 @@ bool known_prologue(int p) { return p >= PRO_PLAIN && p <= PRO_SITU_FAST && p !=
 
 }  // namespace
 
+// The non-PLAIN prologues run as a separate kernel (prologue_rows.hip) into a stream-ordered T[M, K] buffer that the
+// plain quantizer then reads: every prologue ends on a rounding to T, so this is bit-identical to the fused form.
+extern "C" int gpu_internal_quant_prologue(int dtype, int prologue, const void* x, int64_t x_stride, const void* g,
+                                           int64_t g_stride, int64_t up_offset, const float* norm_w, const float* norm_b,
+                                           float eps, const void* mod_scale, const void* mod_shift, void* out, int M, int K,
+                                           void* stream);
+
+namespace {
+template <class F>
+int with_prologue(int dtype, int prologue, const void* x, int64_t x_stride, const void* g, int64_t g_stride,
+                  int64_t up_offset, const float* norm_w, const float* norm_b, float eps, const void* mod_scale,
+                  const void* mod_shift, int M, int K, hipStream_t st, F&& quantize) {
+    if (M <= 0) return 0;
+    void* rows = nullptr;
+    const bool wide = prologue == PRO_SITU || prologue == PRO_SITU_FAST;   // these leave fp32 values
+    hipError_t e = hipMallocAsync(&rows, (size_t)M * K * (dtype == DT_F32 || wide ? 4 : 2), st);
+    if (e != hipSuccess) return (int)e;
+    int rc = gpu_internal_quant_prologue(dtype, prologue, x, x_stride, g, g_stride, up_offset, norm_w, norm_b, eps, mod_scale,
+                                         mod_shift, rows, M, K, st);
+    if (rc == 0) rc = quantize(rows);
+    e = hipFreeAsync(rows, st);
+    return rc == 0 && e != hipSuccess ? (int)e : rc;
+}
+}  // namespace
+
 GPU_API int gpu_quant_rows(int dtype, int prologue, const void* x, int64_t x_stride, const void* g, int64_t g_stride,
                            int64_t up_offset, const float* norm_w, float eps, const void* mod_scale,
                            const void* mod_shift, int8_t* q, float* scales, int M, int K, int rotate, void* stream) {
-    (void)g; (void)g_stride; (void)up_offset; (void)norm_w; (void)eps; (void)mod_scale; (void)mod_shift;
     const int grp = rotate_group(rotate);
     const int need = grp == 0 ? 64 : grp;
     if (K <= 0 || (K % need) != 0) return -1;
     if (dtype != DT_BF16 && dtype != DT_F32) return -4;
     if (!known_prologue(prologue)) return -3;   // the id list of csrc/kernels.cu:280-292
     if (K > 32768) return -2;
-    if (prologue != PRO_PLAIN) return -30;
-    QuantArgs a{x, x_stride, q, scales, nullptr, M, K, 1, 1};
     hipStream_t st = (hipStream_t)stream;
-    return dtype == DT_BF16 ? run_quant<MODE_BF16>(a, grp, st) : run_quant<MODE_F32>(a, grp, st);
+    auto quantize = [&](const void* rows, int64_t stride, bool wide) {
+        QuantArgs a{rows, stride, q, scales, nullptr, M, K, 1, 1};
+        return dtype == DT_F32 ? run_quant<MODE_F32>(a, grp, st)
+                               : wide ? run_quant<MODE_BF16_WIDE>(a, grp, st) : run_quant<MODE_BF16>(a, grp, st);
+    };
+    if (prologue == PRO_PLAIN) return quantize(x, x_stride, false);
+    // PRO_SITU is one float expression whose value is not rounded to T before the quantizer (csrc/kernels.cu:112): its row
+    // buffer is fp32.  PRO_SITU_FAST, defined by NVIDIA's approximate tanh / exp / divide (csrc/common.cuh:88-90, "about
+    // 2^-11 relative error"), runs the same accurate expression.
+    const bool wide = prologue == PRO_SITU || prologue == PRO_SITU_FAST;
+    return with_prologue(dtype, prologue, x, x_stride, g, g_stride, up_offset, norm_w, nullptr, eps, mod_scale, mod_shift, M, K,
+                         st, [&](const void* rows) { return quantize(rows, K, wide); });
 }
 
 GPU_API int gpu_quant_rows_b(int dtype, int prologue, const void* x, int64_t x_stride, const float* norm_w,
                              const float* norm_b, float eps, const void* mod_scale, const void* mod_shift, int8_t* q,
                              float* scales, int M, int K, int rotate, void* stream) {
-    (void)x; (void)x_stride; (void)norm_w; (void)norm_b; (void)eps; (void)mod_scale; (void)mod_shift; (void)q;
-    (void)scales; (void)M; (void)rotate; (void)stream;
     if ((K % 256) != 0) return -1;
     if (dtype != DT_BF16) return -4;
     if (prologue != PRO_LN_MOD && prologue != PRO_LN_AFFINE) return -3;
-    return -30;
+    if (K <= 0) return -1;
+    if (K > 32768) return -2;
+    hipStream_t st = (hipStream_t)stream;
+    const int grp = rotate_group(rotate);
+    return with_prologue(dtype, prologue, x, x_stride, nullptr, 0, 0, norm_w, norm_b, eps, mod_scale, mod_shift, M, K, st,
+                         [&](const void* rows) {
+                             QuantArgs a{rows, K, q, scales, nullptr, M, K, 1, 1};
+                             return run_quant<MODE_BF16>(a, grp, st);
+                         });
 }
 
 GPU_API int gpu_rotate_rows_f32(int prologue, const float* x, int64_t x_stride, int64_t up_offset, const float* norm_w,
                                 float eps, float* out, int M, int K, void* stream) {
-    (void)up_offset; (void)norm_w; (void)eps;
     if (K <= 0 || (K % 256) != 0) return -1;
     if (prologue != PRO_PLAIN && prologue != PRO_RMS && prologue != PRO_SWIGLU) return -3;
     if (K > 32768) return -2;
-    if (prologue != PRO_PLAIN) return -30;
-    QuantArgs a{x, x_stride, nullptr, nullptr, out, M, K, 1, 1};
-    return run_quant<MODE_ROT_F32>(a, 256, (hipStream_t)stream);
+    hipStream_t st = (hipStream_t)stream;
+    if (prologue == PRO_PLAIN) {
+        QuantArgs a{x, x_stride, nullptr, nullptr, out, M, K, 1, 1};
+        return run_quant<MODE_ROT_F32>(a, 256, st);
+    }
+    return with_prologue(DT_F32, prologue, x, x_stride, nullptr, 0, up_offset, norm_w, nullptr, eps, nullptr, nullptr, M, K, st,
+                         [&](const void* rows) {
+                             QuantArgs a{rows, K, nullptr, nullptr, out, M, K, 1, 1};
+                             return run_quant<MODE_ROT_F32>(a, 256, st);
+                         });
 }
 
 GPU_API int gpu_sd_quant_rows(const void* x, int64_t x_stride, int8_t* q, float* scales, int M, int K, int rotate,

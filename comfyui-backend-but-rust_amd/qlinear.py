@@ -29,6 +29,39 @@ def quant_rows(x, rotate=0, K=None, q=None, scales=None):
     return q, scales
 
 
+def quant_rows_pro(x, prologue, K, rotate=0, g=None, up_offset=0, norm_w=None, eps=0.0, mod_scale=None, mod_shift=None):
+    """gpu_quant_rows with a row prologue (src/dit.rs:510-611 call patterns): x [M, x_stride], optional gate logits g."""
+    M = x.shape[0]
+    q = torch.empty((M, K), dtype=torch.int8, device=x.device)
+    scales = torch.empty((M,), dtype=torch.float32, device=x.device)
+    ffi.k("gpu_quant_rows", _TORCH_DT[x.dtype], prologue, _ptr(x), x.stride(0), _ptr(g), 0 if g is None else g.stride(0),
+          up_offset, _ptr(norm_w), float(eps), _ptr(mod_scale), _ptr(mod_shift), _ptr(q), _ptr(scales), M, K, rotate, _stream())
+    return q, scales
+
+
+def quant_rows_b(x, prologue, K, norm_w, norm_b, eps, rotate=0, mod_scale=None, mod_shift=None):
+    M = x.shape[0]
+    q = torch.empty((M, K), dtype=torch.int8, device=x.device)
+    scales = torch.empty((M,), dtype=torch.float32, device=x.device)
+    ffi.k("gpu_quant_rows_b", _TORCH_DT[x.dtype], prologue, _ptr(x), x.stride(0), _ptr(norm_w), _ptr(norm_b), float(eps),
+          _ptr(mod_scale), _ptr(mod_shift), _ptr(q), _ptr(scales), M, K, rotate, _stream())
+    return q, scales
+
+
+def prologue_rows(x, prologue, K, g=None, up_offset=0, norm_w=None, norm_b=None, eps=0.0, mod_scale=None, mod_shift=None,
+                  b_variant=False):
+    """gpu_prologue_rows / gpu_prologue_rows_b: the prologue's output row in x's dtype, [M, K]."""
+    M = x.shape[0]
+    out = torch.empty((M, K), dtype=x.dtype, device=x.device)
+    if b_variant:
+        ffi.k("gpu_prologue_rows_b", _TORCH_DT[x.dtype], prologue, _ptr(x), x.stride(0), _ptr(norm_w), _ptr(norm_b), float(eps),
+              _ptr(mod_scale), _ptr(mod_shift), _ptr(out), K, M, K, _stream())
+    else:
+        ffi.k("gpu_prologue_rows", _TORCH_DT[x.dtype], prologue, _ptr(x), x.stride(0), _ptr(g), 0 if g is None else g.stride(0),
+              up_offset, _ptr(norm_w), float(eps), _ptr(mod_scale), _ptr(mod_shift), _ptr(out), K, M, K, _stream())
+    return out
+
+
 def sd_quant_rows(x, rotate=0, K=None):
     M, x_stride = x.shape
     K = x_stride if K is None else K
@@ -38,11 +71,12 @@ def sd_quant_rows(x, rotate=0, K=None):
     return q, scales
 
 
-def rotate_rows_f32(x, K=None):
+def rotate_rows_f32(x, K=None, prologue=ffi.PRO_PLAIN, up_offset=0, norm_w=None, eps=0.0):
     M, x_stride = x.shape
     K = x_stride if K is None else K
     out = torch.empty((M, K), dtype=torch.float32, device=x.device)
-    ffi.k("gpu_rotate_rows_f32", ffi.PRO_PLAIN, _ptr(x), x.stride(0), 0, 0, 0.0, _ptr(out), M, K, _stream())
+    ffi.k("gpu_rotate_rows_f32", prologue, _ptr(x), x.stride(0), up_offset, _ptr(norm_w), float(eps), _ptr(out), M, K,
+          _stream())
     return out
 
 

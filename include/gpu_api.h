@@ -13,7 +13,6 @@
  *   int8 GEMM   -200 (plain) / -201 (residual): unknown out_dt, null rscale/resid, K == 0 for the residual form,
  *               or a shape the kernels cannot run (K % 16 != 0)
  *   w6 decode   -1 (K % 32 or G % 16)
- *   -30         a prologue id that exists in the reference but is not built in this library yet
  */
 #ifndef GPU_API_H
 #define GPU_API_H
@@ -39,7 +38,13 @@ enum {
  * x: T[M, x_stride] (T = bf16 or f32 by `dtype`; rows 16-byte aligned); q: int8 [M, K]; scales: f32 [M].
  * rotate: 0 = none; 1 or 256 = the reference's 256-wide normalized Hadamard; 64 and 128 select a 64- or 128-wide
  * group (an extension: the reference treats the argument as a flag).  K must be a multiple of 256 (of 64 when
- * rotate is 0 or 64, of 128 when rotate is 128). */
+ * rotate is 0 or 64, of 128 when rotate is 128).
+ * Prologues (x, g, up_offset, norm_w, eps, mod_scale, mod_shift as in QuantParams, csrc/kernels.cu:21-37): all ids of
+ * csrc/kernels.cu:280-292.  A non-PLAIN prologue runs as a kernel of its own into a stream-ordered [M, K] row buffer: of
+ * type T for the prologues that end on a rounding to T (all but the two below), so codes and scales are those of the
+ * fused form; of unrounded fp32 values for PRO_SITU, as its fused form hands them on.  PRO_SITU_FAST, which the reference
+ * defines through NVIDIA's approximate tanh/exp/divide (about 2^-11 relative error), runs PRO_SITU's accurate expression.  Row sums are accumulated in fp64 and exp / erf / tanh / 1/sqrt are correctly rounded, where the reference has
+ * fp32 sums in the order of its thread layout and CUDA's 1-2 ulp routines. */
 int gpu_quant_rows(int dtype, int prologue, const void* x, int64_t x_stride, const void* g, int64_t g_stride,
                    int64_t up_offset, const float* norm_w, float eps, const void* mod_scale, const void* mod_shift,
                    int8_t* q, float* scales, int M, int K, int rotate, void* stream);
@@ -53,6 +58,20 @@ int gpu_quant_rows_b(int dtype, int prologue, const void* x, int64_t x_stride, c
  * Replaces gpu_rotate_rows_f32, src/ffi.rs:35-36 / csrc/kernels.cu:316-327. */
 int gpu_rotate_rows_f32(int prologue, const float* x, int64_t x_stride, int64_t up_offset, const float* norm_w,
                         float eps, float* out, int M, int K, void* stream);
+
+/* The row prologues alone: writes the activation row in T for a non-quantized GEMM.
+ * Replaces gpu_prologue_rows, src/ffi.rs / csrc/kernels.cu:420-446: dtype bf16 or f32 (-4), prologue PLAIN, RMS, GATE,
+ * SWIGLU, LAYERNORM, SILU, GELU, ADALN or SITU (-3).  out: T[M, out_stride]. */
+int gpu_prologue_rows(int dtype, int prologue, const void* x, int64_t x_stride, const void* g, int64_t g_stride,
+                      int64_t up_offset, const float* norm_w, float eps, const void* mod_scale, const void* mod_shift,
+                      void* out, int64_t out_stride, int M, int K, void* stream);
+
+/* The LayerNorm variants with a bias, and the plain activations, in bf16, f16 or f32.
+ * Replaces gpu_prologue_rows_b, csrc/kernels.cu:449-474: prologue PLAIN, LAYERNORM, LN_MOD, LN_AFFINE,
+ * LN_AFFINE_SILU, SILU, GELU or GELU_TANH (-3). */
+int gpu_prologue_rows_b(int dtype, int prologue, const void* x, int64_t x_stride, const float* norm_w,
+                        const float* norm_b, float eps, const void* mod_scale, const void* mod_shift, void* out,
+                        int64_t out_stride, int M, int K, void* stream);
 
 /* fp16 rows -> optional 64/256 rotation -> int8 rows + scales (the SD/SDXL UNet quantizer).
  * Replaces gpu_sd_quant_rows, src/ffi.rs:252 / csrc/sd.cu:599-606.  rotate in {0, 64, 256}, K % 16 == 0. */

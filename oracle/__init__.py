@@ -30,6 +30,10 @@ def lib():
         L.orc_fht.restype = i32; L.orc_fht.argtypes = [vp, i32, i32]
         L.orc_quant_rows.restype = i32; L.orc_quant_rows.argtypes = [i32, vp, i64, vp, vp, i32, i32, i32]
         L.orc_rotate_rows_f32.restype = i32; L.orc_rotate_rows_f32.argtypes = [vp, i64, vp, i32, i32]
+        L.orc_quant_rows_wide.restype = i32; L.orc_quant_rows_wide.argtypes = [i32, vp, i64, vp, vp, i32, i32, i32]
+        L.orc_situ_rows_wide.restype = i32; L.orc_situ_rows_wide.argtypes = [i32, vp, i64, i64, vp, i32, i32]
+        L.orc_prologue_rows.restype = i32
+        L.orc_prologue_rows.argtypes = [i32, i32, vp, i64, vp, i64, i64, vp, vp, f32, vp, vp, vp, i64, i32, i32]
         L.orc_sd_quant_rows.restype = i32; L.orc_sd_quant_rows.argtypes = [vp, i64, vp, vp, i32, i32, i32]
         L.orc_int8_gemm_acc.restype = None; L.orc_int8_gemm_acc.argtypes = [vp, vp, vp, i64, i64, i64]
         L.orc_epilogue.restype = None; L.orc_epilogue.argtypes = [vp, vp, vp, vp, vp, i64, i64, i32, i32]
@@ -107,6 +111,42 @@ def quant_rows(dtype, x, K, rotate, x_stride=None):
     s = np.zeros((M,), np.float32)
     rc = lib().orc_quant_rows(dtype, _p(x), x_stride, _p(q), _p(s), M, K, rotate)
     return rc, q, s
+
+
+def prologue_rows(dtype, prologue, x, K, g=None, up_offset=0, norm_w=None, norm_b=None, eps=0.0, mod_scale=None,
+                  mod_shift=None):
+    """Row prologue (RMS / LayerNorm variants, gate, SwiGLU, activations) -> the T row the quantizer consumes.
+    x, g: [M, stride] arrays in the dtype's storage (uint16 bits or float32); norm_w/norm_b float32 [K];
+    mod_scale/mod_shift [K] in the dtype's storage.  Returns (rc, out [M, K])."""
+    x = _c(x, _IN_NP[dtype])
+    M = x.shape[0]
+    g = None if g is None else _c(g, _IN_NP[dtype])
+    norm_w = None if norm_w is None else _c(norm_w, np.float32)
+    norm_b = None if norm_b is None else _c(norm_b, np.float32)
+    mod_scale = None if mod_scale is None else _c(mod_scale, _IN_NP[dtype])
+    mod_shift = None if mod_shift is None else _c(mod_shift, _IN_NP[dtype])
+    out = np.zeros((M, K), _IN_NP[dtype])
+    rc = lib().orc_prologue_rows(dtype, prologue, _p(x), x.shape[1], _p(g), 0 if g is None else g.shape[1], up_offset,
+                                 _p(norm_w), _p(norm_b), float(eps), _p(mod_scale), _p(mod_shift), _p(out), K, M, K)
+    return rc, out
+
+
+def quant_rows_wide(rd, x, K, rotate):
+    """fp32 rows [M, K] quantized with the rounding of type rd -> (rc, q, scales)."""
+    x = _c(x, np.float32)
+    M = x.shape[0]
+    q = np.zeros((M, K), np.int8)
+    s = np.zeros(M, np.float32)
+    rc = lib().orc_quant_rows_wide(rd, _p(x), x.shape[1], _p(q), _p(s), M, K, rotate)
+    return rc, q, s
+
+
+def situ_rows_wide(dtype, x, K, up_offset):
+    """situ_f(x[:, :K], x[:, up_offset:up_offset+K]) as unrounded fp32 -> (rc, out [M, K])."""
+    x = _c(x, _IN_NP[dtype])
+    out = np.zeros((x.shape[0], K), np.float32)
+    rc = lib().orc_situ_rows_wide(dtype, _p(x), x.shape[1], up_offset, _p(out), x.shape[0], K)
+    return rc, out
 
 
 def rotate_rows_f32(x, K, x_stride=None):

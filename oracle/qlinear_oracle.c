@@ -24,6 +24,13 @@
  *                                      64 codes x 256 scales against the definition; pack/unpack round trip
  *   orc_w6a8_group_gemm                this build's own format (no reference counterpart); integer partials pinned by
  *                                      numpy int64
+ *   orc_quant_rows_wide                pinned: equals orc_quant_rows for f32, torch bf16 arithmetic on fp32 values
+ *   orc_prologue_rows, orc_situ_rows_wide  structure and rounding points pinned: torch float64 / bf16 tensor arithmetic
+ *                                      (normalizations, gates, activations from torch.nn.functional) to one ulp of T,
+ *                                      closed-form rows.  PARITY UNPINNED against the reference in the last bit: its
+ *                                      row sums are fp32 in the order of its thread layout and its expf / erff /
+ *                                      tanhf / rsqrtf are CUDA's 1-2 ulp routines; here sums are fp64 rounded once and
+ *                                      the functions are correctly rounded (fp64 libm rounded to fp32).
  */
 #include <math.h>
 #include <stdint.h>
@@ -162,32 +169,43 @@ static int quant_check(int dtype, int K, int rotate) {
     if (K > 32768) return -2; /* more than 32 warps of 4 groups, csrc/kernels.cu:263-265 */
     return 0;
 }
-ORC_API int orc_quant_rows(int dtype, const void* x, int64_t x_stride, int8_t* q, float* scales, int M, int K,
+/* ld: the type the row is stored in; rd: the type T whose rounding the quantizer applies.  They differ only for the
+ * fused PRO_SITU prologue of a bf16 row, which hands unrounded fp32 values to the quantizer (csrc/kernels.cu:107-112). */
+static int quant_rows_impl(int ld, int rd, const void* x, int64_t x_stride, int8_t* q, float* scales, int M, int K,
                            int rotate) {
-    const int rc = quant_check(dtype, K, rotate);
+    const int rc = quant_check(rd, K, rotate);
     if (rc) return rc;
     const int g = rotate_group(rotate);
-    const float tmax = dtype == ORC_BF16 ? 3.38953139e38f : 3.402823466e+38f; /* csrc/kernels.cu:48-50 */
+    const float tmax = rd == ORC_BF16 ? 3.38953139e38f : 3.402823466e+38f; /* csrc/kernels.cu:48-50 */
 #pragma omp parallel
     {
         float* v = (float*)malloc(sizeof(float) * (size_t)K);
 #pragma omp for schedule(static)
         for (int m = 0; m < M; ++m) {
-            for (int k = 0; k < K; ++k) v[k] = ld_t(dtype, x, (int64_t)m * x_stride + k);
+            for (int k = 0; k < K; ++k) v[k] = ld_t(ld, x, (int64_t)m * x_stride + k);
             if (g) orc_fht(v, K, g);
             float amax = 0.f;
             for (int k = 0; k < K; ++k) amax = fmax_dev(amax, fabsf(v[k]));
             const float scale = fmax_dev(fmin_dev(amax, tmax) * (1.f / 127.f), 1.0e-30f); /* :241 */
             scales[m] = scale;
-            const float st = rnd_t(dtype, scale);                                           /* :243 */
+            const float st = rnd_t(rd, scale);                                              /* :243 */
             for (int k = 0; k < K; ++k) {
-                const float t = rnd_t(dtype, rnd_t(dtype, v[k]) / st);                      /* :254 */
+                const float t = rnd_t(rd, rnd_t(rd, v[k]) / st);                            /* :254 */
                 q[(int64_t)m * K + k] = (int8_t)fmin_dev(127.f, fmax_dev(-128.f, nearbyintf(t)));
             }
         }
         free(v);
     }
     return 0;
+}
+ORC_API int orc_quant_rows(int dtype, const void* x, int64_t x_stride, int8_t* q, float* scales, int M, int K,
+                           int rotate) {
+    return quant_rows_impl(dtype, dtype, x, x_stride, q, scales, M, K, rotate);
+}
+/* fp32 values quantized with T = rd's rounding. */
+ORC_API int orc_quant_rows_wide(int rd, const float* x, int64_t x_stride, int8_t* q, float* scales, int M, int K,
+                                int rotate) {
+    return quant_rows_impl(ORC_F32, rd, x, x_stride, q, scales, M, K, rotate);
 }
 
 /* gpu_rotate_rows_f32, PRO_PLAIN: csrc/kernels.cu:316-327 with :227-238 (rotation always on, f32 in, f32 out). */
@@ -390,6 +408,100 @@ ORC_API int orc_w6a8_group_gemm(const int8_t* A, const uint8_t* packed, const fl
             st_t(out_dt, D, m * N + n, fmaf(accf, xs[m], b));
         }
     free(w);
+    return 0;
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * Row prologues: csrc/kernels.cu:88-182 (inside quant_rows_kernel) and :348-418 (prologue_rows_kernel), helpers
+ * csrc/common.cuh:71-95, ln_finish csrc/kernels.cu:40-46.  Writes the T row the quantizer would consume.
+ * prologue ids: csrc/kernels.cu:13-15.  SITU is the eager chain of :409-417.
+ * ------------------------------------------------------------------------------------------- */
+enum { OP_PLAIN = 0, OP_RMS = 1, OP_GATE = 2, OP_SWIGLU = 3, OP_LAYERNORM = 4, OP_SILU = 5, OP_GELU = 6, OP_ADALN = 7,
+       OP_SITU = 8, OP_LN_MOD = 9, OP_LN_AFFINE = 10, OP_GELU_TANH = 11, OP_LN_AFFINE_SILU = 12 };
+static inline float exp_cr(float x) { return (float)exp((double)x); }
+static inline float silu_o(float x) { return x / (1.f + exp_cr(-x)); }
+static inline float sigmoid_o(float x) { return 1.f / (1.f + exp_cr(-x)); }
+static inline float stable_tanh_o(float x) {
+    const float t = (float)expm1((double)(-2.f * fabsf(x)));
+    return copysignf(-t / (t + 2.f), x);
+}
+static inline float gelu_o(float x) { return 0.5f * x * (1.f + (float)erf((double)(x * 0.70710678118654752f))); }
+static inline float gelu_tanh_o(float x) {
+    const float k0 = 0.7978845608028654f, k1 = 0.044715f;
+    return 0.5f * x * (1.f + (float)tanh((double)(k0 * fmaf(k1 * x * x, x, x))));
+}
+/* situ_f, csrc/common.cuh:80-82: one float expression; the fused PRO_SITU of the quantizer (csrc/kernels.cu:107-112)
+ * hands its unrounded value on.  out: fp32 [M, K]. */
+ORC_API int orc_situ_rows_wide(int dt, const void* x, int64_t x_stride, int64_t up_offset, float* out, int M, int K) {
+    if (dt < 0 || dt > 2) return -4;
+    for (int64_t m = 0; m < M; ++m)
+        for (int k = 0; k < K; ++k) {
+            const float hidden = ld_t(dt, x, m * x_stride + k), gate = ld_t(dt, x, m * x_stride + up_offset + k);
+            out[m * K + k] = 4.f * stable_tanh_o(gate / 4.f) / (1.f + exp_cr(-gate)) * (25.f * stable_tanh_o(hidden / 25.f));
+        }
+    return 0;
+}
+ORC_API int orc_prologue_rows(int dt, int pro, const void* x, int64_t x_stride, const void* g, int64_t g_stride,
+                              int64_t up_offset, const float* norm_w, const float* norm_b, float eps, const void* ms,
+                              const void* sh, void* out, int64_t out_stride, int M, int K) {
+    if (dt < 0 || dt > 2) return -4;
+    if (pro < OP_PLAIN || pro > OP_LN_AFFINE_SILU) return -3;
+    for (int64_t m = 0; m < M; ++m) {
+        const int64_t xb = m * x_stride, ob = m * out_stride;
+#define X(k) ld_t(dt, x, xb + (k))
+#define R(v) rnd_t(dt, (v))
+        if (pro == OP_RMS || pro == OP_ADALN || pro == OP_LAYERNORM || pro >= OP_LN_MOD && pro != OP_GELU_TANH) {
+            const int ln = pro != OP_RMS && pro != OP_ADALN;
+            float mean = 0.f;
+            if (ln) {
+                double s = 0.0;
+                for (int k = 0; k < K; ++k) s += (double)X(k);
+                mean = (float)s / (float)K;
+            }
+            double s2 = 0.0;
+            for (int k = 0; k < K; ++k) { const float v = X(k) - mean; s2 += (double)v * (double)v; }
+            const float ss = (float)s2;
+            const float rstd = (float)(1.0 / sqrt((double)(ss / (float)K + eps)));
+            for (int k = 0; k < K; ++k) {
+                float n = (X(k) - mean) * rstd;
+                const float msv = ms ? ld_t(dt, ms, k) : 0.f, shv = ms ? ld_t(dt, sh, k) : 0.f;
+                float r;
+                if (pro == OP_ADALN) r = fmaf(n, 1.f + msv, shv);
+                else if (pro == OP_LN_MOD) r = fmaf(R(n), R(1.f + msv), shv);
+                else if (pro == OP_LN_AFFINE) r = fmaf(n, norm_w[k], norm_b[k]);
+                else if (pro == OP_LN_AFFINE_SILU) r = silu_o(R(fmaf(n, norm_w[k], norm_b[k])));
+                else {
+                    if (norm_w) n *= norm_w[k];
+                    n = R(n);
+                    if (ms) { const float a = R(1.f + msv); n = R(a * n); n = R(n + shv); }
+                    r = n;
+                }
+                st_t(dt, out, ob + k, r);
+            }
+        } else if (pro == OP_GATE) {
+            for (int k = 0; k < K; ++k) st_t(dt, out, ob + k, X(k) * R(sigmoid_o(ld_t(dt, g, m * g_stride + k))));
+        } else if (pro == OP_SWIGLU) {
+            for (int k = 0; k < K; ++k) st_t(dt, out, ob + k, R(silu_o(X(k))) * X(up_offset + k));
+        } else if (pro == OP_SILU) {
+            for (int k = 0; k < K; ++k) st_t(dt, out, ob + k, silu_o(X(k)));
+        } else if (pro == OP_GELU) {
+            for (int k = 0; k < K; ++k) st_t(dt, out, ob + k, gelu_o(X(k)));
+        } else if (pro == OP_GELU_TANH) {
+            for (int k = 0; k < K; ++k) st_t(dt, out, ob + k, gelu_tanh_o(X(k)));
+        } else if (pro == OP_SITU) {
+            for (int k = 0; k < K; ++k) {
+                const float hidden = X(k), gate = X(up_offset + k);
+                const float capped = R(4.f * R(stable_tanh_o(R(gate / 4.f))));
+                const float gg = R(capped * R(sigmoid_o(gate)));
+                const float h = R(25.f * R(stable_tanh_o(R(hidden / 25.f))));
+                st_t(dt, out, ob + k, gg * h);
+            }
+        } else {
+            for (int k = 0; k < K; ++k) st_t(dt, out, ob + k, X(k));
+        }
+#undef X
+#undef R
+    }
     return 0;
 }
 

@@ -162,6 +162,145 @@ def test_rotate_rows_f32_bit_exact():
     assert np.array_equal(got.cpu().numpy().view(np.uint32), out.view(np.uint32))
 
 
+# ------------------------------------------------------------------------------------------------ row prologues
+def pro_case(dt, seed, M, K, cols):
+    """Inputs of every prologue for one shape, in the oracle's storage form: x rows [M, cols] (a gate/up half at
+    column K + 64), gate logits, norm weight/bias, modulation vectors."""
+    rnd = lambda stream, *shape: synth.normal(seed, stream, int(np.prod(shape))).reshape(shape)
+    conv = {BF16: synth.bf16_bits, F16: synth.f16_bits, F32: lambda a: np.ascontiguousarray(a, dtype=np.float32)}[dt]
+    x = rnd(1, M, cols) * np.float32(1.5)
+    x[0, :6] = [0.0, -0.0, 30.0, -30.0, 6.0, -6.0]
+    if M > 1:
+        x[1, :] = 0
+    return dict(x=conv(x), g=conv(rnd(2, M, K + 8) * np.float32(2)), w=(1 + 0.2 * rnd(3, K)).astype(np.float32),
+                b=(0.1 * rnd(4, K)).astype(np.float32), ms=conv(0.3 * rnd(5, K)), sh=conv(0.3 * rnd(6, K)))
+
+
+def pro_args(name, c, K):
+    """Keyword arguments of one prologue (host arrays)."""
+    a = dict(eps=1e-6)
+    if name == "GATE":
+        a["g"] = c["g"]
+    if name in ("SWIGLU", "SITU"):
+        a["up_offset"] = K + 64
+    if name in ("RMS_W", "LAYERNORM_W", "LN_AFFINE", "LN_AFFINE_SILU", "RMS_W_MOD", "LAYERNORM_B"):
+        a["norm_w"] = c["w"]
+    if name in ("LN_AFFINE", "LN_AFFINE_SILU"):
+        a["norm_b"] = c["b"]
+    if name in ("ADALN", "LN_MOD", "RMS_W_MOD", "LAYERNORM_MOD"):
+        a["mod_scale"], a["mod_shift"] = c["ms"], c["sh"]
+    return a
+
+
+PRO_ID = dict(PLAIN=0, RMS=1, RMS_W=1, RMS_W_MOD=1, GATE=2, SWIGLU=3, LAYERNORM=4, LAYERNORM_W=4, LAYERNORM_MOD=4,
+              LAYERNORM_B=4, SILU=5, GELU=6, ADALN=7, SITU=8, LN_MOD=9, LN_AFFINE=10, GELU_TANH=11, LN_AFFINE_SILU=12)
+A_NAMES = ["PLAIN", "RMS", "RMS_W", "RMS_W_MOD", "GATE", "SWIGLU", "LAYERNORM", "LAYERNORM_W", "LAYERNORM_MOD", "SILU", "GELU",
+           "ADALN", "SITU"]
+B_NAMES = ["PLAIN", "LAYERNORM_B", "LN_MOD", "LN_AFFINE", "LN_AFFINE_SILU", "SILU", "GELU", "GELU_TANH"]
+
+
+def to_dev_args(a, dt):
+    d = dict(a)
+    for k in ("g", "mod_scale", "mod_shift"):
+        if k in d:
+            d[k] = dev_bits(d[k], dt)
+    for k in ("norm_w", "norm_b"):
+        if k in d:
+            d[k] = dev(d[k])
+    return d
+
+
+@pytest.mark.parametrize("dt", [BF16, F32])
+@pytest.mark.parametrize("M,K", [(5, 256), (3, 3072), (2, 200), (3, 5120)])
+def test_prologue_rows_bit_exact(M, K, dt):
+    cols = 2 * K + 64
+    c = pro_case(dt, 500 + K, M, K, cols)
+    xd = dev_bits(c["x"], dt)
+    for name in A_NAMES:
+        say("prologue_rows", name, M, K, dt)
+        a = pro_args(name, c, K)
+        rc, want = oracle.prologue_rows(dt, PRO_ID[name], c["x"], K, **a)
+        assert rc == 0
+        got = ql.prologue_rows(xd, PRO_ID[name], K, **to_dev_args(a, dt))
+        torch.cuda.synchronize()
+        gb, wb = host_bits(got), want
+        assert np.array_equal(gb.view(np.uint32 if dt == F32 else np.uint16), wb.view(np.uint32 if dt == F32 else np.uint16)), name
+
+
+@pytest.mark.parametrize("dt", [BF16, F16, F32])
+@pytest.mark.parametrize("M,K", [(4, 64), (5, 1152), (2, 4096)])
+def test_prologue_rows_b_bit_exact(M, K, dt):
+    c = pro_case(dt, 600 + K, M, K, K + 16)
+    xd = dev_bits(c["x"], dt)
+    for name in B_NAMES:
+        say("prologue_rows_b", name, M, K, dt)
+        a = pro_args(name, c, K)
+        rc, want = oracle.prologue_rows(dt, PRO_ID[name], c["x"], K, **a)
+        assert rc == 0
+        got = ql.prologue_rows(xd, PRO_ID[name], K, b_variant=True, **to_dev_args(a, dt))
+        torch.cuda.synchronize()
+        view = np.uint32 if dt == F32 else np.uint16
+        assert np.array_equal(host_bits(got).view(view), want.view(view)), name
+
+
+@pytest.mark.parametrize("dt", [BF16, F32])
+@pytest.mark.parametrize("M,K,rotate", [(6, 256, 0), (4, 3072, 1), (3, 3072, 128), (2, 1024, 64), (3, 12288, 1)])
+def test_quant_rows_with_prologue_equals_prologue_then_quantizer(M, K, rotate, dt):
+    """gpu_quant_rows(prologue) == quantizer(oracle prologue row): every prologue ends on a rounding to T
+    (csrc/kernels.cu:100-179), so the two-step form has the fused kernel's codes and scales."""
+    cols = 2 * K + 64
+    c = pro_case(dt, 700 + K + rotate, M, K, cols)
+    xd = dev_bits(c["x"], dt)
+    for name in ["RMS_W", "RMS_W_MOD", "GATE", "SWIGLU", "LAYERNORM", "LAYERNORM_MOD", "SILU", "GELU", "ADALN", "LN_MOD", "GELU_TANH"]:
+        say("quant_rows prologue", name, M, K, rotate, dt)
+        a = pro_args(name, c, K)
+        rc, row = oracle.prologue_rows(dt, PRO_ID[name], c["x"], K, **a)
+        rc2, q, s = oracle.quant_rows(dt, row, K, rotate)
+        assert rc == 0 and rc2 == 0
+        qd, sd = ql.quant_rows_pro(xd, PRO_ID[name], K, rotate, **to_dev_args(a, dt))
+        torch.cuda.synchronize()
+        assert np.array_equal(sd.cpu().numpy().view(np.uint32), s.view(np.uint32)), name
+        assert np.array_equal(qd.cpu().numpy(), q), name
+    # the fused SiTU hands unrounded fp32 values to the quantizer (csrc/kernels.cu:107-112); the lossy id runs the same code
+    rc, wide = oracle.situ_rows_wide(dt, c["x"], K, K + 64)
+    rc2, q, s = oracle.quant_rows_wide(dt, wide, K, rotate)
+    assert rc == 0 and rc2 == 0
+    for pro in (ffi.PRO_SITU, ffi.PRO_SITU_FAST):
+        say("quant_rows prologue SITU", pro, M, K, rotate, dt)
+        qd, sd = ql.quant_rows_pro(xd, pro, K, rotate, up_offset=K + 64)
+        torch.cuda.synchronize()
+        assert np.array_equal(sd.cpu().numpy().view(np.uint32), s.view(np.uint32)), pro
+        assert np.array_equal(qd.cpu().numpy(), q), pro
+
+
+def test_quant_rows_b_and_rotate_rows_f32_with_prologues():
+    M, K = 5, 1536
+    c = pro_case(BF16, 801, M, K, K + 16)
+    xd = dev_bits(c["x"], BF16)
+    for name in ("LN_MOD", "LN_AFFINE"):
+        a = pro_args(name, c, K)
+        rc, row = oracle.prologue_rows(BF16, PRO_ID[name], c["x"], K, **a)
+        for rotate in (0, 1):
+            rc2, q, s = oracle.quant_rows(BF16, row, K, rotate)
+            d = to_dev_args(a, BF16)
+            qd, sd = ql.quant_rows_b(xd, PRO_ID[name], K, d.get("norm_w"), d.get("norm_b"), 1e-6, rotate,
+                                     d.get("mod_scale"), d.get("mod_shift"))
+            torch.cuda.synchronize()
+            assert np.array_equal(sd.cpu().numpy().view(np.uint32), s.view(np.uint32)), (name, rotate)
+            assert np.array_equal(qd.cpu().numpy(), q), (name, rotate)
+    K = 1024
+    cf = pro_case(F32, 802, 4, K, 2 * K + 64)
+    xf = dev(cf["x"])
+    for name in ("RMS_W", "SWIGLU"):
+        a = pro_args(name, cf, K)
+        rc, row = oracle.prologue_rows(F32, PRO_ID[name], cf["x"], K, **a)
+        rc2, want = oracle.rotate_rows_f32(row, K)
+        d = to_dev_args(a, F32)
+        got = ql.rotate_rows_f32(xf, K, PRO_ID[name], d.get("up_offset", 0), d.get("norm_w"), 1e-6)
+        torch.cuda.synchronize()
+        assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32)), name
+
+
 def test_rotated_quant_golden_fixture():
     g = json.load(open(os.path.join(ROOT, "tests", "golden", "rotated_quant.json")))
     xb = synth.bf16_bits(synth.activations(11, 8, 1024, "t3"))

@@ -52,7 +52,8 @@ def test_quant_rows_refusals_match_reference_order():
     assert q(dtype=1, pro=99) == -4             # dtype is looked at before the prologue id
     assert q(pro=99) == -3 and q(pro=12) == -3  # :292 (LN_AFFINE_SILU is not in the quantizer's list)
     assert q(K=32768 + 256) == -2               # :265
-    assert q(pro=ffi.PRO_RMS) == -30            # known prologue, not built here
+    assert q(pro=ffi.PRO_SITU, M=0) == 0 and q(pro=ffi.PRO_SITU_FAST, M=0) == 0
+    assert q(pro=ffi.PRO_RMS, M=0) == 0
     assert q(M=0) == 0
     # the oracle agrees on the shared codes
     x = np.zeros((1, 512), np.uint16)
@@ -66,6 +67,10 @@ def test_other_entry_point_refusals():
     assert ffi.raw("gpu_quant_rows_b", 2, ffi.PRO_RMS, 0, 256, 0, 0, 0.0, 0, 0, 0, 0, 1, 256, 0, 0) == -3
     assert ffi.raw("gpu_rotate_rows_f32", ffi.PRO_PLAIN, 0, 320, 0, 0, 0.0, 0, 1, 320, 0) == -1
     assert ffi.raw("gpu_rotate_rows_f32", ffi.PRO_GATE, 0, 256, 0, 0, 0.0, 0, 1, 256, 0) == -3
+    pr = lambda dt, pro: ffi.raw("gpu_prologue_rows", dt, pro, 0, 256, 0, 0, 0, 0, 0.0, 0, 0, 0, 256, 0, 256, 0)
+    assert pr(1, ffi.PRO_RMS) == -4 and pr(2, ffi.PRO_LN_MOD) == -3 and pr(2, 99) == -3 and pr(2, ffi.PRO_RMS) == 0
+    pb = lambda dt, pro: ffi.raw("gpu_prologue_rows_b", dt, pro, 0, 256, 0, 0, 0.0, 0, 0, 0, 256, 0, 256, 0)
+    assert pb(7, ffi.PRO_LN_MOD) == -4 and pb(1, ffi.PRO_RMS) == -3 and pb(1, ffi.PRO_GELU_TANH) == 0
     assert ffi.raw("gpu_sd_quant_rows", 0, 640, 0, 0, 1, 640, 128, 0) == -1     # csrc/sd.cu:600
     assert ffi.raw("gpu_sd_quant_rows", 0, 640, 0, 0, 1, 640, 256, 0) == -1
     assert ffi.raw("gpu_w6_decode", 0, 0, 0, 4, 48, 32, 0) == -1                # csrc/h3.cu:41

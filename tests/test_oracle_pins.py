@@ -408,3 +408,212 @@ def test_w6a8_group_gemm_partials_and_output(synth):
     ref = (want_p * sw[None].astype(np.float64)).sum(-1) * xs[:, None] + oracle.bf16_to_f32(bias)[None]
     got = oracle.bf16_to_f32(D).astype(np.float64)
     assert np.allclose(got, ref, rtol=2.0 ** -7, atol=1e-6)
+
+
+# ----------------------------------------------------------------------------------------------- row prologues
+# The prologue restatement is pinned against torch's float64 routines (silu, gelu, layer_norm, ...) applied to the same
+# rows and rounded once to T: it must land within one unit of T of that, and mostly on it.  Whether the reference's
+# CUDA build (expf, rsqrtf, its fp32 block sums) gives the same last bit is not something this container can tell.
+PRO = dict(PLAIN=0, RMS=1, GATE=2, SWIGLU=3, LAYERNORM=4, SILU=5, GELU=6, ADALN=7, SITU=8, LN_MOD=9, LN_AFFINE=10,
+           GELU_TANH=11, LN_AFFINE_SILU=12)
+_TT = {BF16: torch.bfloat16, F16: torch.float16, F32: torch.float32}
+
+
+def to_storage(dt, a64):
+    """float64 tensor -> T (one rounding) in the oracle's storage form."""
+    t = a64.to(_TT[dt])
+    return t.numpy() if dt == F32 else t.view(torch.int16).numpy().view(np.uint16)
+
+
+def from_storage(dt, a):
+    a = np.ascontiguousarray(a)
+    return torch.from_numpy(a) if dt == F32 else torch.from_numpy(a.view(np.int16)).view(_TT[dt])
+
+
+def units_apart(dt, a, b):
+    """Distance in units of T between two storage arrays (finite values)."""
+    wide = np.int32 if dt == F32 else np.int16
+    mask = 0x7fffffff if dt == F32 else 0x7fff
+    def key(v):
+        i = np.ascontiguousarray(v).view(wide).astype(np.int64)
+        return np.where(i < 0, -(i & mask), i)
+    return np.abs(key(a) - key(b))
+
+
+def pro_inputs(dt, seed, M, K, cols=None):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(M, cols or K, generator=g, dtype=torch.float64) * 1.5
+    x[0, :4] = torch.tensor([0.0, -0.0, 30.0, -30.0], dtype=torch.float64)
+    xs = to_storage(dt, x)
+    return xs, from_storage(dt, xs).double()
+
+
+def check_close(dt, got, want64, max_units, min_exact):
+    """16-bit T: within max_units of the float64 result rounded once, and equal to it on min_exact of the elements.
+    f32: the chain's own fp32 roundings (x - mean cancels) allow a few 2^-24 of (|value| + 1)."""
+    if dt == F32:
+        assert ((torch.from_numpy(got).double() - want64).abs() <= 2.0 ** -20 * (want64.abs() + 1)).all()
+        return
+    want = to_storage(dt, want64)
+    d = units_apart(dt, got, want)
+    assert d.max() <= max_units, d.max()
+    assert (d == 0).mean() >= min_exact, (d == 0).mean()
+
+
+@pytest.mark.parametrize("dt", [BF16, F16, F32])
+@pytest.mark.parametrize("name", ["SILU", "GELU", "GELU_TANH", "PLAIN"])
+def test_prologue_activations_match_torch_float64(dt, name):
+    F = torch.nn.functional
+    xs, x = pro_inputs(dt, 3, 16, 512)
+    rc, out = oracle.prologue_rows(dt, PRO[name], xs, 512)
+    assert rc == 0
+    want = {"SILU": F.silu(x), "GELU": F.gelu(x), "GELU_TANH": F.gelu(x, approximate="tanh"), "PLAIN": x}[name]
+    if name == "PLAIN":
+        assert np.array_equal(out, xs)
+    else:
+        # in the tail of gelu (x below -3) the value is 0.5 x (1 + erf), a small difference of fp32 numbers: only its
+        # absolute error is small there.  Elsewhere: within one unit of T, and for the 16-bit types mostly on it.
+        got = from_storage(dt, out).double()
+        rel = {BF16: 2.0 ** -8, F16: 2.0 ** -11, F32: 2.0 ** -22}[dt]
+        # (f32: 1 + erf also loses a bit or two for moderate negative x)
+        assert ((got - want).abs() <= rel * want.abs() + 1e-7 * (x < (0 if dt == F32 else -3)) + 1e-30).all()
+        if dt != F32:
+            body = (x > -3).numpy()
+            assert (units_apart(dt, out, to_storage(dt, want))[body] == 0).mean() >= 0.99
+    # the anchors: f(0) = 0, f(30) = 30, f(-30) = -0 or 0
+    vals = from_storage(dt, out)[0, :4].double()
+    if name != "PLAIN":
+        assert vals[0] == 0 and vals[1] == 0 and vals[2] == 30 and abs(vals[3]) < 1e-11
+
+
+@pytest.mark.parametrize("dt", [BF16, F32])
+def test_prologue_norms_match_torch_float64(dt):
+    F = torch.nn.functional
+    M, K, eps = 12, 768, 1e-6
+    xs, x = pro_inputs(dt, 5, M, K)
+    g = torch.Generator().manual_seed(6)
+    w = (1 + 0.2 * torch.randn(K, generator=g)).float()
+    b = (0.1 * torch.randn(K, generator=g)).float()
+    ms_s = to_storage(dt, 0.3 * torch.randn(K, generator=g, dtype=torch.float64))
+    sh_s = to_storage(dt, 0.3 * torch.randn(K, generator=g, dtype=torch.float64))
+    ms, sh = from_storage(dt, ms_s).double(), from_storage(dt, sh_s).double()
+    rms = x / torch.sqrt((x * x).mean(1, keepdim=True) + eps)
+    ln = F.layer_norm(x, (K,), eps=eps)
+    one, most = (1, 0.98) if dt == BF16 else (4, 0.5)
+    run = lambda name, **kw: oracle.prologue_rows(dt, PRO[name], xs, K, eps=eps, **kw)[1]
+    check_close(dt, run("RMS", norm_w=w.numpy()), rms * w.double(), one, most)
+    check_close(dt, run("RMS"), rms, one, most)
+    check_close(dt, run("LAYERNORM"), ln, one, most)
+    check_close(dt, run("LAYERNORM", norm_w=w.numpy()), ln * w.double(), one, most)
+    check_close(dt, run("ADALN", mod_scale=ms_s, mod_shift=sh_s), rms * (1 + ms) + sh, one, most)
+    check_close(dt, run("LN_AFFINE", norm_w=w.numpy(), norm_b=b.numpy()), ln * w.double() + b.double(), one, most)
+    # silu of the affine value rounded to T first (csrc/kernels.cu:44); a last-unit difference of that rounding is
+    # magnified by silu's condition number for negative arguments, so: mostly equal, and close everywhere
+    aff = (ln * w.double() + b.double()).to(_TT[dt]).double()
+    got = run("LN_AFFINE_SILU", norm_w=w.numpy(), norm_b=b.numpy())
+    assert (units_apart(dt, got, to_storage(dt, F.silu(aff))) == 0).mean() >= (0.97 if dt == BF16 else 0.3)
+    assert ((from_storage(dt, got).double() - F.silu(aff)).abs() <= 2.0 ** (-6 if dt == BF16 else -19) * (F.silu(aff).abs() + 0.05)).all()
+    # forms that round every intermediate tensor to T, restated with torch tensors of that type
+    T = _TT[dt]
+    lnT = ln.to(T)
+    a = (1 + ms.float()).to(T) if dt == F32 else (1.0 + ms).to(T)
+    got = from_storage(dt, run("LN_MOD", mod_scale=ms_s, mod_shift=sh_s)).double()
+    want = (lnT.double() * a.double() + sh).to(T).double()
+    assert ((got - want).abs() <= 2.0 ** (-7 if dt == BF16 else -21) * want.abs() + 1e-6).all()
+    got = run("LAYERNORM", mod_scale=ms_s, mod_shift=sh_s)
+    want = ((a * lnT).to(T) + from_storage(dt, sh_s)).to(T)
+    d = units_apart(dt, got, to_storage(dt, want.double()))
+    # a last-unit difference of the normalised value can move through the two later roundings
+    assert (d == 0).mean() >= (0.97 if dt == BF16 else 0.4)
+    assert ((from_storage(dt, got).double() - want.double()).abs() <= 2.0 ** (-6 if dt == BF16 else -20) * (want.double().abs() + 1)).all()
+
+
+def test_prologue_norm_closed_forms():
+    K = 256
+    # a constant power-of-two row: rms = |c| exactly, so RMS gives sign(c) and ADALN gives (1 + ms) + sh rounded once
+    x = np.full((2, K), 0.25, np.float32); x[1] = -4.0
+    ms = np.linspace(-0.5, 0.5, K).astype(np.float32)
+    sh = np.linspace(1.0, 2.0, K).astype(np.float32)
+    rc, out = oracle.prologue_rows(F32, PRO["RMS"], x, K)
+    assert rc == 0 and np.array_equal(out, np.sign(x))
+    rc, out = oracle.prologue_rows(F32, PRO["ADALN"], x, K, mod_scale=ms, mod_shift=sh)
+    want = np.stack([(np.float64(1) + ms.astype(np.float64)) + sh, -(np.float64(1) + ms.astype(np.float64)) + sh])
+    # fmaf(n, 1 + ms, sh) with n = +-1: (1 + ms) is rounded to f32 first, the sum once more
+    one_ms = (np.float32(1) + ms).astype(np.float64)
+    assert np.array_equal(out, np.stack([one_ms + sh, -one_ms + sh]).astype(np.float32))
+    del want
+    # alternating +-2: mean 0, variance 4, LayerNorm gives +-1; with weight and bias, +-w + b
+    x = np.tile(np.array([2.0, -2.0], np.float32), K // 2)[None]
+    w = np.arange(K, dtype=np.float32) / 8
+    b = np.arange(K, dtype=np.float32)[::-1].copy() / 4
+    rc, out = oracle.prologue_rows(F32, PRO["LAYERNORM"], x, K)
+    assert np.array_equal(out, np.sign(x))
+    rc, out = oracle.prologue_rows(F32, PRO["LN_AFFINE"], x, K, norm_w=w, norm_b=b)
+    assert np.array_equal(out, np.sign(x) * w + b)
+    # eps enters under the root: an all-zero row with eps = 1/16 has rstd = 4 and stays zero; one of 3s with eps = 7 has
+    # mean square 9, rstd = 1/4
+    x = np.full((1, K), 3.0, np.float32)
+    rc, out = oracle.prologue_rows(F32, PRO["RMS"], x, K, eps=7.0)
+    assert np.array_equal(out, np.full((1, K), 0.75, np.float32))
+    # bf16: the result is rounded to bf16, 1/3 * 3 is not representable but 0.75 is; use 1.00390625 * w to see rounding
+    xb = oracle.bf16_bits(np.full((1, K), 3.0, np.float32))
+    rc, out = oracle.prologue_rows(BF16, PRO["RMS"], xb, K, eps=7.0, norm_w=np.full(K, 1.00390625, np.float32))
+    assert np.array_equal(oracle.bf16_to_f32(out), np.full((1, K), 0.75390625, np.float32))   # 0.7529... -> bf16 tie to even
+
+
+@pytest.mark.parametrize("dt", [BF16, F32])
+def test_prologue_gated_forms_match_torch_float64(dt):
+    F = torch.nn.functional
+    M, K = 8, 512
+    xs, x = pro_inputs(dt, 9, M, K, cols=2 * K + 64)
+    gs, gt = pro_inputs(dt, 10, M, K, cols=K + 8)
+    one, most = (1, 0.97) if dt == BF16 else (4, 0.4)
+    rc, out = oracle.prologue_rows(dt, PRO["GATE"], xs, K, g=gs)
+    assert rc == 0
+    T = _TT[dt]   # the gate / the silu is rounded to T before the product (csrc/kernels.cu:392, :397)
+    check_close(dt, out, x[:, :K] * torch.sigmoid(gt[:, :K]).to(T).double(), one, most)
+    up = K + 64
+    rc, out = oracle.prologue_rows(dt, PRO["SWIGLU"], xs, K, up_offset=up)
+    check_close(dt, out, F.silu(x[:, :K]).to(T).double() * x[:, up:up + K], one, most)
+    rc, out = oracle.prologue_rows(dt, PRO["SITU"], xs, K, up_offset=up)
+    hidden, gate = x[:, :K], x[:, up:up + K]
+    want = (4 * torch.tanh(gate / 4) * torch.sigmoid(gate)) * (25 * torch.tanh(hidden / 25))
+    got = from_storage(dt, out).double()
+    assert ((got - want).abs() <= 2.0 ** (-6 if dt == BF16 else -20) * want.abs() + 1e-30).all()
+
+
+def test_prologue_argument_codes_and_strides():
+    x = np.zeros((2, 256), np.float32)
+    out = np.zeros_like(x)
+    assert oracle.lib().orc_prologue_rows(3, 0, x.ctypes.data, 256, None, 0, 0, None, None, 0.0, None, None, out.ctypes.data, 256, 2, 256) == -4
+    assert oracle.prologue_rows(F32, 13, x, 256)[0] == -3 and oracle.prologue_rows(F32, -1, x, 256)[0] == -3
+    # rows are read at x_stride and only K columns of them
+    xs, _ = pro_inputs(F32, 11, 4, 256, cols=300)
+    a = oracle.prologue_rows(F32, PRO["RMS"], xs, 256, eps=1e-6)[1]
+    b = oracle.prologue_rows(F32, PRO["RMS"], xs[:, :256].copy(), 256, eps=1e-6)[1]
+    assert np.array_equal(a, b)
+
+
+def test_situ_wide_and_wide_quantizer(synth):
+    """The fused SiTU: fp32 values of one float expression (csrc/common.cuh:80-82), then the quantizer with T's rounding."""
+    M, K = 6, 512
+    xs, x = pro_inputs(BF16, 13, M, K, cols=2 * K + 64)
+    rc, wide = oracle.situ_rows_wide(BF16, xs, K, K + 64)
+    assert rc == 0
+    hidden, gate = x[:, :K], x[:, K + 64:2 * K + 64]
+    want = (4 * torch.tanh(gate / 4) * torch.sigmoid(gate)) * (25 * torch.tanh(hidden / 25))
+    assert ((torch.from_numpy(wide).double() - want).abs() <= 2.0 ** -20 * want.abs() + 1e-30).all()
+    # f32 rounding: the wide quantizer is the f32 quantizer
+    for rotate in (0, 1, 128):
+        a = oracle.quant_rows_wide(F32, wide, K, rotate)
+        b = oracle.quant_rows(F32, wide, K, rotate)
+        assert a[0] == 0 and np.array_equal(a[1], b[1]) and np.array_equal(a[2], b[2])
+    # bf16 rounding of fp32 values, restated with torch tensors: amax of the unrounded values, both operands of the
+    # divide rounded to bf16, the quotient rounded to bf16
+    rc, q, s = oracle.quant_rows_wide(BF16, wide, K, 0)
+    w = torch.from_numpy(wide)
+    scale = torch.clamp(w.abs().amax(1) * torch.tensor(1.0 / 127.0, dtype=torch.float32), min=1e-30)
+    t = (w.bfloat16() / scale.bfloat16()[:, None]).float()
+    assert np.array_equal(s, scale.numpy())
+    assert np.array_equal(q, torch.clamp(torch.round(t), -128, 127).to(torch.int8).numpy())
+    assert oracle.quant_rows_wide(F16, wide, K, 0)[0] == -4
