@@ -143,6 +143,91 @@ __global__ void __launch_bounds__(256) prologue_rows_kernel(ProArgs p) {
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------------
+// The SD UNet's fused quantizer sources (csrc/sd.cu:611-663): the half row another kernel would have written -- LayerNorm,
+// GEGLU, head un-padding, GroupNorm -- which the fp16 quantizer then reads.  Same two choices as above for sums and 1/sqrt.
+// ---------------------------------------------------------------------------------------------------------------------
+enum { SDQ_LN = 1, SDQ_GEGLU = 2, SDQ_UNPAD = 3, SDQ_GN = 4 };
+struct SdSrc {
+    const uint16_t* x;
+    int64_t x_stride;     // LN: elements between rows
+    const float* w;       // LN, GN
+    const float* b;
+    float eps;            // LN
+    int heads, d, dp;     // UNPAD: heads of d values, each stored dp wide
+    const float2* stats;  // GN: (mean, rstd) of group ng at stats[2 * ng], the layout csrc/sd.cu:203-207 leaves
+    int groups;
+    int64_t P;            // GN: pixels per image
+    uint16_t* out;        // half rows [M, K]
+    int K;
+};
+
+template <int MODE>
+__global__ void __launch_bounds__(256) sd_source_rows_kernel(SdSrc p) {
+    __shared__ double red[4];
+    const int K = p.K;
+    const int64_t m = blockIdx.x;
+    uint16_t* o = p.out + m * K;
+    if (MODE == SDQ_LN) {                                                 // csrc/sd.cu:629-641
+        const uint16_t* r = p.x + m * p.x_stride;
+        double s = 0.0;
+        for (int k = threadIdx.x; k < K; k += blockDim.x) s += (double)f16_to_f(r[k]);
+        const float mean = block_sum_f64(s, red) / (float)K;
+        double s2 = 0.0;
+        for (int k = threadIdx.x; k < K; k += blockDim.x) {
+            const float d = f16_to_f(r[k]) - mean;
+            s2 += (double)d * (double)d;
+        }
+        const float rstd = (float)(1.0 / sqrt((double)(block_sum_f64(s2, red) / (float)K + p.eps)));
+        for (int k = threadIdx.x; k < K; k += blockDim.x)
+            o[k] = f_to_f16(__builtin_fmaf((f16_to_f(r[k]) - mean) * rstd, p.w[k], p.b[k]));
+    } else if (MODE == SDQ_GEGLU) {                                       // :642-649: [M, 2K] value then gate
+        const uint16_t* r = p.x + m * 2 * K;
+        for (int k = threadIdx.x; k < K; k += blockDim.x)
+            o[k] = f_to_f16(f16_to_f(r[k]) * rnd_dt<DT_F16>(gelu_f(f16_to_f(r[K + k]))));
+    } else if (MODE == SDQ_UNPAD) {                                       // :650-652
+        const uint16_t* r = p.x + m * p.heads * p.dp;
+        for (int k = threadIdx.x; k < K; k += blockDim.x) o[k] = r[(k / p.d) * p.dp + k % p.d];
+    } else {                                                              // :653-662: row m is a pixel of image m / P
+        const uint16_t* r = p.x + m * K;
+        const int n = (int)(m / p.P);
+        for (int c = threadIdx.x; c < K; c += blockDim.x) {
+            const float2 st = p.stats[(n * p.groups + c / (K / p.groups)) * 2];
+            o[c] = f_to_f16(__builtin_fmaf((f16_to_f(r[c]) - st.x) * st.y, p.w[c], p.b[c]));
+        }
+    }
+}
+
+// GroupNorm statistics of fp16 x [N, P, C]: one workgroup per (image, group).  Sums in fp64, then csrc/sd.cu:203-207:
+// mean = s / cnt, var = max(ss / cnt - mean^2, 0), rstd = 1 / sqrt(var + eps), both narrowed to fp32.
+__global__ void __launch_bounds__(256) sd_group_stats_kernel(const uint16_t* x, float2* stats, int64_t P, int C, int G, float eps) {
+    __shared__ double red[4];
+    __shared__ double keep;
+    const int ng = blockIdx.x, n = ng / G, g = ng % G, per = C / G;
+    const uint16_t* base = x + (int64_t)n * P * C + g * per;
+    const int64_t count = P * per;
+    double s = 0.0, ss = 0.0;
+    for (int64_t i = threadIdx.x; i < count; i += blockDim.x) {
+        const double v = (double)f16_to_f(base[(i / per) * C + (i % per)]);
+        s += v;
+        ss += v * v;
+    }
+    // block_sum_f64 narrows to fp32; these sums stay in fp64
+    for (int o = 32; o > 0; o >>= 1) { s += __shfl_xor(s, o); ss += __shfl_xor(ss, o); }
+    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+    if (lane == 0) red[wid] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) keep = red[0] + red[1] + red[2] + red[3];
+    __syncthreads();
+    if (lane == 0) red[wid] = ss;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const double cnt = (double)count, mean = keep / cnt;
+        const double var = fmax((red[0] + red[1] + red[2] + red[3]) / cnt - mean * mean, 0.0);
+        stats[ng * 2] = make_float2((float)mean, (float)(1.0 / sqrt(var + (double)eps)));
+    }
+}
+
 template <int DT, int PRO>
 int launch(const ProArgs& p, int M, hipStream_t st) {
     if (M <= 0) return 0;
@@ -222,4 +307,27 @@ extern "C" int gpu_internal_quant_prologue(int dtype, int prologue, const void* 
     if (dtype == DT_F32) { QPRO(DT_F32) }
 #undef QPRO
     return -4;
+}
+
+// The SD fused sources into a half row buffer [M, K] (mode: 1 LN, 2 GEGLU, 3 UNPAD, 4 GN; for GN `stats` is the caller's
+// `sums` scratch, filled here first).
+extern "C" int gpu_internal_sd_source(int mode, const void* x, int64_t x_stride, const float* w, const float* b, float eps,
+                                      int heads, int d, int dp, void* stats, int groups, int64_t P, int n_images, void* out,
+                                      int M, int K, void* stream) {
+    if (M <= 0) return 0;
+    hipStream_t st = (hipStream_t)stream;
+    SdSrc p{(const uint16_t*)x, x_stride, w, b, eps, heads, d, dp, (const float2*)stats, groups, P, (uint16_t*)out, K};
+    switch (mode) {
+        case SDQ_LN: hipLaunchKernelGGL(sd_source_rows_kernel<SDQ_LN>, dim3((unsigned)M), dim3(256), 0, st, p); break;
+        case SDQ_GEGLU: hipLaunchKernelGGL(sd_source_rows_kernel<SDQ_GEGLU>, dim3((unsigned)M), dim3(256), 0, st, p); break;
+        case SDQ_UNPAD: hipLaunchKernelGGL(sd_source_rows_kernel<SDQ_UNPAD>, dim3((unsigned)M), dim3(256), 0, st, p); break;
+        case SDQ_GN:
+            hipLaunchKernelGGL(sd_group_stats_kernel, dim3((unsigned)(n_images * groups)), dim3(256), 0, st, (const uint16_t*)x,
+                               (float2*)stats, P, K, groups, eps);
+            hipLaunchKernelGGL(sd_source_rows_kernel<SDQ_GN>, dim3((unsigned)M), dim3(256), 0, st, p);
+            break;
+        default: return -3;
+    }
+    KCHECK();
+    return 0;
 }

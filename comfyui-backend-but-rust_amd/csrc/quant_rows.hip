@@ -384,3 +384,49 @@ GPU_API int gpu_sd_quant_rows(const void* x, int64_t x_stride, int8_t* q, float*
     QuantArgs a{x, x_stride, q, scales, nullptr, M, K, 1, 1};
     return run_quant<MODE_SD_F16>(a, rotate, (hipStream_t)stream);
 }
+
+// The SD UNet's fused quantizers (csrc/sd.cu:608-724): the half row of LayerNorm / GEGLU / head un-padding / GroupNorm,
+// then gpu_sd_quant_rows of it.  The row is written to a stream-ordered buffer by a kernel of its own; it is rounded to
+// half in the reference too, so codes and scales are those of the one-kernel form.
+extern "C" int gpu_internal_sd_source(int mode, const void* x, int64_t x_stride, const float* w, const float* b, float eps,
+                                      int heads, int d, int dp, void* stats, int groups, int64_t P, int n_images, void* out,
+                                      int M, int K, void* stream);
+namespace {
+int sd_quant_src(int mode, const void* x, int64_t x_stride, const float* w, const float* b, float eps, int heads, int d, int dp,
+                 void* stats, int groups, int64_t P, int n_images, int8_t* q, float* scales, int M, int K, int rotate,
+                 hipStream_t st) {
+    if ((rotate != 0 && rotate != 64 && rotate != 256) || (rotate && K % rotate)) return -1;   // csrc/sd.cu:682
+    if (K <= 0 || (K % 16) != 0) return -1;
+    if (K > 32768) return -2;
+    if (M <= 0) return 0;
+    void* rows = nullptr;
+    hipError_t e = hipMallocAsync(&rows, (size_t)M * K * 2, st);
+    if (e != hipSuccess) return (int)e;
+    int rc = gpu_internal_sd_source(mode, x, x_stride, w, b, eps, heads, d, dp, stats, groups, P, n_images, rows, M, K, st);
+    if (rc == 0) {
+        QuantArgs a{rows, K, q, scales, nullptr, M, K, 1, 1};
+        rc = run_quant<MODE_SD_F16>(a, rotate, st);
+    }
+    e = hipFreeAsync(rows, st);
+    return rc == 0 && e != hipSuccess ? (int)e : rc;
+}
+}  // namespace
+
+GPU_API int gpu_sd_ln_quant_rows(const void* x, int64_t x_stride, const float* w, const float* b, float eps, int8_t* q,
+                                 float* scales, int M, int K, int rotate, void* stream) {
+    return sd_quant_src(1, x, x_stride, w, b, eps, 0, 0, 0, nullptr, 0, 0, 0, q, scales, M, K, rotate, (hipStream_t)stream);
+}
+GPU_API int gpu_sd_geglu_quant_rows(const void* in, int8_t* q, float* scales, int M, int I, int rotate, void* stream) {
+    return sd_quant_src(2, in, 0, nullptr, nullptr, 0.f, 0, 0, 0, nullptr, 0, 0, 0, q, scales, M, I, rotate, (hipStream_t)stream);
+}
+GPU_API int gpu_sd_unpad_quant_rows(const void* src, int8_t* q, float* scales, int M, int H, int d, int dp, int rotate,
+                                    void* stream) {
+    if (H <= 0 || d <= 0 || dp < d) return -1;
+    return sd_quant_src(3, src, 0, nullptr, nullptr, 0.f, H, d, dp, nullptr, 0, 0, 0, q, scales, M, H * d, rotate,
+                        (hipStream_t)stream);
+}
+GPU_API int gpu_sd_group_norm_quant_rows(const void* x, const float* w, const float* b, void* sums, int N, int64_t P, int C, int G,
+                                         float eps, int8_t* q, float* scales, int rotate, void* stream) {
+    if (G <= 0 || C % G) return -1;                                                             // csrc/sd.cu:713
+    return sd_quant_src(4, x, 0, w, b, eps, 0, 0, 0, sums, G, P, N, q, scales, (int)(N * P), C, rotate, (hipStream_t)stream);
+}

@@ -22,6 +22,10 @@ SIGNATURES = {
     "gpu_quant_rows_b": [_I32, _I32, _P, _I64, _P, _P, _F32, _P, _P, _P, _P, _I32, _I32, _I32, _P],
     "gpu_rotate_rows_f32": [_I32, _P, _I64, _I64, _P, _F32, _P, _I32, _I32, _P],
     "gpu_sd_quant_rows": [_P, _I64, _P, _P, _I32, _I32, _I32, _P],
+    "gpu_sd_ln_quant_rows": [_P, _I64, _P, _P, _F32, _P, _P, _I32, _I32, _I32, _P],
+    "gpu_sd_geglu_quant_rows": [_P, _P, _P, _I32, _I32, _I32, _P],
+    "gpu_sd_unpad_quant_rows": [_P, _P, _P, _I32, _I32, _I32, _I32, _I32, _P],
+    "gpu_sd_group_norm_quant_rows": [_P, _P, _P, _P, _I32, _I64, _I32, _I32, _F32, _P, _P, _I32, _P],
     "gpu_prologue_rows": [_I32, _I32, _P, _I64, _P, _I64, _I64, _P, _F32, _P, _P, _P, _I64, _I32, _I32, _P],
     "gpu_prologue_rows_b": [_I32, _I32, _P, _I64, _P, _P, _F32, _P, _P, _P, _I64, _I32, _I32, _P],
     "gpu_int8_gemm": [_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I32, _P],

@@ -71,6 +71,42 @@ def sd_quant_rows(x, rotate=0, K=None):
     return q, scales
 
 
+def _sd_out(M, K, dev):
+    return torch.empty((M, K), dtype=torch.int8, device=dev), torch.empty((M,), dtype=torch.float32, device=dev)
+
+
+def sd_ln_quant_rows(x, w, b, eps, rotate=0, K=None):
+    """LayerNorm (half) then the fp16 quantizer, src/unet.rs call pattern of gpu_sd_ln_quant_rows."""
+    M = x.shape[0]
+    K = x.shape[1] if K is None else K
+    q, s = _sd_out(M, K, x.device)
+    ffi.k("gpu_sd_ln_quant_rows", _ptr(x), x.stride(0), _ptr(w), _ptr(b), float(eps), _ptr(q), _ptr(s), M, K, rotate, _stream())
+    return q, s
+
+
+def sd_geglu_quant_rows(x, rotate=0):
+    M, I = x.shape[0], x.shape[1] // 2
+    q, s = _sd_out(M, I, x.device)
+    ffi.k("gpu_sd_geglu_quant_rows", _ptr(x), _ptr(q), _ptr(s), M, I, rotate, _stream())
+    return q, s
+
+
+def sd_unpad_quant_rows(x, d, rotate=0):
+    M, H, dp = x.shape
+    q, s = _sd_out(M, H * d, x.device)
+    ffi.k("gpu_sd_unpad_quant_rows", _ptr(x), _ptr(q), _ptr(s), M, H, d, dp, rotate, _stream())
+    return q, s
+
+
+def sd_group_norm_quant_rows(x, w, b, groups, eps, rotate=0):
+    N, P, C = x.shape
+    q, s = _sd_out(N * P, C, x.device)
+    sums = torch.empty(16 * N * groups + 16, dtype=torch.uint8, device=x.device)
+    ffi.k("gpu_sd_group_norm_quant_rows", _ptr(x), _ptr(w), _ptr(b), _ptr(sums), N, P, C, groups, float(eps), _ptr(q), _ptr(s),
+          rotate, _stream())
+    return q, s, sums
+
+
 def rotate_rows_f32(x, K=None, prologue=ffi.PRO_PLAIN, up_offset=0, norm_w=None, eps=0.0):
     M, x_stride = x.shape
     K = x_stride if K is None else K

@@ -78,6 +78,22 @@ int gpu_prologue_rows_b(int dtype, int prologue, const void* x, int64_t x_stride
 int gpu_sd_quant_rows(const void* x, int64_t x_stride, int8_t* q, float* scales, int M, int K, int rotate,
                       void* stream);
 
+/* The SD UNet's fused quantizers: the half row another kernel would have written, then gpu_sd_quant_rows of it.
+ * Replace gpu_sd_ln_quant_rows, gpu_sd_geglu_quant_rows, gpu_sd_unpad_quant_rows, gpu_sd_group_norm_quant_rows,
+ * csrc/sd.cu:691-724.  rotate and K as gpu_sd_quant_rows.  The row goes through a stream-ordered half [M, K] buffer.
+ *   ln:     LayerNorm of x [M, x_stride] with fp32 weight and bias.
+ *   geglu:  in [M, 2I] (value, then gate) -> value * gelu(gate), K = I.
+ *   unpad:  src [M, H, dp] -> the first d of every dp, K = H * d.
+ *   gn:     GroupNorm (no SiLU) of x [N, P, C] per image; rows are pixels, K = C.  sums: 16 * N * G + 16 bytes of device
+ *           scratch, which receives (mean, rstd) as two floats at byte 16 * (n * G + g), as the reference leaves them. */
+int gpu_sd_ln_quant_rows(const void* x, int64_t x_stride, const float* w, const float* b, float eps, int8_t* q,
+                         float* scales, int M, int K, int rotate, void* stream);
+int gpu_sd_geglu_quant_rows(const void* in, int8_t* q, float* scales, int M, int I, int rotate, void* stream);
+int gpu_sd_unpad_quant_rows(const void* src, int8_t* q, float* scales, int M, int H, int d, int dp, int rotate,
+                            void* stream);
+int gpu_sd_group_norm_quant_rows(const void* x, const float* w, const float* b, void* sums, int N, int64_t P, int C, int G,
+                                 float eps, int8_t* q, float* scales, int rotate, void* stream);
+
 /* D[M,N] = Out((A[M,K] . W[N,K]^T) * xs[m] * ws[n] + bias[n]).
  * Replaces gpu_int8_gemm, src/ffi.rs:38 / csrc/gemm.cu:124-129.
  * A, W int8 row-major (K contiguous); xs f32 [M]; ws f32 [N]; bias Out[N] or null; D Out[M,N]; out_dt a DT_* code. */

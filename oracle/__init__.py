@@ -32,6 +32,8 @@ def lib():
         L.orc_rotate_rows_f32.restype = i32; L.orc_rotate_rows_f32.argtypes = [vp, i64, vp, i32, i32]
         L.orc_quant_rows_wide.restype = i32; L.orc_quant_rows_wide.argtypes = [i32, vp, i64, vp, vp, i32, i32, i32]
         L.orc_situ_rows_wide.restype = i32; L.orc_situ_rows_wide.argtypes = [i32, vp, i64, i64, vp, i32, i32]
+        L.orc_sd_source_rows.restype = i32
+        L.orc_sd_source_rows.argtypes = [i32, vp, i64, vp, vp, f32, i32, i32, i32, i32, i64, vp, i32, i32]
         L.orc_prologue_rows.restype = i32
         L.orc_prologue_rows.argtypes = [i32, i32, vp, i64, vp, i64, i64, vp, vp, f32, vp, vp, vp, i64, i32, i32]
         L.orc_sd_quant_rows.restype = i32; L.orc_sd_quant_rows.argtypes = [vp, i64, vp, vp, i32, i32, i32]
@@ -146,6 +148,19 @@ def situ_rows_wide(dtype, x, K, up_offset):
     x = _c(x, _IN_NP[dtype])
     out = np.zeros((x.shape[0], K), np.float32)
     rc = lib().orc_situ_rows_wide(dtype, _p(x), x.shape[1], up_offset, _p(out), x.shape[0], K)
+    return rc, out
+
+
+SD_LN, SD_GEGLU, SD_UNPAD, SD_GN = 1, 2, 3, 4
+
+
+def sd_source_rows(mode, x, M, K, x_stride=0, w=None, b=None, eps=0.0, heads=0, d=0, dp=0, groups=0, P=0):
+    """The half row of the SD fused quantizer sources (LayerNorm, GEGLU, head un-padding, GroupNorm) -> (rc, [M, K] bits)."""
+    x = _c(x, np.uint16)
+    w = None if w is None else _c(w, np.float32)
+    b = None if b is None else _c(b, np.float32)
+    out = np.zeros((M, K), np.uint16)
+    rc = lib().orc_sd_source_rows(mode, _p(x), x_stride, _p(w), _p(b), float(eps), heads, d, dp, groups, P, _p(out), M, K)
     return rc, out
 
 

@@ -25,6 +25,8 @@
  *   orc_w6a8_group_gemm                this build's own format (no reference counterpart); integer partials pinned by
  *                                      numpy int64
  *   orc_quant_rows_wide                pinned: equals orc_quant_rows for f32, torch bf16 arithmetic on fp32 values
+ *   orc_sd_source_rows                 LN / GEGLU / GroupNorm against torch float64 layer_norm, gelu, group_norm rounded to
+ *                                      half; un-padding against a numpy gather.  Last bit vs the reference unpinned, as below
  *   orc_prologue_rows, orc_situ_rows_wide  structure and rounding points pinned: torch float64 / bf16 tensor arithmetic
  *                                      (normalizations, gates, activations from torch.nn.functional) to one ulp of T,
  *                                      closed-form rows.  PARITY UNPINNED against the reference in the last bit: its
@@ -501,6 +503,54 @@ ORC_API int orc_prologue_rows(int dt, int pro, const void* x, int64_t x_stride, 
         }
 #undef X
 #undef R
+    }
+    return 0;
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * The SD UNet's fused quantizer sources, csrc/sd.cu:611-663: the half row that LayerNorm (:629-641), GEGLU (:642-649),
+ * head un-padding (:650-652) or GroupNorm without SiLU (:653-662, statistics :203-207) would have written; the fp16
+ * quantizer (orc_sd_quant_rows) then reads it.  Sums in fp64 rounded once, 1/sqrt correctly rounded, as in the prologues.
+ * mode: 1 LN, 2 GEGLU, 3 UNPAD, 4 GN.  out: half bits [M, K].
+ * ------------------------------------------------------------------------------------------- */
+ORC_API int orc_sd_source_rows(int mode, const uint16_t* x, int64_t x_stride, const float* w, const float* b, float eps,
+                               int heads, int d, int dp, int groups, int64_t P, uint16_t* out, int M, int K) {
+    if (mode < 1 || mode > 4) return -3;
+    if (mode == 4 && (groups <= 0 || K % groups)) return -1;
+    for (int64_t m = 0; m < M; ++m) {
+        uint16_t* o = out + m * K;
+        if (mode == 1) {
+            const uint16_t* r = x + m * x_stride;
+            double s = 0.0;
+            for (int k = 0; k < K; ++k) s += (double)orc_f16_to_f32(r[k]);
+            const float mean = (float)s / (float)K;
+            double s2 = 0.0;
+            for (int k = 0; k < K; ++k) { const float dd = orc_f16_to_f32(r[k]) - mean; s2 += (double)dd * (double)dd; }
+            const float rstd = (float)(1.0 / sqrt((double)((float)s2 / (float)K + eps)));
+            for (int k = 0; k < K; ++k) o[k] = orc_f32_to_f16(fmaf((orc_f16_to_f32(r[k]) - mean) * rstd, w[k], b[k]));
+        } else if (mode == 2) {
+            const uint16_t* r = x + m * 2 * K;
+            for (int k = 0; k < K; ++k)
+                o[k] = orc_f32_to_f16(orc_f16_to_f32(r[k]) * orc_f16_round(gelu_o(orc_f16_to_f32(r[K + k]))));
+        } else if (mode == 3) {
+            const uint16_t* r = x + m * heads * dp;
+            for (int k = 0; k < K; ++k) o[k] = r[(k / d) * dp + k % d];
+        } else {
+            const int per = K / groups;
+            const int64_t n = m / P;
+            const uint16_t* img = x + n * P * K;
+            for (int g = 0; g < groups; ++g) {
+                /* statistics of (image n, group g); recomputed per row for simplicity, rows of one image agree */
+                double s = 0.0, ss = 0.0;
+                for (int64_t pp = 0; pp < P; ++pp)
+                    for (int c = 0; c < per; ++c) { const double v = (double)orc_f16_to_f32(img[pp * K + g * per + c]); s += v; ss += v * v; }
+                const double cnt = (double)P * per, mean = s / cnt;
+                const double var = fmax(ss / cnt - mean * mean, 0.0);
+                const float mf = (float)mean, rf = (float)(1.0 / sqrt(var + (double)eps));
+                for (int c = g * per; c < (g + 1) * per; ++c)
+                    o[c] = orc_f32_to_f16(fmaf((orc_f16_to_f32(x[m * K + c]) - mf) * rf, w[c], b[c]));
+            }
+        }
     }
     return 0;
 }

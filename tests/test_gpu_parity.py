@@ -301,6 +301,57 @@ def test_quant_rows_b_and_rotate_rows_f32_with_prologues():
         assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32)), name
 
 
+@pytest.mark.parametrize("rotate", [0, 64, 256])
+def test_sd_fused_quantizers_equal_source_then_quantizer(rotate):
+    """gpu_sd_{ln,geglu,unpad,group_norm}_quant_rows == fp16 quantizer of the oracle's half row (csrc/sd.cu:608-724)."""
+    def check(tag, got, row, K):
+        rc, q, s = oracle.sd_quant_rows(row, K, rotate)
+        torch.cuda.synchronize()
+        assert rc == 0
+        assert np.array_equal(got[1].cpu().numpy().view(np.uint32), s.view(np.uint32)), tag
+        assert np.array_equal(got[0].cpu().numpy(), q), tag
+    M, K = 37, 1280
+    rnd = lambda stream, *shape: synth.normal(900 + rotate, stream, int(np.prod(shape))).reshape(shape)
+    w = (1 + 0.2 * rnd(1, K)).astype(np.float32)
+    b = (0.1 * rnd(2, K)).astype(np.float32)
+    x = synth.f16_bits(rnd(3, M, K + 64) * np.float32(1.5))
+    x[1, :] = 0
+    say("sd ln", rotate)
+    rc, row = oracle.sd_source_rows(oracle.SD_LN, x, M, K, x_stride=K + 64, w=w, b=b, eps=1e-5)
+    check("ln", ql.sd_ln_quant_rows(dev_bits(x, F16), dev(w), dev(b), 1e-5, rotate, K=K), row, K)
+    say("sd geglu", rotate)
+    xg = synth.f16_bits(rnd(4, M, 2 * K) * np.float32(2))
+    rc, row = oracle.sd_source_rows(oracle.SD_GEGLU, xg, M, K)
+    check("geglu", ql.sd_geglu_quant_rows(dev_bits(xg, F16), rotate), row, K)
+    say("sd unpad", rotate)
+    H, d, dp = 16, 80, 96                                                # K = 1280
+    xu = synth.f16_bits(rnd(5, M, H * dp))
+    rc, row = oracle.sd_source_rows(oracle.SD_UNPAD, xu, M, H * d, heads=H, d=d, dp=dp)
+    check("unpad", ql.sd_unpad_quant_rows(dev_bits(xu, F16).view(M, H, dp), d, rotate), row, H * d)
+    say("sd gn", rotate)
+    N, P, C, G = 2, 40, 512, 32
+    xn = synth.f16_bits(rnd(6, N * P, C) * np.float32(1.5) + np.float32(0.3))
+    rc, row = oracle.sd_source_rows(oracle.SD_GN, xn, N * P, C, w=w[:C], b=b[:C], eps=1e-5, groups=G, P=P)
+    qd, sd, sums = ql.sd_group_norm_quant_rows(dev_bits(xn, F16).view(N, P, C), dev(w[:C].copy()), dev(b[:C].copy()), G, 1e-5, rotate)
+    check("gn", (qd, sd), row, C)
+    # the statistics are left where the reference leaves them: (mean, rstd) floats at byte 16 * (n * G + g)
+    st = sums.cpu().numpy()[:16 * N * G].view(np.float32).reshape(N * G, 4)[:, :2]
+    xf = oracle.to_f32(xn, F16).astype(np.float64).reshape(N, P, G, C // G)
+    mean = xf.mean(axis=(1, 3)).reshape(-1)
+    var = xf.var(axis=(1, 3)).reshape(-1)
+    assert np.allclose(st[:, 0], mean, rtol=1e-6, atol=1e-7) and np.allclose(st[:, 1], 1 / np.sqrt(var + 1e-5), rtol=1e-6)
+
+
+def test_sd_fused_quantizer_argument_checks():
+    z = torch.zeros(64, dtype=torch.float16, device=DEV)
+    p = z.data_ptr()
+    assert ffi.raw("gpu_sd_ln_quant_rows", p, 640, p, p, 0.0, p, p, 1, 640, 128, 0) == -1
+    assert ffi.raw("gpu_sd_geglu_quant_rows", p, p, p, 1, 320, 256, 0) == -1
+    assert ffi.raw("gpu_sd_unpad_quant_rows", p, p, p, 1, 8, 40, 32, 0, 0) == -1      # dp < d
+    assert ffi.raw("gpu_sd_group_norm_quant_rows", p, p, p, p, 1, 4, 30, 4, 0.0, p, p, 0, 0) == -1
+    assert ffi.raw("gpu_sd_geglu_quant_rows", p, p, p, 0, 320, 0, 0) == 0
+
+
 def test_rotated_quant_golden_fixture():
     g = json.load(open(os.path.join(ROOT, "tests", "golden", "rotated_quant.json")))
     xb = synth.bf16_bits(synth.activations(11, 8, 1024, "t3"))

@@ -9,6 +9,9 @@ import torch
 
 import oracle
 from oracle import BF16, F16, F32
+from conftest import pkg
+
+synth = pkg("synth")
 
 H4 = np.array([[1, 1, 1, -1], [1, 1, -1, 1], [1, -1, 1, 1], [-1, 1, 1, 1]], dtype=np.float64)
 
@@ -617,3 +620,66 @@ def test_situ_wide_and_wide_quantizer(synth):
     assert np.array_equal(s, scale.numpy())
     assert np.array_equal(q, torch.clamp(torch.round(t), -128, 127).to(torch.int8).numpy())
     assert oracle.quant_rows_wide(F16, wide, K, 0)[0] == -4
+
+
+# ----------------------------------------------------------------------------------------------- SD fused sources
+def half_units(a, b):
+    return units_apart(F16, a, b)
+
+
+def test_sd_source_rows_match_torch_float64():
+    F = torch.nn.functional
+    g = torch.Generator().manual_seed(21)
+    M, K = 10, 640
+    xs, x = pro_inputs(F16, 21, M, K, cols=K + 32)
+    w = (1 + 0.2 * torch.randn(K, generator=g)).float()
+    b = (0.1 * torch.randn(K, generator=g)).float()
+    rc, out = oracle.sd_source_rows(oracle.SD_LN, xs, M, K, x_stride=K + 32, w=w.numpy(), b=b.numpy(), eps=1e-5)
+    assert rc == 0
+    want = to_storage(F16, F.layer_norm(x[:, :K], (K,), w.double(), b.double(), eps=1e-5))
+    d = half_units(out, want)
+    assert d.max() <= 1 and (d == 0).mean() > 0.98
+    # GEGLU: value * half(gelu(gate)), the product rounded to half
+    xs2, x2 = pro_inputs(F16, 22, M, 2 * K, cols=2 * K)
+    rc, out = oracle.sd_source_rows(oracle.SD_GEGLU, xs2, M, K)
+    want = to_storage(F16, x2[:, :K] * F.gelu(x2[:, K:]).half().double())
+    d = half_units(out, want)
+    body = (x2[:, K:] > -3).numpy()
+    assert d[body].max() <= 1 and (d[body] == 0).mean() > 0.98
+    assert (np.abs(oracle.to_f32(out, F16).astype(np.float64) - oracle.to_f32(want, F16)) <= 1e-3).all()
+    # un-padding is a gather
+    H, dd, dp = 5, 40, 64
+    src = synth.f16_bits(synth.normal(23, 1, 3 * H * dp).reshape(3, H * dp))
+    rc, out = oracle.sd_source_rows(oracle.SD_UNPAD, src, 3, H * dd, heads=H, d=dd, dp=dp)
+    assert rc == 0 and np.array_equal(out, src.reshape(3, H, dp)[:, :, :dd].reshape(3, H * dd))
+    # GroupNorm of [N, P, C] per image and group
+    N, P, C, G = 2, 24, 64, 8
+    xs3, x3 = pro_inputs(F16, 24, N * P, C, cols=C)
+    w3, b3 = w[:C], b[:C]
+    rc, out = oracle.sd_source_rows(oracle.SD_GN, xs3, N * P, C, w=w3.numpy(), b=b3.numpy(), eps=1e-5, groups=G, P=P)
+    assert rc == 0
+    ref = F.group_norm(x3.reshape(N, P, C).permute(0, 2, 1), G, w3.double(), b3.double(), eps=1e-5).permute(0, 2, 1).reshape(N * P, C)
+    d = half_units(out, to_storage(F16, ref))
+    assert d.max() <= 1 and (d == 0).mean() > 0.98
+    assert oracle.sd_source_rows(oracle.SD_GN, xs3, N * P, C, w=w3.numpy(), b=b3.numpy(), groups=7, P=P)[0] == -1
+    assert oracle.sd_source_rows(9, xs3, 1, C)[0] == -3
+
+
+def test_sd_source_closed_forms():
+    # alternating +-2 with eps 0: LayerNorm gives +-1, so the row is +-w + b exactly where that is a half number
+    K = 64
+    x = synth.f16_bits(np.tile(np.array([2.0, -2.0], np.float32), K // 2)[None])
+    w = np.arange(K, dtype=np.float32) / 8
+    b = np.arange(K, dtype=np.float32)[::-1].copy() / 4
+    rc, out = oracle.sd_source_rows(oracle.SD_LN, x, 1, K, x_stride=K, w=w, b=b, eps=0.0)
+    sign = np.tile(np.array([1.0, -1.0], np.float32), K // 2)
+    assert np.array_equal(oracle.to_f32(out, F16)[0], sign * w + b)
+    # a group of constant value c: mean c, variance 0, rstd = 1/sqrt(eps); every output is b
+    N, P, C, G = 1, 4, 16, 2
+    xg = synth.f16_bits(np.full((P, C), 3.0, np.float32))
+    rc, out = oracle.sd_source_rows(oracle.SD_GN, xg, P, C, w=np.ones(C, np.float32), b=np.full(C, 0.5, np.float32), eps=0.25, groups=G, P=P)
+    assert np.array_equal(oracle.to_f32(out, F16), np.full((P, C), 0.5, np.float32))
+    # geglu with gate 0 and a large gate: gelu(0) = 0, gelu(12) = 12
+    r = synth.f16_bits(np.array([[1.5, -2.0, 0.0, 12.0]], np.float32))
+    rc, out = oracle.sd_source_rows(oracle.SD_GEGLU, r, 1, 2)
+    assert oracle.to_f32(out, F16)[0].tolist() == [0.0, -24.0]
