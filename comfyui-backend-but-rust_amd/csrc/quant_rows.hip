@@ -7,8 +7,10 @@
 // a lane; for the wider strides the chunk makes one trip through a wave-private LDS tile so that those butterflies are
 // again lane-local, then returns to row order for the 16-byte code stores.
 #include "common.hpp"
+#include "convrot.hpp"
 
 namespace {
+using namespace convrot;
 
 // MODE_BF16_WIDE: fp32 values quantized with bf16 rounding (a bf16 row whose prologue leaves unrounded fp32 values).
 enum { MODE_BF16 = 0, MODE_F32 = 1, MODE_SD_F16 = 2, MODE_ROT_F32 = 3, MODE_BF16_WIDE = 4 };
@@ -22,26 +24,24 @@ struct QuantArgs {
     int M, K;
     int wpr;           // waves per row
     int rpb;           // rows per block
+    uint64_t seed;     // nonzero: stochastic rounding keyed by element index + seed (gpu_convrot_requant)
 };
 
-constexpr int kChunk = 1024;           // values per wave-chunk (64 lanes x 16)
-constexpr int kLdsPerWave = 1024 + 64; // floats: one chunk plus 16 pad floats per 256
-
-// LDS position of chunk element e.  Each lane's 16 consecutive values are four 16-byte vectors; vector i of lane L is
-// rotated to slot (i + L/2) & 3 so that 8 neighbouring lanes cover all 32 banks in a 128-bit access, and every 256
-// elements are padded by 16 floats so that the stride-16 accesses of the second phase spread over both bank halves.
-__device__ __forceinline__ int lds_pos(int e) {
-    const int L = e >> 4, i = (e >> 2) & 3, j = e & 3;
-    return (L << 4) + (((i + (L >> 1)) & 3) << 2) + j + ((e >> 8) << 4);
+// csrc/kernels.cu:1355-1359
+__device__ __forceinline__ uint32_t pcg_hash(uint32_t x) {
+    const uint32_t state = x * 747796405u + 2891336453u;
+    const uint32_t word = ((state >> ((state >> 28u) + 4u)) ^ state) * 277803737u;
+    return (word >> 22u) ^ word;
 }
-
-// h4_row x 4 outputs with the reference's left-to-right adds, scaled by 0.5 (csrc/common.cuh:99-106,119-122).
-__device__ __forceinline__ void bfly4(float& a, float& b, float& c, float& d) {
-    const float x0 = a, x1 = b, x2 = c, x3 = d;
-    a = 0.5f * (x0 + x1 + x2 - x3);
-    b = 0.5f * (x0 + x1 - x2 + x3);
-    c = 0.5f * (x0 - x1 + x2 + x3);
-    d = 0.5f * (-x0 + x1 + x2 + x3);
+// a + b of two bf16 values rounded once to bf16, what the bf16 add instruction behind __hadd gives
+// (csrc/kernels.cu:1341-1343): the exact sum fits a double, which is then cut to 8 significant bits, ties to even.
+__device__ __forceinline__ float bf16_add_once(float a, float b) {
+    const double s = (double)a + (double)b;
+    uint64_t u = __builtin_bit_cast(uint64_t, s);
+    const uint64_t rem = u & ((1ull << 45) - 1), half = 1ull << 44;
+    u >>= 45;
+    if (rem > half || (rem == half && (u & 1))) ++u;
+    return (float)__builtin_bit_cast(double, u << 45);
 }
 
 template <int MODE> __device__ __forceinline__ void load16(const void* x, int64_t off, float* v) {
@@ -71,81 +71,6 @@ template <int MODE> __device__ __forceinline__ void load16(const void* x, int64_
             v[4 * i] = f.x; v[4 * i + 1] = f.y; v[4 * i + 2] = f.z; v[4 * i + 3] = f.w;
         }
     }
-}
-
-// Rotate one chunk held as v[16] per lane (element 16*lane + i).  wl is the wave's LDS tile.
-// The LDS tile is private to the wave and the LDS unit executes one wave's accesses in program order, so between the
-// phases of rotate_chunk it is enough to stop the compiler from reordering them: no workgroup barrier is needed.
-#define LDS_WAVE_ORDER() asm volatile("" ::: "memory")
-
-template <int G> __device__ __forceinline__ void rotate_chunk(float* v, float* wl, int lane) {
-    // strides 1 and 4: inside the lane
-#pragma unroll
-    for (int i = 0; i < 4; ++i) bfly4(v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) bfly4(v[j], v[j + 4], v[j + 8], v[j + 12]);
-    // to LDS in row order
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-        *reinterpret_cast<float4*>(wl + lds_pos(16 * lane + 4 * i)) = make_float4(v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]);
-    LDS_WAVE_ORDER();
-    if (G == 256) {
-        // lane (R = lane/16, b = lane%16) takes elements R*256 + a*16 + b, a = 0..15: strides 16 and 64 are lane-local
-        const int base = (lane >> 4) * 256 + (lane & 15);
-        float w[16];
-#pragma unroll
-        for (int a = 0; a < 16; ++a) w[a] = wl[lds_pos(base + a * 16)];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) bfly4(w[4 * i], w[4 * i + 1], w[4 * i + 2], w[4 * i + 3]);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) bfly4(w[j], w[j + 4], w[j + 8], w[j + 12]);
-#pragma unroll
-        for (int a = 0; a < 16; ++a) wl[lds_pos(base + a * 16)] = w[a];
-    } else if (G == 64) {
-        // lane (Q = lane/4, p = lane%4) takes elements Q*64 + d*16 + 4p + j: stride 16 is lane-local
-        const int base = (lane >> 2) * 64 + (lane & 3) * 4;
-        float4 w[4];
-#pragma unroll
-        for (int d = 0; d < 4; ++d) w[d] = *reinterpret_cast<float4*>(wl + lds_pos(base + d * 16));
-        bfly4(w[0].x, w[1].x, w[2].x, w[3].x);
-        bfly4(w[0].y, w[1].y, w[2].y, w[3].y);
-        bfly4(w[0].z, w[1].z, w[2].z, w[3].z);
-        bfly4(w[0].w, w[1].w, w[2].w, w[3].w);
-#pragma unroll
-        for (int d = 0; d < 4; ++d) *reinterpret_cast<float4*>(wl + lds_pos(base + d * 16)) = w[d];
-    } else {
-        // G == 128: lane (O = lane/8, p = lane%8) takes O*128 + t*64 + d*16 + 2p + j: stride 16 (radix 4) and the
-        // closing radix-2 stage at stride 64, scaled by 1/sqrt(2)
-        const int base = (lane >> 3) * 128 + (lane & 7) * 2;
-        float2 w[2][4];
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int d = 0; d < 4; ++d) w[t][d] = *reinterpret_cast<float2*>(wl + lds_pos(base + t * 64 + d * 16));
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            bfly4(w[t][0].x, w[t][1].x, w[t][2].x, w[t][3].x);
-            bfly4(w[t][0].y, w[t][1].y, w[t][2].y, w[t][3].y);
-        }
-        const float c = 0.70710678118654752f;
-#pragma unroll
-        for (int d = 0; d < 4; ++d) {
-            const float ax = w[0][d].x, bx = w[1][d].x, ay = w[0][d].y, by = w[1][d].y;
-            w[0][d].x = (ax + bx) * c; w[1][d].x = (ax - bx) * c;
-            w[0][d].y = (ay + by) * c; w[1][d].y = (ay - by) * c;
-        }
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int d = 0; d < 4; ++d) *reinterpret_cast<float2*>(wl + lds_pos(base + t * 64 + d * 16)) = w[t][d];
-    }
-    LDS_WAVE_ORDER();
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const float4 f = *reinterpret_cast<float4*>(wl + lds_pos(16 * lane + 4 * i));
-        v[4 * i] = f.x; v[4 * i + 1] = f.y; v[4 * i + 2] = f.z; v[4 * i + 3] = f.w;
-    }
-    LDS_WAVE_ORDER();
 }
 
 __device__ __forceinline__ float wave_max(float v) {
@@ -239,7 +164,15 @@ __global__ void __launch_bounds__(512) quant_rows_kernel(QuantArgs p) {
                 } else {
                     t = x / st;
                 }
-                const int qi = (int)fminf(127.f, fmaxf(-128.f, nearbyintf(t)));
+                float r;
+                if (p.seed != 0 && (MODE == MODE_BF16 || MODE == MODE_F32)) {   // csrc/kernels.cu:1385-1388
+                    const uint64_t key = (uint64_t)(m * (int64_t)p.K + e0 + 4 * i + j) + p.seed;
+                    const float noise = (float)(pcg_hash((uint32_t)key ^ (uint32_t)(key >> 32)) >> 8) * 0x1.0p-24f;
+                    r = floorf(MODE == MODE_F32 ? t + noise : bf16_add_once(t, rnd_dt<DT_BF16>(noise)));
+                } else {
+                    r = nearbyintf(t);
+                }
+                const int qi = (int)fminf(127.f, fmaxf(-128.f, r));
                 acc |= ((uint32_t)qi & 0xffu) << (8 * j);
             }
             w[i] = acc;
@@ -429,4 +362,14 @@ GPU_API int gpu_sd_group_norm_quant_rows(const void* x, const float* w, const fl
                                          float eps, int8_t* q, float* scales, int rotate, void* stream) {
     if (G <= 0 || C % G) return -1;                                                             // csrc/sd.cu:713
     return sd_quant_src(4, x, 0, w, b, eps, 0, 0, 0, sums, G, P, N, q, scales, (int)(N * P), C, rotate, (hipStream_t)stream);
+}
+
+// x [N, K] in its original basis -> rotated int8 rows + row scales: the 256-wide quantizer with rounding to nearest
+// (seed 0) or stochastic rounding keyed by element index + seed.  Replaces gpu_convrot_requant, csrc/kernels.cu:1361-1420;
+// as there, any dtype other than DT_F32 is read as bf16.
+GPU_API int gpu_convrot_requant(int dtype, const void* x, void* q, void* s, int64_t N, int K, uint64_t seed, void* stream) {
+    if (K <= 0 || (K % 256) != 0) return -1;
+    if (K > 32768 || N > 0x7fffffff) return -2;
+    QuantArgs a{x, K, (int8_t*)q, (float*)s, nullptr, (int)N, K, 1, 1, seed};
+    return dtype == DT_F32 ? run_quant<MODE_F32>(a, 256, (hipStream_t)stream) : run_quant<MODE_BF16>(a, 256, (hipStream_t)stream);
 }

@@ -14,7 +14,7 @@ DT_F32, DT_F16, DT_BF16 = 0, 1, 2
 (PRO_PLAIN, PRO_RMS, PRO_GATE, PRO_SWIGLU, PRO_LAYERNORM, PRO_SILU, PRO_GELU, PRO_ADALN, PRO_SITU, PRO_LN_MOD,
  PRO_LN_AFFINE, PRO_GELU_TANH, PRO_LN_AFFINE_SILU, PRO_SITU_FAST) = range(14)
 
-_P, _I64, _I32, _F32 = C.c_void_p, C.c_int64, C.c_int, C.c_float
+_P, _I64, _I32, _F32, _U64 = C.c_void_p, C.c_int64, C.c_int, C.c_float, C.c_uint64
 
 # name -> argtypes, in the order of include/gpu_api.h
 SIGNATURES = {
@@ -26,6 +26,10 @@ SIGNATURES = {
     "gpu_sd_geglu_quant_rows": [_P, _P, _P, _I32, _I32, _I32, _P],
     "gpu_sd_unpad_quant_rows": [_P, _P, _P, _I32, _I32, _I32, _I32, _I32, _P],
     "gpu_sd_group_norm_quant_rows": [_P, _P, _P, _P, _I32, _I64, _I32, _I32, _F32, _P, _P, _I32, _P],
+    "gpu_dequant_i8": [_P, _P, _P, _I64, _I64, _P],
+    "gpu_embed_dequant": [_P, _P, _P, _I32, _I32, _I32, _P],
+    "gpu_convrot_dequant": [_I32, _P, _P, _P, _I64, _I32, _P],
+    "gpu_convrot_requant": [_I32, _P, _P, _P, _I64, _I32, _U64, _P],
     "gpu_prologue_rows": [_I32, _I32, _P, _I64, _P, _I64, _I64, _P, _F32, _P, _P, _P, _I64, _I32, _I32, _P],
     "gpu_prologue_rows_b": [_I32, _I32, _P, _I64, _P, _P, _F32, _P, _P, _P, _I64, _I32, _I32, _P],
     "gpu_int8_gemm": [_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I32, _P],

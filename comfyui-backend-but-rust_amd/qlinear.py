@@ -71,6 +71,35 @@ def sd_quant_rows(x, rotate=0, K=None):
     return q, scales
 
 
+def dequant_i8(q, s):
+    out = torch.empty(q.shape, dtype=torch.float32, device=q.device)
+    ffi.k("gpu_dequant_i8", _ptr(q), _ptr(s), _ptr(out), q.shape[0], q.shape[1], _stream())
+    return out
+
+
+def embed_dequant(q, s):
+    """Rows of an int8 ConvRot embedding table -> fp32 rows of bf16 values (src/te.rs:441)."""
+    out = torch.empty(q.shape, dtype=torch.float32, device=q.device)
+    ffi.k("gpu_embed_dequant", _ptr(q), _ptr(s), _ptr(out), q.shape[0], q.shape[1], 1, _stream())
+    return out
+
+
+def convrot_dequant(q, s, dtype=torch.bfloat16):
+    """Rotated int8 weight + row scales -> the weight in its original basis (src/lora.rs:589)."""
+    out = torch.empty(q.shape, dtype=dtype, device=q.device)
+    ffi.k("gpu_convrot_dequant", _TORCH_DT[dtype], _ptr(q), _ptr(s), _ptr(out), q.shape[0], q.shape[1], _stream())
+    return out
+
+
+def convrot_requant(w, seed=0):
+    """Weight in its original basis -> rotated int8 + row scales (src/lora.rs:592, src/moss.rs:91)."""
+    N, K = w.shape
+    q = torch.empty((N, K), dtype=torch.int8, device=w.device)
+    s = torch.empty((N,), dtype=torch.float32, device=w.device)
+    ffi.k("gpu_convrot_requant", _TORCH_DT[w.dtype], _ptr(w), _ptr(q), _ptr(s), N, K, seed, _stream())
+    return q, s
+
+
 def _sd_out(M, K, dev):
     return torch.empty((M, K), dtype=torch.int8, device=dev), torch.empty((M,), dtype=torch.float32, device=dev)
 

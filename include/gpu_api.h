@@ -94,6 +94,19 @@ int gpu_sd_unpad_quant_rows(const void* src, int8_t* q, float* scales, int M, in
 int gpu_sd_group_norm_quant_rows(const void* x, const float* w, const float* b, void* sums, int N, int64_t P, int C, int G,
                                  float eps, int8_t* q, float* scales, int rotate, void* stream);
 
+/* Weight-side kernels of the int8 ConvRot format (weights are stored rotated; H256 is its own inverse).
+ *   gpu_dequant_i8       out f32 [N,K] = q * s[row].  Replaces csrc/kernels.cu:329-343 (K % 4, else -1).
+ *   gpu_embed_dequant    rows of an int8 ConvRot embedding table -> f32 rows holding bf16 values, H256(q * s).
+ *                        Replaces csrc/kernels.cu:620-639 (rotate == 0: -1).  K % 256.
+ *   gpu_convrot_dequant  the weight in its original basis, f32 (DT_F32) or bf16 (any other code).  csrc/kernels.cu:1345-1407.
+ *   gpu_convrot_requant  x [N,K] f32 or bf16 in its original basis -> rotated q [N,K] + row scales; seed 0 rounds to
+ *                        nearest, any other seed rounds stochastically with the reference's hash of (element index + seed).
+ *                        csrc/kernels.cu:1361-1420.  K % 256, K <= 32768. */
+int gpu_dequant_i8(const int8_t* q, const float* s, float* out, int64_t N, int64_t K, void* stream);
+int gpu_embed_dequant(const int8_t* q, const float* s, float* out, int M, int K, int rotate, void* stream);
+int gpu_convrot_dequant(int dtype, const void* q, const void* s, void* out, int64_t N, int K, void* stream);
+int gpu_convrot_requant(int dtype, const void* x, void* q, void* s, int64_t N, int K, uint64_t seed, void* stream);
+
 /* D[M,N] = Out((A[M,K] . W[N,K]^T) * xs[m] * ws[n] + bias[n]).
  * Replaces gpu_int8_gemm, src/ffi.rs:38 / csrc/gemm.cu:124-129.
  * A, W int8 row-major (K contiguous); xs f32 [M]; ws f32 [N]; bias Out[N] or null; D Out[M,N]; out_dt a DT_* code. */

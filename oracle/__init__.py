@@ -34,6 +34,9 @@ def lib():
         L.orc_situ_rows_wide.restype = i32; L.orc_situ_rows_wide.argtypes = [i32, vp, i64, i64, vp, i32, i32]
         L.orc_sd_source_rows.restype = i32
         L.orc_sd_source_rows.argtypes = [i32, vp, i64, vp, vp, f32, i32, i32, i32, i32, i64, vp, i32, i32]
+        L.orc_convrot_requant.restype = i32; L.orc_convrot_requant.argtypes = [i32, vp, vp, vp, i32, i32, C.c_uint64]
+        L.orc_convrot_dequant.restype = i32; L.orc_convrot_dequant.argtypes = [i32, vp, vp, vp, i64, i32]
+        L.orc_dequant_i8.restype = i32; L.orc_dequant_i8.argtypes = [vp, vp, vp, i64, i64]
         L.orc_prologue_rows.restype = i32
         L.orc_prologue_rows.argtypes = [i32, i32, vp, i64, vp, i64, i64, vp, vp, f32, vp, vp, vp, i64, i32, i32]
         L.orc_sd_quant_rows.restype = i32; L.orc_sd_quant_rows.argtypes = [vp, i64, vp, vp, i32, i32, i32]
@@ -148,6 +151,34 @@ def situ_rows_wide(dtype, x, K, up_offset):
     x = _c(x, _IN_NP[dtype])
     out = np.zeros((x.shape[0], K), np.float32)
     rc = lib().orc_situ_rows_wide(dtype, _p(x), x.shape[1], up_offset, _p(out), x.shape[0], K)
+    return rc, out
+
+
+def convrot_requant(dtype, x, seed=0):
+    """Weight rows [N, K] (float32, or bf16 bits) -> (rc, rotated int8 codes, row scales); seed 0 rounds to nearest."""
+    x = _c(x, _IN_NP[dtype])
+    N, K = x.shape
+    q = np.zeros((N, K), np.int8)
+    s = np.zeros(N, np.float32)
+    rc = lib().orc_convrot_requant(dtype, _p(x), _p(q), _p(s), N, K, seed)
+    return rc, q, s
+
+
+def convrot_dequant(mode, q, s):
+    """H256(q * s[row]); mode 0 float32, 1 bf16 bits, 2 float32 holding bf16 values (the embedding form)."""
+    q = _c(q, np.int8)
+    s = _c(s, np.float32)
+    N, K = q.shape
+    out = np.zeros((N, K), np.uint16 if mode == 1 else np.float32)
+    rc = lib().orc_convrot_dequant(mode, _p(q), _p(s), _p(out), N, K)
+    return rc, out
+
+
+def dequant_i8(q, s):
+    q = _c(q, np.int8)
+    s = _c(s, np.float32)
+    out = np.zeros(q.shape, np.float32)
+    rc = lib().orc_dequant_i8(_p(q), _p(s), _p(out), q.shape[0], q.shape[1])
     return rc, out
 
 

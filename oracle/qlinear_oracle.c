@@ -25,6 +25,9 @@
  *   orc_w6a8_group_gemm                this build's own format (no reference counterpart); integer partials pinned by
  *                                      numpy int64
  *   orc_quant_rows_wide                pinned: equals orc_quant_rows for f32, torch bf16 arithmetic on fp32 values
+ *   orc_convrot_requant                seed 0 equals orc_quant_rows(rotate 256); the stochastic form against exact
+ *                                      rational arithmetic on the same hash values, unbiasedness, hash known answers
+ *   orc_convrot_dequant, orc_dequant_i8  numpy products and the dense Kronecker matrix
  *   orc_sd_source_rows                 LN / GEGLU / GroupNorm against torch float64 layer_norm, gelu, group_norm rounded to
  *                                      half; un-padding against a numpy gather.  Last bit vs the reference unpinned, as below
  *   orc_prologue_rows, orc_situ_rows_wide  structure and rounding points pinned: torch float64 / bf16 tensor arithmetic
@@ -173,8 +176,29 @@ static int quant_check(int dtype, int K, int rotate) {
 }
 /* ld: the type the row is stored in; rd: the type T whose rounding the quantizer applies.  They differ only for the
  * fused PRO_SITU prologue of a bf16 row, which hands unrounded fp32 values to the quantizer (csrc/kernels.cu:107-112). */
+/* csrc/kernels.cu:1355-1359 */
+static inline uint32_t pcg_hash(uint32_t x) {
+    const uint32_t state = x * 747796405u + 2891336453u;
+    const uint32_t word = ((state >> ((state >> 28u) + 4u)) ^ state) * 277803737u;
+    return (word >> 22u) ^ word;
+}
+/* bf16 + bf16 rounded once to bf16 (the add instruction behind __hadd, csrc/kernels.cu:1341-1343): the sum is exact in
+ * long double / double for the magnitudes here and is rounded by the integer form on the double's bits. */
+ORC_API float orc_bf16_add_once(float a, float b);
+static inline float bf16_add_once(float a, float b) {
+    const double sum = (double)a + (double)b;
+    uint64_t u; memcpy(&u, &sum, 8);
+    const uint64_t rem = u & ((1ull << 45) - 1), half = 1ull << 44;
+    u >>= 45;
+    if (rem > half || (rem == half && (u & 1))) ++u;
+    u <<= 45;
+    double r; memcpy(&r, &u, 8);
+    return (float)r;
+}
+ORC_API float orc_bf16_add_once(float a, float b) { return bf16_add_once(a, b); }
+/* seed != 0: the stochastic rounding of gpu_convrot_requant, csrc/kernels.cu:1379-1389. */
 static int quant_rows_impl(int ld, int rd, const void* x, int64_t x_stride, int8_t* q, float* scales, int M, int K,
-                           int rotate) {
+                           int rotate, uint64_t seed) {
     const int rc = quant_check(rd, K, rotate);
     if (rc) return rc;
     const int g = rotate_group(rotate);
@@ -193,7 +217,13 @@ static int quant_rows_impl(int ld, int rd, const void* x, int64_t x_stride, int8
             const float st = rnd_t(rd, scale);                                              /* :243 */
             for (int k = 0; k < K; ++k) {
                 const float t = rnd_t(rd, rnd_t(rd, v[k]) / st);                            /* :254 */
-                q[(int64_t)m * K + k] = (int8_t)fmin_dev(127.f, fmax_dev(-128.f, nearbyintf(t)));
+                float r = nearbyintf(t);
+                if (seed) {
+                    const uint64_t key = (uint64_t)((int64_t)m * K + k) + seed;
+                    const float noise = (float)(pcg_hash((uint32_t)key ^ (uint32_t)(key >> 32)) >> 8) * 0x1.0p-24f;
+                    r = floorf(rd == ORC_F32 ? t + noise : bf16_add_once(t, orc_bf16_round(noise)));
+                }
+                q[(int64_t)m * K + k] = (int8_t)fmin_dev(127.f, fmax_dev(-128.f, r));
             }
         }
         free(v);
@@ -202,12 +232,39 @@ static int quant_rows_impl(int ld, int rd, const void* x, int64_t x_stride, int8
 }
 ORC_API int orc_quant_rows(int dtype, const void* x, int64_t x_stride, int8_t* q, float* scales, int M, int K,
                            int rotate) {
-    return quant_rows_impl(dtype, dtype, x, x_stride, q, scales, M, K, rotate);
+    return quant_rows_impl(dtype, dtype, x, x_stride, q, scales, M, K, rotate, 0);
 }
 /* fp32 values quantized with T = rd's rounding. */
 ORC_API int orc_quant_rows_wide(int rd, const float* x, int64_t x_stride, int8_t* q, float* scales, int M, int K,
                                 int rotate) {
-    return quant_rows_impl(ORC_F32, rd, x, x_stride, q, scales, M, K, rotate);
+    return quant_rows_impl(ORC_F32, rd, x, x_stride, q, scales, M, K, rotate, 0);
+}
+/* gpu_convrot_requant, csrc/kernels.cu:1361-1420: weight rows [N, K] (f32, else bf16) -> rotated codes + row scales. */
+ORC_API int orc_convrot_requant(int dtype, const void* x, int8_t* q, float* scales, int N, int K, uint64_t seed) {
+    const int dt = dtype == ORC_F32 ? ORC_F32 : ORC_BF16;
+    return quant_rows_impl(dt, dt, x, K, q, scales, N, K, 1, seed);
+}
+/* gpu_convrot_dequant (csrc/kernels.cu:1345-1353, out f32 or bf16 bits) and gpu_embed_dequant (:620-631, mode 2: f32
+ * holding bf16 values): out = H256(q * s[row]). */
+ORC_API int orc_convrot_dequant(int mode, const int8_t* q, const float* s, void* out, int64_t N, int K) {
+    if (K <= 0 || K % 256) return -1;
+    float* row = (float*)malloc(sizeof(float) * (size_t)K);
+    for (int64_t m = 0; m < N; ++m) {
+        for (int k = 0; k < K; ++k) row[k] = (float)q[m * K + k] * s[m];
+        orc_fht(row, K, 256);
+        for (int k = 0; k < K; ++k) {
+            if (mode == 1) ((uint16_t*)out)[m * K + k] = orc_f32_to_bf16(row[k]);
+            else ((float*)out)[m * K + k] = mode == 2 ? orc_bf16_round(row[k]) : row[k];
+        }
+    }
+    free(row);
+    return 0;
+}
+/* gpu_dequant_i8, csrc/kernels.cu:329-343 */
+ORC_API int orc_dequant_i8(const int8_t* q, const float* s, float* out, int64_t N, int64_t K) {
+    if (K % 4) return -1;
+    for (int64_t i = 0; i < N * K; ++i) out[i] = (float)q[i] * s[i / K];
+    return 0;
 }
 
 /* gpu_rotate_rows_f32, PRO_PLAIN: csrc/kernels.cu:316-327 with :227-238 (rotation always on, f32 in, f32 out). */

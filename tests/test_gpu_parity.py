@@ -352,6 +352,62 @@ def test_sd_fused_quantizer_argument_checks():
     assert ffi.raw("gpu_sd_geglu_quant_rows", p, p, p, 0, 320, 0, 0) == 0
 
 
+# ------------------------------------------------------------------------------------------------ weight-side formats
+@pytest.mark.parametrize("N,K", [(7, 256), (33, 3072), (5, 1280), (2, 12288), (1030, 512)])
+def test_convrot_dequant_and_embed_bit_exact(N, K):
+    say("convrot_dequant", N, K)
+    q = synth.randint(40 + K, 1, N * K, -128, 127).astype(np.int8).reshape(N, K)
+    s = synth.uniform(40 + K, 2, N, 1e-3, 1e-2)
+    qd, sd = dev(q), dev(s)
+    for mode, dt in ((0, torch.float32), (1, torch.bfloat16)):
+        rc, want = oracle.convrot_dequant(mode, q, s)
+        got = ql.convrot_dequant(qd, sd, dt)
+        torch.cuda.synchronize()
+        assert rc == 0 and np.array_equal(host_bits(got).view(want.dtype if mode else np.uint32), want.view(np.uint32) if not mode else want)
+    rc, want = oracle.convrot_dequant(2, q, s)
+    got = ql.embed_dequant(qd, sd)
+    torch.cuda.synchronize()
+    assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    assert ffi.raw("gpu_embed_dequant", qd.data_ptr(), sd.data_ptr(), got.data_ptr(), N, K, 0, 0) == -1
+    assert ffi.raw("gpu_convrot_dequant", 0, qd.data_ptr(), sd.data_ptr(), got.data_ptr(), N, 200, 0) == -1
+
+
+@pytest.mark.parametrize("N,K", [(9, 64), (5, 100), (3, 4096), (1025, 48)])
+def test_dequant_i8_bit_exact(N, K):
+    q = synth.randint(50 + K, 1, N * K, -128, 127).astype(np.int8).reshape(N, K)
+    s = synth.uniform(50 + K, 2, N, 1e-3, 1e-2)
+    rc, want = oracle.dequant_i8(q, s)
+    got = ql.dequant_i8(dev(q), dev(s))
+    torch.cuda.synchronize()
+    assert rc == 0 and np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    assert ffi.raw("gpu_dequant_i8", 0, 0, 0, 4, 6, 0) == -1
+
+
+@pytest.mark.parametrize("dt", [BF16, F32])
+@pytest.mark.parametrize("N,K", [(6, 256), (40, 3072), (3, 12288)])
+def test_convrot_requant_bit_exact(N, K, dt):
+    say("convrot_requant", N, K, dt)
+    w = synth.normal(60 + K, 1, N * K).reshape(N, K) * np.float32(0.05)
+    w[0, :] = 0
+    x = synth.bf16_bits(w) if dt == BF16 else w
+    xd = dev_bits(x, dt)
+    for seed in (0, 1, 0x1234_5678_9abc, 2 ** 63 + 12345):
+        rc, q, s = oracle.convrot_requant(dt, x, seed)
+        qd, sd = ql.convrot_requant(xd, seed)
+        torch.cuda.synchronize()
+        assert rc == 0
+        assert np.array_equal(sd.cpu().numpy().view(np.uint32), s.view(np.uint32)), seed
+        assert np.array_equal(qd.cpu().numpy(), q), seed
+    # the round trip of the LoRA baker (src/lora.rs:589-592): dequant to the original basis, requant with rounding to
+    # nearest, gives the codes back when the weight was exactly representable (bf16 storage costs at most one code)
+    rc, q0, s0 = oracle.convrot_requant(dt, x, 0)
+    back = ql.convrot_dequant(dev(q0), dev(s0), torch.float32)
+    q1, s1 = ql.convrot_requant(back, 0)
+    torch.cuda.synchronize()
+    assert np.abs(q1.cpu().numpy().astype(np.int32) - q0).max() <= 1
+    assert ffi.raw("gpu_convrot_requant", 0, xd.data_ptr(), qd.data_ptr(), sd.data_ptr(), N, 300, 0, 0) == -1
+
+
 def test_rotated_quant_golden_fixture():
     g = json.load(open(os.path.join(ROOT, "tests", "golden", "rotated_quant.json")))
     xb = synth.bf16_bits(synth.activations(11, 8, 1024, "t3"))

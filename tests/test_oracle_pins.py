@@ -1,6 +1,7 @@
 """Pins for the CPU oracle: every function is checked against something that does not share its code --
 library casts and arithmetic (torch bf16/f16/float8 tensors, numpy int64 matmul), closed forms (the Kronecker
 Hadamard matrix), exact rational arithmetic, and hand-worked special cases."""
+import ctypes
 from fractions import Fraction
 
 import numpy as np
@@ -683,3 +684,115 @@ def test_sd_source_closed_forms():
     r = synth.f16_bits(np.array([[1.5, -2.0, 0.0, 12.0]], np.float32))
     rc, out = oracle.sd_source_rows(oracle.SD_GEGLU, r, 1, 2)
     assert oracle.to_f32(out, F16)[0].tolist() == [0.0, -24.0]
+
+
+# ----------------------------------------------------------------------------------------------- weight-side formats
+def py_pcg(x):
+    """The hash of csrc/kernels.cu:1355-1359 in Python integers."""
+    m = 0xffffffff
+    state = (x * 747796405 + 2891336453) & m
+    word = (((state >> ((state >> 28) + 4)) ^ state) * 277803737) & m
+    return ((word >> 22) ^ word) & m
+
+
+def round_sig8(a):
+    """float64 array rounded to 8 significant bits, ties to even: a bf16 rounding done with frexp/rint."""
+    m, e = np.frexp(a)
+    return np.ldexp(np.rint(m * 256.0), e - 8)
+
+
+def test_convrot_dequant_and_dequant_i8(synth):
+    N, K = 5, 768
+    q = synth.randint(31, 1, N * K, -127, 127).astype(np.int8).reshape(N, K)
+    s = synth.uniform(31, 2, N, 1e-3, 1e-2)
+    rc, out = oracle.dequant_i8(q, s)
+    assert rc == 0 and np.array_equal(out, q.astype(np.float32) * s[:, None])
+    assert oracle.dequant_i8(q[:, :6], s)[0] == -1
+    H = kron_h(4)
+    want = np.einsum("ngk,jk->ngj", (q.astype(np.float32) * s[:, None]).astype(np.float64).reshape(N, K // 256, 256), H).reshape(N, K)
+    rc, o32 = oracle.convrot_dequant(0, q, s)
+    assert rc == 0 and np.allclose(o32, want, rtol=0, atol=2e-6)
+    rc, ob = oracle.convrot_dequant(1, q, s)
+    assert np.array_equal(ob, oracle.bf16_bits(o32))
+    rc, oe = oracle.convrot_dequant(2, q, s)
+    assert np.array_equal(oe, oracle.bf16_to_f32(ob))
+    assert oracle.convrot_dequant(0, q[:, :300], s)[0] == -1
+    # a weight that is exact in the rotated basis comes back exactly: q = 16 e_j, s = 1 -> a row of the Hadamard matrix
+    q1 = np.zeros((1, 256), np.int8); q1[0, 37] = 16
+    rc, o1 = oracle.convrot_dequant(0, q1, np.ones(1, np.float32))
+    assert np.array_equal(o1[0], (H[:, 37] * 16).astype(np.float32))
+
+
+def test_convrot_requant_nearest_and_stochastic(synth):
+    N, K = 6, 512
+    w = synth.normal(32, 1, N * K).reshape(N, K) * np.float32(0.05)
+    for dt, x in ((F32, w), (BF16, oracle.bf16_bits(w))):
+        rc, q0, s0 = oracle.convrot_requant(dt, x, 0)
+        rc1, q1, s1 = oracle.quant_rows(dt, x, K, 1)
+        assert rc == 0 and np.array_equal(q0, q1) and np.array_equal(s0, s1)
+        # requant(dequant(q, s)) is the identity for codes that are exactly representable after the round trip:
+        # stochastic rounding: floor(t + u), u = hash(index + seed) / 2^24 in [0, 1)
+        seed = 0x1234_5678_9abc
+        rc, qs, ss = oracle.convrot_requant(dt, x, seed)
+        assert rc == 0 and np.array_equal(ss, s0)
+        d = qs.astype(np.int32) - q0.astype(np.int32)
+        assert np.abs(d).max() <= 1 and 0.2 < (d != 0).mean() < 0.8
+        # restated from the rotated values: t as the quantizer computes it, then the draw
+        xf = oracle.to_f32(x, dt) if dt == BF16 else x
+        rot = np.einsum("ngk,jk->ngj", xf.astype(np.float64).reshape(N, K // 256, 256), kron_h(4)).reshape(N, K)
+        idx = np.arange(N * K, dtype=np.uint64) + np.uint64(seed)
+        folded = (idx & np.uint64(0xffffffff)) ^ (idx >> np.uint64(32))
+        u = np.array([py_pcg(int(v)) >> 8 for v in folded], np.float64).reshape(N, K) * 2.0 ** -24
+        st = s0.astype(np.float64) if dt == F32 else oracle.bf16_to_f32(oracle.bf16_bits(s0)).astype(np.float64)
+        t = rot / st[:, None]
+        if dt == F32:
+            total, slack = t + u, 2.0 ** -14
+        else:
+            # every step of the bf16 path is a bf16 number: t, the noise, and their sum rounded once
+            total, slack = round_sig8(round_sig8(round_sig8(rot) / st[:, None]) + round_sig8(u)), 2.0 ** -7
+            t = round_sig8(round_sig8(rot) / st[:, None])
+        want = np.clip(np.floor(total), -128, 127)
+        # rot carries the fp32 rounding of the butterflies: a draw can differ only where that error crosses a boundary
+        if dt == F32:
+            near = np.abs(total - np.rint(total)) < slack
+            assert (qs[~near] == want[~near]).all() and near.mean() < 0.01
+        else:
+            assert (qs != want).sum() <= 3
+    # the mean over many seeds is unbiased: E[floor(t + u)] = t
+    x1 = np.tile(w[:1], (1, 1))
+    acc = np.zeros(K)
+    for sd in range(1, 201):
+        acc += oracle.convrot_requant(F32, x1, sd * 7919)[1][0]
+    rot = np.einsum("gk,jk->gj", x1.astype(np.float64).reshape(K // 256, 256), kron_h(4)).reshape(K)
+    t = rot / oracle.convrot_requant(F32, x1, 0)[2][0]
+    assert np.abs(acc / 200 - t).max() < 0.15 and abs((acc / 200 - t).mean()) < 0.01
+    # hash known answers, worked by hand from the definition for x = 0: state = 2891336453, shift = (state >> 28) + 4 = 14
+    st0 = 2891336453
+    w0 = (((st0 >> 14) ^ st0) * 277803737) & 0xffffffff
+    assert py_pcg(0) == ((w0 >> 22) ^ w0)
+
+
+def test_bf16_add_with_one_rounding():
+    """The stochastic bf16 path adds two bf16 numbers with one rounding (the bf16 add instruction), not fp32 add then
+    bf16 rounding.  Checked against exact rational arithmetic, and on a pair where the two differ."""
+    L = oracle.lib()
+    L.orc_bf16_add_once.restype = ctypes.c_float
+    L.orc_bf16_add_once.argtypes = [ctypes.c_float, ctypes.c_float]
+    rng = np.random.default_rng(5)
+    a = oracle.bf16_to_f32(oracle.bf16_bits((rng.standard_normal(4000) * 60).astype(np.float32)))
+    b = oracle.bf16_to_f32(oracle.bf16_bits(rng.random(4000).astype(np.float32)))
+    for x, y in zip(a.tolist(), b.tolist()):
+        exact = Fraction(x) + Fraction(y)
+        got = Fraction(L.orc_bf16_add_once(x, y))
+        if exact == 0:
+            assert got == 0
+            continue
+        e = 0
+        while abs(exact) >= Fraction(2) ** (e + 1): e += 1
+        while abs(exact) < Fraction(2) ** e: e -= 1
+        ulp = Fraction(2) ** (e - 7)
+        assert abs(got - exact) <= ulp / 2 and got / ulp == int(got / ulp)
+        if abs(got - exact) == ulp / 2:
+            assert int(got / ulp) % 2 == 0
+    # 100 + 0.2578125 (= 0.25 + 2^-7): the exact sum lies above the tie 100.25 and rounds up to 100.5
+    assert L.orc_bf16_add_once(100.0, 0.2578125) == 100.5
