@@ -120,6 +120,64 @@ def time_w6a8(torch, ffi, M, K, N, steps, warmup):
     return e0.elapsed_time(e1) / steps * 1e3
 
 
+def time_row_kernels(torch, ffi, steps):
+    """The HBM-bound kernels either side of the GEMM, each timed alone with HIP events on the launch stream: name,
+    microseconds and algorithmic GB/s (bytes the call must read and write once)."""
+    dev = "cuda:0"
+    st = torch.cuda.current_stream()
+    s = st.cuda_stream
+    g = torch.Generator(device=dev).manual_seed(7)
+    P = lambda t: 0 if t is None else t.data_ptr()
+    out = []
+
+    def timed(name, nbytes, fn):
+        for _ in range(3):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record(st)
+        for _ in range(steps):
+            fn()
+        e1.record(st)
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / steps
+        out.append({"name": name, "us": round(us, 2), "GBs": round(nbytes / us / 1e3, 1),
+                    "frac_hbm": round(nbytes / us / 1e3 / PEAK_HBM_GBS, 4)})
+
+    M, K = 4608, 3072
+    x = torch.randn(M, 2 * K, device=dev, generator=g).to(torch.bfloat16)
+    w = torch.rand(K, device=dev, generator=g) + 0.5
+    ms = (torch.randn(K, device=dev, generator=g) * 0.3).to(torch.bfloat16)
+    q = torch.empty((M, K), dtype=torch.int8, device=dev)
+    xs = torch.empty((M,), dtype=torch.float32, device=dev)
+    quant = lambda pro, xs_, up, nw, m_, sh_: ffi.k("gpu_quant_rows", ffi.DT_BF16, pro, x.data_ptr(), xs_, 0, 0, up, P(nw), 1e-6,
+                                                    P(m_), P(sh_), q.data_ptr(), xs.data_ptr(), M, K, 1, s)
+    timed("gpu_quant_rows PLAIN rotate 256, M=4608 K=3072 bf16", M * K * 3, lambda: quant(ffi.PRO_PLAIN, 2 * K, 0, None, None, None))
+    timed("gpu_quant_rows RMS + modulation, rotate 256 (prologue kernel + quantizer)", M * K * 3,
+          lambda: quant(ffi.PRO_RMS, 2 * K, 0, w, ms, ms))
+    timed("gpu_quant_rows SWIGLU, rotate 256 (prologue kernel + quantizer)", M * K * 5, lambda: quant(ffi.PRO_SWIGLU, 2 * K, K, None, None, None))
+    Ms, I = 8192, 2560
+    xg = torch.randn(Ms, 2 * I, device=dev, generator=g).to(torch.float16)
+    qs = torch.empty((Ms, I), dtype=torch.int8, device=dev)
+    ss = torch.empty((Ms,), dtype=torch.float32, device=dev)
+    timed("gpu_sd_quant_rows rotate 64, M=8192 K=2560 f16", Ms * I * 3,
+          lambda: ffi.k("gpu_sd_quant_rows", xg.data_ptr(), 2 * I, qs.data_ptr(), ss.data_ptr(), Ms, I, 64, s))
+    timed("gpu_sd_geglu_quant_rows rotate 64, M=8192 I=2560 (source kernel + quantizer)", Ms * I * 5,
+          lambda: ffi.k("gpu_sd_geglu_quant_rows", xg.data_ptr(), qs.data_ptr(), ss.data_ptr(), Ms, I, 64, s))
+    N = 12288
+    wq = torch.randint(-127, 128, (N, K), dtype=torch.int8, device=dev, generator=g)
+    wsc = torch.rand(N, device=dev, generator=g) * 0.01 + 0.001
+    wf = torch.empty((N, K), dtype=torch.bfloat16, device=dev)
+    w32 = torch.empty((N, K), dtype=torch.float32, device=dev)
+    timed("gpu_convrot_dequant bf16, N=12288 K=3072", N * K * 3,
+          lambda: ffi.k("gpu_convrot_dequant", ffi.DT_BF16, wq.data_ptr(), wsc.data_ptr(), wf.data_ptr(), N, K, s))
+    timed("gpu_convrot_requant bf16 stochastic, N=12288 K=3072", N * K * 3,
+          lambda: ffi.k("gpu_convrot_requant", ffi.DT_BF16, wf.data_ptr(), wq.data_ptr(), wsc.data_ptr(), N, K, 12345, s))
+    timed("gpu_dequant_i8, N=12288 K=3072", N * K * 5,
+          lambda: ffi.k("gpu_dequant_i8", wq.data_ptr(), wsc.data_ptr(), w32.data_ptr(), N, K, s))
+    return out
+
+
 def cpu_baseline(host, M, K, N, rotate, target_s):
     """The oracle's whole linear (quantize, int32 GEMM, epilogue) on a row sample sized for about `target_s` seconds."""
     import oracle
@@ -223,6 +281,7 @@ def main():
             w6.append({"name": name, "M": m, "K": k, "N": n, "kernel": "gpu_w6a8_group_gemm", "us": round(us, 1),
                        "TOPS": round(2.0 * m * n * k / us / 1e6, 1), "frac_int8_peak": round(2.0 * m * n * k / us / 1e6 / PEAK_INT8_TOPS, 4)})
         out["w6a8"] = w6
+        out["row_kernels"] = time_row_kernels(torch, ffi, few)
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(host, M, K, N, a.rotate, a.cpu_seconds)
     print(json.dumps(out))

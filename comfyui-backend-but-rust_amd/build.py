@@ -36,11 +36,25 @@ def _compile(src):
     return obj
 
 
+BLAS_OUT = os.path.join(HERE, "libgpu_blas.so")
+
+
+def build_blas():
+    """The dense-GEMM library over hipBLASLt: host code only."""
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    subprocess.check_call(["hipcc", "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden",
+                           os.path.join(CSRC, "blas_gemm.cpp"), "-o", BLAS_OUT, "-L" + os.path.join(rocm, "lib"), "-lhipblaslt",
+                           "-Wl,-rpath," + os.path.join(rocm, "lib")])
+    return BLAS_OUT
+
+
 def stale():
     if not os.path.exists(OUT):
         return True
     t = os.path.getmtime(OUT)
-    deps = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".hip", ".hpp"))]
+    if not os.path.exists(BLAS_OUT):
+        return True
+    deps = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".hip", ".hpp", ".cpp"))]
     deps.append(os.path.join(os.path.dirname(HERE), "include", "gpu_api.h"))
     return any(os.path.getmtime(d) > t for d in deps)
 
@@ -51,6 +65,7 @@ def build(force=True):
     with concurrent.futures.ThreadPoolExecutor(max_workers=len(SOURCES)) as ex:
         objs = list(ex.map(_compile, SOURCES))
     subprocess.check_call(["hipcc", "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", OUT, *objs])
+    build_blas()
     return OUT
 
 

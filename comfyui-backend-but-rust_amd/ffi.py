@@ -100,5 +100,35 @@ def raw(name, *args):
     return getattr(lib, name)(*args)
 
 
+# The dense GEMM beside the path lives in a library of its own (include/gpu_blas_api.h), loaded on first use so that the
+# int8 path does not depend on hipBLASLt.
+BLAS_LIB_PATH = os.path.join(_HERE, "libgpu_blas.so")
+_SZ = C.c_size_t
+BLAS_SIGNATURES = {
+    "gpu_blas_init": [_SZ],
+    "gpu_gemm": [_P, _I64, _P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I32, _I32, _I32, _F32, _F32, _P],
+}
+_blas = None
+
+
+def blas():
+    global _blas
+    if _blas is None:
+        if not os.path.exists(BLAS_LIB_PATH):
+            raise ImportError("libgpu_blas.so is not built (%s); run the package's build.py" % BLAS_LIB_PATH)
+        L = C.CDLL(BLAS_LIB_PATH)
+        for name, args in BLAS_SIGNATURES.items():
+            fn = getattr(L, name)
+            fn.argtypes = args
+            fn.restype = _I32
+        _blas = L
+    return _blas
+
+
+def kb(name, *args):
+    """Checked call into the dense-GEMM library."""
+    ok(getattr(blas(), name)(*args), name)
+
+
 def build_info():
     return lib.gpu_kernels_build_info().decode()

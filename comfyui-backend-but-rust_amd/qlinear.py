@@ -71,6 +71,18 @@ def sd_quant_rows(x, rotate=0, K=None):
     return q, scales
 
 
+def gemm(A, B, bias=None, transb=True, out_dtype=None, alpha=1.0, beta=0.0, D=None):
+    """gpu_gemm (src/ffi.rs, csrc/gemm.cu:55): D = alpha * A . B^T (transb) or A . B, + bias, + beta * D."""
+    ffi.kb("gpu_blas_init", 32 << 20)
+    M, K = A.shape
+    N = B.shape[0] if transb else B.shape[1]
+    out_dtype = A.dtype if out_dtype is None else out_dtype
+    D = torch.empty((M, N), dtype=out_dtype, device=A.device) if D is None else D
+    ffi.kb("gpu_gemm", _ptr(A), A.stride(0), _ptr(B), B.stride(0), _ptr(D), D.stride(0), _ptr(bias), M, N, K, 1 if transb else 0,
+           _TORCH_DT[A.dtype], _TORCH_DT[out_dtype], float(alpha), float(beta), _stream())
+    return D
+
+
 def dequant_i8(q, s):
     out = torch.empty(q.shape, dtype=torch.float32, device=q.device)
     ffi.k("gpu_dequant_i8", _ptr(q), _ptr(s), _ptr(out), q.shape[0], q.shape[1], _stream())

@@ -408,6 +408,35 @@ def test_convrot_requant_bit_exact(N, K, dt):
     assert ffi.raw("gpu_convrot_requant", 0, xd.data_ptr(), qd.data_ptr(), sd.data_ptr(), N, 300, 0, 0) == -1
 
 
+# ------------------------------------------------------------------------------------------------ dense GEMM
+@pytest.mark.parametrize("in_dt,out_dt", [(torch.bfloat16, torch.bfloat16), (torch.float16, torch.float16),
+                                          (torch.float32, torch.float32), (torch.bfloat16, torch.float32)])
+@pytest.mark.parametrize("M,N,K,transb,with_bias", [(64, 256, 512, True, True), (130, 96, 320, True, False),
+                                                     (48, 128, 256, False, True), (1, 3072, 256, True, True)])
+def test_gpu_gemm_against_float64(M, N, K, transb, with_bias, in_dt, out_dt):
+    """gpu_gemm over hipBLASLt: fp32 accumulation of the inputs' products, checked against a float64 product of the same
+    rounded inputs.  Tolerance: two units of the output type plus the fp32 accumulation error over K."""
+    say("gpu_gemm", M, N, K, transb, with_bias, in_dt, out_dt)
+    g = torch.Generator().manual_seed(M + N + K)
+    A = torch.randn(M, K, generator=g).to(in_dt)
+    B = (torch.randn(N, K, generator=g) if transb else torch.randn(K, N, generator=g)).to(in_dt) * 0.1
+    bias = torch.randn(N, generator=g).to(out_dt) if with_bias else None
+    want = A.double() @ (B.double().T if transb else B.double())
+    if with_bias:
+        want = want + bias.double()
+    got = ql.gemm(A.to(DEV), B.to(DEV), None if bias is None else bias.to(DEV), transb, out_dt)
+    torch.cuda.synchronize()
+    unit = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11, torch.float32: 2.0 ** -24}[out_dt]
+    mag = A.double().abs() @ (B.double().abs().T if transb else B.double().abs())
+    assert ((got.cpu().double() - want).abs() <= 2 * unit * want.abs() + K * 2.0 ** -24 * mag + 1e-30).all()
+    # alpha and beta
+    D = torch.ones((M, N), dtype=out_dt, device=DEV)
+    ql.gemm(A.to(DEV), B.to(DEV), None, transb, out_dt, alpha=0.5, beta=2.0, D=D)
+    torch.cuda.synchronize()
+    want2 = 0.5 * (want - (bias.double() if with_bias else 0)) + 2.0
+    assert ((D.cpu().double() - want2).abs() <= 2 * unit * (want2.abs() + 2) + K * 2.0 ** -24 * mag + 1e-30).all()
+
+
 def test_rotated_quant_golden_fixture():
     g = json.load(open(os.path.join(ROOT, "tests", "golden", "rotated_quant.json")))
     xb = synth.bf16_bits(synth.activations(11, 8, 1024, "t3"))

@@ -14,8 +14,8 @@ from conftest import ROOT, pkg
 ffi = pkg("ffi")
 
 
-def header_functions():
-    text = open(os.path.join(ROOT, "include", "gpu_api.h")).read()
+def header_functions(name="gpu_api.h"):
+    text = open(os.path.join(ROOT, "include", name)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return re.findall(r"\b(gpu_[a-z0-9_]+)\s*\(", text)
 
@@ -30,6 +30,13 @@ def test_library_exports_every_declared_symbol():
     for n in ffi.SIGNATURES:
         assert n in names, "ffi.py binds %s, which the header does not declare" % n
     assert "gfx950" in ffi.build_info()
+    # the dense-GEMM library: loads (hipBLASLt resolves) and exports what its header declares
+    blas_names = header_functions("gpu_blas_api.h")
+    assert set(blas_names) == {"gpu_blas_init", "gpu_gemm"} == set(ffi.BLAS_SIGNATURES)
+    blas = ctypes.CDLL(ffi.BLAS_LIB_PATH)
+    for n in blas_names:
+        assert hasattr(blas, n), n
+    assert ffi.blas().gpu_gemm(0, 0, 0, 0, 0, 0, 0, 4, 4, 4, 1, 2, 2, 1.0, 0.0, 0) == -100    # before gpu_blas_init
 
 
 def test_header_constants_match_reference_codes():
