@@ -153,9 +153,9 @@ def time_row_kernels(torch, ffi, steps):
     quant = lambda pro, xs_, up, nw, m_, sh_: ffi.k("gpu_quant_rows", ffi.DT_BF16, pro, x.data_ptr(), xs_, 0, 0, up, P(nw), 1e-6,
                                                     P(m_), P(sh_), q.data_ptr(), xs.data_ptr(), M, K, 1, s)
     timed("gpu_quant_rows PLAIN rotate 256, M=4608 K=3072 bf16", M * K * 3, lambda: quant(ffi.PRO_PLAIN, 2 * K, 0, None, None, None))
-    timed("gpu_quant_rows RMS + modulation, rotate 256 (prologue kernel + quantizer)", M * K * 3,
+    timed("gpu_quant_rows RMS + modulation, rotate 256", M * K * 3,
           lambda: quant(ffi.PRO_RMS, 2 * K, 0, w, ms, ms))
-    timed("gpu_quant_rows SWIGLU, rotate 256 (prologue kernel + quantizer)", M * K * 5, lambda: quant(ffi.PRO_SWIGLU, 2 * K, K, None, None, None))
+    timed("gpu_quant_rows SWIGLU, rotate 256", M * K * 5, lambda: quant(ffi.PRO_SWIGLU, 2 * K, K, None, None, None))
     Ms, I = 8192, 2560
     xg = torch.randn(Ms, 2 * I, device=dev, generator=g).to(torch.float16)
     qs = torch.empty((Ms, I), dtype=torch.int8, device=dev)

@@ -1,8 +1,7 @@
 // Row prologues of the quantizer (csrc/kernels.cu:88-182 inside quant_rows_kernel, :348-474 as prologue_rows_kernel):
 // RMSNorm / LayerNorm with modulation, gates, SwiGLU, activations.  Every prologue ends on a rounding to the row dtype
-// T, so writing its result as a T row and quantizing that row is bit-identical to the fused form; this file writes the
-// row (gpu_prologue_rows[_b], which the reference also exports for its bf16/f32 GEMMs) and quant_rows.hip runs its
-// plain quantizer on it for the non-PLAIN prologues of gpu_quant_rows / gpu_quant_rows_b / gpu_rotate_rows_f32.
+// T.  This file writes that row (gpu_prologue_rows[_b], which the reference exports for its bf16/f32 GEMMs); the
+// quantizer entry points apply the same expressions inside their own kernel (quant_rows.hip).
 //
 // Arithmetic: the reference's expressions and rounding points (rnd<T> after the same operations), with two choices
 // where its result depends on things a port cannot copy:
@@ -13,6 +12,7 @@
 //   * a*b + c written as one expression is contracted to an fma, as nvcc does by default.
 // One workgroup per row.
 #include "common.hpp"
+#include "rowmath.hpp"
 
 namespace {
 
@@ -31,26 +31,6 @@ struct ProArgs {
     int64_t out_stride;
     int K;
 };
-
-__device__ __forceinline__ float exp_cr(float x) { return (float)exp((double)x); }
-__device__ __forceinline__ float silu_f(float x) { return x / (1.f + exp_cr(-x)); }          // csrc/common.cuh:71
-__device__ __forceinline__ float sigmoid_f(float x) { return 1.f / (1.f + exp_cr(-x)); }     // :72
-__device__ __forceinline__ float stable_tanh(float x) {                                      // :74-77
-    const float t = (float)expm1((double)(-2.f * fabsf(x)));
-    return copysignf(-t / (t + 2.f), x);
-}
-__device__ __forceinline__ float gelu_f(float x) { return 0.5f * x * (1.f + (float)erf((double)(x * 0.70710678118654752f))); }  // :91
-__device__ __forceinline__ float gelu_tanh_f(float x) {                                      // :92-95
-    const float k0 = 0.7978845608028654f, k1 = 0.044715f;
-    return 0.5f * x * (1.f + (float)tanh((double)(k0 * __builtin_fmaf(k1 * x * x, x, x))));
-}
-
-// MOSS Image's soft-capped gated activation as one float expression, csrc/common.cuh:80-82
-__device__ __forceinline__ float situ_f(float hidden, float gate) {
-    return 4.f * stable_tanh(gate / 4.f) / (1.f + exp_cr(-gate)) * (25.f * stable_tanh(hidden / 25.f));
-}
-// Internal id: situ_f of a T row written as unrounded fp32 (what the fused quantizer consumes, csrc/kernels.cu:107-112).
-constexpr int PRO_SITU_WIDE = 100;
 
 template <int PRO> __device__ __forceinline__ constexpr bool is_ln() {
     return PRO == PRO_LAYERNORM || PRO == PRO_LN_MOD || PRO == PRO_LN_AFFINE || PRO == PRO_LN_AFFINE_SILU;
@@ -135,9 +115,6 @@ __global__ void __launch_bounds__(256) prologue_rows_kernel(ProArgs p) {
             const float h = R(25.f * R(stable_tanh(R(hidden / 25.f))));
             st_dt<DT>(o, k, g * h);
         }
-    } else if (PRO == PRO_SITU_WIDE) {
-        float* of = (float*)p.out + m * p.out_stride;
-        for (int k = threadIdx.x; k < K; k += blockDim.x) of[k] = situ_f(ld_dt<DT>(x, k), ld_dt<DT>(x, p.up_offset + k));
     } else {
         for (int k = threadIdx.x; k < K; k += blockDim.x) st_dt<DT>(o, k, ld_dt<DT>(x, k));
     }
@@ -276,36 +253,6 @@ GPU_API int gpu_prologue_rows_b(int dtype, int prologue, const void* x, int64_t 
     if (dtype == DT_BF16) return dispatch<DT_BF16>(prologue, p, M, (hipStream_t)stream, true);
     if (dtype == DT_F16) return dispatch<DT_F16>(prologue, p, M, (hipStream_t)stream, true);
     if (dtype == DT_F32) return dispatch<DT_F32>(prologue, p, M, (hipStream_t)stream, true);
-    return -4;
-}
-
-// The prologues of the quantizer entry points, into a T row buffer the caller (quant_rows.hip) provides: the ids of
-// csrc/kernels.cu:280-292 (gpu_quant_rows), :308-312 (gpu_quant_rows_b) and :322-327 (gpu_rotate_rows_f32).
-extern "C" int gpu_internal_quant_prologue(int dtype, int prologue, const void* x, int64_t x_stride, const void* g,
-                                           int64_t g_stride, int64_t up_offset, const float* norm_w, const float* norm_b,
-                                           float eps, const void* mod_scale, const void* mod_shift, void* out, int M, int K,
-                                           void* stream) {
-    ProArgs p{x, x_stride, g, g_stride, up_offset, norm_w, norm_b, eps, mod_scale, mod_shift, out, K, K};
-    hipStream_t st = (hipStream_t)stream;
-#define QPRO(DT)                                                           \
-    switch (prologue) {                                                    \
-        case PRO_RMS: return launch<DT, PRO_RMS>(p, M, st);                \
-        case PRO_GATE: return launch<DT, PRO_GATE>(p, M, st);              \
-        case PRO_SWIGLU: return launch<DT, PRO_SWIGLU>(p, M, st);          \
-        case PRO_LAYERNORM: return launch<DT, PRO_LAYERNORM>(p, M, st);    \
-        case PRO_SILU: return launch<DT, PRO_SILU>(p, M, st);              \
-        case PRO_GELU: return launch<DT, PRO_GELU>(p, M, st);              \
-        case PRO_ADALN: return launch<DT, PRO_ADALN>(p, M, st);            \
-        case PRO_LN_MOD: return launch<DT, PRO_LN_MOD>(p, M, st);          \
-        case PRO_LN_AFFINE: return launch<DT, PRO_LN_AFFINE>(p, M, st);    \
-        case PRO_GELU_TANH: return launch<DT, PRO_GELU_TANH>(p, M, st);    \
-        case PRO_SITU:                                                     \
-        case PRO_SITU_FAST: return launch<DT, PRO_SITU_WIDE>(p, M, st);    \
-        default: return -3;                                                \
-    }
-    if (dtype == DT_BF16) { QPRO(DT_BF16) }
-    if (dtype == DT_F32) { QPRO(DT_F32) }
-#undef QPRO
     return -4;
 }
 

@@ -8,12 +8,12 @@
 // again lane-local, then returns to row order for the 16-byte code stores.
 #include "common.hpp"
 #include "convrot.hpp"
+#include "rowmath.hpp"
 
 namespace {
 using namespace convrot;
 
-// MODE_BF16_WIDE: fp32 values quantized with bf16 rounding (a bf16 row whose prologue leaves unrounded fp32 values).
-enum { MODE_BF16 = 0, MODE_F32 = 1, MODE_SD_F16 = 2, MODE_ROT_F32 = 3, MODE_BF16_WIDE = 4 };
+enum { MODE_BF16 = 0, MODE_F32 = 1, MODE_SD_F16 = 2, MODE_ROT_F32 = 3 };
 
 struct QuantArgs {
     const void* x;
@@ -25,6 +25,16 @@ struct QuantArgs {
     int wpr;           // waves per row
     int rpb;           // rows per block
     uint64_t seed;     // nonzero: stochastic rounding keyed by element index + seed (gpu_convrot_requant)
+    // row prologue (csrc/kernels.cu:21-37), PRO kernels only
+    int pro;
+    const void* g;          // GATE: logits [M, g_stride]
+    int64_t g_stride;
+    int64_t up_offset;      // SWIGLU, SITU: column of the second half inside the x row
+    const float* norm_w;    // RMS, LAYERNORM, LN_AFFINE
+    const float* norm_b;    // LN_AFFINE
+    float eps;
+    const void* mod_scale;  // [K] in the row dtype
+    const void* mod_shift;
 };
 
 // csrc/kernels.cu:1355-1359
@@ -79,18 +89,40 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
-template <int MODE, int G, int C>
+// Sum over the waves of one row in fp64, rounded to fp32 once (every wave of the block calls it).
+__device__ __forceinline__ float row_sum_f64(double v, double* red, int wave, int lane, int wpr, int rloc) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    __syncthreads();
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    double t = 0.0;
+    for (int i = 0; i < wpr; ++i) t += red[rloc * wpr + i];
+    return (float)t;
+}
+
+// PRO: the row prologue (csrc/kernels.cu:88-182) runs on the values as they are loaded, with the reference's rounding
+// points; p.pro selects it at run time.  Row sums are fp64, rounded once; the activation functions are correctly rounded.
+template <int MODE, int G, int C, bool PRO>
 __global__ void __launch_bounds__(512) quant_rows_kernel(QuantArgs p) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     __shared__ float red[8];
+    __shared__ double dred[8];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int rloc = wave / p.wpr, wr = wave - rloc * p.wpr;
     const int64_t m = (int64_t)blockIdx.x * p.rpb + rloc;
     const bool row_ok = m < p.M;
     float* wl = lds + wave * kLdsPerWave;
+    constexpr int TD = MODE == MODE_BF16 ? DT_BF16 : DT_F32;            // the row dtype T of the prologue's roundings
+    constexpr int TMODE = MODE == MODE_BF16 ? MODE_BF16 : MODE_F32;     // how a T vector is loaded
+    auto R = [](float x) { return rnd_dt<TD>(x); };
 
     float v[C][16];
     float amax = 0.f;
+    const int pro = PRO ? p.pro : PRO_PLAIN;
+    const bool ln = pro == PRO_LAYERNORM || pro == PRO_LN_MOD || pro == PRO_LN_AFFINE;
+    const bool norm = ln || pro == PRO_RMS || pro == PRO_ADALN;
+    double part = 0.0;
 #pragma unroll
     for (int c = 0; c < C; ++c) {
         const int e0 = (wr + c * p.wpr) * kChunk + lane * 16;
@@ -101,6 +133,96 @@ __global__ void __launch_bounds__(512) quant_rows_kernel(QuantArgs p) {
 #pragma unroll
             for (int i = 0; i < 16; ++i) v[c][i] = 0.f;
         }
+        if (PRO && act) {
+            if (pro == PRO_GATE) {                                                   // csrc/kernels.cu:95-100
+                float gg[16];
+                load16<TMODE>(p.g, m * p.g_stride + e0, gg);
+#pragma unroll
+                for (int i = 0; i < 16; ++i) v[c][i] = R(v[c][i] * R(sigmoid_f(gg[i])));
+            } else if (pro == PRO_SWIGLU || pro == PRO_SITU || pro == PRO_SITU_FAST) {  // :101-112
+                float u[16];
+                load16<TMODE>(p.x, m * p.x_stride + p.up_offset + e0, u);
+                if (pro == PRO_SWIGLU) {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) v[c][i] = R(R(silu_f(v[c][i])) * u[i]);
+                } else {   // one float expression, not rounded to T; the lossy id runs the same accurate form
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) v[c][i] = situ_f(v[c][i], u[i]);
+                }
+            } else if (pro == PRO_SILU) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) v[c][i] = R(silu_f(v[c][i]));
+            } else if (pro == PRO_GELU) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) v[c][i] = R(gelu_f(v[c][i]));
+            } else if (pro == PRO_GELU_TANH) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) v[c][i] = R(gelu_tanh_f(v[c][i]));
+            } else if (ln) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) part += (double)v[c][i];
+            } else if (norm) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) part += (double)v[c][i] * (double)v[c][i];
+            }
+        }
+    }
+    if (PRO && norm) {   // uniform over the block
+        if (ln) {        // :133-145
+            const float mean = row_sum_f64(part, dred, wave, lane, p.wpr, rloc) / (float)p.K;
+            part = 0.0;
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+                const int e0 = (wr + c * p.wpr) * kChunk + lane * 16;
+                if (!(row_ok && e0 < p.K)) continue;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    v[c][i] -= mean;
+                    part += (double)v[c][i] * (double)v[c][i];
+                }
+            }
+        }
+        const float ss = row_sum_f64(part, dred, wave, lane, p.wpr, rloc);
+        const float rstd = (float)(1.0 / sqrt((double)(ss / (float)p.K + p.eps)));   // :148
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const int e0 = (wr + c * p.wpr) * kChunk + lane * 16;
+            if (!(row_ok && e0 < p.K)) continue;
+            float msv[16], shv[16], nw[16], nb[16];
+            const bool mod = p.mod_scale != nullptr;
+            if (mod) {
+                load16<TMODE>(p.mod_scale, e0, msv);
+                load16<TMODE>(p.mod_shift, e0, shv);
+            }
+            if (p.norm_w && (pro == PRO_RMS || pro == PRO_LAYERNORM || pro == PRO_LN_AFFINE)) load16<MODE_F32>(p.norm_w, e0, nw);
+            if (pro == PRO_LN_AFFINE) load16<MODE_F32>(p.norm_b, e0, nb);
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                float n = v[c][i] * rstd;
+                const float a = mod ? msv[i] : 0.f, sh = mod ? shv[i] : 0.f;
+                if (pro == PRO_ADALN) {                                              // :163-166, one rounding
+                    n = R(__builtin_fmaf(n, 1.f + a, sh));
+                } else if (pro == PRO_LN_MOD) {                                      // ln_finish, :40-46
+                    n = R(__builtin_fmaf(R(n), R(1.f + a), sh));
+                } else if (pro == PRO_LN_AFFINE) {
+                    n = R(__builtin_fmaf(n, nw[i], nb[i]));
+                } else {                                                             // RMS, LAYERNORM: :171-179
+                    if (p.norm_w) n *= nw[i];
+                    n = R(n);
+                    if (mod) {
+                        const float aa = R(1.f + a);
+                        n = R(aa * n);
+                        n = R(n + sh);
+                    }
+                }
+                v[c][i] = n;
+            }
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+        const int e0 = (wr + c * p.wpr) * kChunk + lane * 16;
+        const bool act = row_ok && e0 < p.K;
         if (G != 0) rotate_chunk<G>(v[c], wl, lane);
         if (MODE == MODE_ROT_F32) {
             if (act) {
@@ -132,7 +254,7 @@ __global__ void __launch_bounds__(512) quant_rows_kernel(QuantArgs p) {
         scale = fmaxf(amax, 1e-30f) / 127.f;                       // csrc/sd.cu:589
         const float sh = rnd_dt<DT_F16>(scale);
         st = sh > 0.f ? sh : scale;                                // :593
-    } else if (MODE == MODE_BF16 || MODE == MODE_BF16_WIDE) {
+    } else if (MODE == MODE_BF16) {
         scale = fmaxf(fminf(amax, 3.38953139e38f) * (1.f / 127.f), 1.0e-30f);  // csrc/kernels.cu:241
         st = rnd_dt<DT_BF16>(scale);
         rinv = __builtin_amdgcn_rcpf(st);
@@ -154,7 +276,7 @@ __global__ void __launch_bounds__(512) quant_rows_kernel(QuantArgs p) {
             for (int j = 0; j < 4; ++j) {
                 const float x = v[c][4 * i + j];
                 float t;
-                if (MODE == MODE_BF16 || MODE == MODE_BF16_WIDE) {
+                if (MODE == MODE_BF16) {
                     // Both operands carry 8 significant bits, so their exact quotient is never closer than 2^-17
                     // (relative) to a bf16 rounding boundary: a 1-ulp reciprocal times the numerator rounds to the
                     // same bf16 value as the IEEE quotient does.
@@ -185,7 +307,11 @@ template <int MODE, int G, int C>
 int launch(const QuantArgs& a, int nw, hipStream_t st) {
     const int grid = (a.M + a.rpb - 1) / a.rpb;
     const size_t smem = G ? (size_t)nw * kLdsPerWave * sizeof(float) : 0;
-    hipLaunchKernelGGL((quant_rows_kernel<MODE, G, C>), dim3(grid), dim3(nw * 64), smem, st, a);
+    constexpr bool CAN_PRO = MODE == MODE_BF16 || MODE == MODE_F32 || MODE == MODE_ROT_F32;
+    if (CAN_PRO && a.pro != PRO_PLAIN)
+        hipLaunchKernelGGL((quant_rows_kernel<MODE, G, C, CAN_PRO>), dim3(grid), dim3(nw * 64), smem, st, a);
+    else
+        hipLaunchKernelGGL((quant_rows_kernel<MODE, G, C, false>), dim3(grid), dim3(nw * 64), smem, st, a);
     KCHECK();
     return 0;
 }
@@ -215,7 +341,7 @@ int run_quant(QuantArgs a, int g, hipStream_t st) {
     switch (g) {
         case 0: return launch_c<MODE, 0>(a, nw, C, st);
         case 64: return launch_c<MODE, 64>(a, nw, C, st);
-        case 128: if (MODE == MODE_SD_F16 || MODE == MODE_ROT_F32) return -1; return launch_c<MODE == MODE_F32 || MODE == MODE_BF16 || MODE == MODE_BF16_WIDE ? MODE : MODE_BF16, 128>(a, nw, C, st);
+        case 128: if (MODE == MODE_SD_F16 || MODE == MODE_ROT_F32) return -1; return launch_c<MODE == MODE_F32 || MODE == MODE_BF16 ? MODE : MODE_BF16, 128>(a, nw, C, st);
         default: return launch_c<MODE, 256>(a, nw, C, st);
     }
 }
@@ -224,31 +350,6 @@ int rotate_group(int rotate) { return rotate == 0 ? 0 : (rotate == 64 || rotate 
 
 bool known_prologue(int p) { return p >= PRO_PLAIN && p <= PRO_SITU_FAST && p != PRO_LN_AFFINE_SILU; }
 
-}  // namespace
-
-// The non-PLAIN prologues run as a separate kernel (prologue_rows.hip) into a stream-ordered T[M, K] buffer that the
-// plain quantizer then reads: every prologue ends on a rounding to T, so this is bit-identical to the fused form.
-extern "C" int gpu_internal_quant_prologue(int dtype, int prologue, const void* x, int64_t x_stride, const void* g,
-                                           int64_t g_stride, int64_t up_offset, const float* norm_w, const float* norm_b,
-                                           float eps, const void* mod_scale, const void* mod_shift, void* out, int M, int K,
-                                           void* stream);
-
-namespace {
-template <class F>
-int with_prologue(int dtype, int prologue, const void* x, int64_t x_stride, const void* g, int64_t g_stride,
-                  int64_t up_offset, const float* norm_w, const float* norm_b, float eps, const void* mod_scale,
-                  const void* mod_shift, int M, int K, hipStream_t st, F&& quantize) {
-    if (M <= 0) return 0;
-    void* rows = nullptr;
-    const bool wide = prologue == PRO_SITU || prologue == PRO_SITU_FAST;   // these leave fp32 values
-    hipError_t e = hipMallocAsync(&rows, (size_t)M * K * (dtype == DT_F32 || wide ? 4 : 2), st);
-    if (e != hipSuccess) return (int)e;
-    int rc = gpu_internal_quant_prologue(dtype, prologue, x, x_stride, g, g_stride, up_offset, norm_w, norm_b, eps, mod_scale,
-                                         mod_shift, rows, M, K, st);
-    if (rc == 0) rc = quantize(rows);
-    e = hipFreeAsync(rows, st);
-    return rc == 0 && e != hipSuccess ? (int)e : rc;
-}
 }  // namespace
 
 GPU_API int gpu_quant_rows(int dtype, int prologue, const void* x, int64_t x_stride, const void* g, int64_t g_stride,
@@ -260,19 +361,9 @@ GPU_API int gpu_quant_rows(int dtype, int prologue, const void* x, int64_t x_str
     if (dtype != DT_BF16 && dtype != DT_F32) return -4;
     if (!known_prologue(prologue)) return -3;   // the id list of csrc/kernels.cu:280-292
     if (K > 32768) return -2;
-    hipStream_t st = (hipStream_t)stream;
-    auto quantize = [&](const void* rows, int64_t stride, bool wide) {
-        QuantArgs a{rows, stride, q, scales, nullptr, M, K, 1, 1};
-        return dtype == DT_F32 ? run_quant<MODE_F32>(a, grp, st)
-                               : wide ? run_quant<MODE_BF16_WIDE>(a, grp, st) : run_quant<MODE_BF16>(a, grp, st);
-    };
-    if (prologue == PRO_PLAIN) return quantize(x, x_stride, false);
-    // PRO_SITU is one float expression whose value is not rounded to T before the quantizer (csrc/kernels.cu:112): its row
-    // buffer is fp32.  PRO_SITU_FAST, defined by NVIDIA's approximate tanh / exp / divide (csrc/common.cuh:88-90, "about
-    // 2^-11 relative error"), runs the same accurate expression.
-    const bool wide = prologue == PRO_SITU || prologue == PRO_SITU_FAST;
-    return with_prologue(dtype, prologue, x, x_stride, g, g_stride, up_offset, norm_w, nullptr, eps, mod_scale, mod_shift, M, K,
-                         st, [&](const void* rows) { return quantize(rows, K, wide); });
+    QuantArgs a{x, x_stride, q, scales, nullptr, M, K, 1, 1, 0, prologue, g, g_stride, up_offset, norm_w, nullptr, eps, mod_scale,
+                mod_shift};
+    return dtype == DT_BF16 ? run_quant<MODE_BF16>(a, grp, (hipStream_t)stream) : run_quant<MODE_F32>(a, grp, (hipStream_t)stream);
 }
 
 GPU_API int gpu_quant_rows_b(int dtype, int prologue, const void* x, int64_t x_stride, const float* norm_w,
@@ -283,13 +374,8 @@ GPU_API int gpu_quant_rows_b(int dtype, int prologue, const void* x, int64_t x_s
     if (prologue != PRO_LN_MOD && prologue != PRO_LN_AFFINE) return -3;
     if (K <= 0) return -1;
     if (K > 32768) return -2;
-    hipStream_t st = (hipStream_t)stream;
-    const int grp = rotate_group(rotate);
-    return with_prologue(dtype, prologue, x, x_stride, nullptr, 0, 0, norm_w, norm_b, eps, mod_scale, mod_shift, M, K, st,
-                         [&](const void* rows) {
-                             QuantArgs a{rows, K, q, scales, nullptr, M, K, 1, 1};
-                             return run_quant<MODE_BF16>(a, grp, st);
-                         });
+    QuantArgs a{x, x_stride, q, scales, nullptr, M, K, 1, 1, 0, prologue, nullptr, 0, 0, norm_w, norm_b, eps, mod_scale, mod_shift};
+    return run_quant<MODE_BF16>(a, rotate_group(rotate), (hipStream_t)stream);
 }
 
 GPU_API int gpu_rotate_rows_f32(int prologue, const float* x, int64_t x_stride, int64_t up_offset, const float* norm_w,
@@ -297,16 +383,9 @@ GPU_API int gpu_rotate_rows_f32(int prologue, const float* x, int64_t x_stride, 
     if (K <= 0 || (K % 256) != 0) return -1;
     if (prologue != PRO_PLAIN && prologue != PRO_RMS && prologue != PRO_SWIGLU) return -3;
     if (K > 32768) return -2;
-    hipStream_t st = (hipStream_t)stream;
-    if (prologue == PRO_PLAIN) {
-        QuantArgs a{x, x_stride, nullptr, nullptr, out, M, K, 1, 1};
-        return run_quant<MODE_ROT_F32>(a, 256, st);
-    }
-    return with_prologue(DT_F32, prologue, x, x_stride, nullptr, 0, up_offset, norm_w, nullptr, eps, nullptr, nullptr, M, K, st,
-                         [&](const void* rows) {
-                             QuantArgs a{rows, K, nullptr, nullptr, out, M, K, 1, 1};
-                             return run_quant<MODE_ROT_F32>(a, 256, st);
-                         });
+    QuantArgs a{x, x_stride, nullptr, nullptr, out, M, K, 1, 1, 0, prologue, nullptr, 0, up_offset, norm_w, nullptr, eps, nullptr,
+                nullptr};
+    return run_quant<MODE_ROT_F32>(a, 256, (hipStream_t)stream);
 }
 
 GPU_API int gpu_sd_quant_rows(const void* x, int64_t x_stride, int8_t* q, float* scales, int M, int K, int rotate,

@@ -40,11 +40,10 @@ enum {
  * group (an extension: the reference treats the argument as a flag).  K must be a multiple of 256 (of 64 when
  * rotate is 0 or 64, of 128 when rotate is 128).
  * Prologues (x, g, up_offset, norm_w, eps, mod_scale, mod_shift as in QuantParams, csrc/kernels.cu:21-37): all ids of
- * csrc/kernels.cu:280-292.  A non-PLAIN prologue runs as a kernel of its own into a stream-ordered [M, K] row buffer: of
- * type T for the prologues that end on a rounding to T (all but the two below), so codes and scales are those of the
- * fused form; of unrounded fp32 values for PRO_SITU, as its fused form hands them on.  PRO_SITU_FAST, which the reference
- * defines through NVIDIA's approximate tanh/exp/divide (about 2^-11 relative error), runs PRO_SITU's accurate expression.  Row sums are accumulated in fp64 and exp / erf / tanh / 1/sqrt are correctly rounded, where the reference has
- * fp32 sums in the order of its thread layout and CUDA's 1-2 ulp routines. */
+ * csrc/kernels.cu:280-292, applied inside the quantizer kernel with the reference's rounding points.  Row sums are
+ * accumulated in fp64 and rounded once, exp / erf / tanh / 1/sqrt are correctly rounded (the reference has fp32 sums in the
+ * order of its thread layout and CUDA's 1-2 ulp routines).  PRO_SITU_FAST, which the reference defines through NVIDIA's
+ * approximate tanh/exp/divide (about 2^-11 relative error), runs PRO_SITU's accurate expression. */
 int gpu_quant_rows(int dtype, int prologue, const void* x, int64_t x_stride, const void* g, int64_t g_stride,
                    int64_t up_offset, const float* norm_w, float eps, const void* mod_scale, const void* mod_shift,
                    int8_t* q, float* scales, int M, int K, int rotate, void* stream);
