@@ -162,7 +162,7 @@ def time_row_kernels(torch, ffi, steps):
     ss = torch.empty((Ms,), dtype=torch.float32, device=dev)
     timed("gpu_sd_quant_rows rotate 64, M=8192 K=2560 f16", Ms * I * 3,
           lambda: ffi.k("gpu_sd_quant_rows", xg.data_ptr(), 2 * I, qs.data_ptr(), ss.data_ptr(), Ms, I, 64, s))
-    timed("gpu_sd_geglu_quant_rows rotate 64, M=8192 I=2560 (source kernel + quantizer)", Ms * I * 5,
+    timed("gpu_sd_geglu_quant_rows rotate 64, M=8192 I=2560", Ms * I * 5,
           lambda: ffi.k("gpu_sd_geglu_quant_rows", xg.data_ptr(), qs.data_ptr(), ss.data_ptr(), Ms, I, 64, s))
     N = 12288
     wq = torch.randint(-127, 128, (N, K), dtype=torch.int8, device=dev, generator=g)

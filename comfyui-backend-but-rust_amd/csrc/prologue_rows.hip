@@ -13,6 +13,7 @@
 // One workgroup per row.
 #include "common.hpp"
 #include "rowmath.hpp"
+#include "act_tables.hpp"
 
 namespace {
 
@@ -30,6 +31,7 @@ struct ProArgs {
     void* out;
     int64_t out_stride;
     int K;
+    ActTables tab;   // activation tables for bf16 rows (null members: evaluate per element)
 };
 
 template <int PRO> __device__ __forceinline__ constexpr bool is_ln() {
@@ -57,6 +59,11 @@ __global__ void __launch_bounds__(256) prologue_rows_kernel(ProArgs p) {
     const uint8_t* x = (const uint8_t*)p.x + m * p.x_stride * SZ;
     uint8_t* o = (uint8_t*)p.out + m * p.out_stride * SZ;
     auto R = [](float v) { return rnd_dt<DT>(v); };
+    // rnd(f(x)) of a bf16 value through the table of all 65536 inputs, when it is there
+    auto via = [](const uint16_t* tab, float v, auto f) {
+        if (DT == DT_BF16 && tab) return bf16_to_f(tab[f2u(v) >> 16]);
+        return rnd_dt<DT>(f(v));
+    };
     if (PRO == PRO_RMS || is_ln<PRO>() || PRO == PRO_ADALN) {
         float mean = 0.f;
         if (is_ln<PRO>()) {
@@ -97,16 +104,16 @@ __global__ void __launch_bounds__(256) prologue_rows_kernel(ProArgs p) {
         }
     } else if (PRO == PRO_GATE) {                                         // :108-113
         const uint8_t* g = (const uint8_t*)p.g + m * p.g_stride * SZ;
-        for (int k = threadIdx.x; k < K; k += blockDim.x) st_dt<DT>(o, k, ld_dt<DT>(x, k) * R(sigmoid_f(ld_dt<DT>(g, k))));
+        for (int k = threadIdx.x; k < K; k += blockDim.x) st_dt<DT>(o, k, ld_dt<DT>(x, k) * via(p.tab.sigmoid_bf16, ld_dt<DT>(g, k), [](float t) { return sigmoid_f(t); }));
     } else if (PRO == PRO_SWIGLU) {                                       // :114-119
         for (int k = threadIdx.x; k < K; k += blockDim.x)
-            st_dt<DT>(o, k, R(silu_f(ld_dt<DT>(x, k))) * ld_dt<DT>(x, p.up_offset + k));
+            st_dt<DT>(o, k, via(p.tab.silu_bf16, ld_dt<DT>(x, k), [](float t) { return silu_f(t); }) * ld_dt<DT>(x, p.up_offset + k));
     } else if (PRO == PRO_SILU) {
-        for (int k = threadIdx.x; k < K; k += blockDim.x) st_dt<DT>(o, k, silu_f(ld_dt<DT>(x, k)));
+        for (int k = threadIdx.x; k < K; k += blockDim.x) st_dt<DT>(o, k, via(p.tab.silu_bf16, ld_dt<DT>(x, k), [](float t) { return silu_f(t); }));
     } else if (PRO == PRO_GELU) {
-        for (int k = threadIdx.x; k < K; k += blockDim.x) st_dt<DT>(o, k, gelu_f(ld_dt<DT>(x, k)));
+        for (int k = threadIdx.x; k < K; k += blockDim.x) st_dt<DT>(o, k, via(p.tab.gelu_bf16, ld_dt<DT>(x, k), [](float t) { return gelu_f(t); }));
     } else if (PRO == PRO_GELU_TANH) {
-        for (int k = threadIdx.x; k < K; k += blockDim.x) st_dt<DT>(o, k, gelu_tanh_f(ld_dt<DT>(x, k)));
+        for (int k = threadIdx.x; k < K; k += blockDim.x) st_dt<DT>(o, k, via(p.tab.gelu_tanh_bf16, ld_dt<DT>(x, k), [](float t) { return gelu_tanh_f(t); }));
     } else if (PRO == PRO_SITU) {                                         // csrc/kernels.cu:409-417, the eager chain
         for (int k = threadIdx.x; k < K; k += blockDim.x) {
             const float hidden = ld_dt<DT>(x, k), gate = ld_dt<DT>(x, p.up_offset + k);
@@ -117,61 +124,6 @@ __global__ void __launch_bounds__(256) prologue_rows_kernel(ProArgs p) {
         }
     } else {
         for (int k = threadIdx.x; k < K; k += blockDim.x) st_dt<DT>(o, k, ld_dt<DT>(x, k));
-    }
-}
-
-// ---------------------------------------------------------------------------------------------------------------------
-// The SD UNet's fused quantizer sources (csrc/sd.cu:611-663): the half row another kernel would have written -- LayerNorm,
-// GEGLU, head un-padding, GroupNorm -- which the fp16 quantizer then reads.  Same two choices as above for sums and 1/sqrt.
-// ---------------------------------------------------------------------------------------------------------------------
-enum { SDQ_LN = 1, SDQ_GEGLU = 2, SDQ_UNPAD = 3, SDQ_GN = 4 };
-struct SdSrc {
-    const uint16_t* x;
-    int64_t x_stride;     // LN: elements between rows
-    const float* w;       // LN, GN
-    const float* b;
-    float eps;            // LN
-    int heads, d, dp;     // UNPAD: heads of d values, each stored dp wide
-    const float2* stats;  // GN: (mean, rstd) of group ng at stats[2 * ng], the layout csrc/sd.cu:203-207 leaves
-    int groups;
-    int64_t P;            // GN: pixels per image
-    uint16_t* out;        // half rows [M, K]
-    int K;
-};
-
-template <int MODE>
-__global__ void __launch_bounds__(256) sd_source_rows_kernel(SdSrc p) {
-    __shared__ double red[4];
-    const int K = p.K;
-    const int64_t m = blockIdx.x;
-    uint16_t* o = p.out + m * K;
-    if (MODE == SDQ_LN) {                                                 // csrc/sd.cu:629-641
-        const uint16_t* r = p.x + m * p.x_stride;
-        double s = 0.0;
-        for (int k = threadIdx.x; k < K; k += blockDim.x) s += (double)f16_to_f(r[k]);
-        const float mean = block_sum_f64(s, red) / (float)K;
-        double s2 = 0.0;
-        for (int k = threadIdx.x; k < K; k += blockDim.x) {
-            const float d = f16_to_f(r[k]) - mean;
-            s2 += (double)d * (double)d;
-        }
-        const float rstd = (float)(1.0 / sqrt((double)(block_sum_f64(s2, red) / (float)K + p.eps)));
-        for (int k = threadIdx.x; k < K; k += blockDim.x)
-            o[k] = f_to_f16(__builtin_fmaf((f16_to_f(r[k]) - mean) * rstd, p.w[k], p.b[k]));
-    } else if (MODE == SDQ_GEGLU) {                                       // :642-649: [M, 2K] value then gate
-        const uint16_t* r = p.x + m * 2 * K;
-        for (int k = threadIdx.x; k < K; k += blockDim.x)
-            o[k] = f_to_f16(f16_to_f(r[k]) * rnd_dt<DT_F16>(gelu_f(f16_to_f(r[K + k]))));
-    } else if (MODE == SDQ_UNPAD) {                                       // :650-652
-        const uint16_t* r = p.x + m * p.heads * p.dp;
-        for (int k = threadIdx.x; k < K; k += blockDim.x) o[k] = r[(k / p.d) * p.dp + k % p.d];
-    } else {                                                              // :653-662: row m is a pixel of image m / P
-        const uint16_t* r = p.x + m * K;
-        const int n = (int)(m / p.P);
-        for (int c = threadIdx.x; c < K; c += blockDim.x) {
-            const float2 st = p.stats[(n * p.groups + c / (K / p.groups)) * 2];
-            o[c] = f_to_f16(__builtin_fmaf((f16_to_f(r[c]) - st.x) * st.y, p.w[c], p.b[c]));
-        }
     }
 }
 
@@ -214,7 +166,10 @@ int launch(const ProArgs& p, int M, hipStream_t st) {
 }
 
 template <int DT>
-int dispatch(int prologue, const ProArgs& p, int M, hipStream_t st, bool b_variant) {
+int dispatch(int prologue, ProArgs p, int M, hipStream_t st, bool b_variant) {
+    if (DT == DT_BF16 && M > 0 &&
+        (prologue == PRO_GATE || prologue == PRO_SWIGLU || prologue == PRO_SILU || prologue == PRO_GELU || prologue == PRO_GELU_TANH))
+        if (const ActTables* t = act_tables()) p.tab = *t;
     switch (prologue) {
         case PRO_PLAIN: return launch<DT, PRO_PLAIN>(p, M, st);
         case PRO_RMS: return b_variant ? -3 : launch<DT, PRO_RMS>(p, M, st);
@@ -256,25 +211,12 @@ GPU_API int gpu_prologue_rows_b(int dtype, int prologue, const void* x, int64_t 
     return -4;
 }
 
-// The SD fused sources into a half row buffer [M, K] (mode: 1 LN, 2 GEGLU, 3 UNPAD, 4 GN; for GN `stats` is the caller's
-// `sums` scratch, filled here first).
-extern "C" int gpu_internal_sd_source(int mode, const void* x, int64_t x_stride, const float* w, const float* b, float eps,
-                                      int heads, int d, int dp, void* stats, int groups, int64_t P, int n_images, void* out,
-                                      int M, int K, void* stream) {
-    if (M <= 0) return 0;
-    hipStream_t st = (hipStream_t)stream;
-    SdSrc p{(const uint16_t*)x, x_stride, w, b, eps, heads, d, dp, (const float2*)stats, groups, P, (uint16_t*)out, K};
-    switch (mode) {
-        case SDQ_LN: hipLaunchKernelGGL(sd_source_rows_kernel<SDQ_LN>, dim3((unsigned)M), dim3(256), 0, st, p); break;
-        case SDQ_GEGLU: hipLaunchKernelGGL(sd_source_rows_kernel<SDQ_GEGLU>, dim3((unsigned)M), dim3(256), 0, st, p); break;
-        case SDQ_UNPAD: hipLaunchKernelGGL(sd_source_rows_kernel<SDQ_UNPAD>, dim3((unsigned)M), dim3(256), 0, st, p); break;
-        case SDQ_GN:
-            hipLaunchKernelGGL(sd_group_stats_kernel, dim3((unsigned)(n_images * groups)), dim3(256), 0, st, (const uint16_t*)x,
-                               (float2*)stats, P, K, groups, eps);
-            hipLaunchKernelGGL(sd_source_rows_kernel<SDQ_GN>, dim3((unsigned)M), dim3(256), 0, st, p);
-            break;
-        default: return -3;
-    }
+// GroupNorm statistics for gpu_sd_group_norm_quant_rows: (mean, rstd) of group ng as two floats at stats + 16 * ng bytes,
+// the layout csrc/sd.cu:203-207 leaves.
+extern "C" int gpu_internal_sd_group_stats(const void* x, void* stats, int n_images, int64_t P, int C, int G, float eps,
+                                           void* stream) {
+    hipLaunchKernelGGL(sd_group_stats_kernel, dim3((unsigned)(n_images * G)), dim3(256), 0, (hipStream_t)stream,
+                       (const uint16_t*)x, (float2*)stats, P, C, G, eps);
     KCHECK();
     return 0;
 }

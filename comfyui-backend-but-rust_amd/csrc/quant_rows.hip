@@ -9,6 +9,7 @@
 #include "common.hpp"
 #include "convrot.hpp"
 #include "rowmath.hpp"
+#include "act_tables.hpp"
 
 namespace {
 using namespace convrot;
@@ -35,7 +36,13 @@ struct QuantArgs {
     float eps;
     const void* mod_scale;  // [K] in the row dtype
     const void* mod_shift;
+    int d, dp;              // PRO_SD_UNPAD: heads of d values, each stored dp wide
+    int per;                // PRO_SD_GN: channels per group; g holds the (mean, rstd) pairs, g_stride the pixels per image
+    ActTables tab;          // activation tables for 16-bit rows (null members: evaluate per element)
 };
+
+// Sources of the SD UNet's fused quantizers (csrc/sd.cu:611-663), fp16 rows only.  Its LayerNorm source is PRO_LN_AFFINE.
+enum { PRO_SD_GEGLU = 101, PRO_SD_UNPAD = 102, PRO_SD_GN = 103 };
 
 // csrc/kernels.cu:1355-1359
 __device__ __forceinline__ uint32_t pcg_hash(uint32_t x) {
@@ -113,9 +120,15 @@ __global__ void __launch_bounds__(512) quant_rows_kernel(QuantArgs p) {
     const int64_t m = (int64_t)blockIdx.x * p.rpb + rloc;
     const bool row_ok = m < p.M;
     float* wl = lds + wave * kLdsPerWave;
-    constexpr int TD = MODE == MODE_BF16 ? DT_BF16 : DT_F32;            // the row dtype T of the prologue's roundings
-    constexpr int TMODE = MODE == MODE_BF16 ? MODE_BF16 : MODE_F32;     // how a T vector is loaded
+    // the row dtype T of the prologue's roundings, and how a T vector is loaded
+    constexpr int TD = MODE == MODE_BF16 ? DT_BF16 : MODE == MODE_SD_F16 ? DT_F16 : DT_F32;
+    constexpr int TMODE = MODE == MODE_BF16 ? MODE_BF16 : MODE == MODE_SD_F16 ? MODE_SD_F16 : MODE_F32;
     auto R = [](float x) { return rnd_dt<TD>(x); };
+    // rnd(f(x)) of a bf16 value x through a table of all 65536 inputs, when the table is there
+    auto via = [](const uint16_t* tab, float x, auto f) {
+        if (MODE == MODE_BF16 && tab) return bf16_to_f(tab[f2u(x) >> 16]);
+        return rnd_dt<TD>(f(x));
+    };
 
     float v[C][16];
     float amax = 0.f;
@@ -127,37 +140,71 @@ __global__ void __launch_bounds__(512) quant_rows_kernel(QuantArgs p) {
     for (int c = 0; c < C; ++c) {
         const int e0 = (wr + c * p.wpr) * kChunk + lane * 16;
         const bool act = row_ok && e0 < p.K;
-        if (act) {
+        if (PRO && MODE == MODE_SD_F16 && pro == PRO_SD_UNPAD) {                     // csrc/sd.cu:650-652
+            const uint16_t* r = (const uint16_t*)p.x + m * p.x_stride;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int k = e0 + i;
+                v[c][i] = act ? f16_to_f(r[(k / p.d) * p.dp + k % p.d]) : 0.f;
+            }
+        } else if (act) {
             load16<MODE>(p.x, m * p.x_stride + e0, v[c]);
         } else {
 #pragma unroll
             for (int i = 0; i < 16; ++i) v[c][i] = 0.f;
         }
         if (PRO && act) {
-            if (pro == PRO_GATE) {                                                   // csrc/kernels.cu:95-100
+            if (MODE == MODE_SD_F16) {
+                if (pro == PRO_SD_GEGLU) {                                           // :642-649, row = [value | gate]
+                    float gg[16];
+                    load16<TMODE>(p.x, m * p.x_stride + p.up_offset + e0, gg);
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const float gl = p.tab.gelu_f16 ? f16_to_f(p.tab.gelu_f16[f_to_f16(gg[i])]) : R(gelu_f(gg[i]));
+                        v[c][i] = R(v[c][i] * gl);
+                    }
+                } else if (pro == PRO_SD_GN) {                                       // :653-662
+                    const float2* stats = (const float2*)p.g + (m / p.g_stride) * (int64_t)(p.K / p.per) * 2;
+                    float nw[16], nb[16];
+                    load16<MODE_F32>(p.norm_w, e0, nw);
+                    load16<MODE_F32>(p.norm_b, e0, nb);
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const float2 st = stats[((e0 + i) / p.per) * 2];
+                        v[c][i] = R(__builtin_fmaf((v[c][i] - st.x) * st.y, nw[i], nb[i]));
+                    }
+                } else if (ln) {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) part += (double)v[c][i];
+                }
+            } else if (pro == PRO_GATE) {                                            // csrc/kernels.cu:95-100
                 float gg[16];
                 load16<TMODE>(p.g, m * p.g_stride + e0, gg);
 #pragma unroll
-                for (int i = 0; i < 16; ++i) v[c][i] = R(v[c][i] * R(sigmoid_f(gg[i])));
+                for (int i = 0; i < 16; ++i) v[c][i] = R(v[c][i] * via(p.tab.sigmoid_bf16, gg[i], [](float x) { return sigmoid_f(x); }));
             } else if (pro == PRO_SWIGLU || pro == PRO_SITU || pro == PRO_SITU_FAST) {  // :101-112
                 float u[16];
                 load16<TMODE>(p.x, m * p.x_stride + p.up_offset + e0, u);
                 if (pro == PRO_SWIGLU) {
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) v[c][i] = R(R(silu_f(v[c][i])) * u[i]);
+                    for (int i = 0; i < 16; ++i) v[c][i] = R(via(p.tab.silu_bf16, v[c][i], [](float x) { return silu_f(x); }) * u[i]);
+                } else if (MODE == MODE_BF16 && p.tab.situ_gate_bf16) {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i)
+                        v[c][i] = p.tab.situ_gate_bf16[f2u(u[i]) >> 16] * p.tab.situ_hidden_bf16[f2u(v[c][i]) >> 16];
                 } else {   // one float expression, not rounded to T; the lossy id runs the same accurate form
 #pragma unroll
                     for (int i = 0; i < 16; ++i) v[c][i] = situ_f(v[c][i], u[i]);
                 }
             } else if (pro == PRO_SILU) {
 #pragma unroll
-                for (int i = 0; i < 16; ++i) v[c][i] = R(silu_f(v[c][i]));
+                for (int i = 0; i < 16; ++i) v[c][i] = via(p.tab.silu_bf16, v[c][i], [](float x) { return silu_f(x); });
             } else if (pro == PRO_GELU) {
 #pragma unroll
-                for (int i = 0; i < 16; ++i) v[c][i] = R(gelu_f(v[c][i]));
+                for (int i = 0; i < 16; ++i) v[c][i] = via(p.tab.gelu_bf16, v[c][i], [](float x) { return gelu_f(x); });
             } else if (pro == PRO_GELU_TANH) {
 #pragma unroll
-                for (int i = 0; i < 16; ++i) v[c][i] = R(gelu_tanh_f(v[c][i]));
+                for (int i = 0; i < 16; ++i) v[c][i] = via(p.tab.gelu_tanh_bf16, v[c][i], [](float x) { return gelu_tanh_f(x); });
             } else if (ln) {
 #pragma unroll
                 for (int i = 0; i < 16; ++i) part += (double)v[c][i];
@@ -307,7 +354,7 @@ template <int MODE, int G, int C>
 int launch(const QuantArgs& a, int nw, hipStream_t st) {
     const int grid = (a.M + a.rpb - 1) / a.rpb;
     const size_t smem = G ? (size_t)nw * kLdsPerWave * sizeof(float) : 0;
-    constexpr bool CAN_PRO = MODE == MODE_BF16 || MODE == MODE_F32 || MODE == MODE_ROT_F32;
+    constexpr bool CAN_PRO = true;
     if (CAN_PRO && a.pro != PRO_PLAIN)
         hipLaunchKernelGGL((quant_rows_kernel<MODE, G, C, CAN_PRO>), dim3(grid), dim3(nw * 64), smem, st, a);
     else
@@ -346,6 +393,14 @@ int run_quant(QuantArgs a, int g, hipStream_t st) {
     }
 }
 
+// The activation tables, for the prologues that evaluate exp / erf / tanh on a 16-bit row.
+void attach_tables(QuantArgs& a) {
+    const int p = a.pro;
+    if (p == PRO_GATE || p == PRO_SWIGLU || p == PRO_SITU || p == PRO_SITU_FAST || p == PRO_SILU || p == PRO_GELU || p == PRO_GELU_TANH ||
+        p == PRO_SD_GEGLU)
+        if (const ActTables* t = act_tables()) a.tab = *t;
+}
+
 int rotate_group(int rotate) { return rotate == 0 ? 0 : (rotate == 64 || rotate == 128) ? rotate : 256; }
 
 bool known_prologue(int p) { return p >= PRO_PLAIN && p <= PRO_SITU_FAST && p != PRO_LN_AFFINE_SILU; }
@@ -363,6 +418,7 @@ GPU_API int gpu_quant_rows(int dtype, int prologue, const void* x, int64_t x_str
     if (K > 32768) return -2;
     QuantArgs a{x, x_stride, q, scales, nullptr, M, K, 1, 1, 0, prologue, g, g_stride, up_offset, norm_w, nullptr, eps, mod_scale,
                 mod_shift};
+    if (dtype == DT_BF16 && M > 0) attach_tables(a);
     return dtype == DT_BF16 ? run_quant<MODE_BF16>(a, grp, (hipStream_t)stream) : run_quant<MODE_F32>(a, grp, (hipStream_t)stream);
 }
 
@@ -398,49 +454,46 @@ GPU_API int gpu_sd_quant_rows(const void* x, int64_t x_stride, int8_t* q, float*
 }
 
 // The SD UNet's fused quantizers (csrc/sd.cu:608-724): the half row of LayerNorm / GEGLU / head un-padding / GroupNorm,
-// then gpu_sd_quant_rows of it.  The row is written to a stream-ordered buffer by a kernel of its own; it is rounded to
-// half in the reference too, so codes and scales are those of the one-kernel form.
-extern "C" int gpu_internal_sd_source(int mode, const void* x, int64_t x_stride, const float* w, const float* b, float eps,
-                                      int heads, int d, int dp, void* stats, int groups, int64_t P, int n_images, void* out,
-                                      int M, int K, void* stream);
+// computed on the values as the fp16 quantizer loads them; it is rounded to half there as in the reference.
+extern "C" int gpu_internal_sd_group_stats(const void* x, void* stats, int n_images, int64_t P, int C, int G, float eps,
+                                           void* stream);
 namespace {
-int sd_quant_src(int mode, const void* x, int64_t x_stride, const float* w, const float* b, float eps, int heads, int d, int dp,
-                 void* stats, int groups, int64_t P, int n_images, int8_t* q, float* scales, int M, int K, int rotate,
-                 hipStream_t st) {
-    if ((rotate != 0 && rotate != 64 && rotate != 256) || (rotate && K % rotate)) return -1;   // csrc/sd.cu:682
-    if (K <= 0 || (K % 16) != 0) return -1;
-    if (K > 32768) return -2;
-    if (M <= 0) return 0;
-    void* rows = nullptr;
-    hipError_t e = hipMallocAsync(&rows, (size_t)M * K * 2, st);
-    if (e != hipSuccess) return (int)e;
-    int rc = gpu_internal_sd_source(mode, x, x_stride, w, b, eps, heads, d, dp, stats, groups, P, n_images, rows, M, K, st);
-    if (rc == 0) {
-        QuantArgs a{rows, K, q, scales, nullptr, M, K, 1, 1};
-        rc = run_quant<MODE_SD_F16>(a, rotate, st);
-    }
-    e = hipFreeAsync(rows, st);
-    return rc == 0 && e != hipSuccess ? (int)e : rc;
+int sd_fused(QuantArgs a, int rotate, hipStream_t st) {
+    if ((rotate != 0 && rotate != 64 && rotate != 256) || (rotate && a.K % rotate)) return -1;   // csrc/sd.cu:682
+    if (a.K <= 0 || (a.K % 16) != 0) return -1;
+    if (a.K > 32768) return -2;
+    if (a.M <= 0) return 0;
+    attach_tables(a);
+    return run_quant<MODE_SD_F16>(a, rotate, st);
 }
 }  // namespace
 
 GPU_API int gpu_sd_ln_quant_rows(const void* x, int64_t x_stride, const float* w, const float* b, float eps, int8_t* q,
                                  float* scales, int M, int K, int rotate, void* stream) {
-    return sd_quant_src(1, x, x_stride, w, b, eps, 0, 0, 0, nullptr, 0, 0, 0, q, scales, M, K, rotate, (hipStream_t)stream);
+    QuantArgs a{x, x_stride, q, scales, nullptr, M, K, 1, 1, 0, PRO_LN_AFFINE, nullptr, 0, 0, w, b, eps, nullptr, nullptr};
+    return sd_fused(a, rotate, (hipStream_t)stream);
 }
 GPU_API int gpu_sd_geglu_quant_rows(const void* in, int8_t* q, float* scales, int M, int I, int rotate, void* stream) {
-    return sd_quant_src(2, in, 0, nullptr, nullptr, 0.f, 0, 0, 0, nullptr, 0, 0, 0, q, scales, M, I, rotate, (hipStream_t)stream);
+    QuantArgs a{in, 2 * (int64_t)I, q, scales, nullptr, M, I, 1, 1, 0, PRO_SD_GEGLU, nullptr, 0, I, nullptr, nullptr, 0.f, nullptr,
+                nullptr};
+    return sd_fused(a, rotate, (hipStream_t)stream);
 }
 GPU_API int gpu_sd_unpad_quant_rows(const void* src, int8_t* q, float* scales, int M, int H, int d, int dp, int rotate,
                                     void* stream) {
     if (H <= 0 || d <= 0 || dp < d) return -1;
-    return sd_quant_src(3, src, 0, nullptr, nullptr, 0.f, H, d, dp, nullptr, 0, 0, 0, q, scales, M, H * d, rotate,
-                        (hipStream_t)stream);
+    QuantArgs a{src, (int64_t)H * dp, q, scales, nullptr, M, H * d, 1, 1, 0, PRO_SD_UNPAD, nullptr, 0, 0, nullptr, nullptr, 0.f,
+                nullptr, nullptr, d, dp};
+    return sd_fused(a, rotate, (hipStream_t)stream);
 }
 GPU_API int gpu_sd_group_norm_quant_rows(const void* x, const float* w, const float* b, void* sums, int N, int64_t P, int C, int G,
                                          float eps, int8_t* q, float* scales, int rotate, void* stream) {
     if (G <= 0 || C % G) return -1;                                                             // csrc/sd.cu:713
-    return sd_quant_src(4, x, 0, w, b, eps, 0, 0, 0, sums, G, P, N, q, scales, (int)(N * P), C, rotate, (hipStream_t)stream);
+    if ((rotate != 0 && rotate != 64 && rotate != 256) || (rotate && C % rotate) || C <= 0 || C % 16) return -1;
+    if (N <= 0 || P <= 0) return 0;
+    const int rc = gpu_internal_sd_group_stats(x, sums, N, P, C, G, eps, stream);
+    if (rc) return rc;
+    QuantArgs a{x, C, q, scales, nullptr, (int)(N * P), C, 1, 1, 0, PRO_SD_GN, sums, P, 0, w, b, eps, nullptr, nullptr, 0, 0, C / G};
+    return sd_fused(a, rotate, (hipStream_t)stream);
 }
 
 // x [N, K] in its original basis -> rotated int8 rows + row scales: the 256-wide quantizer with rounding to nearest

@@ -18,7 +18,9 @@ static __device__ __attribute__((noinline)) float gelu_tanh_f(float x) {        
     return 0.5f * x * (1.f + (float)tanh((double)(k0 * __builtin_fmaf(k1 * x * x, x, x))));
 }
 
-// MOSS Image's soft-capped gated activation as one float expression, csrc/common.cuh:80-82
-__device__ __forceinline__ float situ_f(float hidden, float gate) {
-    return 4.f * stable_tanh(gate / 4.f) / (1.f + exp_cr(-gate)) * (25.f * stable_tanh(hidden / 25.f));
-}
+// MOSS Image's soft-capped gated activation as one float expression, csrc/common.cuh:80-82:
+//   4.f * stable_tanh(gate / 4.f) / (1.f + expf(-gate)) * (25.f * stable_tanh(hidden / 25.f))
+// evaluated left to right: (gate factor) * (hidden factor), each an fp32 value of one argument.
+__device__ __forceinline__ float situ_gate_f(float gate) { return 4.f * stable_tanh(gate / 4.f) / (1.f + exp_cr(-gate)); }
+__device__ __forceinline__ float situ_hidden_f(float hidden) { return 25.f * stable_tanh(hidden / 25.f); }
+__device__ __forceinline__ float situ_f(float hidden, float gate) { return situ_gate_f(gate) * situ_hidden_f(hidden); }

@@ -79,7 +79,7 @@ int gpu_sd_quant_rows(const void* x, int64_t x_stride, int8_t* q, float* scales,
 
 /* The SD UNet's fused quantizers: the half row another kernel would have written, then gpu_sd_quant_rows of it.
  * Replace gpu_sd_ln_quant_rows, gpu_sd_geglu_quant_rows, gpu_sd_unpad_quant_rows, gpu_sd_group_norm_quant_rows,
- * csrc/sd.cu:691-724.  rotate and K as gpu_sd_quant_rows.  The row goes through a stream-ordered half [M, K] buffer.
+ * csrc/sd.cu:691-724.  rotate and K as gpu_sd_quant_rows.  The source runs inside the quantizer kernel.
  *   ln:     LayerNorm of x [M, x_stride] with fp32 weight and bias.
  *   geglu:  in [M, 2I] (value, then gate) -> value * gelu(gate), K = I.
  *   unpad:  src [M, H, dp] -> the first d of every dp, K = H * d.
