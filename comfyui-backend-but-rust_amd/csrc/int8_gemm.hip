@@ -6,6 +6,8 @@
 // one row), so tiles go global -> LDS as 16-byte chunks with an XOR swizzle and come back as ds_read_b128 fragments.
 // W rides in src0 and A in src1, which leaves every lane holding runs of four consecutive n for one m: the epilogue
 // stores 8-byte (bf16/f16) or 16-byte (f32) vectors straight from the accumulators.
+#include <cstdlib>
+
 #include "common.hpp"
 
 // Nothing is scheduled across this point: it pins hand-interleaved instruction orders and keeps live ranges short.
@@ -29,6 +31,10 @@ struct GemmArgs {
     int M, N, K;
     int tiles_m, tiles_n;
     int kslice;   // ring kernel only: K elements per split-K slice (a multiple of 128), 0 = no split
+    int stagger;  // ring kernel only: start delay, in shader clocks, spread over the workgroups that have a tile to spare
+#ifdef GEMM_TRACE
+    long long* trace;   // [workgroup][16] shader-clock stamps: start, then (K loop end, epilogue end) per tile
+#endif
 };
 
 template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int OCC_>
@@ -51,6 +57,13 @@ struct Cfg {
 // 16-byte bank groups.  Rows are BK bytes apart: with 128-byte rows an even/odd row pair already covers the two halves
 // of the bank space, so the chunk index is XORed with bits 1..3 of the row; with 64-byte rows four rows span the banks
 // and bits 2..3 are used.  (Measured: XOR with the low row bits instead costs 25 % of the read bandwidth.)
+// The lane number from the execution mask counters: two instructions, and no register held across a loop for it.
+__device__ __forceinline__ int hw_lane() {
+    int l = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    asm volatile("" : "+v"(l));
+    return l;
+}
+
 template <int BK> __device__ __forceinline__ int swz(int row, int chunk) {
     return BK == 64 ? (chunk ^ ((row >> 2) & 3)) : (chunk ^ ((row >> 1) & 7));
 }
@@ -126,8 +139,11 @@ __device__ __forceinline__ void epilogue_store(const GemmArgs& p, v16i (&acc)[TN
 // writes whole rows: 16 bytes per lane, consecutive lanes on consecutive addresses.  For the residual form the LDS
 // holds z = Out(acc*xs*ws + bias), exactly the intermediate the reference rounds, and fma(z, rscale, resid) is applied
 // on the way out.  Needs row starts of D (and resid) 16-byte aligned; the caller falls back to epilogue_store otherwise.
-template <int TM, int TN, int OUT_DT, int EPI, int PW = TN * 32, bool UNTRACKED = false>
-__device__ __forceinline__ void epilogue_shuffle(const GemmArgs& p, v16i (&acc)[TN][TM], int mb, int nb, int lane, uint8_t* wl) {
+// STAGED: the per-column constants (ws and bias as floats, 2 x 32*TN values) are kept in the wave's LDS area `cst` and
+// read back per piece, instead of 96 registers that a persistent kernel cannot spare next to its pipeline state.
+template <int TM, int TN, int OUT_DT, int EPI, int PW = TN * 32, bool UNTRACKED = false, bool STAGED = false>
+__device__ __forceinline__ void epilogue_shuffle(const GemmArgs& p, v16i (&acc)[TN][TM], int mb, int nb, int lane, uint8_t* wl,
+                                                 uint8_t* wl2 = nullptr, float* cst = nullptr) {
     // a piece is 32 rows x PW columns of the wave tile: PW*SZ bytes per LDS row, 32*PW*SZ bytes per wave
     constexpr int SZ = (EPI == EPI_ACC || OUT_DT == DT_F32) ? 4 : 2;
     constexpr int WTN = TN * 32, NP = WTN / PW, TNP = PW / 32;
@@ -141,13 +157,43 @@ __device__ __forceinline__ void epilogue_shuffle(const GemmArgs& p, v16i (&acc)[
     // the stores, each behind a full memory wait.  Making the lane number opaque here keeps the address arithmetic local.
     asm volatile("" : "+v"(lane));
     const int frow = lane & 31, fhalf = lane >> 5;
+#ifdef GEMM_TRACE
+    int estamp = 8;
+    auto stamp_e = [&]() {
+        if (p.trace && threadIdx.x == 0 && estamp < 15 && p.trace[blockIdx.x * 16 + 8 + 6] == 0)
+            p.trace[blockIdx.x * 16 + estamp] = (long long)__builtin_readcyclecounter();
+        ++estamp;
+    };
+    stamp_e();
+#else
+    auto stamp_e = [&]() {};
+#endif
 
     // per-lane column constants, loaded once and in one batch (no branches between the loads, so a single wait covers
     // them): ws and the raw bias words for the 4 n of every (in, rb).  Columns past N read the last valid vector.
     constexpr int BW = SZ == 4 ? 4 : 2;            // 32-bit words holding 4 bias values
-    float wsr[TN][4][4];
-    uint32_t braw[TN][4][BW];
-    if (EPI != EPI_ACC) {
+    float wsr[STAGED ? 1 : TN][4][4];
+    uint32_t braw[STAGED ? 1 : TN][4][BW];
+    if (EPI != EPI_ACC && STAGED) {
+        // two columns per lane and pass
+#pragma unroll
+        for (int c0 = 0; c0 < WTN; c0 += 128) {
+            const int c = c0 + lane * 2;
+            if (c < WTN) {
+                int n = nb + c;
+                n = n < p.N ? n : p.N - 2;
+                const float2 w2 = *reinterpret_cast<const float2*>(p.ws + n);
+                float2 b2 = make_float2(0.f, 0.f);
+                if (p.bias) {
+                    b2.x = ld_dt<(SZ == 4 ? DT_F32 : OUT_DT)>(p.bias, n);
+                    b2.y = ld_dt<(SZ == 4 ? DT_F32 : OUT_DT)>(p.bias, n + 1);
+                }
+                *reinterpret_cast<float2*>(cst + c) = w2;
+                *reinterpret_cast<float2*>(cst + WTN + c) = b2;
+            }
+        }
+    }
+    if (EPI != EPI_ACC && !STAGED) {
 #pragma unroll
         for (int in = 0; in < TN; ++in)
 #pragma unroll
@@ -210,80 +256,118 @@ __device__ __forceinline__ void epilogue_shuffle(const GemmArgs& p, v16i (&acc)[
         }
     };
 
-#pragma unroll
-    for (int im = 0; im < TM; ++im) {
+    // write phase of piece (im, np): row frow of the piece into `buf`
+    auto write_piece = [&](int im, int np, uint8_t* buf) {
         const float xs = xsr[im];
 #pragma unroll
-        for (int np = 0; np < NP; ++np) {
-            // The residual rows of this piece are requested before its write phase, whose arithmetic covers their latency
-            // (and that of the previous piece's stores, which retire ahead of them).
-            uint4 rv[PASSES];
-            if (EPI == EPI_RESID) load_resid(im, np, rv);
-            // write phase: row frow of the piece
+        for (int ip = 0; ip < TNP; ++ip)
 #pragma unroll
-            for (int ip = 0; ip < TNP; ++ip)
-#pragma unroll
-                for (int rb = 0; rb < 4; ++rb) {
-                    const int in = np * TNP + ip;
-                    const int byte = (ip * 32 + rb * 8 + fhalf * 4) * SZ;
-                    uint8_t* dst = wl + frow * ROWB + ((((byte >> 4) ^ frow) & MASK) << 4) + (byte & 15);
-                    if (EPI == EPI_ACC) {
-                        *reinterpret_cast<v4i*>(dst) = v4i{acc[in][im][4 * rb], acc[in][im][4 * rb + 1], acc[in][im][4 * rb + 2], acc[in][im][4 * rb + 3]};
+            for (int rb = 0; rb < 4; ++rb) {
+                const int in = np * TNP + ip;
+                const int byte = (ip * 32 + rb * 8 + fhalf * 4) * SZ;
+                uint8_t* dst = buf + frow * ROWB + ((((byte >> 4) ^ frow) & MASK) << 4) + (byte & 15);
+                if (EPI == EPI_ACC) {
+                    *reinterpret_cast<v4i*>(dst) = v4i{acc[in][im][4 * rb], acc[in][im][4 * rb + 1], acc[in][im][4 * rb + 2], acc[in][im][4 * rb + 3]};
+                } else {
+                    float o[4];
+                    if (STAGED) {
+                        const float4 w4 = *reinterpret_cast<const float4*>(cst + in * 32 + rb * 8 + fhalf * 4);
+                        const float4 b4 = *reinterpret_cast<const float4*>(cst + WTN + in * 32 + rb * 8 + fhalf * 4);
+                        o[0] = __builtin_fmaf((float)acc[in][im][4 * rb] * xs, w4.x, b4.x);
+                        o[1] = __builtin_fmaf((float)acc[in][im][4 * rb + 1] * xs, w4.y, b4.y);
+                        o[2] = __builtin_fmaf((float)acc[in][im][4 * rb + 2] * xs, w4.z, b4.z);
+                        o[3] = __builtin_fmaf((float)acc[in][im][4 * rb + 3] * xs, w4.w, b4.w);
                     } else {
-                        float o[4];
 #pragma unroll
                         for (int j = 0; j < 4; ++j) o[j] = __builtin_fmaf((float)acc[in][im][4 * rb + j] * xs, wsr[in][rb][j], bias_f(in, rb, j));
-                        if (OUT_DT == DT_F32) {
-                            *reinterpret_cast<float4*>(dst) = make_float4(o[0], o[1], o[2], o[3]);
-                        } else if (OUT_DT == DT_BF16) {
-                            *reinterpret_cast<uint2*>(dst) = make_uint2(pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]));
-                        } else {
-                            *reinterpret_cast<uint2*>(dst) = make_uint2((uint32_t)f_to_f16(o[0]) | ((uint32_t)f_to_f16(o[1]) << 16),
-                                                                        (uint32_t)f_to_f16(o[2]) | ((uint32_t)f_to_f16(o[3]) << 16));
-                        }
                     }
-                }
-            asm volatile("" ::: "memory");   // the wave's own LDS writes are ordered before its reads by the LDS queue
-            // read phase: whole rows out
-            const int ncol = nb + np * PW + rc * EPC;
-#pragma unroll
-            for (int t = 0; t < PASSES; ++t) {
-                const int r = t * RPI + rrow;
-                const uint4 v = *reinterpret_cast<const uint4*>(wl + r * ROWB + (((rc ^ r) & MASK) << 4));
-                const int m = mb + im * 32 + r;
-                if (m >= p.M || ncol >= p.N) continue;
-                const int64_t o = (int64_t)m * p.N + ncol;
-                if (EPI != EPI_RESID) {
-                    if (UNTRACKED) store16_untracked((uint8_t*)p.D + o * SZ, v);
-                    else *reinterpret_cast<uint4*>((uint8_t*)p.D + o * SZ) = v;
-                } else {
-                    const uint32_t zw[4] = {v.x, v.y, v.z, v.w}, rw[4] = {rv[t].x, rv[t].y, rv[t].z, rv[t].w};
-                    uint32_t ow[4];
                     if (OUT_DT == DT_F32) {
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) ow[j] = f2u(__builtin_fmaf(u2f(zw[j]), rs[np][j], u2f(rw[j])));
+                        *reinterpret_cast<float4*>(dst) = make_float4(o[0], o[1], o[2], o[3]);
+                    } else if (OUT_DT == DT_BF16) {
+                        *reinterpret_cast<uint2*>(dst) = make_uint2(pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]));
                     } else {
+                        *reinterpret_cast<uint2*>(dst) = make_uint2((uint32_t)f_to_f16(o[0]) | ((uint32_t)f_to_f16(o[1]) << 16),
+                                                                    (uint32_t)f_to_f16(o[2]) | ((uint32_t)f_to_f16(o[3]) << 16));
+                    }
+                }
+            }
+    };
+    // read phase, first half: the piece's rows back from `buf`, 16 bytes per lane and pass, all passes in one batch
+    auto read_piece = [&](const uint8_t* buf, uint4* v) {
 #pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            float z0, z1, r0, r1;
-                            if (OUT_DT == DT_BF16) {
-                                z0 = u2f(zw[j] << 16); z1 = u2f(zw[j] & 0xffff0000u); r0 = u2f(rw[j] << 16); r1 = u2f(rw[j] & 0xffff0000u);
-                                ow[j] = pack_bf16x2(__builtin_fmaf(z0, rs[np][2 * j], r0), __builtin_fmaf(z1, rs[np][2 * j + 1], r1));
-                            } else {
-                                z0 = f16_to_f((uint16_t)(zw[j] & 0xffffu)); z1 = f16_to_f((uint16_t)(zw[j] >> 16));
-                                r0 = f16_to_f((uint16_t)(rw[j] & 0xffffu)); r1 = f16_to_f((uint16_t)(rw[j] >> 16));
-                                ow[j] = (uint32_t)f_to_f16(__builtin_fmaf(z0, rs[np][2 * j], r0)) | ((uint32_t)f_to_f16(__builtin_fmaf(z1, rs[np][2 * j + 1], r1)) << 16);
-                            }
+        for (int t = 0; t < PASSES; ++t) {
+            const int r = t * RPI + rrow;
+            v[t] = *reinterpret_cast<const uint4*>(buf + r * ROWB + (((rc ^ r) & MASK) << 4));
+        }
+    };
+    // read phase, second half: whole rows out
+    auto store_piece = [&](int im, int np, const uint4* v, const uint4* rv) {
+        const int ncol = nb + np * PW + rc * EPC;
+        uint8_t* base = (uint8_t*)p.D + ((int64_t)(mb + im * 32 + rrow) * p.N + ncol) * SZ;
+        const int64_t step = (int64_t)RPI * p.N * SZ;
+#pragma unroll
+        for (int t = 0; t < PASSES; ++t) {
+            const int m = mb + im * 32 + t * RPI + rrow;
+            if (m >= p.M || ncol >= p.N) continue;
+            uint8_t* out = base + t * step;
+            if (EPI != EPI_RESID) {
+                if (UNTRACKED) store16_untracked(out, v[t]);
+                else *reinterpret_cast<uint4*>(out) = v[t];
+            } else {
+                const uint32_t zw[4] = {v[t].x, v[t].y, v[t].z, v[t].w}, rw[4] = {rv[t].x, rv[t].y, rv[t].z, rv[t].w};
+                uint32_t ow[4];
+                if (OUT_DT == DT_F32) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) ow[j] = f2u(__builtin_fmaf(u2f(zw[j]), rs[np][j], u2f(rw[j])));
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        float z0, z1, r0, r1;
+                        if (OUT_DT == DT_BF16) {
+                            z0 = u2f(zw[j] << 16); z1 = u2f(zw[j] & 0xffff0000u); r0 = u2f(rw[j] << 16); r1 = u2f(rw[j] & 0xffff0000u);
+                            ow[j] = pack_bf16x2(__builtin_fmaf(z0, rs[np][2 * j], r0), __builtin_fmaf(z1, rs[np][2 * j + 1], r1));
+                        } else {
+                            z0 = f16_to_f((uint16_t)(zw[j] & 0xffffu)); z1 = f16_to_f((uint16_t)(zw[j] >> 16));
+                            r0 = f16_to_f((uint16_t)(rw[j] & 0xffffu)); r1 = f16_to_f((uint16_t)(rw[j] >> 16));
+                            ow[j] = (uint32_t)f_to_f16(__builtin_fmaf(z0, rs[np][2 * j], r0)) | ((uint32_t)f_to_f16(__builtin_fmaf(z1, rs[np][2 * j + 1], r1)) << 16);
                         }
                     }
-                    if (UNTRACKED) store16_untracked((uint8_t*)p.D + o * SZ, make_uint4(ow[0], ow[1], ow[2], ow[3]));
-                    else *reinterpret_cast<uint4*>((uint8_t*)p.D + o * SZ) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
                 }
-                SCHED_FENCE();
+                if (UNTRACKED) store16_untracked(out, make_uint4(ow[0], ow[1], ow[2], ow[3]));
+                else *reinterpret_cast<uint4*>(out) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
             }
+        }
+    };
+
+    // Pieces go through the LDS one after the other.  With a second region (wl2) the loop is software-pipelined: the
+    // LDS reads of piece i are issued, then the arithmetic and LDS writes of piece i+1 (into the other region) cover
+    // their latency, then piece i is stored.  The LDS queue runs one wave's accesses in program order, so a piece's
+    // reads see its writes, and a region is rewritten only after the reads of its previous piece have returned (they
+    // are waited for by the stores in between).  The residual rows of a piece are requested before its write phase.
+    constexpr int NPIECE = TM * NP;
+    uint8_t* bufs[2] = {wl, wl2 ? wl2 : wl};
+    uint4 rv[2][PASSES];
+    if (EPI == EPI_RESID) load_resid(0, 0, rv[0]);
+    write_piece(0, 0, bufs[0]);
+#pragma unroll
+    for (int i = 0; i < NPIECE; ++i) {
+        const int im = i / NP, np = i % NP;
+        uint4 v[PASSES];
+        asm volatile("" ::: "memory");
+        read_piece(bufs[i & 1], v);
+        asm volatile("" ::: "memory");
+        if (wl2 && i + 1 < NPIECE) {
+            if (EPI == EPI_RESID) load_resid((i + 1) / NP, (i + 1) % NP, rv[(i + 1) & 1]);
+            write_piece((i + 1) / NP, (i + 1) % NP, bufs[(i + 1) & 1]);
+        }
+        store_piece(im, np, v, rv[i & 1]);
+        if (!wl2 && i + 1 < NPIECE) {
+            if (EPI == EPI_RESID) load_resid((i + 1) / NP, (i + 1) % NP, rv[(i + 1) & 1]);
             asm volatile("" ::: "memory");
+            write_piece((i + 1) / NP, (i + 1) % NP, bufs[0]);
         }
     }
+    asm volatile("" ::: "memory");
 }
 
 // Chooses the coalesced epilogue when row starts are 16-byte aligned.  Must be called by all waves of the workgroup:
@@ -812,10 +896,9 @@ struct RingCfg {
         return true;
     }
     static_assert(slots_ok(), "DMA slots must be distinct, inside the iteration, and early for a two-stage A");
-    // columns of one epilogue shuffle piece for an output element of SZ bytes: 64..256-byte LDS rows
-    static constexpr int piece_cols(int sz) {
-        return sz == 2 ? (WTN % 128 == 0 ? 128 : WTN % 64 == 0 ? 64 : 32) : (WTN % 64 == 0 ? 64 : 32);
-    }
+    // columns of one epilogue shuffle piece for an output element of SZ bytes: 128-byte LDS rows, i.e. four 16-byte
+    // vectors per lane in flight between the read and the store half of a piece
+    static constexpr int piece_cols(int sz) { return 128 / sz; }
 };
 
 template <class C, int OUT_DT, int EPI>
@@ -846,27 +929,33 @@ __global__ void __launch_bounds__(256, 1) int8_gemm_ring_kernel(GemmArgs p) {
     // DMA streams.  Each walks (tile, K tile) pairs in the order the MFMAs will consume them and stops on the last one
     // (re-fetching it into a stage nothing reads again keeps the loop free of branches around the DMA slots).
     // rows come in blocks of 8 (block index wave + 4j has the parity of wave): swz<128> of the row
-    const int lrow = lane >> 3, lch = ((lane & 7) ^ (((wave & 1) << 2) | (lrow >> 1))) * 16;
     uint32_t ga[C::A_LD], gw[C::W_LD];
     int a_tile = 0, a_kt = 0, a_stage = 0, w_tile = 0, w_kt = 0, w_stage = 0;
+    // The row and chunk of a lane are recomputed from the hardware lane number each time a stream moves to its next
+    // tile: as loop invariants the compiler would keep sixteen of them live across the K loop, spill them, and reload
+    // them here behind full memory waits that drain the DMA pipeline (a spilled copy of the lane number does the same).
     auto set_a = [&](int i) {
         int m0, n0;
         tile_origin(i, m0, n0);
+        const int l = hw_lane();
+        const int lr = l >> 3, lc = ((l & 7) ^ (((wave & 1) << 2) | (lr >> 1))) * 16;
 #pragma unroll
         for (int j = 0; j < C::A_LD; ++j) {
-            const int row = (wave + 4 * j) * 8 + lrow;
+            const int row = (wave + 4 * j) * 8 + lr;
             const int gr = m0 + row < p.M ? m0 + row : p.M - 1;
-            ga[j] = (uint32_t)gr * (uint32_t)ld + lch;
+            ga[j] = (uint32_t)gr * (uint32_t)ld + lc;
         }
     };
     auto set_w = [&](int i) {
         int m0, n0;
         tile_origin(i, m0, n0);
+        const int l = hw_lane();
+        const int lr = l >> 3, lc = ((l & 7) ^ (((wave & 1) << 2) | (lr >> 1))) * 16;
 #pragma unroll
         for (int j = 0; j < C::W_LD; ++j) {
-            const int row = (wave + 4 * j) * 8 + lrow;
+            const int row = (wave + 4 * j) * 8 + lr;
             const int gr = n0 + row < p.N ? n0 + row : p.N - 1;
-            gw[j] = (uint32_t)gr * (uint32_t)ld + lch;
+            gw[j] = (uint32_t)gr * (uint32_t)ld + lc;
         }
     };
     // The DMA is written as inline assembly: through the builtin the compiler, unable to prove that a fragment read and
@@ -931,6 +1020,25 @@ __global__ void __launch_bounds__(256, 1) int8_gemm_ring_kernel(GemmArgs p) {
         }
     };
 
+    // Workgroups with one tile less than the others have a tile's time to spare.  Left alone, every workgroup reaches its
+    // epilogue at the same moment and the burst of output stores saturates HBM while all matrix cores wait; the spare
+    // time is spent up front instead, as a start delay that grows with the workgroup's index, so that the epilogues of
+    // those workgroups fall between the others'.
+    if (p.stagger > 0) {
+        const int nmax = (ntiles + G - 1) / G, first_short = ntiles % G;
+        if (nt_b < nmax && first_short > 0) {
+            const int64_t delay = (int64_t)p.stagger * ((int)blockIdx.x - first_short) / (G - first_short);
+            const int64_t t0 = (int64_t)__builtin_readcyclecounter();
+            while ((int64_t)__builtin_readcyclecounter() - t0 < delay) __builtin_amdgcn_s_sleep(16);
+        }
+    }
+
+#ifdef GEMM_TRACE
+    auto stamp = [&](int i) { if (p.trace && tid == 0 && i < 16) p.trace[blockIdx.x * 16 + i] = (long long)__builtin_readcyclecounter(); };
+    stamp(0);
+#else
+    auto stamp = [&](int) {};
+#endif
     // prologue: A(0), W(0), [A(1),] W(1) in flight; A(0) and W(0) must land
     set_a(0);
     set_w(0);
@@ -966,7 +1074,7 @@ __global__ void __launch_bounds__(256, 1) int8_gemm_ring_kernel(GemmArgs p) {
         // draining the DMA pipeline every iteration.  (Waits it derives for its own loads stay correct: the memory
         // counter retires in order, so instructions it does not know about only make those waits stricter.)
 
-        int pa = 0;
+        int pa = 0, pw = 0;
         for (int kt = 0; kt < nk; ++kt) {
             const uint8_t* sa = smem + ca * C::A_STAGE;
             const uint8_t* sw = smem + C::W_BASE + cw * C::W_STAGE;
@@ -981,6 +1089,7 @@ __global__ void __launch_bounds__(256, 1) int8_gemm_ring_kernel(GemmArgs p) {
             advance_a();
             advance_w();
             pa = ca;
+            pw = cw;
             ca = na;
             cw = nw;
         }
@@ -989,18 +1098,27 @@ __global__ void __launch_bounds__(256, 1) int8_gemm_ring_kernel(GemmArgs p) {
         // (The launcher only picks this kernel when the coalesced epilogue's alignment conditions hold.)
         int m0, n0;
         tile_origin(ti, m0, n0);
+        stamp(1 + 2 * ti);
         __syncthreads();   // every wave is done reading that stage
         constexpr int SZ = (EPI == EPI_ACC || OUT_DT == DT_F32) ? 4 : 2;
         constexpr int PW = C::piece_cols(SZ);
-        static_assert(32 * PW * SZ <= 8192, "shuffle piece");
-        epilogue_shuffle<TM, TN, OUT_DT, EPI, PW, true>(p, acc, m0 + wm * C::WTM, n0 + wn * C::WTN, lane,
-                                                         smem + pa * C::A_STAGE + wave * 8192);
+        static_assert(32 * PW * SZ <= 8192 && C::A_STAGE >= 4 * 8192 && C::W_STAGE >= 4 * 8192, "shuffle piece");
+        // Shuffle scratch, 8 KB per wave and region: the A stage and the W stage that were just multiplied (the DMA in
+        // flight fills the other stages; the next write into these two is issued inside the next iteration).
+        // A piece takes 4 KB of a region; the wave's column constants sit behind the first one.
+        static_assert(32 * PW * SZ <= 4096 && 2 * C::WTN * 4 <= 4096, "shuffle piece and constants share 8 KB");
+        epilogue_shuffle<TM, TN, OUT_DT, EPI, PW, true, true>(p, acc, m0 + wm * C::WTM, n0 + wn * C::WTN, hw_lane(),
+                                                               smem + pa * C::A_STAGE + wave * 8192,
+                                                               smem + C::W_BASE + pw * C::W_STAGE + wave * 8192,
+                                                               reinterpret_cast<float*>(smem + pa * C::A_STAGE + wave * 8192 + 4096));
         // The first fragments of the next tile were prefetched by the last sub-step; fetching them again here instead of
         // carrying 32 registers across the epilogue keeps the epilogue free of spills.
 #pragma unroll
         for (int j = 0; j < NF; ++j) f0[j] = frag(smem + ca * C::A_STAGE, smem + C::W_BASE + cw * C::W_STAGE, 0, j);
+        stamp(2 + 2 * ti);
     }
     wait_vmcnt<0>();   // no DMA may still be writing this workgroup's LDS when it retires
+    stamp(15);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -1185,7 +1303,7 @@ __global__ void __launch_bounds__(StreamCfg::NT, 1) int8_gemm_stream_kernel(Gemm
             for (int im = 0; im < TM; ++im)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc[in][im][r] = 0;
-        int pa = 0;
+        int pa = 0, pw = 0;
         for (int kt = 0; kt < nk; ++kt) {
             const uint8_t* sa = smem + ca * C::A_STAGE;
             const uint8_t* sw = smem + C::W_BASE + cw * C::W_STAGE;
@@ -1197,6 +1315,7 @@ __global__ void __launch_bounds__(StreamCfg::NT, 1) int8_gemm_stream_kernel(Gemm
             wg_barrier();                                                   // Y
             substep(f1, f0, smem + na * C::A_STAGE, smem + C::W_BASE + nw * C::W_STAGE, 0);
             pa = ca;
+            pw = cw;
             ca = na;
             cw = nw;
         }
@@ -1290,6 +1409,17 @@ int launch_ring_cfg(GemmArgs a, int slices, hipStream_t st) {
     const int num_cu = device_cu_count();
     const int64_t per_slice = slices > 1 ? (num_cu / slices > 0 ? num_cu / slices : 1) : num_cu;
     const unsigned grid = (unsigned)(ntiles < per_slice ? ntiles : per_slice);
+    a.stagger = 0;
+    if (slices == 1 && ntiles > grid) {
+        static const char* env = getenv("GEMM_STAGGER_PER_KTILE");
+        a.stagger = (env ? atoi(env) : 0) * (a.K / C::BK);
+    }
+#ifdef GEMM_TRACE
+    {
+        const char* tp = getenv("GEMM_TRACE_PTR");
+        a.trace = tp ? (long long*)strtoull(tp, nullptr, 0) : nullptr;
+    }
+#endif
     hipLaunchKernelGGL(kern, dim3(grid, (unsigned)slices), dim3(C::NT), C::SMEM, st, a);
     KCHECK();
     return 0;
@@ -1338,6 +1468,17 @@ int launch_stream(GemmArgs a, int slices, hipStream_t st) {
     const int num_cu = device_cu_count();
     const int64_t per_slice = slices > 1 ? (num_cu / slices > 0 ? num_cu / slices : 1) : num_cu;
     const unsigned grid = (unsigned)(ntiles < per_slice ? ntiles : per_slice);
+    a.stagger = 0;
+    if (slices == 1 && ntiles > grid) {
+        static const char* env = getenv("GEMM_STAGGER_PER_KTILE");
+        a.stagger = (env ? atoi(env) : 0) * (a.K / C::BK);
+    }
+#ifdef GEMM_TRACE
+    {
+        const char* tp = getenv("GEMM_TRACE_PTR");
+        a.trace = tp ? (long long*)strtoull(tp, nullptr, 0) : nullptr;
+    }
+#endif
     hipLaunchKernelGGL(kern, dim3(grid, (unsigned)slices), dim3(C::NT), C::SMEM, st, a);
     KCHECK();
     return 0;
