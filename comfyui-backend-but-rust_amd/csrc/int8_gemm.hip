@@ -863,9 +863,9 @@ template <int V> struct ic { static constexpr int value = V; };
 
 // BN: tile width; WGM x WGN: wave grid (four waves); NSA: LDS stages of A (2 for the 256-wide tile, where 160 KB of LDS
 // leave no room for a third; 3 where a narrower tile leaves room).  W always has three stages.
-template <int BN_, int WGM_, int WGN_, int NSA_>
+template <int BN_, int WGM_, int WGN_, int NSA_, int BM_ = 256>
 struct RingCfg {
-    static constexpr int BM = 256, BN = BN_, BK = 128, WGM = WGM_, WGN = WGN_, NT = 256, NSA = NSA_, NSW = 3;
+    static constexpr int BM = BM_, BN = BN_, BK = 128, WGM = WGM_, WGN = WGN_, NT = 256, NSA = NSA_, NSW = 3;
     static constexpr int WTM = BM / WGM, WTN = BN / WGN, TM = WTM / 32, TN = WTN / 32;
     static constexpr int A_LD = BM / 32, W_LD = BN / 32;     // DMA instructions per wave per stage (8 rows each)
     static constexpr int NDMA = A_LD + W_LD, NM = TM * TN, NF = TM + TN;
@@ -896,9 +896,15 @@ struct RingCfg {
         return true;
     }
     static_assert(slots_ok(), "DMA slots must be distinct, inside the iteration, and early for a two-stage A");
-    // columns of one epilogue shuffle piece for an output element of SZ bytes: 128-byte LDS rows, i.e. four 16-byte
-    // vectors per lane in flight between the read and the store half of a piece
-    static constexpr int piece_cols(int sz) { return 128 / sz; }
+    // columns of one epilogue shuffle piece for an output element of SZ bytes: 128-byte LDS rows (four 16-byte vectors
+    // per lane in flight between the read and the store half of a piece) where the wave tile's width allows
+    static constexpr int piece_cols(int sz) { return WTN % (128 / sz) == 0 ? 128 / sz : 32; }
+    // Epilogue scratch of one wave inside a stage that was just multiplied: a shuffle piece in each of an A and a W
+    // stage, and the wave's column constants (2 x WTN floats) behind the piece in the W stage.
+    static constexpr int A_REGION = A_STAGE / 4, W_REGION = W_STAGE / 4;
+    static constexpr int piece_bytes(int sz) { return 32 * piece_cols(sz) * sz; }
+    static constexpr bool scratch_ok(int sz) { return piece_bytes(sz) <= A_REGION && piece_bytes(sz) + 2 * WTN * 4 <= W_REGION; }
+    static_assert(scratch_ok(2) && scratch_ok(4), "epilogue scratch fits the stages");
 };
 
 template <class C, int OUT_DT, int EPI>
@@ -1061,6 +1067,9 @@ __global__ void __launch_bounds__(256, 1) int8_gemm_ring_kernel(GemmArgs p) {
 #pragma unroll
     for (int j = 0; j < NF; ++j) f0[j] = frag(smem, smem + C::W_BASE, 0, j);
 
+#ifdef GEMM_TRACE
+    long long qs[5] = {0, 0, 0, 0, 0};
+#endif
     int ca = 0, cw = 0;   // stages of the iteration being multiplied
     for (int ti = 0; ti < nt_b; ++ti) {
 #pragma unroll
@@ -1079,13 +1088,32 @@ __global__ void __launch_bounds__(256, 1) int8_gemm_ring_kernel(GemmArgs p) {
             const uint8_t* sa = smem + ca * C::A_STAGE;
             const uint8_t* sw = smem + C::W_BASE + cw * C::W_STAGE;
             const int na = ca == NSA - 1 ? 0 : ca + 1, nw = cw == C::NSW - 1 ? 0 : cw + 1;
+#ifdef GEMM_TRACE
+            const long long q0 = (long long)__builtin_readcyclecounter();
+#endif
             wg_barrier();                                                   // X
+#ifdef GEMM_TRACE
+            const long long q1 = (long long)__builtin_readcyclecounter();
+#endif
             substep(ic<0>{}, f0, f1, sa, sw, 1);
             substep(ic<NM>{}, f1, f0, sa, sw, 2);
             substep(ic<2 * NM>{}, f0, f1, sa, sw, 3);
+#ifdef GEMM_TRACE
+            const long long q2 = (long long)__builtin_readcyclecounter();
+#endif
             wait_vmcnt<C::in_flight_at_y()>();
+#ifdef GEMM_TRACE
+            const long long q3 = (long long)__builtin_readcyclecounter();
+#endif
             wg_barrier();                                                   // Y
+#ifdef GEMM_TRACE
+            const long long q4 = (long long)__builtin_readcyclecounter();
+#endif
             substep(ic<3 * NM>{}, f1, f0, smem + na * C::A_STAGE, smem + C::W_BASE + nw * C::W_STAGE, 0);
+#ifdef GEMM_TRACE
+            const long long q5 = (long long)__builtin_readcyclecounter();
+            qs[0] += q1 - q0; qs[1] += q2 - q1; qs[2] += q3 - q2; qs[3] += q4 - q3; qs[4] += q5 - q4;
+#endif
             advance_a();
             advance_w();
             pa = ca;
@@ -1102,15 +1130,12 @@ __global__ void __launch_bounds__(256, 1) int8_gemm_ring_kernel(GemmArgs p) {
         __syncthreads();   // every wave is done reading that stage
         constexpr int SZ = (EPI == EPI_ACC || OUT_DT == DT_F32) ? 4 : 2;
         constexpr int PW = C::piece_cols(SZ);
-        static_assert(32 * PW * SZ <= 8192 && C::A_STAGE >= 4 * 8192 && C::W_STAGE >= 4 * 8192, "shuffle piece");
         // Shuffle scratch, 8 KB per wave and region: the A stage and the W stage that were just multiplied (the DMA in
         // flight fills the other stages; the next write into these two is issued inside the next iteration).
-        // A piece takes 4 KB of a region; the wave's column constants sit behind the first one.
-        static_assert(32 * PW * SZ <= 4096 && 2 * C::WTN * 4 <= 4096, "shuffle piece and constants share 8 KB");
-        epilogue_shuffle<TM, TN, OUT_DT, EPI, PW, true, true>(p, acc, m0 + wm * C::WTM, n0 + wn * C::WTN, hw_lane(),
-                                                               smem + pa * C::A_STAGE + wave * 8192,
-                                                               smem + C::W_BASE + pw * C::W_STAGE + wave * 8192,
-                                                               reinterpret_cast<float*>(smem + pa * C::A_STAGE + wave * 8192 + 4096));
+        uint8_t* ra = smem + pa * C::A_STAGE + wave * C::A_REGION;
+        uint8_t* rw = smem + C::W_BASE + pw * C::W_STAGE + wave * C::W_REGION;
+        epilogue_shuffle<TM, TN, OUT_DT, EPI, PW, true, true>(p, acc, m0 + wm * C::WTM, n0 + wn * C::WTN, hw_lane(), ra, rw,
+                                                               reinterpret_cast<float*>(rw + C::piece_bytes(SZ)));
         // The first fragments of the next tile were prefetched by the last sub-step; fetching them again here instead of
         // carrying 32 registers across the epilogue keeps the epilogue free of spills.
 #pragma unroll
@@ -1119,6 +1144,10 @@ __global__ void __launch_bounds__(256, 1) int8_gemm_ring_kernel(GemmArgs p) {
     }
     wait_vmcnt<0>();   // no DMA may still be writing this workgroup's LDS when it retires
     stamp(15);
+#ifdef GEMM_TRACE
+    if (p.trace && lane == 0 && wave < 2)
+        for (int i = 0; i < 5; ++i) p.trace[4096 + (blockIdx.x * 2 + wave) * 5 + i] = qs[i];
+#endif
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -1295,6 +1324,9 @@ __global__ void __launch_bounds__(StreamCfg::NT, 1) int8_gemm_stream_kernel(Gemm
     wg_barrier();   // A(0) and W(0) have landed
 #pragma unroll
     for (int j = 0; j < NF; ++j) f0[j] = frag(smem, smem + C::W_BASE, 0, j);
+#ifdef GEMM_TRACE
+    long long qs[5] = {0, 0, 0, 0, 0};
+#endif
     int ca = 0, cw = 0;   // stages of the iteration being multiplied
     for (int ti = 0; ti < nt_b; ++ti) {
 #pragma unroll
@@ -1425,13 +1457,46 @@ int launch_ring_cfg(GemmArgs a, int slices, hipStream_t st) {
     return 0;
 }
 
-using RingL = RingCfg<256, 2, 2, 2>;    // 256x256, waves 2x2 of 128x128: the compute-bound workhorse
+using RingL = RingCfg<256, 2, 2, 2>;         // 256x256, waves 2x2 of 128x128: the compute-bound workhorse
+using RingS = RingCfg<192, 2, 2, 3, 128>;    // 128x192, waves 2x2 of 64x96: re-tiles what the last round of RingL leaves
 
+// Rows [row0, row0 + rows) of the problem as a problem of its own.
+template <int OUT_DT, int EPI>
+GemmArgs row_band(const GemmArgs& a, int64_t row0, int64_t rows) {
+    constexpr int SZ = (EPI == EPI_ACC || OUT_DT == DT_F32) ? 4 : 2;
+    GemmArgs b = a;
+    b.A = a.A + row0 * a.K;
+    b.xs = a.xs ? a.xs + row0 : nullptr;
+    b.D = (uint8_t*)a.D + row0 * a.N * SZ;
+    b.resid = a.resid ? (const uint8_t*)a.resid + row0 * a.N * SZ : nullptr;
+    b.M = (int)rows;
+    return b;
+}
+
+// The persistent kernel gives every CU whole 256x256 tiles: when the tile count is not a multiple of the CU count, the
+// last round keeps only some CUs busy for a full tile's time (864 tiles on 256 CUs: 96 busy, 160 idle, a sixth of the
+// launch).  The tile rows that fill whole rounds go to the 256x256 kernel; the rows left over are re-tiled 128x192 and
+// run as a second launch when that is estimated to be shorter (a small tile costs about 0.45 of a large one).
 template <int OUT_DT, int EPI>
 int launch_ring(GemmArgs a, hipStream_t st) {
     bool vec_ok, aligned;
     epilogue_alignment<OUT_DT, EPI>(a, vec_ok, aligned);
     if (!aligned) return launch_cfg<CfgL, OUT_DT, EPI>(a, st);   // the ring kernel has only the coalesced epilogue
+    const int64_t G = device_cu_count();
+    const int64_t tm = (a.M + RingL::BM - 1) / RingL::BM, tn = (a.N + RingL::BN - 1) / RingL::BN;
+    const int64_t full = tm * tn / G, rem = tm * tn % G;
+    if (full >= 1 && rem > 0 && tm > 1) {
+        int64_t main_rows = full * G / tn;
+        if (main_rows >= tm) main_rows = tm - 1;
+        const int64_t m_main = main_rows * RingL::BM, m_rest = a.M - m_main;
+        const int64_t small = ((m_rest + RingS::BM - 1) / RingS::BM) * ((a.N + RingS::BN - 1) / RingS::BN);
+        const double split_cost = (double)((main_rows * tn + G - 1) / G) + 0.45 * (double)((small + G - 1) / G);
+        if (main_rows > 0 && split_cost < (double)(full + 1) - 0.1) {
+            const int rc = launch_ring_cfg<RingL, OUT_DT, EPI>(row_band<OUT_DT, EPI>(a, 0, m_main), 1, st);
+            if (rc) return rc;
+            return launch_ring_cfg<RingS, OUT_DT, EPI>(row_band<OUT_DT, EPI>(a, m_main, m_rest), 1, st);
+        }
+    }
     return launch_ring_cfg<RingL, OUT_DT, EPI>(a, 1, st);
 }
 
