@@ -31,7 +31,6 @@ struct GemmArgs {
     int M, N, K;
     int tiles_m, tiles_n;
     int kslice;   // ring kernel only: K elements per split-K slice (a multiple of 128), 0 = no split
-    int stagger;  // ring kernel only: start delay, in shader clocks, spread over the workgroups that have a tile to spare
 #ifdef GEMM_TRACE
     long long* trace;   // [workgroup][16] shader-clock stamps: start, then (K loop end, epilogue end) per tile
 #endif
@@ -1026,19 +1025,6 @@ __global__ void __launch_bounds__(256, 1) int8_gemm_ring_kernel(GemmArgs p) {
         }
     };
 
-    // Workgroups with one tile less than the others have a tile's time to spare.  Left alone, every workgroup reaches its
-    // epilogue at the same moment and the burst of output stores saturates HBM while all matrix cores wait; the spare
-    // time is spent up front instead, as a start delay that grows with the workgroup's index, so that the epilogues of
-    // those workgroups fall between the others'.
-    if (p.stagger > 0) {
-        const int nmax = (ntiles + G - 1) / G, first_short = ntiles % G;
-        if (nt_b < nmax && first_short > 0) {
-            const int64_t delay = (int64_t)p.stagger * ((int)blockIdx.x - first_short) / (G - first_short);
-            const int64_t t0 = (int64_t)__builtin_readcyclecounter();
-            while ((int64_t)__builtin_readcyclecounter() - t0 < delay) __builtin_amdgcn_s_sleep(16);
-        }
-    }
-
 #ifdef GEMM_TRACE
     auto stamp = [&](int i) { if (p.trace && tid == 0 && i < 16) p.trace[blockIdx.x * 16 + i] = (long long)__builtin_readcyclecounter(); };
     stamp(0);
@@ -1441,11 +1427,6 @@ int launch_ring_cfg(GemmArgs a, int slices, hipStream_t st) {
     const int num_cu = device_cu_count();
     const int64_t per_slice = slices > 1 ? (num_cu / slices > 0 ? num_cu / slices : 1) : num_cu;
     const unsigned grid = (unsigned)(ntiles < per_slice ? ntiles : per_slice);
-    a.stagger = 0;
-    if (slices == 1 && ntiles > grid) {
-        static const char* env = getenv("GEMM_STAGGER_PER_KTILE");
-        a.stagger = (env ? atoi(env) : 0) * (a.K / C::BK);
-    }
 #ifdef GEMM_TRACE
     {
         const char* tp = getenv("GEMM_TRACE_PTR");
@@ -1533,11 +1514,6 @@ int launch_stream(GemmArgs a, int slices, hipStream_t st) {
     const int num_cu = device_cu_count();
     const int64_t per_slice = slices > 1 ? (num_cu / slices > 0 ? num_cu / slices : 1) : num_cu;
     const unsigned grid = (unsigned)(ntiles < per_slice ? ntiles : per_slice);
-    a.stagger = 0;
-    if (slices == 1 && ntiles > grid) {
-        static const char* env = getenv("GEMM_STAGGER_PER_KTILE");
-        a.stagger = (env ? atoi(env) : 0) * (a.K / C::BK);
-    }
 #ifdef GEMM_TRACE
     {
         const char* tp = getenv("GEMM_TRACE_PTR");
