@@ -30,6 +30,7 @@ SIGNATURES = {
     "gpu_embed_dequant": [_P, _P, _P, _I32, _I32, _I32, _P],
     "gpu_convrot_dequant": [_I32, _P, _P, _P, _I64, _I32, _P],
     "gpu_convrot_requant": [_I32, _P, _P, _P, _I64, _I32, _U64, _P],
+    "gpu_w6_requant": [_P, _P, _P, _P, _I64, _I32, _U64, _P],
     "gpu_prologue_rows": [_I32, _I32, _P, _I64, _P, _I64, _I64, _P, _F32, _P, _P, _P, _I64, _I32, _I32, _P],
     "gpu_prologue_rows_b": [_I32, _I32, _P, _I64, _P, _P, _F32, _P, _P, _P, _I64, _I32, _I32, _P],
     "gpu_int8_gemm": [_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I32, _P],

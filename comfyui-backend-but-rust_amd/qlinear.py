@@ -112,6 +112,16 @@ def convrot_requant(w, seed=0):
     return q, s
 
 
+def w6_requant(w, seed):
+    """bf16 weight [N, K] -> (packed uint8 [N, 3K/4], s_rel e4m3 bits uint8 [N, K/32], s_channel f32 [N]), src/lora.rs:630."""
+    N, K = w.shape
+    packed = torch.empty((N, K * 3 // 4), dtype=torch.uint8, device=w.device)
+    s_rel = torch.empty((N, K // 32), dtype=torch.uint8, device=w.device)
+    s_ch = torch.empty((N,), dtype=torch.float32, device=w.device)
+    ffi.k("gpu_w6_requant", _ptr(w), _ptr(packed), _ptr(s_rel), _ptr(s_ch), N, K, seed, _stream())
+    return packed, s_rel, s_ch
+
+
 def _sd_out(M, K, dev):
     return torch.empty((M, K), dtype=torch.int8, device=dev), torch.empty((M,), dtype=torch.float32, device=dev)
 

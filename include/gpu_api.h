@@ -106,6 +106,14 @@ int gpu_embed_dequant(const int8_t* q, const float* s, float* out, int M, int K,
 int gpu_convrot_dequant(int dtype, const void* q, const void* s, void* out, int64_t N, int K, void* stream);
 int gpu_convrot_requant(int dtype, const void* x, void* q, void* s, int64_t N, int K, uint64_t seed, void* stream);
 
+/* bf16 weight [N,K] in its original basis -> the reference's W6 format: ConvRot256, two alternating-least-squares rounds
+ * for the step of every 32 columns, packed [N, 3K/4] (nibble plane then 2-bit plane, code = q + 32), s_rel fp8-e4m3
+ * [N, K/32], s_channel f32 [N]; every value is rounded stochastically between its two bracketing grid levels, keyed by
+ * element index and seed.  Replaces gpu_w6_requant, src/ffi.rs:132 / csrc/vendor/w6a8_requant.cu:242-252.
+ * K % 256 (-1), K <= 39 680 (-2: the rotated row is held in LDS). */
+int gpu_w6_requant(const void* weight, void* packed, void* s_rel, void* s_channel, int64_t N, int K, uint64_t seed,
+                   void* stream);
+
 /* D[M,N] = Out((A[M,K] . W[N,K]^T) * xs[m] * ws[n] + bias[n]).
  * Replaces gpu_int8_gemm, src/ffi.rs:38 / csrc/gemm.cu:124-129.
  * A, W int8 row-major (K contiguous); xs f32 [M]; ws f32 [N]; bias Out[N] or null; D Out[M,N]; out_dt a DT_* code. */

@@ -37,6 +37,8 @@ def lib():
         L.orc_convrot_requant.restype = i32; L.orc_convrot_requant.argtypes = [i32, vp, vp, vp, i32, i32, C.c_uint64]
         L.orc_convrot_dequant.restype = i32; L.orc_convrot_dequant.argtypes = [i32, vp, vp, vp, i64, i32]
         L.orc_dequant_i8.restype = i32; L.orc_dequant_i8.argtypes = [vp, vp, vp, i64, i64]
+        L.orc_f32_to_e4m3.restype = C.c_uint8; L.orc_f32_to_e4m3.argtypes = [f32]
+        L.orc_w6_requant.restype = i32; L.orc_w6_requant.argtypes = [vp, vp, vp, vp, i64, i32, C.c_uint64]
         L.orc_prologue_rows.restype = i32
         L.orc_prologue_rows.argtypes = [i32, i32, vp, i64, vp, i64, i64, vp, vp, f32, vp, vp, vp, i64, i32, i32]
         L.orc_sd_quant_rows.restype = i32; L.orc_sd_quant_rows.argtypes = [vp, i64, vp, vp, i32, i32, i32]
@@ -180,6 +182,17 @@ def dequant_i8(q, s):
     out = np.zeros(q.shape, np.float32)
     rc = lib().orc_dequant_i8(_p(q), _p(s), _p(out), q.shape[0], q.shape[1])
     return rc, out
+
+
+def w6_requant(w_bits, seed):
+    """bf16 weight bits [N, K] in the original basis -> (rc, packed [N, 3K/4], s_rel e4m3 bits [N, K/32], s_channel [N])."""
+    w = _c(w_bits, np.uint16)
+    N, K = w.shape
+    packed = np.zeros((N, K * 3 // 4), np.uint8)
+    s_rel = np.zeros((N, K // 32), np.uint8)
+    s_ch = np.zeros(N, np.float32)
+    rc = lib().orc_w6_requant(_p(w), _p(packed), _p(s_rel), _p(s_ch), N, K, seed)
+    return rc, packed, s_rel, s_ch
 
 
 SD_LN, SD_GEGLU, SD_UNPAD, SD_GN = 1, 2, 3, 4

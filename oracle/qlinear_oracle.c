@@ -22,6 +22,10 @@
  *                                      are provided and differ by at most one ulp of the output type.
  *   orc_e4m3_to_f32 / orc_w6_decode    pinned: exhaustive 256 bytes against torch.float8_e4m3fn; exhaustive
  *                                      64 codes x 256 scales against the definition; pack/unpack round trip
+ *   orc_f32_to_e4m3 / orc_w6_requant   encoder pinned exhaustively against torch.float8_e4m3fn casts; the requantizer by
+ *                                      its invariants (decoded weight within half a grid step of the rotated input in
+ *                                      expectation, codes 1..63, scales reproduce the least-squares steps in numpy) --
+ *                                      the fma contractions are assumptions about nvcc's default: PARITY UNPINNED
  *   orc_w6a8_group_gemm                this build's own format (no reference counterpart); integer partials pinned by
  *                                      numpy int64
  *   orc_quant_rows_wide                pinned: equals orc_quant_rows for f32, torch bf16 arithmetic on fp32 values
@@ -419,6 +423,104 @@ ORC_API void orc_w6_pack_planes(const uint8_t* codes, uint8_t* q, int64_t N, int
             hi[e / 4] |= (uint8_t)((c >> 4) << (2 * (e & 3)));
         }
     }
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * W6 requantizer, reference format: csrc/vendor/w6a8_requant.cu (one launch: bf16 weight in its original basis ->
+ * ConvRot256 -> two-plane 6-bit codes + e4m3 s_rel per 32 + f32 s_channel).  Cited by line below.  Expressions of the
+ * form a*b + c are contracted to an fma where nvcc's default would (num += w*q, den += q*q, lo + u*(hi - lo)).
+ * ------------------------------------------------------------------------------------------- */
+/* __nv_cvt_float_to_fp8(x, __NV_SATFINITE, __NV_E4M3) for finite x: round to nearest even, saturate at 448. */
+ORC_API uint8_t orc_f32_to_e4m3(float x) {
+    const uint8_t sgn = (uint8_t)((f2u(x) >> 31) << 7);
+    const float a = fabsf(x);
+    if (a != a) return (uint8_t)(sgn | 0x7f);
+    if (a > 448.f) return (uint8_t)(sgn | 0x7e);
+    if (a < 0.015625f) return (uint8_t)(sgn | (uint8_t)nearbyintf(a * 512.f));   /* subnormals: multiples of 2^-9 */
+    int ex;
+    const float f = frexpf(a, &ex);                                               /* a = f * 2^ex, f in [0.5, 1) */
+    int m = (int)nearbyintf((2.f * f - 1.f) * 8.f), e = ex - 1;
+    if (m == 8) { m = 0; ++e; }
+    const int code = ((e + 7) << 3) | m;
+    return (uint8_t)(sgn | (code > 0x7e ? 0x7e : code));
+}
+static inline float w6_level(int i, float s) {                                    /* :59-61 */
+    return fmin_dev(127.f, fmax_dev(-127.f, nearbyintf((float)(i - 31) * s)));
+}
+static inline int w6_lower_bound(float t, float s, float inv_s) {                 /* :63-69 */
+    const float est = nearbyintf((ceilf(t) - 0.5f) * inv_s);                      /* __float2int_rn saturates */
+    int i = (est > 2.0e9f ? 2000000000 : est < -2.0e9f ? -2000000000 : (int)est) + 31;
+    i = i < 0 ? 0 : i > 63 ? 63 : i;
+    while (i > 0 && w6_level(i - 1, s) >= t) --i;
+    while (i < 63 && w6_level(i, s) < t) ++i;
+    return i;
+}
+static inline float rq_uniform(int64_t idx, uint64_t seed) {                      /* :27-31 */
+    const uint32_t h = pcg_hash((uint32_t)idx ^ (uint32_t)seed ^ (uint32_t)(seed >> 32));
+    return (float)(h >> 8) * (1.0f / 16777216.0f);
+}
+ORC_API int orc_w6_requant(const uint16_t* w, uint8_t* packed, uint8_t* s_rel, float* s_channel, int64_t N, int K,
+                           uint64_t seed) {
+    if (K % 256) return -1;                                                        /* :243 */
+    enum { G = 32 };
+    float* row = (float*)malloc(sizeof(float) * (size_t)K);
+    float* gscale = (float*)malloc(sizeof(float) * (size_t)(K / G));
+    for (int64_t n = 0; n < N; ++n) {
+        /* rotation, the result rounded to the weight dtype: :174-218 (the butterflies of orc_fht, group 256) */
+        for (int k = 0; k < K; ++k) row[k] = orc_bf16_to_f32(w[n * K + k]);
+        orc_fht(row, K, 256);
+        for (int k = 0; k < K; ++k) row[k] = orc_bf16_round(row[k]);
+        /* phase 1: per-group step, two alternating-least-squares rounds; row amax of the decoded weight (:94-120) */
+        float row_amax = 0.f;
+        for (int g = 0; g < K / G; ++g) {
+            const float* x = row + g * G;
+            float amax = 0.f;
+            for (int i = 0; i < G; ++i) amax = fmax_dev(amax, fabsf(x[i]));
+            float gs = fmax_dev(amax / 31.0f, 1e-8f), inv = 1.0f / gs;
+            for (int it = 0; it < 2; ++it) {
+                float num = 0.f, den = 0.f;
+                for (int i = 0; i < G; ++i) {
+                    const float q = fmin_dev(31.0f, fmax_dev(-31.0f, nearbyintf(x[i] * inv)));
+                    num = fmaf(x[i], q, num);
+                    den = fmaf(q, q, den);
+                }
+                gs = fmax_dev(num / fmax_dev(den, 1e-8f), 1e-8f);
+                inv = 1.0f / gs;
+            }
+            gscale[g] = gs;
+            for (int i = 0; i < G; ++i)
+                row_amax = fmax_dev(row_amax, fabsf(fmin_dev(31.0f, fmax_dev(-31.0f, nearbyintf(x[i] * inv))) * gs));
+        }
+        const float sc = fmax_dev(row_amax / 127.0f, 1e-8f), inv_sc = 1.0f / sc;    /* :121-123 */
+        s_channel[n] = sc;
+        /* phase 2: e4m3 s_rel, stochastic grid assignment (the launcher always passes stochastic = true, :249),
+         * code = level index + 1 = q + 32, two-plane pack (:126-151) */
+        uint8_t* lo = packed + n * (K * 3 / 4);
+        uint8_t* hi = lo + K / 2;
+        memset(lo, 0, (size_t)(K * 3 / 4));
+        for (int g = 0; g < K / G; ++g) {
+            const uint8_t bits = orc_f32_to_e4m3(gscale[g] / sc);
+            s_rel[n * (K / G) + g] = bits;
+            const float sr = orc_e4m3_to_f32(bits), inv_sr = 1.0f / fmax_dev(sr, 1e-30f);
+            for (int i = 0; i < G; ++i) {
+                const int e = g * G + i;
+                const float t = row[e] * inv_sc;
+                const int pos = w6_lower_bound(t, sr, inv_sr);
+                int l = pos - 1;                                                  /* :75-80 */
+                l = l < 0 ? 0 : l > 61 ? 61 : l;
+                const float level_lo = w6_level(l, sr);
+                const float thr = fmaf(rq_uniform(n * K + e, seed), w6_level(l + 1, sr) - level_lo, level_lo);
+                int lev = l + (t > thr ? 1 : 0);
+                lev = lev > 62 ? 62 : lev;
+                const unsigned c = (unsigned)(lev + 1);
+                lo[e / 2] |= (uint8_t)((c & 0xFu) << (4 * (e & 1)));
+                hi[e / 4] |= (uint8_t)((c >> 4) << (2 * (e & 3)));
+            }
+        }
+    }
+    free(row);
+    free(gscale);
+    return 0;
 }
 
 /* ---------------------------------------------------------------------------------------------

@@ -408,6 +408,31 @@ def test_convrot_requant_bit_exact(N, K, dt):
     assert ffi.raw("gpu_convrot_requant", 0, xd.data_ptr(), qd.data_ptr(), sd.data_ptr(), N, 300, 0, 0) == -1
 
 
+@pytest.mark.parametrize("N,K", [(5, 256), (33, 3072), (3, 13824), (300, 512)])
+def test_w6_requant_bit_exact(N, K):
+    say("w6_requant", N, K)
+    w = synth.normal(70 + K, 1, N * K).reshape(N, K) * np.float32(0.04)
+    w[0, :32] = 0
+    if N > 2:
+        w[2, :] = 0
+    wb = synth.bf16_bits(w)
+    wd = dev_bits(wb, BF16)
+    for seed in (0, 99, 2 ** 40 + 5):
+        rc, packed, s_rel, s_ch = oracle.w6_requant(wb, seed)
+        pd, rd, cd = ql.w6_requant(wd, seed)
+        torch.cuda.synchronize()
+        assert rc == 0
+        assert np.array_equal(cd.cpu().numpy().view(np.uint32), s_ch.view(np.uint32)), seed
+        assert np.array_equal(rd.cpu().numpy(), s_rel), seed
+        assert np.array_equal(pd.cpu().numpy(), packed), seed
+    # what it writes is what gpu_w6_decode reads
+    rc, grid = oracle.w6_decode(packed, s_rel, N, K, 32)
+    got = ql.w6_decode(pd, rd, N, K, 32)
+    torch.cuda.synchronize()
+    assert np.array_equal(got.cpu().numpy(), grid)
+    assert ffi.raw("gpu_w6_requant", wd.data_ptr(), pd.data_ptr(), rd.data_ptr(), cd.data_ptr(), N, 300, 1, 0) == -1
+
+
 # ------------------------------------------------------------------------------------------------ dense GEMM
 @pytest.mark.parametrize("in_dt,out_dt", [(torch.bfloat16, torch.bfloat16), (torch.float16, torch.float16),
                                           (torch.float32, torch.float32), (torch.bfloat16, torch.float32)])

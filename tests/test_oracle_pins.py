@@ -796,3 +796,73 @@ def test_bf16_add_with_one_rounding():
             assert int(got / ulp) % 2 == 0
     # 100 + 0.2578125 (= 0.25 + 2^-7): the exact sum lies above the tie 100.25 and rounds up to 100.5
     assert L.orc_bf16_add_once(100.0, 0.2578125) == 100.5
+
+
+# ----------------------------------------------------------------------------------------------- W6 requantizer
+def test_e4m3_encoder_matches_torch_float8():
+    L = oracle.lib()
+    rng = np.random.default_rng(9)
+    # every code, every midpoint between neighbouring codes, and random values inside the finite range
+    vals = np.array([oracle.lib().orc_e4m3_to_f32(b) for b in range(0x7f)], np.float32)
+    mids = ((vals[:-1].astype(np.float64) + vals[1:]) / 2).astype(np.float32)
+    x = np.concatenate([vals, mids, np.nextafter(mids, np.float32(0)), np.nextafter(mids, np.float32(1000)),
+                        (rng.random(20000) * 448).astype(np.float32), (rng.random(5000) * 0.05).astype(np.float32)])
+    x = np.concatenate([x, -x])
+    want = torch.from_numpy(x).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    got = np.array([L.orc_f32_to_e4m3(float(v)) for v in x], np.uint8)
+    same = (got == want) | ((got & 0x7f) == 0) & ((want & 0x7f) == 0)          # +0 and -0 of tiny inputs
+    assert same.all(), (x[~same][:5], got[~same][:5], want[~same][:5])
+    assert L.orc_f32_to_e4m3(1.0e6) == 0x7e and L.orc_f32_to_e4m3(-500.0) == 0xfe   # saturating, unlike torch's cast
+
+
+def w6_codes_of(packed, K):
+    lo, hi = packed[:, :K // 2], packed[:, K // 2:]
+    e = np.arange(K)
+    return ((lo[:, e // 2] >> (4 * (e & 1))) & 0xF) | (((hi[:, e // 4] >> (2 * (e & 3))) & 3) << 4)
+
+
+def test_w6_requant_invariants_and_closed_form(synth):
+    N, K = 6, 768
+    w = synth.normal(41, 1, N * K).reshape(N, K) * np.float32(0.04)
+    wb = oracle.bf16_bits(w)
+    rc, packed, s_rel, s_ch = oracle.w6_requant(wb, 7)
+    assert rc == 0 and (s_ch > 0).all()
+    codes = w6_codes_of(packed, K)
+    assert codes.min() >= 1 and codes.max() <= 63
+    # the rotated row (bf16) the codes describe
+    rot = np.einsum("ngk,jk->ngj", oracle.bf16_to_f32(wb).astype(np.float64).reshape(N, K // 256, 256), kron_h(4)).reshape(N, K)
+    rot = oracle.bf16_to_f32(oracle.bf16_bits(rot.astype(np.float32))).astype(np.float64)
+    # decoded weight: the int8 grid of gpu_w6_decode times the row scale; stochastic rounding picks one of the two bracketing
+    # levels, so the error is below one level spacing (s_rel * s_channel, plus the rounding of the level to an integer)
+    rc2, grid = oracle.w6_decode(packed, s_rel, N, K, 32)
+    dec = grid.astype(np.float64) * s_ch[:, None]
+    sr = np.array([[oracle.lib().orc_e4m3_to_f32(int(b)) for b in r] for r in s_rel], np.float64)
+    step = (np.repeat(sr, 32, axis=1) + 1.0) * s_ch[:, None]
+    err = dec - rot
+    inside = np.abs(rot) <= 30.5 * np.repeat(sr, 32, axis=1) * s_ch[:, None]        # beyond the last level values clip
+    assert (np.abs(err)[inside] <= step[inside] * 1.001).all()
+    assert abs(err[inside].mean()) < 0.03 * step.mean()                              # unbiased
+    # the group steps are the least-squares steps: restated in numpy (float64), compared through the e4m3 rounding
+    x = rot.reshape(N, K // 32, 32)
+    gs = np.maximum(np.abs(x).max(-1) / 31, 1e-8)
+    for _ in range(2):
+        q = np.clip(np.rint(x / gs[..., None]), -31, 31)
+        gs = np.maximum((x * q).sum(-1) / np.maximum((q * q).sum(-1), 1e-8), 1e-8)
+    q = np.clip(np.rint(x / gs[..., None]), -31, 31)
+    sc = np.maximum(np.abs(q * gs[..., None]).max(axis=(1, 2)) / 127, 1e-8)
+    assert np.allclose(s_ch, sc, rtol=1e-5)
+    assert np.allclose(sr, gs / sc[:, None], rtol=2.0 ** -4)
+    # same seed, same bits; another seed moves codes but not scales
+    again = oracle.w6_requant(wb, 7)
+    assert np.array_equal(again[1], packed) and np.array_equal(again[2], s_rel)
+    other = oracle.w6_requant(wb, 8)
+    assert np.array_equal(other[2], s_rel) and np.array_equal(other[3], s_ch)
+    d = np.abs(w6_codes_of(other[1], K).astype(int) - codes.astype(int))
+    assert d.max() <= 1 and 0.05 < (d != 0).mean() < 0.6
+    assert oracle.w6_requant(wb[:, :300], 1)[0] == -1
+    # closed form: a constant row is an eigenvector of the rotation (eigenvalue 1); with c = 31 * 2^-6 every group has
+    # step 2^-6, the row scale is c/127, s_rel = e4m3(127/31 = 4.097) = 4.0 (0x48), t = 127 lies above the last level pair
+    # (120, 124), so every code is 63 whatever the draw
+    c = np.float32(31 * 2.0 ** -6)
+    rc, p1, r1, s1 = oracle.w6_requant(oracle.bf16_bits(np.full((1, 256), c, np.float32)), 12345)
+    assert (w6_codes_of(p1, 256) == 63).all() and (r1 == 0x48).all() and s1[0] == c / np.float32(127)
