@@ -119,7 +119,7 @@ def w6_srel_bytes(seed, N, K, G=32):
 
 
 def config0(seed=0):
-    """BASELINE config 0: X bf16 [256,1024] with 8 outlier columns x20; W int8 [1024,1024]; per-channel scales; bias."""
+    """The CPU-runnable anchor case: X bf16 [256,1024] with 8 outlier columns x20; W int8 [1024,1024]; per-channel scales; bias."""
     M, K, N = 256, 1024, 1024
     x = activations(seed, M, K, "normal", C0_OUTLIER_COLS)
     W, ws, bias = w8_weights(seed, N, K)

@@ -530,6 +530,14 @@ def test_int8_gemm_many_tiles_bit_exact(M, N, K):
     assert np.array_equal(got.cpu().numpy(), want)
     assert np.array_equal(host_bits(d), want_d)
     assert np.array_equal(host_bits(r), want_r)
+    if M == 4352:   # the other output types through the same split into 256x256 rounds and a 128x192 remainder
+        for dt, tdt, tob in ((F32, torch.float32, lambda a: a.astype(np.float32)), (F16, torch.float16, oracle.f16_bits)):
+            b2 = tob(synth.normal(4, 5, N) * np.float32(0.02))
+            w2 = oracle.epilogue(want, xs, ws, b2, dt, fma=1)
+            d2 = ql.int8_gemm(Ad, Wd, dev(xs), dev(ws), dev_bits(b2, dt), tdt)
+            torch.cuda.synchronize()
+            view = np.uint32 if dt == F32 else np.uint16
+            assert np.array_equal(host_bits(d2).view(view), w2.view(view)), dt
 
 
 @pytest.mark.parametrize("out_dt", [BF16, F16, F32])
