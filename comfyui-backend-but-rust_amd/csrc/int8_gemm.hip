@@ -1481,6 +1481,15 @@ int launch_ring(GemmArgs a, hipStream_t st) {
     return launch_ring_cfg<RingL, OUT_DT, EPI>(a, 1, st);
 }
 
+// The 128x192 ring kernel on the whole problem: shapes with too few 256x256 tiles to fill the CUs.
+template <int OUT_DT, int EPI>
+int launch_ring_small(GemmArgs a, hipStream_t st) {
+    bool vec_ok, aligned;
+    epilogue_alignment<OUT_DT, EPI>(a, vec_ok, aligned);
+    if (!aligned) return launch_cfg<CfgM, OUT_DT, EPI>(a, st);
+    return launch_ring_cfg<RingS, OUT_DT, EPI>(a, 1, st);
+}
+
 // Keep freed scratch in the device's default pool instead of returning it to the driver at every synchronization, as
 // the reference's runtime layer does at start-up (src/cuda.rs:88-97): otherwise each call that needs scratch pays a
 // fresh allocation.
@@ -1593,6 +1602,9 @@ int choose_cfg(int64_t M, int64_t N, int64_t K) {
     if (M <= 256 && N >= 1024 && (K % 128) == 0 && K >= 512 && dma_ok) return 6;
     const int64_t tiles_l = ((M + 255) / 256) * ((N + 255) / 256);
     if (M >= 512 && N >= 512 && tiles_l >= 192) return !dma_ok ? 0 : (K % 128) == 0 ? 5 : (K % 64) == 0 ? 3 : 0;
+    // too few 256x256 tiles for the CUs: the persistent kernel on 128x192 tiles, where those fill at least a third of them
+    const int64_t tiles_s = ((M + 127) / 128) * ((N + 191) / 192);
+    if (dma_ok && (K % 128) == 0 && M > 128 && N >= 192 && tiles_s >= 96) return 7;
     const int64_t tiles_m = ((M + 127) / 128) * ((N + 127) / 128);
     if (M > 64 && N > 64 && tiles_m >= 128) return 1;
     return 2;
@@ -1605,6 +1617,7 @@ int dispatch_cfg(const GemmArgs& a, hipStream_t st) {
         case 4: return launch_dma2<Dma2L, OUT_DT, EPI>(a, st);
         case 5: return launch_ring<OUT_DT, EPI>(a, st);
         case 6: return launch_skinny<OUT_DT, EPI>(a, st);
+        case 7: return launch_ring_small<OUT_DT, EPI>(a, st);
         case 0: return launch_cfg<CfgL, OUT_DT, EPI>(a, st);
         case 1: return launch_cfg<CfgM, OUT_DT, EPI>(a, st);
         default: return launch_cfg<CfgS, OUT_DT, EPI>(a, st);
@@ -1669,7 +1682,8 @@ GPU_API int gpu_int8_gemm_acc(const int8_t* A, const int8_t* W, int32_t* acc, in
     return rc < 0 ? -200 : rc;
 }
 
-// Test hook: force a tile configuration (0 = 256x256, 1 = 128x128, 2 = 64x64, -1 = automatic).
+// Test hook: force a kernel family (0 = 256x256, 1 = 128x128, 2 = 64x64 register-staged tiles; 3, 4 = the earlier
+// direct-to-LDS kernels; 5 = persistent ring, 256x256; 6 = weight streaming; 7 = persistent ring, 128x192; -1 = automatic).
 GPU_API int gpu_int8_gemm_force_config(int cfg) {
     g_force_cfg = cfg;
     return 0;

@@ -486,7 +486,7 @@ ACC_CASES = [(1, 96, 256), (3, 32, 16), (64, 64, 64), (65, 72, 48), (100, 104, 3
              (77, 4096, 1280), (250, 25000, 128)]
 
 
-@pytest.mark.parametrize("cfg", [2, 1, 0, 3, 4, 5, 6])
+@pytest.mark.parametrize("cfg", [2, 1, 0, 3, 4, 5, 6, 7])
 @pytest.mark.parametrize("M,N,K", ACC_CASES)
 def test_int8_gemm_acc_bit_exact(M, N, K, cfg):
     say("gemm_acc", M, N, K, "cfg", cfg)
@@ -541,7 +541,8 @@ def test_int8_gemm_many_tiles_bit_exact(M, N, K):
 
 
 @pytest.mark.parametrize("out_dt", [BF16, F16, F32])
-@pytest.mark.parametrize("M,N,K,with_bias", [(37, 96, 256, True), (130, 264, 192, False), (256, 1024, 1024, True), (100, 2048, 1024, True)])
+@pytest.mark.parametrize("M,N,K,with_bias", [(37, 96, 256, True), (130, 264, 192, False), (256, 1024, 1024, True), (100, 2048, 1024, True),
+                                                     (4100, 648, 384, True)])
 def test_int8_gemm_epilogue(M, N, K, with_bias, out_dt):
     say("gemm", M, N, K, with_bias, out_dt)
     A = rand_i8(2, 1, M, K, -127, 127)
