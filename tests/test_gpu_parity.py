@@ -433,6 +433,50 @@ def test_w6_requant_bit_exact(N, K):
     assert ffi.raw("gpu_w6_requant", wd.data_ptr(), pd.data_ptr(), rd.data_ptr(), cd.data_ptr(), N, 300, 1, 0) == -1
 
 
+def test_checkpoint_linears_run_like_the_reference_sequence(tmp_path):
+    """Weights as the reference's checkpoints store them (safetensors: int8 ConvRot with row scales, W6 triplet, dense),
+    loaded and run through quantize -> GEMM; int8 and W6 outputs bit-exact against the oracle's sequence."""
+    from safetensors import safe_open
+    from safetensors.torch import save_file
+    wts = pkg("weights")
+    N, K, M = 96, 512, 40
+    W = synth.randint(81, 1, N * K, -127, 127).astype(np.int8).reshape(N, K)
+    ws = synth.uniform(81, 2, N, 1e-3, 1e-2)
+    bias = oracle.bf16_bits(synth.normal(81, 3, N) * np.float32(0.02))
+    codes = (synth.w6_codes(81, N, K).astype(np.int16) + 32).astype(np.uint8)
+    packed = oracle.w6_pack_planes(codes)
+    s_rel = synth.randint(81, 4, N * (K // 32), 0x38, 0x48).astype(np.uint8).reshape(N, K // 32)
+    s_ch = synth.uniform(81, 5, N, 1e-3, 1e-2)
+    dense = synth.normal(81, 6, N * K).reshape(N, K) * np.float32(0.05)
+    path = str(tmp_path / "m.safetensors")
+    save_file({
+        "a.weight": torch.from_numpy(W), "a.weight_scale": torch.from_numpy(ws),
+        "a.bias": torch.from_numpy(bias.view(np.int16)).view(torch.bfloat16),
+        "a.comfy_quant": torch.tensor(list(json.dumps({"format": "int8_tensorwise", "convrot": True, "convrot_groupsize": 256}).encode()), dtype=torch.uint8),
+        "b.weight": torch.from_numpy(packed), "b.weight_s_rel": torch.from_numpy(s_rel).view(torch.float8_e4m3fn),
+        "b.weight_s_channel": torch.from_numpy(s_ch),
+        "c.weight": torch.from_numpy(oracle.bf16_bits(dense).view(np.int16)).view(torch.bfloat16),
+    }, path)
+    xb = synth.bf16_bits(synth.activations(82, M, K, "t3"))
+    x = dev_bits(xb, BF16)
+    rc, q, xs = oracle.quant_rows(BF16, xb, K, 1)
+    with safe_open(path, framework="pt") as st:
+        a = wts.load_linear(st, "a", DEV)
+        b = wts.load_linear(st, "b", DEV)
+        c = wts.load_linear(st, "c", DEV)
+    ya = wts.forward(a, x)
+    yb = wts.forward(b, x)
+    yc = wts.forward(c, x)
+    torch.cuda.synchronize()
+    want_a = oracle.epilogue(oracle.int8_gemm_acc(q, W), xs, ws, bias, BF16, fma=1)
+    assert np.array_equal(host_bits(ya), want_a)
+    rc, grid = oracle.w6_decode(packed, s_rel, N, K, 32)
+    want_b = oracle.epilogue(oracle.int8_gemm_acc(q, grid), xs, s_ch, None, BF16, fma=1)
+    assert np.array_equal(host_bits(yb), want_b)
+    ref = oracle.bf16_to_f32(xb).astype(np.float64) @ oracle.bf16_to_f32(oracle.bf16_bits(dense)).astype(np.float64).T
+    assert np.allclose(yc.float().cpu().numpy(), ref, rtol=2.0 ** -7, atol=1e-3)
+
+
 # ------------------------------------------------------------------------------------------------ dense GEMM
 @pytest.mark.parametrize("in_dt,out_dt", [(torch.bfloat16, torch.bfloat16), (torch.float16, torch.float16),
                                           (torch.float32, torch.float32), (torch.bfloat16, torch.float32)])

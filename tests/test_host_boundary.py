@@ -127,3 +127,56 @@ def test_oracle_reproduces_golden_fixtures(synth):
     for grp in (64, 128, 256):
         rc, q2, s2 = oracle.quant_rows(oracle.BF16, xr, 1024, grp)
         assert dig(q2) == r["q_g%d_sha256" % grp] and dig(s2.view(np.uint32)) == r["xs_bits_g%d_sha256" % grp]
+
+
+def _write_checkpoint(path, extra=None, groupsize=256, scalar_scale=False):
+    import torch
+    from safetensors.torch import save_file
+    g = torch.Generator().manual_seed(3)
+    N, K = 64, 512
+    t = {
+        "blk.fc.weight": torch.randint(-127, 128, (N, K), dtype=torch.int8, generator=g),
+        "blk.fc.weight_scale": torch.tensor([0.01]) if scalar_scale else torch.rand(N, generator=g) * 0.01 + 0.001,
+        "blk.fc.bias": (torch.randn(N, generator=g) * 0.02).to(torch.bfloat16),
+        "blk.fc.comfy_quant": torch.tensor(list(json.dumps({"format": "int8_tensorwise", "convrot": True,
+                                                            "convrot_groupsize": groupsize}).encode()), dtype=torch.uint8),
+        "blk.w6.weight": torch.randint(0, 256, (N, K * 3 // 4), dtype=torch.uint8, generator=g),
+        "blk.w6.weight_s_rel": torch.randint(0x30, 0x50, (N, K // 32), dtype=torch.uint8, generator=g).view(torch.float8_e4m3fn),
+        "blk.w6.weight_s_channel": torch.rand(N, generator=g) * 0.01,
+        "blk.dense.weight": torch.randn(N, K, generator=g).to(torch.bfloat16),
+    }
+    t.update(extra or {})
+    save_file(t, path)
+    return t
+
+
+def test_checkpoint_layouts_are_read_like_the_reference(tmp_path):
+    import torch
+    from safetensors import safe_open
+    wts = pkg("weights")
+    p = str(tmp_path / "a.safetensors")
+    t = _write_checkpoint(p)
+    with safe_open(p, framework="pt") as st:
+        fc = wts.load_linear(st, "blk.fc", device="cpu")
+        assert fc.kind == "int8_convrot" and (fc.n, fc.k) == (64, 512) and fc.scale.shape == (64,)
+        assert torch.equal(fc.weight, t["blk.fc.weight"]) and fc.bias.dtype == torch.bfloat16
+        w6 = wts.load_linear(st, "blk.w6", device="cpu")
+        assert w6.kind == "w6" and (w6.n, w6.k) == (64, 512) and w6.s_rel.dtype == torch.uint8 and w6.s_rel.shape == (64, 16)
+        assert wts.load_linear(st, "blk.dense", device="cpu").kind == "dense"
+    # one scale for all rows is expanded on the host (src/relayvsr.rs:141-149)
+    p2 = str(tmp_path / "b.safetensors")
+    _write_checkpoint(p2, scalar_scale=True)
+    with safe_open(p2, framework="pt") as st:
+        s = wts.load_linear(st, "blk.fc", device="cpu").scale
+        assert s.shape == (64,) and (s == s[0]).all()
+    # other group sizes and scale counts are refused
+    p3 = str(tmp_path / "c.safetensors")
+    _write_checkpoint(p3, groupsize=64)
+    with safe_open(p3, framework="pt") as st:
+        with pytest.raises(wts.CheckpointError, match="groups of 256"):
+            wts.load_linear(st, "blk.fc", device="cpu")
+    p4 = str(tmp_path / "d.safetensors")
+    _write_checkpoint(p4, extra={"blk.fc.weight_scale": torch.ones(7)})
+    with safe_open(p4, framework="pt") as st:
+        with pytest.raises(wts.CheckpointError, match="7 weight scales for 64 rows"):
+            wts.load_linear(st, "blk.fc", device="cpu")
