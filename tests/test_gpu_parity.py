@@ -477,6 +477,58 @@ def test_checkpoint_linears_run_like_the_reference_sequence(tmp_path):
     assert np.allclose(yc.float().cpu().numpy(), ref, rtol=2.0 ** -7, atol=1e-3)
 
 
+def test_dit_block_linear_chain_matches_oracle_composition():
+    """The linear launches of one DiT block in the order and with the argument patterns of src/dit.rs:545-611: RMS +
+    modulation prologue -> fused QKV+gate GEMM; gate prologue reading the gate columns inside the QKV buffer -> output
+    projection with the residual added in place; RMS + modulation -> MLP gate|up GEMM; SwiGLU prologue on the two halves of
+    that buffer -> down projection with the residual in place.  (Attention itself is outside this path: the q columns
+    stand in for its output.)  The final hidden state must equal the oracle's composition bit for bit."""
+    rows, F, QKV, MLP, eps = 70, 512, 1024, 1024, 1e-6
+    QKVG = QKV + F
+    rnd = lambda st, *shape: synth.normal(91, st, int(np.prod(shape))).reshape(shape)
+    wq = lambda st, n, k: synth.randint(91, st, n * k, -127, 127).astype(np.int8).reshape(n, k)
+    x0 = synth.bf16_bits(rnd(1, rows, F))
+    pre, post = (1 + 0.1 * rnd(2, F)).astype(np.float32), (1 + 0.1 * rnd(3, F)).astype(np.float32)
+    mv = [synth.bf16_bits(0.2 * rnd(10 + i, F)) for i in range(6)]
+    Wqkvg, Wo, Wgu, Wd = wq(20, QKVG, F), wq(21, F, F), wq(22, 2 * MLP, F), wq(23, F, MLP)
+    sc = lambda st, n: synth.uniform(91, st, n, 2e-4, 1e-3)
+    sqkvg, so, sgu, sd = sc(30, QKVG), sc(31, F), sc(32, 2 * MLP), sc(33, F)
+
+    # oracle composition
+    def o_quant(pro, xb, K, **kw):
+        rc, row = oracle.prologue_rows(BF16, pro, xb, K, **kw)
+        rc2, q, s = oracle.quant_rows(BF16, row, K, 1)
+        assert rc == 0 and rc2 == 0
+        return q, s
+    x = x0.copy()
+    q, s = o_quant(1, x, F, norm_w=pre, eps=eps, mod_scale=mv[0], mod_shift=mv[1])
+    qkvg = oracle.epilogue(oracle.int8_gemm_acc(q, Wqkvg), s, sqkvg, None, BF16, fma=1)
+    attn = np.ascontiguousarray(qkvg[:, :F])
+    q, s = o_quant(2, attn, F, g=np.ascontiguousarray(qkvg[:, QKV:]))
+    x = oracle.epilogue_residual(oracle.int8_gemm_acc(q, Wo), s, so, None, mv[2], x, BF16, fma=1)
+    q, s = o_quant(1, x, F, norm_w=post, eps=eps, mod_scale=mv[3], mod_shift=mv[4])
+    gu = oracle.epilogue(oracle.int8_gemm_acc(q, Wgu), s, sgu, None, BF16, fma=1)
+    q, s = o_quant(3, gu, MLP, up_offset=MLP)
+    x = oracle.epilogue_residual(oracle.int8_gemm_acc(q, Wd), s, sd, None, mv[5], x, BF16, fma=1)
+
+    # the same launches through the C ABI
+    xd = dev_bits(x0, BF16)
+    mvd = [dev_bits(m, BF16) for m in mv]
+    a8, asc = ql.quant_rows_pro(xd, ffi.PRO_RMS, F, 1, norm_w=dev(pre), eps=eps, mod_scale=mvd[0], mod_shift=mvd[1])
+    qkvg_d = ql.int8_gemm(a8, dev(Wqkvg), asc, dev(sqkvg), None, torch.bfloat16)
+    attn_d = qkvg_d[:, :F].contiguous()
+    gate_view = qkvg_d[:, QKV:]                               # the gate columns where they lie: row stride QKVG
+    a8, asc = ql.quant_rows_pro(attn_d, ffi.PRO_GATE, F, 1, g=gate_view)
+    ql.int8_gemm_residual(a8, dev(Wo), asc, dev(so), None, mvd[2], xd, D=xd)
+    a8, asc = ql.quant_rows_pro(xd, ffi.PRO_RMS, F, 1, norm_w=dev(post), eps=eps, mod_scale=mvd[3], mod_shift=mvd[4])
+    gu_d = ql.int8_gemm(a8, dev(Wgu), asc, dev(sgu), None, torch.bfloat16)
+    a8, asc = ql.quant_rows_pro(gu_d, ffi.PRO_SWIGLU, MLP, 1, up_offset=MLP)
+    ql.int8_gemm_residual(a8, dev(Wd), asc, dev(sd), None, mvd[5], xd, D=xd)
+    torch.cuda.synchronize()
+    assert np.array_equal(host_bits(qkvg_d), qkvg) and np.array_equal(host_bits(gu_d), gu)
+    assert np.array_equal(host_bits(xd), x)
+
+
 # ------------------------------------------------------------------------------------------------ dense GEMM
 @pytest.mark.parametrize("in_dt,out_dt", [(torch.bfloat16, torch.bfloat16), (torch.float16, torch.float16),
                                           (torch.float32, torch.float32), (torch.bfloat16, torch.float32)])
