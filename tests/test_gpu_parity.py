@@ -529,6 +529,37 @@ def test_dit_block_linear_chain_matches_oracle_composition():
     assert np.array_equal(host_bits(xd), x)
 
 
+def test_unet_feed_forward_chain_matches_oracle_composition():
+    """The feed-forward of an SD/SDXL transformer block as src/unet.rs:429-456 launches it, fp16 throughout: LayerNorm
+    fused into the quantizer -> GEGLU up-projection with bias; GEGLU fused into the quantizer -> down-projection added to
+    the hidden state in place (residual scale of ones)."""
+    M, C, I, rot = 130, 640, 2560, 64
+    rnd = lambda st, *shape: synth.normal(95, st, int(np.prod(shape))).reshape(shape)
+    wq = lambda st, n, k: synth.randint(95, st, n * k, -127, 127).astype(np.int8).reshape(n, k)
+    x0 = synth.f16_bits(rnd(1, M, C))
+    lw, lb = (1 + 0.1 * rnd(2, C)).astype(np.float32), (0.05 * rnd(3, C)).astype(np.float32)
+    Wup, Wdn = wq(4, 2 * I, C), wq(5, C, I)
+    sup, sdn = synth.uniform(95, 6, 2 * I, 2e-4, 1e-3), synth.uniform(95, 7, C, 1e-4, 5e-4)
+    bup, bdn = synth.f16_bits(0.02 * rnd(8, 2 * I)), synth.f16_bits(0.02 * rnd(9, C))
+    ones = synth.f16_bits(np.ones(C, np.float32))
+    # oracle
+    rc, row = oracle.sd_source_rows(oracle.SD_LN, x0, M, C, x_stride=C, w=lw, b=lb, eps=1e-5)
+    rc, q, s = oracle.sd_quant_rows(row, C, rot)
+    h = oracle.epilogue(oracle.int8_gemm_acc(q, Wup), s, sup, bup, F16, fma=1)
+    rc, row = oracle.sd_source_rows(oracle.SD_GEGLU, h, M, I)
+    rc, q, s = oracle.sd_quant_rows(row, I, rot)
+    want = oracle.epilogue_residual(oracle.int8_gemm_acc(q, Wdn), s, sdn, bdn, ones, x0, F16, fma=1)
+    # C ABI
+    xd = dev_bits(x0, F16)
+    a8, asc = ql.sd_ln_quant_rows(xd, dev(lw), dev(lb), 1e-5, rot)
+    hd = ql.int8_gemm(a8, dev(Wup), asc, dev(sup), dev_bits(bup, F16), torch.float16)
+    a8, asc = ql.sd_geglu_quant_rows(hd, rot)
+    ql.int8_gemm_residual(a8, dev(Wdn), asc, dev(sdn), dev_bits(bdn, F16), dev_bits(ones, F16), xd, D=xd)
+    torch.cuda.synchronize()
+    assert np.array_equal(host_bits(hd), h)
+    assert np.array_equal(host_bits(xd), want)
+
+
 # ------------------------------------------------------------------------------------------------ dense GEMM
 @pytest.mark.parametrize("in_dt,out_dt", [(torch.bfloat16, torch.bfloat16), (torch.float16, torch.float16),
                                           (torch.float32, torch.float32), (torch.bfloat16, torch.float32)])
