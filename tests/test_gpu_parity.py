@@ -560,6 +560,38 @@ def test_unet_feed_forward_chain_matches_oracle_composition():
     assert np.array_equal(host_bits(xd), want)
 
 
+def test_text_encoder_mlp_chain_weight_only_int8():
+    """A text-encoder MLP as src/te.rs:490-513 runs it: weight-only int8 ConvRot weights, fp32 activations rotated
+    instead of the weights (x @ ((q s) H)^T == (x H) @ (q s)^T), fp32 GEMMs, the residual through beta = 1.  The rotated
+    rows are bit-exact against the oracle; the GEMM results are checked against float64."""
+    M, D, FF, eps = 24, 512, 1024, 1e-6
+    rnd = lambda st, *shape: synth.normal(97, st, int(np.prod(shape))).reshape(shape)
+    wq = lambda st, n, k: synth.randint(97, st, n * k, -127, 127).astype(np.int8).reshape(n, k)
+    x0 = rnd(1, M, D).astype(np.float32)
+    ln = (1 + 0.1 * rnd(2, D)).astype(np.float32)
+    Wgu, Wd = wq(3, 2 * FF, D), wq(4, D, FF)
+    sgu, sd = synth.uniform(97, 5, 2 * FF, 2e-4, 1e-3), synth.uniform(97, 6, D, 2e-4, 1e-3)
+    # oracle for the rotated rows, float64 for the products
+    rc, row = oracle.prologue_rows(F32, 1, x0, D, norm_w=ln, eps=eps)
+    rc, xr = oracle.rotate_rows_f32(row, D)
+    gu64 = xr.astype(np.float64) @ (Wgu.astype(np.float64) * sgu[:, None].astype(np.float64)).T
+    xd = dev(x0)
+    xr_d = ql.rotate_rows_f32(xd, D, ffi.PRO_RMS, 0, dev(ln), eps)
+    gu_d = ql.gemm(xr_d, ql.dequant_i8(dev(Wgu), dev(sgu)), None, True, torch.float32)
+    torch.cuda.synchronize()
+    assert np.array_equal(xr_d.cpu().numpy().view(np.uint32), xr.view(np.uint32))
+    assert np.allclose(gu_d.cpu().numpy(), gu64, rtol=1e-4, atol=1e-4)
+    gu = gu_d.cpu().numpy()
+    rc, row2 = oracle.prologue_rows(F32, 3, gu, FF, up_offset=FF)
+    rc, xr2 = oracle.rotate_rows_f32(row2, FF)
+    xr2_d = ql.rotate_rows_f32(gu_d, FF, ffi.PRO_SWIGLU, FF)
+    out = ql.gemm(xr2_d, ql.dequant_i8(dev(Wd), dev(sd)), None, True, torch.float32, beta=1.0, D=xd)   # x += mlp(x)
+    torch.cuda.synchronize()
+    assert np.array_equal(xr2_d.cpu().numpy().view(np.uint32), xr2.view(np.uint32))
+    want = x0.astype(np.float64) + xr2.astype(np.float64) @ (Wd.astype(np.float64) * sd[:, None].astype(np.float64)).T
+    assert np.allclose(out.cpu().numpy(), want, rtol=1e-4, atol=1e-4)
+
+
 # ------------------------------------------------------------------------------------------------ dense GEMM
 @pytest.mark.parametrize("in_dt,out_dt", [(torch.bfloat16, torch.bfloat16), (torch.float16, torch.float16),
                                           (torch.float32, torch.float32), (torch.bfloat16, torch.float32)])
