@@ -381,6 +381,8 @@ int run_quant(QuantArgs a, int g, hipStream_t st) {
     int wpr = 1;
     while ((nchunks + wpr - 1) / wpr > 4) wpr *= 2;
     if (wpr > 8) return -2;
+    // few rows: more waves per row (down to one chunk per wave) so that the launch has enough waves to hide latency
+    while (wpr < 8 && wpr < nchunks && (int64_t)a.M * wpr < 2048) wpr *= 2;
     const int C = (nchunks + wpr - 1) / wpr;
     const int nw = wpr < 4 ? 4 : wpr;
     a.wpr = wpr;
