@@ -110,7 +110,9 @@ __device__ __forceinline__ float row_sum_f64(double v, double* red, int wave, in
 
 // PRO: the row prologue (csrc/kernels.cu:88-182) runs on the values as they are loaded, with the reference's rounding
 // points; p.pro selects it at run time.  Row sums are fp64, rounded once; the activation functions are correctly rounded.
-template <int MODE, int G, int C, bool PRO>
+// SR: stochastic rounding keyed by element index + p.seed (gpu_convrot_requant); a kernel variant of its own, so that the
+// plain quantizer carries neither the hash nor a branch per element.
+template <int MODE, int G, int C, bool PRO, bool SR = false>
 __global__ void __launch_bounds__(512) quant_rows_kernel(QuantArgs p) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     __shared__ float red[8];
@@ -334,7 +336,7 @@ __global__ void __launch_bounds__(512) quant_rows_kernel(QuantArgs p) {
                     t = x / st;
                 }
                 float r;
-                if (p.seed != 0 && (MODE == MODE_BF16 || MODE == MODE_F32)) {   // csrc/kernels.cu:1385-1388
+                if (SR && (MODE == MODE_BF16 || MODE == MODE_F32)) {   // csrc/kernels.cu:1385-1388
                     const uint64_t key = (uint64_t)(m * (int64_t)p.K + e0 + 4 * i + j) + p.seed;
                     const float noise = (float)(pcg_hash((uint32_t)key ^ (uint32_t)(key >> 32)) >> 8) * 0x1.0p-24f;
                     r = floorf(MODE == MODE_F32 ? t + noise : bf16_add_once(t, rnd_dt<DT_BF16>(noise)));
@@ -355,7 +357,10 @@ int launch(const QuantArgs& a, int nw, hipStream_t st) {
     const int grid = (a.M + a.rpb - 1) / a.rpb;
     const size_t smem = G ? (size_t)nw * kLdsPerWave * sizeof(float) : 0;
     constexpr bool CAN_PRO = true;
-    if (CAN_PRO && a.pro != PRO_PLAIN)
+    constexpr bool CAN_SR = (MODE == MODE_BF16 || MODE == MODE_F32) && G == 256;
+    if (CAN_SR && a.seed != 0 && a.pro == PRO_PLAIN)
+        hipLaunchKernelGGL((quant_rows_kernel<MODE, G, C, false, CAN_SR>), dim3(grid), dim3(nw * 64), smem, st, a);
+    else if (CAN_PRO && a.pro != PRO_PLAIN)
         hipLaunchKernelGGL((quant_rows_kernel<MODE, G, C, CAN_PRO>), dim3(grid), dim3(nw * 64), smem, st, a);
     else
         hipLaunchKernelGGL((quant_rows_kernel<MODE, G, C, false>), dim3(grid), dim3(nw * 64), smem, st, a);
