@@ -126,10 +126,16 @@ __global__ void __launch_bounds__(512) quant_rows_kernel(QuantArgs p) {
     constexpr int TD = MODE == MODE_BF16 ? DT_BF16 : MODE == MODE_SD_F16 ? DT_F16 : DT_F32;
     constexpr int TMODE = MODE == MODE_BF16 ? MODE_BF16 : MODE == MODE_SD_F16 ? MODE_SD_F16 : MODE_F32;
     auto R = [](float x) { return rnd_dt<TD>(x); };
-    // rnd(f(x)) of a bf16 value x through a table of all 65536 inputs, when the table is there
-    auto via = [](const uint16_t* tab, float x, auto f) {
-        if (MODE == MODE_BF16 && tab) return bf16_to_f(tab[f2u(x) >> 16]);
-        return rnd_dt<TD>(f(x));
+    // dst[i] = rnd(f(src[i])) for the 16 values of a lane: through a table of all 65536 bf16 inputs when it is there (one
+    // test for the 16 lookups, which then issue as a batch), else evaluated
+    auto map16 = [](const uint16_t* tab, const float* src, float* dst, auto f) {
+        if (MODE == MODE_BF16 && tab) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) dst[i] = bf16_to_f(tab[f2u(src[i]) >> 16]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) dst[i] = rnd_dt<TD>(f(src[i]));
+        }
     };
 
     float v[C][16];
@@ -160,11 +166,15 @@ __global__ void __launch_bounds__(512) quant_rows_kernel(QuantArgs p) {
                 if (pro == PRO_SD_GEGLU) {                                           // :642-649, row = [value | gate]
                     float gg[16];
                     load16<TMODE>(p.x, m * p.x_stride + p.up_offset + e0, gg);
+                    if (p.tab.gelu_f16) {
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        const float gl = p.tab.gelu_f16 ? f16_to_f(p.tab.gelu_f16[f_to_f16(gg[i])]) : R(gelu_f(gg[i]));
-                        v[c][i] = R(v[c][i] * gl);
+                        for (int i = 0; i < 16; ++i) gg[i] = f16_to_f(p.tab.gelu_f16[f_to_f16(gg[i])]);
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < 16; ++i) gg[i] = R(gelu_f(gg[i]));
                     }
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) v[c][i] = R(v[c][i] * gg[i]);
                 } else if (pro == PRO_SD_GN) {                                       // :653-662
                     const float2* stats = (const float2*)p.g + (m / p.g_stride) * (int64_t)(p.K / p.per) * 2;
                     float nw[16], nb[16];
@@ -182,14 +192,16 @@ __global__ void __launch_bounds__(512) quant_rows_kernel(QuantArgs p) {
             } else if (pro == PRO_GATE) {                                            // csrc/kernels.cu:95-100
                 float gg[16];
                 load16<TMODE>(p.g, m * p.g_stride + e0, gg);
+                map16(p.tab.sigmoid_bf16, gg, gg, [](float x) { return sigmoid_f(x); });
 #pragma unroll
-                for (int i = 0; i < 16; ++i) v[c][i] = R(v[c][i] * via(p.tab.sigmoid_bf16, gg[i], [](float x) { return sigmoid_f(x); }));
+                for (int i = 0; i < 16; ++i) v[c][i] = R(v[c][i] * gg[i]);
             } else if (pro == PRO_SWIGLU || pro == PRO_SITU || pro == PRO_SITU_FAST) {  // :101-112
                 float u[16];
                 load16<TMODE>(p.x, m * p.x_stride + p.up_offset + e0, u);
                 if (pro == PRO_SWIGLU) {
+                    map16(p.tab.silu_bf16, v[c], v[c], [](float x) { return silu_f(x); });
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) v[c][i] = R(via(p.tab.silu_bf16, v[c][i], [](float x) { return silu_f(x); }) * u[i]);
+                    for (int i = 0; i < 16; ++i) v[c][i] = R(v[c][i] * u[i]);
                 } else if (MODE == MODE_BF16 && p.tab.situ_gate_bf16) {
 #pragma unroll
                     for (int i = 0; i < 16; ++i)
@@ -199,14 +211,11 @@ __global__ void __launch_bounds__(512) quant_rows_kernel(QuantArgs p) {
                     for (int i = 0; i < 16; ++i) v[c][i] = situ_f(v[c][i], u[i]);
                 }
             } else if (pro == PRO_SILU) {
-#pragma unroll
-                for (int i = 0; i < 16; ++i) v[c][i] = via(p.tab.silu_bf16, v[c][i], [](float x) { return silu_f(x); });
+                map16(p.tab.silu_bf16, v[c], v[c], [](float x) { return silu_f(x); });
             } else if (pro == PRO_GELU) {
-#pragma unroll
-                for (int i = 0; i < 16; ++i) v[c][i] = via(p.tab.gelu_bf16, v[c][i], [](float x) { return gelu_f(x); });
+                map16(p.tab.gelu_bf16, v[c], v[c], [](float x) { return gelu_f(x); });
             } else if (pro == PRO_GELU_TANH) {
-#pragma unroll
-                for (int i = 0; i < 16; ++i) v[c][i] = via(p.tab.gelu_tanh_bf16, v[c][i], [](float x) { return gelu_tanh_f(x); });
+                map16(p.tab.gelu_tanh_bf16, v[c], v[c], [](float x) { return gelu_tanh_f(x); });
             } else if (ln) {
 #pragma unroll
                 for (int i = 0; i < 16; ++i) part += (double)v[c][i];
@@ -245,26 +254,31 @@ __global__ void __launch_bounds__(512) quant_rows_kernel(QuantArgs p) {
             }
             if (p.norm_w && (pro == PRO_RMS || pro == PRO_LAYERNORM || pro == PRO_LN_AFFINE)) load16<MODE_F32>(p.norm_w, e0, nw);
             if (pro == PRO_LN_AFFINE) load16<MODE_F32>(p.norm_b, e0, nb);
+            // the form is chosen once per 16 values, not per value
+            if (pro == PRO_ADALN) {                                                  // :163-166, one rounding
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                float n = v[c][i] * rstd;
-                const float a = mod ? msv[i] : 0.f, sh = mod ? shv[i] : 0.f;
-                if (pro == PRO_ADALN) {                                              // :163-166, one rounding
-                    n = R(__builtin_fmaf(n, 1.f + a, sh));
-                } else if (pro == PRO_LN_MOD) {                                      // ln_finish, :40-46
-                    n = R(__builtin_fmaf(R(n), R(1.f + a), sh));
-                } else if (pro == PRO_LN_AFFINE) {
-                    n = R(__builtin_fmaf(n, nw[i], nb[i]));
-                } else {                                                             // RMS, LAYERNORM: :171-179
-                    if (p.norm_w) n *= nw[i];
-                    n = R(n);
-                    if (mod) {
-                        const float aa = R(1.f + a);
-                        n = R(aa * n);
-                        n = R(n + sh);
+                for (int i = 0; i < 16; ++i) v[c][i] = R(__builtin_fmaf(v[c][i] * rstd, 1.f + (mod ? msv[i] : 0.f), mod ? shv[i] : 0.f));
+            } else if (pro == PRO_LN_MOD) {                                          // ln_finish, :40-46
+#pragma unroll
+                for (int i = 0; i < 16; ++i) v[c][i] = R(__builtin_fmaf(R(v[c][i] * rstd), R(1.f + (mod ? msv[i] : 0.f)), mod ? shv[i] : 0.f));
+            } else if (pro == PRO_LN_AFFINE) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) v[c][i] = R(__builtin_fmaf(v[c][i] * rstd, nw[i], nb[i]));
+            } else {                                                                 // RMS, LAYERNORM: :171-179
+                if (p.norm_w) {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) v[c][i] = R(v[c][i] * rstd * nw[i]);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) v[c][i] = R(v[c][i] * rstd);
+                }
+                if (mod) {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const float aa = R(1.f + msv[i]);
+                        v[c][i] = R(R(aa * v[c][i]) + shv[i]);
                     }
                 }
-                v[c][i] = n;
             }
         }
     }
