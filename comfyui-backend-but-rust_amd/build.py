@@ -11,7 +11,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "libgpu_kernels.so")
 ARCH = os.environ.get("HIP_ARCH", "gfx950")
-SOURCES = ["quant_rows.hip", "prologue_rows.hip", "weight_formats.hip", "act_tables.hip", "int8_gemm.hip", "w6.hip", "w6_requant.hip", "w6a8_group_gemm.hip"]
+SOURCES = ["quant_rows.hip", "prologue_rows.hip", "weight_formats.hip", "act_tables.hip", "int8_gemm.hip", "w6.hip", "w6_requant.hip", "w6a8_group_gemm.hip", "attn_int8.hip"]
 FLAGS = [
     "--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
     # exact arithmetic: no contraction except where fmaf is written, IEEE divide, no fast-math

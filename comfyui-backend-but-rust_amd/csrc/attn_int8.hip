@@ -1,0 +1,512 @@
+// INT8 attention for head dim 128 on gfx950: Q and K rotated and quantized per scale group, V per channel, integer
+// scores and integer P.V partials on v_mfma_i32_32x32x32_i8, softmax state in fp32.
+//
+// Semantics follow the reference's Sage-style path (csrc/attn_int8.cu:118-160 chains the stages;
+// csrc/vendor/sage/quant_qk_int8.cu:72-157 rotation, :296-413 Q groups, :422-575 K groups, :591-756 K anchor;
+// csrc/vendor/sage/quant_v_int8.cu:94-190 V; csrc/vendor/sage/qk_int_sv_i8_cuda.cuh + attn_utils.cuh:700-800 the tile
+// update with u8 probabilities).  The design is for CDNA4:
+//   * keys ride in src0 and queries in src1 of the score MFMA, so a lane ends up with one query row and 16 keys per
+//     32-key block: row maxima and sums are in-lane plus one exchange with lane ^ 32;
+//   * those 16 scores are, in order, exactly the 16 K-bytes that lane must supply as src1 of the P.V MFMA when V^T is
+//     stored with the matching key order, so probabilities never cross lanes;
+//   * the matrix cores multiply signed bytes only: probabilities 0..255 are fed as p - 128 and the accumulator starts
+//     at 128 * (column sums of the V tile), which the V quantizer leaves in the workspace.  The integers are exact.
+// The workspace layout is private to this file.
+#include <cstdio>
+
+#include "common.hpp"
+
+namespace {
+
+constexpr int D = 128;
+constexpr float kU8Offset = 7.9943534f;
+
+struct AttnArgs {
+    const void *q, *k, *v;
+    void* o;
+    int8_t *qi, *ki, *vt;
+    float *qs, *ks, *vs;
+    int* anchors;
+    uint32_t* vmax;
+    int* vsum;
+    int b, lq, lk, h, hk, rep, qg, kb, ck, nblk;
+    int64_t q_bs, q_rs, q_hs, k_bs, k_rs, k_hs, v_bs, v_rs, v_hs, o_bs, o_rs, o_hs;
+    float sm;
+    int vec_ok;
+};
+
+__device__ __forceinline__ float fmax_nn(float a, float b) { return a > b ? a : b; }
+
+__device__ __forceinline__ int8_t rn_s8(float v) {
+    if (v != v) return 0;
+    const float r = __builtin_rintf(v);
+    return (int8_t)(r > 127.f ? 127.f : r < -128.f ? -128.f : r);
+}
+
+// Sign diagonal and normalized Walsh-Hadamard over the 128 channels of one row held by 32 consecutive lanes, four
+// adjacent channels per lane.  Same operation order as the oracle: H4 in the lane, butterflies over lane bits, scale.
+__device__ __forceinline__ void rot128(float (&v)[4], int lane32) {
+    const uint32_t signs = lane32 < 8 ? 0x1035997bu : lane32 < 16 ? 0x8087f5eeu : lane32 < 24 ? 0xee2e4e1au : 0x71132418u;
+    const int shift = (lane32 & 7) * 4;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) v[c] = u2f(f2u(v[c]) ^ ((((signs >> (shift + c)) & 1u) ^ 1u) << 31));
+    const float a0 = v[0] + v[1], a1 = v[0] - v[1], a2 = v[2] + v[3], a3 = v[2] - v[3];
+    v[0] = (a0 + a2) * 0.5f;
+    v[1] = (a1 + a3) * 0.5f;
+    v[2] = (a0 - a2) * 0.5f;
+    v[3] = (a1 - a3) * 0.5f;
+#pragma unroll
+    for (int bit = 1; bit < 32; bit <<= 1) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const float other = __shfl_xor(v[c], bit);
+            v[c] = (lane32 & bit) ? other - v[c] : v[c] + other;
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < 4; ++c) v[c] *= 0.1767766952966369f;
+}
+
+__device__ __forceinline__ float max32(float m) {
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) m = fmax_nn(m, __shfl_xor(m, off));
+    return m;
+}
+
+__global__ void attn_zero_kernel(uint32_t* p, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0u;
+}
+
+// One workgroup of 128 threads per (kv head, batch): thread = channel.  The shuffle trees of the reference are summed
+// by thread 0 in their order.
+template <int DT>
+__global__ __launch_bounds__(128) void attn_anchor_kernel(AttnArgs a) {
+    __shared__ float s[9][D];
+    __shared__ float energy[D], best_energy[D], amax[D], bmax[D], dist[9][D];
+    __shared__ int chosen;
+    const int c = threadIdx.x, hi = blockIdx.x, bi = blockIdx.y;
+    const int64_t base = bi * a.k_bs + hi * a.k_hs;
+    float e = 0.f, m = 0.f, sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 9; ++i) {
+        const int row = (int)((int64_t)i * (a.lk - 1) / 8);
+        const float x = ld_dt<DT>(a.k, base + (int64_t)row * a.k_rs + c);
+        s[i][c] = x;
+        e = fmaf(x, x, e);
+        m = fmax_nn(m, fabsf(x));
+        sum += x;
+    }
+    energy[c] = e;
+    amax[c] = m;
+#pragma unroll
+    for (int i = 0; i < 9; ++i) {
+        const float d = fmaf(9.f, s[i][c], -sum);
+        dist[i][c] = fmaf(d, d, 0.f);
+    }
+    __syncthreads();
+    auto tree = [](const float* x) {
+        float t[32];
+        for (int i = 0; i < 32; ++i) t[i] = x[i];
+        for (int off = 16; off > 0; off >>= 1)
+            for (int i = 0; i < off; ++i) t[i] += t[i + off];
+        return t[0];
+    };
+    if (c == 0) {
+        int best = 0;
+        float best_d = 3.402823466e+38F;
+        for (int i = 0; i < 9; ++i) {
+            float d = 0.f;
+            for (int w = 0; w < 4; ++w) d += tree(&dist[i][w * 32]);
+            if (d < best_d) { best = i; best_d = d; }
+        }
+        chosen = best;
+    }
+    __syncthreads();
+    const int best = chosen;
+    float be = 0.f, bm = 0.f;
+#pragma unroll
+    for (int i = 0; i < 9; ++i) {
+        const float r = s[i][c] - s[best][c];
+        be = fmaf(r, r, be);
+        bm = fmax_nn(bm, fabsf(r));
+    }
+    best_energy[c] = be;
+    bmax[c] = bm;
+    __syncthreads();
+    if (c == 0) {
+        float e0 = 0.f, e1 = 0.f, m0 = 0.f, m1 = 0.f;
+        for (int w = 0; w < 4; ++w) {
+            e0 += tree(&energy[w * 32]);
+            e1 += tree(&best_energy[w * 32]);
+        }
+        for (int i = 0; i < D; ++i) {
+            m0 = fmax_nn(m0, amax[i]);
+            m1 = fmax_nn(m1, bmax[i]);
+        }
+        a.anchors[bi * a.hk + hi] = (e1 < e0 && m1 <= m0 * 1.125f) ? (int)((int64_t)best * (a.lk - 1) / 8) : -1;
+    }
+}
+
+// Q: one workgroup of 256 threads per 32 rows; each run of 32 lanes is one scale group (rows g, g+8, g+16, g+24).
+template <int DT>
+__global__ __launch_bounds__(256) void attn_quant_q_kernel(AttnArgs a) {
+    const int lane32 = threadIdx.x & 31, g = threadIdx.x >> 5;
+    const int t = blockIdx.x, hi = blockIdx.y, bi = blockIdx.z;
+    const int64_t bh = (int64_t)bi * a.h + hi, base = bi * a.q_bs + hi * a.q_hs + lane32 * 4;
+    float v[4][4];
+    float mx = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int row = t * 32 + g + 8 * j;
+        const int rowc = row < a.lq ? row : a.lq - 1;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) v[j][c] = ld_dt<DT>(a.q, base + (int64_t)rowc * a.q_rs + c);
+        rot128(v[j], lane32);
+        if (row < a.lq) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) mx = fmax_nn(mx, fabsf(v[j][c]));
+        }
+    }
+    mx = max32(mx);
+    const float sc = mx / 127.f + 1e-7f, inv = 1.f / sc;
+    if (lane32 == 0) a.qs[(bh * a.qg + t) * 8 + g] = sc;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int row = t * 32 + g + 8 * j;
+        if (row < a.lq) {
+            uint32_t w = 0;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) w |= (uint32_t)(uint8_t)rn_s8(v[j][c] * inv) << (8 * c);
+            *reinterpret_cast<uint32_t*>(a.qi + (bh * a.lq + row) * D + lane32 * 4) = w;
+        }
+    }
+}
+
+// K: one workgroup of 128 threads per tile of ck keys; each run of 32 lanes is one scale group (keys with
+// (key % 8) / 2 == g).  Two passes over the group's rows: abs-max, then codes.
+template <int DT>
+__global__ __launch_bounds__(128) void attn_quant_k_kernel(AttnArgs a) {
+    const int lane32 = threadIdx.x & 31, g = threadIdx.x >> 5;
+    const int t = blockIdx.x, hi = blockIdx.y, bi = blockIdx.z;
+    const int64_t bh = (int64_t)bi * a.hk + hi, base = bi * a.k_bs + hi * a.k_hs + lane32 * 4;
+    const int anchor = a.anchors[bh];
+    float bias[4] = {0.f, 0.f, 0.f, 0.f};
+    if (anchor >= 0) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) bias[c] = ld_dt<DT>(a.k, base + (int64_t)anchor * a.k_rs + c);
+    }
+    const int n = a.ck / 4;
+    float mx = 0.f, inv = 0.f;
+    for (int pass = 0; pass < 2; ++pass) {
+        for (int i = 0; i < n; ++i) {
+            const int row = t * a.ck + (i / 2) * 8 + g * 2 + (i % 2);
+            const int rowc = row < a.lk ? row : a.lk - 1;
+            float v[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) v[c] = ld_dt<DT>(a.k, base + (int64_t)rowc * a.k_rs + c) - bias[c];
+            rot128(v, lane32);
+            if (row < a.lk) {
+                if (pass == 0) {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) mx = fmax_nn(mx, fabsf(v[c]));
+                } else {
+                    uint32_t w = 0;
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) w |= (uint32_t)(uint8_t)rn_s8(v[c] * inv) << (8 * c);
+                    *reinterpret_cast<uint32_t*>(a.ki + (bh * a.lk + row) * D + lane32 * 4) = w;
+                }
+            }
+        }
+        if (pass == 0) {
+            mx = max32(mx);
+            const float sc = mx / 127.f + 1e-7f;
+            inv = 1.f / sc;
+            if (lane32 == 0) a.ks[(bh * a.kb + t) * 4 + g] = sc;
+        }
+    }
+}
+
+// V abs-max per channel: 256 threads take 128 rows of one (kv head, batch); non-negative floats order as their bits.
+template <int DT>
+__global__ __launch_bounds__(256) void attn_v_absmax_kernel(AttnArgs a) {
+    const int c = threadIdx.x & 127, half = threadIdx.x >> 7;
+    const int hi = blockIdx.y, bi = blockIdx.z;
+    const int64_t base = bi * a.v_bs + hi * a.v_hs + c;
+    float mx = 0.f;
+    const int r0 = blockIdx.x * 128;
+    for (int r = r0 + half; r < r0 + 128 && r < a.lk; r += 2) mx = fmax_nn(mx, fabsf(ld_dt<DT>(a.v, base + (int64_t)r * a.v_rs)));
+    atomicMax(&a.vmax[((int64_t)bi * a.hk + hi) * D + c], f2u(mx));
+}
+
+// V codes: one workgroup per block of 32 keys.  vt[(kv head, block)][d][32]: position h*16 + j of a row holds key
+// (j/4)*8 + h*4 + j%4 of the block, which is the order a lane of the attention kernel holds its 16 scores in.  Keys past
+// lk are zeros.  128 x the column sums go to vsum[(kv head, key tile)][d] by integer atomics.
+template <int DT>
+__global__ __launch_bounds__(256) void attn_v_quant_kernel(AttnArgs a) {
+    const int d = threadIdx.x & 127, hh = threadIdx.x >> 7;
+    const int s = blockIdx.x, hi = blockIdx.y, bi = blockIdx.z;
+    const int64_t bh = (int64_t)bi * a.hk + hi, base = bi * a.v_bs + hi * a.v_hs + d;
+    const float sc = fmax_nn(u2f(a.vmax[bh * D + d]) * (1.f / 127.f), 1e-12f), inv = 1.f / sc;
+    if (s == 0 && hh == 0) a.vs[bh * D + d] = sc;
+    uint32_t w[4] = {0u, 0u, 0u, 0u};
+    int sum = 0;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        const int key = s * 32 + (j / 4) * 8 + hh * 4 + (j % 4);
+        int q = 0;
+        if (key < a.lk) q = rn_s8(ld_dt<DT>(a.v, base + (int64_t)key * a.v_rs) * inv);
+        sum += q;
+        w[j / 4] |= (uint32_t)(uint8_t)q << (8 * (j % 4));
+    }
+    *reinterpret_cast<uint4*>(a.vt + ((bh * a.nblk + s) * D + d) * 32 + hh * 16) = make_uint4(w[0], w[1], w[2], w[3]);
+    atomicAdd(&a.vsum[(bh * a.kb + s / (a.ck / 32)) * D + d], 128 * sum);
+}
+
+// The attention: a wave owns 32 query rows and walks the key tiles on its own (no LDS, no barriers); four waves per
+// workgroup share K and V tiles through the caches.
+template <int OUT_DT, int CK>
+__global__ __launch_bounds__(256) void attn_int8_kernel(AttnArgs a) {
+    constexpr int NB = CK / 32;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int l32 = lane & 31, hh = lane >> 5;
+    const int hi = blockIdx.y, bi = blockIdx.z;
+    const int row0 = blockIdx.x * 128 + wave * 32;
+    if (row0 >= a.lq) return;
+    const int64_t bh = (int64_t)bi * a.h + hi, kvh = (int64_t)bi * a.hk + hi / a.rep;
+    const int r = row0 + l32, rc = r < a.lq ? r : a.lq - 1;
+
+    v4i qf[4];
+    {
+        const int8_t* qrow = a.qi + (bh * a.lq + rc) * D + hh * 16;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) qf[s] = *reinterpret_cast<const v4i*>(qrow + s * 32);
+    }
+    const float q_scale = a.qs[(bh * a.qg + r / 32) * 8 + (r & 7)];
+
+    float ro[4][16];
+#pragma unroll
+    for (int x = 0; x < 4; ++x)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) ro[x][i] = 0.f;
+    float m = -50000.f, dsum = 1.f;
+
+    for (int t = 0; t < a.kb; ++t) {
+        const int key0 = t * CK;
+        const bool last = t == a.kb - 1;
+        v16i S[NB];
+#pragma unroll
+        for (int blk = 0; blk < NB; ++blk) {
+            const int key = key0 + blk * 32 + l32;
+            const int8_t* krow = a.ki + (kvh * a.lk + (key < a.lk ? key : a.lk - 1)) * D + hh * 16;
+            v16i acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const v4i kf = *reinterpret_cast<const v4i*>(krow + s * 32);
+                acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf, qf[s], acc, 0, 0, 0);
+            }
+            S[blk] = acc;
+        }
+        const float* ksc = a.ks + (kvh * a.kb + t) * 4 + hh * 2;
+        const float gs0 = a.sm * (q_scale * ksc[0]), gs1 = a.sm * (q_scale * ksc[1]);
+
+        float m0 = last ? -50000.f : -3.0e38f, m1 = m0;
+#pragma unroll
+        for (int blk = 0; blk < NB; ++blk)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int key = key0 + blk * 32 + (i / 4) * 8 + hh * 4 + (i % 4);
+                const float sv = (float)S[blk][i];
+                if (key < a.lk) {
+                    if ((i % 4) < 2) m0 = fmax_nn(m0, sv);
+                    else m1 = fmax_nn(m1, sv);
+                }
+            }
+        float tile_m = fmax_nn(fmaf(m0, gs0, -kU8Offset), fmaf(m1, gs1, -kU8Offset));
+        tile_m = fmax_nn(tile_m, __shfl_xor(tile_m, 32));
+        const float smaller = __builtin_amdgcn_exp2f(-fabsf(m - tile_m));
+        const float o_scale = m < tile_m ? smaller : 1.f, t_scale = tile_m < m ? smaller : 1.f;
+        m = fmax_nn(m, tile_m);
+        dsum *= o_scale;
+
+        v4i pf[NB];
+        int psum = 0;
+#pragma unroll
+        for (int blk = 0; blk < NB; ++blk) {
+            uint32_t w[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int key = key0 + blk * 32 + (i / 4) * 8 + hh * 4 + (i % 4);
+                int p = 0;
+                if (key < a.lk) {
+                    float e = __builtin_amdgcn_exp2f(fmaf((float)S[blk][i], (i % 4) < 2 ? gs0 : gs1, -tile_m));
+                    e = e > 255.f ? 255.f : e;
+                    p = (int)__builtin_rintf(e);
+                }
+                psum += p;
+                w[i / 4] |= (uint32_t)((p - 128) & 0xff) << (8 * (i % 4));
+            }
+            pf[blk] = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+        }
+        dsum += (float)psum * t_scale;
+
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            const int* vsp = a.vsum + (kvh * a.kb + t) * D + x * 32 + hh * 4;
+            v16i acc;
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const v4i c4 = *reinterpret_cast<const v4i*>(vsp + g4 * 8);
+                acc[g4 * 4 + 0] = c4[0];
+                acc[g4 * 4 + 1] = c4[1];
+                acc[g4 * 4 + 2] = c4[2];
+                acc[g4 * 4 + 3] = c4[3];
+            }
+#pragma unroll
+            for (int blk = 0; blk < NB; ++blk) {
+                const int8_t* vp = a.vt + ((kvh * a.nblk + (t * NB + blk)) * D + x * 32 + l32) * 32 + hh * 16;
+                const v4i vf = *reinterpret_cast<const v4i*>(vp);
+                acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf, pf[blk], acc, 0, 0, 0);
+            }
+#pragma unroll
+            for (int i = 0; i < 16; ++i) ro[x][i] = fmaf((float)acc[i], t_scale, ro[x][i] * o_scale);
+        }
+    }
+
+    const float dtot = dsum + __shfl_xor(dsum, 32);
+    const float rcp = 1.f / dtot;
+    if (r < a.lq) {
+        const int64_t ob = bi * a.o_bs + (int64_t)r * a.o_rs + hi * a.o_hs;
+#pragma unroll
+        for (int x = 0; x < 4; ++x)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const int d0 = x * 32 + g4 * 8 + hh * 4;
+                const float4 s4 = *reinterpret_cast<const float4*>(a.vs + kvh * D + d0);
+                float out[4] = {ro[x][g4 * 4] * rcp * s4.x, ro[x][g4 * 4 + 1] * rcp * s4.y, ro[x][g4 * 4 + 2] * rcp * s4.z,
+                                ro[x][g4 * 4 + 3] * rcp * s4.w};
+                if (a.vec_ok) store4<OUT_DT>(a.o, ob + d0, out);
+                else
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) st_dt<OUT_DT>(a.o, ob + d0 + c, out[c]);
+            }
+    }
+}
+
+int cta_k_for(int lk, int d) { return lk > 1024 && d != 64 ? 128 : 64; }   // csrc/attn_int8.cu:56
+
+struct Plan {
+    int64_t qi, ki, qs, ks, vt, vs, anchors, vmax, vsum, total;
+    int ck, kb, qg, nblk;
+};
+
+Plan plan_for(int64_t b, int64_t h, int64_t hk, int64_t lq, int64_t lk) {
+    Plan p;
+    p.ck = cta_k_for((int)lk, D);
+    p.kb = (int)((lk + p.ck - 1) / p.ck);
+    p.qg = (int)((lq + 127) / 128 * 4);
+    p.nblk = p.kb * (p.ck / 32);
+    int64_t n = 0;
+    auto add = [&](int64_t bytes) { const int64_t at = n; n += (bytes + 255) / 256 * 256; return at; };
+    p.qi = add(b * h * lq * D);
+    p.ki = add(b * hk * lk * D);
+    p.qs = add(b * h * p.qg * 8 * 4);
+    p.ks = add(b * hk * p.kb * 4 * 4);
+    p.vt = add(b * hk * (int64_t)p.nblk * D * 32);
+    p.vs = add(b * hk * D * 4);
+    p.anchors = add(b * hk * 4);
+    p.vmax = add(b * hk * D * 4);                  // vmax and vsum are adjacent: one fill clears both
+    p.vsum = add(b * hk * (int64_t)p.kb * D * 4);
+    p.total = n;
+    return p;
+}
+
+template <int DT>
+int run(AttnArgs a, hipStream_t st) {
+    const int64_t nz = ((char*)a.vsum - (char*)a.vmax) / 4 + (int64_t)a.b * a.hk * a.kb * D;
+    attn_zero_kernel<<<dim3((unsigned)((nz + 255) / 256)), 256, 0, st>>>(a.vmax, nz);
+    attn_anchor_kernel<DT><<<dim3(a.hk, a.b), 128, 0, st>>>(a);
+    attn_quant_q_kernel<DT><<<dim3(a.qg, a.h, a.b), 256, 0, st>>>(a);
+    attn_quant_k_kernel<DT><<<dim3(a.kb, a.hk, a.b), 128, 0, st>>>(a);
+    attn_v_absmax_kernel<DT><<<dim3((a.lk + 127) / 128, a.hk, a.b), 256, 0, st>>>(a);
+    attn_v_quant_kernel<DT><<<dim3(a.nblk, a.hk, a.b), 256, 0, st>>>(a);
+    const dim3 grid((a.lq + 127) / 128, a.h, a.b);
+    if (a.ck == 64) attn_int8_kernel<DT, 64><<<grid, 256, 0, st>>>(a);
+    else attn_int8_kernel<DT, 128><<<grid, 256, 0, st>>>(a);
+    return hipGetLastError() == hipSuccess ? 0 : -401;
+}
+
+int int8_attn(const void* q, const void* k, const void* v, void* o, void* ws, int b, int lq, int lk, int h, int hk, int Dh,
+              int64_t q_bs, int64_t q_rs, int64_t q_hs, int64_t k_bs, int64_t k_rs, int64_t k_hs, int64_t v_bs, int64_t v_rs,
+              int64_t v_hs, int64_t o_bs, int64_t o_rs, int64_t o_hs, float scale, int dt, void* stream) {
+    const char* why = nullptr;
+    if (Dh != D) why = "only head dim 128 is built";
+    else if (!q || !k || !v || !o || !ws) why = "null pointer";
+    else if (b <= 0 || lq <= 0 || lk <= 0 || h <= 0 || hk <= 0 || h % hk != 0) why = "bad sizes";
+    else if (b > 65535 || h > 65535) why = "batch or head count beyond the grid limit";
+    else if (((uintptr_t)ws & 255) != 0) why = "workspace must be 256-byte aligned";
+    if (why) {
+        fprintf(stderr, "int8 attention: %s\n", why);
+        return -400;
+    }
+    const Plan p = plan_for(b, h, hk, lq, lk);
+    char* w = (char*)ws;
+    AttnArgs a;
+    a.q = q; a.k = k; a.v = v; a.o = o;
+    a.qi = (int8_t*)(w + p.qi); a.ki = (int8_t*)(w + p.ki); a.vt = (int8_t*)(w + p.vt);
+    a.qs = (float*)(w + p.qs); a.ks = (float*)(w + p.ks); a.vs = (float*)(w + p.vs);
+    a.anchors = (int*)(w + p.anchors); a.vmax = (uint32_t*)(w + p.vmax); a.vsum = (int*)(w + p.vsum);
+    a.b = b; a.lq = lq; a.lk = lk; a.h = h; a.hk = hk; a.rep = h / hk;
+    a.qg = p.qg; a.kb = p.kb; a.ck = p.ck; a.nblk = p.nblk;
+    a.q_bs = q_bs; a.q_rs = q_rs; a.q_hs = q_hs; a.k_bs = k_bs; a.k_rs = k_rs; a.k_hs = k_hs;
+    a.v_bs = v_bs; a.v_rs = v_rs; a.v_hs = v_hs; a.o_bs = o_bs; a.o_rs = o_rs; a.o_hs = o_hs;
+    a.sm = scale * 1.44269504088896340736f;
+    a.vec_ok = ((o_bs | o_rs | o_hs) % 4 == 0 && ((uintptr_t)o & 7) == 0) ? 1 : 0;
+    return dt == DT_F16 ? run<DT_F16>(a, (hipStream_t)stream) : run<DT_BF16>(a, (hipStream_t)stream);
+}
+
+}  // namespace
+
+GPU_API int64_t gpu_int8_attn_workspace_d(int b, int h, int hk, int lq, int lk, int head_dim) {
+    (void)head_dim;
+    if (b <= 0 || h <= 0 || hk <= 0 || lq <= 0 || lk <= 0) return 0;
+    return plan_for(b, h, hk, lq, lk).total;
+}
+
+GPU_API int64_t gpu_int8_attn_workspace(int b, int h, int hk, int lq, int lk) {
+    return gpu_int8_attn_workspace_d(b, h, hk, lq, lk, D);
+}
+
+GPU_API int gpu_int8_attn_d(const void* q, const void* k, const void* v, void* o, void* ws, int b, int lq, int lk, int h,
+                            int hk, int head_dim, int64_t q_bs, int64_t q_rs, int64_t q_hs, int64_t k_bs, int64_t k_rs,
+                            int64_t k_hs, int64_t v_bs, int64_t v_rs, int64_t v_hs, int64_t o_bs, int64_t o_rs, int64_t o_hs,
+                            float scale, void* stream) {
+    return int8_attn(q, k, v, o, ws, b, lq, lk, h, hk, head_dim, q_bs, q_rs, q_hs, k_bs, k_rs, k_hs, v_bs, v_rs, v_hs, o_bs,
+                     o_rs, o_hs, scale, DT_BF16, stream);
+}
+
+GPU_API int gpu_int8_attn_f16(const void* q, const void* k, const void* v, void* o, void* ws, int b, int lq, int lk, int h,
+                              int hk, int head_dim, int64_t q_bs, int64_t q_rs, int64_t q_hs, int64_t k_bs, int64_t k_rs,
+                              int64_t k_hs, int64_t v_bs, int64_t v_rs, int64_t v_hs, int64_t o_bs, int64_t o_rs,
+                              int64_t o_hs, float scale, void* stream) {
+    return int8_attn(q, k, v, o, ws, b, lq, lk, h, hk, head_dim, q_bs, q_rs, q_hs, k_bs, k_rs, k_hs, v_bs, v_rs, v_hs, o_bs,
+                     o_rs, o_hs, scale, DT_F16, stream);
+}
+
+GPU_API int gpu_int8_attn(const void* q, const void* k, const void* v, void* o, void* ws, int b, int lq, int lk, int h,
+                          int hk, int64_t q_bs, int64_t q_rs, int64_t q_hs, int64_t k_bs, int64_t k_rs, int64_t k_hs,
+                          int64_t v_bs, int64_t v_rs, int64_t v_hs, int64_t o_bs, int64_t o_rs, int64_t o_hs, float scale,
+                          void* stream) {
+    return int8_attn(q, k, v, o, ws, b, lq, lk, h, hk, D, q_bs, q_rs, q_hs, k_bs, k_rs, k_hs, v_bs, v_rs, v_hs, o_bs, o_rs,
+                     o_hs, scale, DT_BF16, stream);
+}
+
+// Test hook: where the pieces of the workspace lie (byte offsets), and the tiling.  out[0..9] = qi, ki, qs, ks, vt, vs,
+// anchors, vsum, key tile length, key tiles.
+GPU_API int gpu_internal_attn_layout(int b, int h, int hk, int lq, int lk, int64_t* out) {
+    if (b <= 0 || h <= 0 || hk <= 0 || lq <= 0 || lk <= 0 || !out) return -400;
+    const Plan p = plan_for(b, h, hk, lq, lk);
+    const int64_t v[10] = {p.qi, p.ki, p.qs, p.ks, p.vt, p.vs, p.anchors, p.vsum, p.ck, p.kb};
+    for (int i = 0; i < 10; ++i) out[i] = v[i];
+    return 0;
+}

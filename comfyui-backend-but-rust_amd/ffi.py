@@ -39,6 +39,10 @@ SIGNATURES = {
     "gpu_int8_gemm_acc": [_P, _P, _P, _I64, _I64, _I64, _P],
     "gpu_w6a8_gemm": [_P, _P, _P, _I32, _P, _P, _P, _P, _I64, _I64, _I64, _I32, _P],
     "gpu_w6a8_group_gemm": [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I32, _P],
+    "gpu_int8_attn_d": [_P, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _I32, _I32] + [_I64] * 12 + [_F32, _P],
+    "gpu_int8_attn_f16": [_P, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _I32, _I32] + [_I64] * 12 + [_F32, _P],
+    "gpu_int8_attn": [_P, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _I32] + [_I64] * 12 + [_F32, _P],
+    "gpu_internal_attn_layout": [_I32, _I32, _I32, _I32, _I32, _P],
     "gpu_int8_gemm_force_config": [_I32],
     "gpu_mfma_layout_probe": [_P, _P],
 }
@@ -53,6 +57,10 @@ def _load():
         fn = getattr(lib, name)
         fn.argtypes = args
         fn.restype = _I32
+    lib.gpu_int8_attn_workspace_d.argtypes = [_I32] * 6
+    lib.gpu_int8_attn_workspace_d.restype = _I64
+    lib.gpu_int8_attn_workspace.argtypes = [_I32] * 5
+    lib.gpu_int8_attn_workspace.restype = _I64
     lib.gpu_kernels_build_info.restype = C.c_char_p
     lib.gpu_kernels_build_info.argtypes = []
     return lib

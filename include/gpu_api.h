@@ -114,6 +114,31 @@ int gpu_convrot_requant(int dtype, const void* x, void* q, void* s, int64_t N, i
 int gpu_w6_requant(const void* weight, void* packed, void* s_rel, void* s_channel, int64_t N, int K, uint64_t seed,
                    void* stream);
 
+/* INT8 attention, head dim 128: o = softmax(q . k^T * scale) . v with q and k rotated (sign diagonal + Walsh-Hadamard
+ * 128) and quantized per scale group (eight groups per 32 query rows, four per key tile), an optional K anchor
+ * subtracted first, v quantized per channel, probabilities as u8 per key tile (64 keys, 128 beyond lk = 1024) and integer
+ * P.V partials folded in fp32.  q/k/v/o: [b, seq, heads, 128] through element strides (batch, row, head), bf16
+ * (gpu_int8_attn, gpu_int8_attn_d) or f16 (gpu_int8_attn_f16); h % hk == 0 (grouped-query heads); ws: 256-byte aligned
+ * device scratch of gpu_int8_attn_workspace[_d] bytes, layout private to the library.
+ * Replaces gpu_int8_attn_workspace_d / gpu_int8_attn_workspace (csrc/attn_int8.cu:62-82), gpu_int8_attn_d (:101-108),
+ * gpu_int8_attn_f16 (:111-118), gpu_int8_attn (:225-231); src/ffi.rs binds them under the same names.
+ * Returns 0, -400 (argument the library refuses: message on stderr; head dims other than 128 are not built) or -401
+ * (launch failure), the reference's codes.  Not built: gpu_int8_attn_norm_rope, gpu_int8_attn_sink,
+ * gpu_int8_attn_key_bias (csrc/attn_int8.cu:166-223). */
+int64_t gpu_int8_attn_workspace_d(int b, int h, int hk, int lq, int lk, int head_dim);
+int64_t gpu_int8_attn_workspace(int b, int h, int hk, int lq, int lk);
+int gpu_int8_attn_d(const void* q, const void* k, const void* v, void* o, void* ws, int b, int lq, int lk, int h, int hk,
+                    int head_dim, int64_t q_bs, int64_t q_rs, int64_t q_hs, int64_t k_bs, int64_t k_rs, int64_t k_hs,
+                    int64_t v_bs, int64_t v_rs, int64_t v_hs, int64_t o_bs, int64_t o_rs, int64_t o_hs, float scale,
+                    void* stream);
+int gpu_int8_attn_f16(const void* q, const void* k, const void* v, void* o, void* ws, int b, int lq, int lk, int h, int hk,
+                      int head_dim, int64_t q_bs, int64_t q_rs, int64_t q_hs, int64_t k_bs, int64_t k_rs, int64_t k_hs,
+                      int64_t v_bs, int64_t v_rs, int64_t v_hs, int64_t o_bs, int64_t o_rs, int64_t o_hs, float scale,
+                      void* stream);
+int gpu_int8_attn(const void* q, const void* k, const void* v, void* o, void* ws, int b, int lq, int lk, int h, int hk,
+                  int64_t q_bs, int64_t q_rs, int64_t q_hs, int64_t k_bs, int64_t k_rs, int64_t k_hs, int64_t v_bs,
+                  int64_t v_rs, int64_t v_hs, int64_t o_bs, int64_t o_rs, int64_t o_hs, float scale, void* stream);
+
 /* D[M,N] = Out((A[M,K] . W[N,K]^T) * xs[m] * ws[n] + bias[n]).
  * Replaces gpu_int8_gemm, src/ffi.rs:38 / csrc/gemm.cu:124-129.
  * A, W int8 row-major (K contiguous); xs f32 [M]; ws f32 [N]; bias Out[N] or null; D Out[M,N]; out_dt a DT_* code. */

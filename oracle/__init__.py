@@ -58,6 +58,13 @@ def lib():
         L.orc_linear_w8a8.restype = i32
         L.orc_linear_w8a8.argtypes = [i32, vp, i64, i32, vp, vp, vp, vp, i32, i32, i32, i32, i32, vp]
         L.orc_set_threads.restype = None; L.orc_set_threads.argtypes = [i32]
+        L.orc_attn_rot128.restype = None; L.orc_attn_rot128.argtypes = [vp]
+        L.orc_attn_quant_qk.restype = i32
+        L.orc_attn_quant_qk.argtypes = [i32, vp, vp, i32, i32, i32, i32, i32, i64, i64, i64, i64, i64, i64, i32, i32, vp, vp, vp, vp, vp]
+        L.orc_attn_quant_v.restype = i32; L.orc_attn_quant_v.argtypes = [i32, vp, i32, i32, i32, i64, i64, i64, vp, vp]
+        L.orc_attn_int8.restype = i32
+        L.orc_attn_int8.argtypes = [i32, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, vp, i64, i64, i64]
+        L.orc_attn_cta_k.restype = i32; L.orc_attn_cta_k.argtypes = [i32, i32]
         _lib = L
     return _lib
 
@@ -326,3 +333,45 @@ def linear_w8a8(dtype, x, rotate, W, ws, bias, out_dt, fma=1, threads=None):
     rc = lib().orc_linear_w8a8(dtype, _p(x), K, rotate, _p(W), _p(ws), _p(bias), _p(D), M, N, K, out_dt, int(fma),
                                C.byref(t))
     return rc, D, t.value
+
+
+def attn_rot128(row):
+    """Sign diagonal + normalized Walsh-Hadamard over 128 channels, in place on a copy."""
+    r = np.ascontiguousarray(row, dtype=np.float32).copy()
+    assert r.shape == (128,)
+    lib().orc_attn_rot128(_p(r))
+    return r
+
+
+def attn_quant(dt, q, k, v, use_anchor=True):
+    """q [b,lq,h,128], k/v [b,lk,hk,128] contiguous (uint16 bits for bf16/f16).  Returns a dict with the int8 tensors
+    in [b,heads,len,128] order, the scales, the anchors and the key tile length."""
+    b, lq, h, D = q.shape
+    _, lk, hk, _ = k.shape
+    assert D == 128 and v.shape == k.shape
+    q, k, v = np.ascontiguousarray(q), np.ascontiguousarray(k), np.ascontiguousarray(v)
+    ck = lib().orc_attn_cta_k(lk, D)
+    qg, kb = (lq + 127) // 128 * 4, (lk + ck - 1) // ck
+    out = dict(ck=ck, qi=np.zeros((b, h, lq, D), np.int8), qs=np.zeros((b, h, qg * 8), np.float32),
+               ki=np.zeros((b, hk, lk, D), np.int8), ks=np.zeros((b, hk, kb * 4), np.float32),
+               anchors=np.zeros((b, hk), np.int32), vi=np.zeros((b, hk, lk, D), np.int8),
+               vs=np.zeros((b, hk, D), np.float32))
+    rc = lib().orc_attn_quant_qk(dt, _p(q), _p(k), b, lq, lk, h, hk, lq * h * D, h * D, D, lk * hk * D, hk * D, D, ck,
+                                 1 if use_anchor else 0, _p(out["qi"]), _p(out["qs"]), _p(out["ki"]), _p(out["ks"]),
+                                 _p(out["anchors"]))
+    assert rc == 0
+    rc = lib().orc_attn_quant_v(dt, _p(v), b, lk, hk, lk * hk * D, hk * D, D, _p(out["vi"]), _p(out["vs"]))
+    assert rc == 0
+    return out
+
+
+def attn_int8(dt, q, k, v, scale, use_anchor=True, quant=None):
+    """The whole int8 attention: o [b,lq,h,128] in dtype dt (uint16 bits for bf16/f16)."""
+    b, lq, h, D = q.shape
+    lk, hk = k.shape[1], k.shape[2]
+    z = quant if quant is not None else attn_quant(dt, q, k, v, use_anchor)
+    o = np.zeros((b, lq, h, D), np.float32 if dt == F32 else np.uint16)
+    rc = lib().orc_attn_int8(dt, _p(z["qi"]), _p(z["ki"]), _p(z["vi"]), _p(z["qs"]), _p(z["ks"]), _p(z["vs"]), b, lq, lk,
+                             h, hk, z["ck"], float(scale), _p(o), lq * h * D, h * D, D)
+    assert rc == 0
+    return o

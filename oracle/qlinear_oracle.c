@@ -745,3 +745,262 @@ ORC_API void orc_set_threads(int n) {
     (void)n;
 #endif
 }
+
+/* ---------------------------------------------------------------------------------------------
+ * INT8 attention, head dim 128 (csrc/attn_int8.cu:118-160 chains the three stages below).
+ *
+ * PARITY UNPINNED against a run of the reference: its exp2 and reciprocal are PTX approximations
+ * (csrc/vendor/sage/math.cuh:54-58,111-115) and its build may pass --use_fast_math (build.rs:140); here exp2 is
+ * fp64 libm rounded to fp32 and divisions are IEEE.  The structure (rotation, scale groups, anchor, tile maxima, u8
+ * probabilities, integer P.V partials folded with fmaf) is pinned by the tests against a dense Hadamard matrix, the
+ * quantizer's half-step bound and exact fp64 softmax attention.
+ * ------------------------------------------------------------------------------------------- */
+#define ATTN_D 128
+#define ATTN_U8_OFFSET 7.9943534f   /* csrc/vendor/sage/attn_utils.cuh:40 */
+
+/* Sign diagonal, then a normalized Walsh-Hadamard transform over 128 channels: H4 on each run of four channels, then
+ * radix-2 butterflies over channel bits 2..6, then one scaling (csrc/vendor/sage/quant_qk_int8.cu:72-109,136-157). */
+ORC_API void orc_attn_rot128(float* v) {
+    static const uint32_t signs[4] = {0x1035997bu, 0x8087f5eeu, 0xee2e4e1au, 0x71132418u};
+    for (int ch = 0; ch < ATTN_D; ++ch) {
+        const int lane = ch >> 2, c = ch & 3;
+        const uint32_t flip = ((signs[lane >> 3] >> ((lane & 7) * 4 + c)) & 1u) ^ 1u;
+        v[ch] = u2f(f2u(v[ch]) ^ (flip << 31));
+    }
+    for (int g = 0; g < ATTN_D; g += 4) {
+        const float a0 = v[g] + v[g + 1], a1 = v[g] - v[g + 1], a2 = v[g + 2] + v[g + 3], a3 = v[g + 2] - v[g + 3];
+        v[g] = (a0 + a2) * 0.5f;
+        v[g + 1] = (a1 + a3) * 0.5f;
+        v[g + 2] = (a0 - a2) * 0.5f;
+        v[g + 3] = (a1 - a3) * 0.5f;
+    }
+    for (int bit = 1; bit < 32; bit <<= 1)
+        for (int lane = 0; lane < 32; ++lane) {
+            if (lane & bit) continue;
+            for (int c = 0; c < 4; ++c) {
+                const float lo = v[lane * 4 + c], hi = v[(lane | bit) * 4 + c];
+                v[lane * 4 + c] = lo + hi;
+                v[(lane | bit) * 4 + c] = lo - hi;
+            }
+        }
+    for (int ch = 0; ch < ATTN_D; ++ch) v[ch] *= 0.1767766952966369f;
+}
+
+static inline int8_t attn_rn_s8(float v) {                       /* cvt.rni.sat.s8.f32, float_utils.cuh:39-45 */
+    if (isnan(v)) return 0;
+    const float r = rintf(v);
+    return (int8_t)(r > 127.f ? 127.f : r < -128.f ? -128.f : r);
+}
+
+/* The 32-lane shfl_down tree as lane 0 sees it (quant_qk_int8.cu:664-674). */
+static float attn_tree_sum32(const float* x) {
+    float t[32];
+    memcpy(t, x, sizeof t);
+    for (int off = 16; off > 0; off >>= 1)
+        for (int i = 0; i < off; ++i) t[i] += t[i + off];
+    return t[0];
+}
+
+/* K anchor for one (batch, head): nine evenly spaced keys, the one closest to their mean, kept only when it lowers
+ * the sampled energy without raising the sampled abs-max by more than 12.5 % (quant_qk_int8.cu:591-756, C = 128: one
+ * channel per thread, four warps).  The distance 9*s - sum is taken as one fma, nvcc's default contraction. */
+static int attn_detect_anchor(int dt, const void* k, int64_t base, int64_t stride_n, int Lk) {
+    float s[9][ATTN_D];
+    for (int i = 0; i < 9; ++i) {
+        const int row = (int)((int64_t)i * (Lk - 1) / 8);
+        for (int c = 0; c < ATTN_D; ++c) s[i][c] = ld_t(dt, k, base + (int64_t)row * stride_n + c);
+    }
+    float energy[ATTN_D], amax[ATTN_D], dist[9][ATTN_D];
+    for (int c = 0; c < ATTN_D; ++c) {
+        float e = 0.f, m = 0.f, sum = 0.f;
+        for (int i = 0; i < 9; ++i) {
+            e = fmaf(s[i][c], s[i][c], e);
+            m = fmax_dev(m, fabsf(s[i][c]));
+            sum += s[i][c];
+        }
+        energy[c] = e;
+        amax[c] = m;
+        for (int i = 0; i < 9; ++i) {
+            const float d = fmaf(9.f, s[i][c], -sum);
+            dist[i][c] = fmaf(d, d, 0.f);
+        }
+    }
+    int best = 0;
+    float best_d = 3.402823466e+38F;
+    for (int i = 0; i < 9; ++i) {
+        float d = 0.f;
+        for (int w = 0; w < 4; ++w) d += attn_tree_sum32(&dist[i][w * 32]);
+        if (d < best_d) { best = i; best_d = d; }
+    }
+    float e0 = 0.f, m0 = 0.f, e1 = 0.f, m1 = 0.f;
+    float be[ATTN_D];
+    for (int c = 0; c < ATTN_D; ++c) {
+        float e = 0.f;
+        for (int i = 0; i < 9; ++i) {
+            const float r = s[i][c] - s[best][c];
+            e = fmaf(r, r, e);
+            m1 = fmax_dev(m1, fabsf(r));
+        }
+        be[c] = e;
+        m0 = fmax_dev(m0, amax[c]);
+    }
+    for (int w = 0; w < 4; ++w) {
+        e0 += attn_tree_sum32(&energy[w * 32]);
+        e1 += attn_tree_sum32(&be[w * 32]);
+    }
+    return (e1 < e0 && m1 <= m0 * 1.125f) ? (int)((int64_t)best * (Lk - 1) / 8) : -1;
+}
+
+/* One scale group: rows[0..n) (absolute row numbers, those >= L skipped) of one head, minus `bias` when given,
+ * rotated, abs-max over the group, scale = max/127 + 1e-7, codes = rn(v * (1/scale))
+ * (quant_qk_int8.cu:296-413 for Q, :422-575 for K). */
+static void attn_quant_group(int dt, const void* x, int64_t base, int64_t stride_n, const int* rows, int n, int L,
+                             const float* bias, int8_t* out, float* scale) {
+    float buf[32][ATTN_D];
+    float mx = 0.f;
+    for (int i = 0; i < n; ++i) {
+        if (rows[i] >= L) continue;
+        for (int c = 0; c < ATTN_D; ++c) {
+            buf[i][c] = ld_t(dt, x, base + (int64_t)rows[i] * stride_n + c);
+            if (bias) buf[i][c] -= bias[c];
+        }
+        orc_attn_rot128(buf[i]);
+        for (int c = 0; c < ATTN_D; ++c) mx = fmax_dev(mx, fabsf(buf[i][c]));
+    }
+    const float sc = mx / 127.f + 1e-7f, inv = 1.f / sc;
+    *scale = sc;
+    for (int i = 0; i < n; ++i) {
+        if (rows[i] >= L) continue;
+        for (int c = 0; c < ATTN_D; ++c) out[(int64_t)rows[i] * ATTN_D + c] = attn_rn_s8(buf[i][c] * inv);
+    }
+}
+
+/* q [b, lq, h, 128], k [b, lk, hk, 128] through element strides (batch, row, head).  qi [b,h,lq,128],
+ * qs [b,h,ceil(lq/128)*32] (eight groups per 32 rows: rows r, r+8, r+16, r+24), ki [b,hk,lk,128],
+ * ks [b,hk,ceil(lk/ck)*4] (four groups per ck keys: keys with (key % 8) / 2 equal), anchors [b,hk]. */
+ORC_API int orc_attn_quant_qk(int dt, const void* q, const void* k, int b, int lq, int lk, int h, int hk, int64_t q_bs,
+                              int64_t q_rs, int64_t q_hs, int64_t k_bs, int64_t k_rs, int64_t k_hs, int ck, int use_anchor,
+                              int8_t* qi, float* qs, int8_t* ki, float* ks, int32_t* anchors) {
+    if (ck != 64 && ck != 128) return -1;
+    const int qg = (lq + 127) / 128 * 4, kb = (lk + ck - 1) / ck;
+    for (int bi = 0; bi < b; ++bi)
+        for (int hi = 0; hi < h; ++hi)
+            for (int t = 0; t < qg; ++t)
+                for (int g = 0; g < 8; ++g) {
+                    int rows[4];
+                    for (int j = 0; j < 4; ++j) rows[j] = t * 32 + g + 8 * j;
+                    const int64_t bh = (int64_t)bi * h + hi;
+                    attn_quant_group(dt, q, bi * q_bs + hi * q_hs, q_rs, rows, 4, lq, NULL, qi + bh * lq * ATTN_D,
+                                     &qs[(bh * qg + t) * 8 + g]);
+                }
+    for (int bi = 0; bi < b; ++bi)
+        for (int hi = 0; hi < hk; ++hi) {
+            const int64_t bh = (int64_t)bi * hk + hi, base = bi * k_bs + hi * k_hs;
+            const int anchor = use_anchor ? attn_detect_anchor(dt, k, base, k_rs, lk) : -1;
+            anchors[bh] = anchor;
+            float bias[ATTN_D];
+            if (anchor >= 0)
+                for (int c = 0; c < ATTN_D; ++c) bias[c] = ld_t(dt, k, base + (int64_t)anchor * k_rs + c);
+            for (int t = 0; t < kb; ++t)
+                for (int g = 0; g < 4; ++g) {
+                    int rows[32];
+                    const int n = ck / 4;
+                    for (int i = 0; i < n; ++i) rows[i] = t * ck + (i / 2) * 8 + g * 2 + (i % 2);
+                    attn_quant_group(dt, k, base, k_rs, rows, n, lk, anchor >= 0 ? bias : NULL, ki + bh * lk * ATTN_D,
+                                     &ks[(bh * kb + t) * 4 + g]);
+                }
+        }
+    return 0;
+}
+
+/* v [b, lk, hk, 128] -> vi [b,hk,lk,128] (plain order; the reference stores it transposed and permuted for its MMA,
+ * quant_v_int8.cu:178-190), vs [b,hk,128]: scale = max(absmax/127 as a product with 1/127, 1e-12) (:163-168). */
+ORC_API int orc_attn_quant_v(int dt, const void* v, int b, int lk, int hk, int64_t v_bs, int64_t v_rs, int64_t v_hs,
+                             int8_t* vi, float* vs) {
+    for (int bi = 0; bi < b; ++bi)
+        for (int hi = 0; hi < hk; ++hi) {
+            const int64_t bh = (int64_t)bi * hk + hi, base = bi * v_bs + hi * v_hs;
+            for (int c = 0; c < ATTN_D; ++c) {
+                float mx = 0.f;
+                for (int n = 0; n < lk; ++n) mx = fmax_dev(mx, fabsf(ld_t(dt, v, base + (int64_t)n * v_rs + c)));
+                const float sc = fmax_dev(mx * (1.f / 127.f), 1e-12f), inv = 1.f / sc;
+                vs[bh * ATTN_D + c] = sc;
+                for (int n = 0; n < lk; ++n)
+                    vi[(bh * lk + n) * ATTN_D + c] = attn_rn_s8(ld_t(dt, v, base + (int64_t)n * v_rs + c) * inv);
+            }
+        }
+    return 0;
+}
+
+static inline float attn_exp2(float x) { return (float)exp2((double)x); }
+
+/* The attention proper over the quantized tensors (csrc/vendor/sage/qk_int_sv_i8_cuda.cuh, mask none).  Per query row
+ * and tile of ck keys: integer scores; per key group the maximum score times that group's scale, minus the u8 offset
+ * (attn_utils.cuh:719-741; the last tile takes the float path with its -50000 floor, :569-596); probabilities
+ * exp2(fma(score, scale, -tile_max)) rounded to u8 (:700-717, mma.cuh:793-804); denominators and outputs rescaled by
+ * exp2(-|m_prev - tile_max|) on whichever side is smaller (:742-756); outputs += float(sum p*v) * tile_scale by fmaf
+ * (:1254-1258); O = RO / d * v_scale (:1130-1146, qk_int_sv_i8_cuda.cuh:1056-1072).  The denominator is summed here
+ * per row in key order; the reference keeps four per-thread partials. */
+ORC_API int orc_attn_int8(int out_dt, const int8_t* qi, const int8_t* ki, const int8_t* vi, const float* qs,
+                          const float* ks, const float* vs, int b, int lq, int lk, int h, int hk, int ck, float scale,
+                          void* o, int64_t o_bs, int64_t o_rs, int64_t o_hs) {
+    if ((ck != 64 && ck != 128) || hk <= 0 || h % hk != 0) return -1;
+    const int qg = (lq + 127) / 128 * 4, kb = (lk + ck - 1) / ck, rep = h / hk;
+    const float sm = scale * 1.44269504088896340736f;
+    #pragma omp parallel for collapse(2) schedule(dynamic, 8)
+    for (int bh = 0; bh < b * h; ++bh)
+        for (int r = 0; r < lq; ++r) {
+            const int bi = bh / h, hi = bh % h;
+            const int64_t kvh = (int64_t)bi * hk + hi / rep;
+            const int8_t* qrow = qi + ((int64_t)bh * lq + r) * ATTN_D;
+            const float q_scale = qs[((int64_t)bh * qg + r / 32) * 8 + r % 8];
+            float m = -50000.f, d = 1.f, ro[ATTN_D];
+            for (int c = 0; c < ATTN_D; ++c) ro[c] = 0.f;
+            int32_t s[128];
+            for (int t = 0; t < kb; ++t) {
+                const int n = lk - t * ck < ck ? lk - t * ck : ck;
+                const int last = t == kb - 1;
+                float gs[4], tile_m = 0.f;
+                for (int g = 0; g < 4; ++g) gs[g] = sm * (q_scale * ks[(kvh * kb + t) * 4 + g]);
+                for (int j = 0; j < n; ++j) {
+                    const int8_t* krow = ki + ((int64_t)kvh * lk + t * ck + j) * ATTN_D;
+                    int32_t acc = 0;
+                    for (int c = 0; c < ATTN_D; ++c) acc += (int32_t)qrow[c] * (int32_t)krow[c];
+                    s[j] = acc;
+                }
+                for (int g = 0; g < 4; ++g) {
+                    float mg = last ? -50000.f : -3.0e38f;
+                    int any = 0;
+                    for (int j = 0; j < n; ++j)
+                        if ((j % 8) / 2 == g) { mg = fmax_dev(mg, (float)s[j]); any = 1; }
+                    if (!any && !last) continue;
+                    const float cand = fmaf(mg, gs[g], -ATTN_U8_OFFSET);
+                    tile_m = (g == 0 || cand > tile_m) ? cand : tile_m;
+                }
+                const float smaller = attn_exp2(-fabsf(m - tile_m));
+                const float o_scale = m < tile_m ? smaller : 1.f, t_scale = tile_m < m ? smaller : 1.f;
+                m = m > tile_m ? m : tile_m;
+                d *= o_scale;
+                int32_t pv[ATTN_D];
+                int32_t psum = 0;
+                for (int c = 0; c < ATTN_D; ++c) pv[c] = 0;
+                for (int j = 0; j < n; ++j) {
+                    float p = attn_exp2(fmaf((float)s[j], gs[(j % 8) / 2], -tile_m));
+                    p = rintf(p > 255.f ? 255.f : p);
+                    const int32_t pi = (int32_t)p;
+                    psum += pi;
+                    const int8_t* vrow = vi + ((int64_t)kvh * lk + t * ck + j) * ATTN_D;
+                    for (int c = 0; c < ATTN_D; ++c) pv[c] += pi * (int32_t)vrow[c];
+                }
+                d += (float)psum * t_scale;
+                for (int c = 0; c < ATTN_D; ++c) ro[c] = fmaf((float)pv[c], t_scale, ro[c] * o_scale);
+            }
+            const float rcp = 1.f / d;
+            for (int c = 0; c < ATTN_D; ++c)
+                st_t(out_dt, o, bi * o_bs + (int64_t)r * o_rs + hi * o_hs + c, ro[c] * rcp * vs[kvh * ATTN_D + c]);
+        }
+    return 0;
+}
+
+/* csrc/attn_int8.cu:56 */
+ORC_API int orc_attn_cta_k(int lk, int d) { return lk > 1024 && d != 64 ? 128 : 64; }

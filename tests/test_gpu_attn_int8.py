@@ -1,0 +1,172 @@
+"""INT8 attention on the GPU against the CPU oracle (quantizer stages bit-exact, outputs within a stated tolerance) and
+against exact softmax attention.
+
+The quantizer stages are integer/rounding work and must match the oracle bit for bit.  The attention output is floating
+point: the kernel's exp2 is the hardware instruction (1 ulp) where the oracle's is correctly rounded, so a u8
+probability can land one step away when the exponent sits on a rounding boundary, and the denominators are summed in a
+different order; the tolerance below is what one such step per row can move an output.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from conftest import pkg
+
+pytestmark = pytest.mark.gpu
+
+
+def _pkg():
+    return pkg("qlinear"), pkg("ffi")
+
+
+def _bits(t):
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def _to_f32(bits, dt):
+    return oracle.bf16_to_f32(bits) if dt == oracle.BF16 else oracle.f16_to_f32(bits)
+
+
+def _inputs(b, lq, lk, h, hk, dtype, seed, k_offset=0.0, v_scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(b, lq, h, 128, generator=g)
+    k = torch.randn(b, lk, hk, 128, generator=g) + k_offset
+    v = torch.randn(b, lk, hk, 128, generator=g) * v_scale
+    return q.to(dtype), k.to(dtype), v.to(dtype)
+
+
+def _exact(q, k, v, scale):
+    h, hk = q.shape[2], k.shape[2]
+    qq = q.double().permute(0, 2, 1, 3)
+    kk = k.double().permute(0, 2, 1, 3).repeat_interleave(h // hk, 1)
+    vv = v.double().permute(0, 2, 1, 3).repeat_interleave(h // hk, 1)
+    return (torch.softmax(qq @ kk.transpose(-1, -2) * scale, -1) @ vv).permute(0, 2, 1, 3).numpy()
+
+
+def _layout(ffi, b, h, hk, lq, lk):
+    out = (C.c_int64 * 10)()
+    assert ffi.raw("gpu_internal_attn_layout", b, h, hk, lq, lk, C.cast(out, C.c_void_p)) == 0
+    return list(out)
+
+
+CASES = [
+    # b, lq, lk, h, hk, dtype, k_offset
+    (1, 200, 300, 4, 2, torch.bfloat16, 0.0),
+    (2, 77, 64, 2, 2, torch.bfloat16, 0.0),
+    (1, 1, 1, 1, 1, torch.bfloat16, 0.0),
+    (1, 129, 65, 2, 1, torch.float16, 0.0),
+    (1, 257, 63, 3, 3, torch.bfloat16, 4.0),      # a K offset large enough for the anchor to switch on
+    (1, 96, 1025, 2, 2, torch.bfloat16, 0.0),     # 128-key tiles with a ragged last tile of one key
+    (1, 130, 1500, 4, 1, torch.float16, 2.0),
+    (1, 33, 1152, 1, 1, torch.bfloat16, 0.0),     # 128-key tiles, no ragged tail
+]
+
+
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "b%d_lq%d_lk%d_h%d_hk%d_%s_off%g" % (c[0], c[1], c[2], c[3], c[4], str(c[5])[6:], c[6]))
+def test_attention_against_oracle(case):
+    ql, ffi = _pkg()
+    b, lq, lk, h, hk, dtype, off = case
+    dt = oracle.BF16 if dtype == torch.bfloat16 else oracle.F16
+    q, k, v = _inputs(b, lq, lk, h, hk, dtype, seed=lq * 7 + lk, k_offset=off)
+    scale = 128 ** -0.5
+    ref_q = oracle.attn_quant(dt, _bits(q), _bits(k), _bits(v))
+    ref = _to_f32(oracle.attn_int8(dt, _bits(q), _bits(k), _bits(v), scale, quant=ref_q), dt)
+
+    ws_bytes = ffi.lib.gpu_int8_attn_workspace_d(b, h, hk, lq, lk, 128)
+    ws = torch.zeros((ws_bytes,), dtype=torch.uint8, device="cuda")
+    o = ql.int8_attn(q.cuda(), k.cuda(), v.cuda(), scale, ws=ws)
+    torch.cuda.synchronize()
+    w = ws.cpu().numpy()
+    qi_o, ki_o, qs_o, ks_o, vt_o, vs_o, an_o, vsum_o, ck, kb = _layout(ffi, b, h, hk, lq, lk)
+    assert ck == ref_q["ck"]
+
+    def take(at, n, dtp):
+        return w[at:at + n * np.dtype(dtp).itemsize].view(dtp)
+
+    # quantizer stages: bit-exact
+    assert np.array_equal(take(an_o, b * hk, np.int32).reshape(b, hk), ref_q["anchors"])
+    if off >= 2.0:
+        assert (ref_q["anchors"] >= 0).all(), "this case is meant to exercise the anchor"
+    assert np.array_equal(take(qi_o, b * h * lq * 128, np.int8).reshape(b, h, lq, 128), ref_q["qi"])
+    assert np.array_equal(take(ki_o, b * hk * lk * 128, np.int8).reshape(b, hk, lk, 128), ref_q["ki"])
+    qs = take(qs_o, ref_q["qs"].size, np.float32).reshape(ref_q["qs"].shape)
+    # groups with no row below lq are never read; compare the groups that own a row
+    own = np.zeros(ref_q["qs"].shape[-1], bool)
+    for r in range(lq):
+        own[(r // 32) * 8 + r % 8] = True
+    assert np.array_equal(qs[..., own].view(np.uint32), ref_q["qs"][..., own].view(np.uint32))
+    assert np.array_equal(take(ks_o, ref_q["ks"].size, np.float32).view(np.uint32), ref_q["ks"].reshape(-1).view(np.uint32))
+    assert np.array_equal(take(vs_o, b * hk * 128, np.float32).view(np.uint32), ref_q["vs"].reshape(-1).view(np.uint32))
+    nblk = kb * (ck // 32)
+    vt = take(vt_o, b * hk * nblk * 128 * 32, np.int8).reshape(b, hk, nblk, 128, 32)
+    pos = np.arange(32)
+    key_of_pos = ((pos % 16) // 4) * 8 + (pos // 16) * 4 + pos % 4
+    vi_pad = np.zeros((b, hk, nblk * 32, 128), np.int8)
+    vi_pad[:, :, :lk] = ref_q["vi"]
+    want_vt = vi_pad.reshape(b, hk, nblk, 32, 128)[:, :, :, key_of_pos, :].transpose(0, 1, 2, 4, 3)
+    assert np.array_equal(vt, want_vt)
+    vsum = take(vsum_o, b * hk * kb * 128, np.int32).reshape(b, hk, kb, 128)
+    want_sum = 128 * vi_pad.reshape(b, hk, kb, ck, 128).astype(np.int64).sum(3)
+    assert np.array_equal(vsum, want_sum)
+
+    # outputs
+    got = _to_f32(_bits(o), dt)
+    vmax = float(v.float().abs().max())
+    ulp = 2.0 ** (-8 if dt == oracle.BF16 else -11)
+    tol = 2 * vmax / 255.0 + 2 * ulp * np.abs(ref)
+    err = np.abs(got - ref)
+    assert (err <= tol).all(), "max excess %g" % float((err - tol).max())
+    assert (err <= ulp * np.abs(ref) + 1e-30).mean() > 0.97, "more than 3 % of outputs differ from the oracle by over one ulp"
+
+    # and the whole thing is attention: close to exact softmax attention of the same rounded inputs
+    ex = _exact(q, k, v, scale)
+    cos = float((got * ex).sum() / np.sqrt((got * got).sum() * (ex * ex).sum()))
+    assert cos > 0.9995, cos
+
+
+def test_attention_strided_views_match_contiguous():
+    """q, k, v as slices of one packed [b, l, 3, h, 128] tensor and o written into a wider buffer."""
+    ql, ffi = _pkg()
+    b, l, h = 2, 150, 3
+    g = torch.Generator().manual_seed(5)
+    qkv = torch.randn(b, l, 3, h, 128, generator=g).bfloat16().cuda()
+    q, k, v = qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2]
+    scale = 0.11
+    a = ql.int8_attn(q, k, v, scale)
+    c = ql.int8_attn(q.contiguous(), k.contiguous(), v.contiguous(), scale)
+    assert torch.equal(a, c)
+
+
+def test_attention_refuses_what_it_does_not_build():
+    ql, ffi = _pkg()
+    x = torch.zeros(1, 4, 1, 128, dtype=torch.bfloat16, device="cuda")
+    ws = torch.zeros(1 << 16, dtype=torch.uint8, device="cuda")
+    p = lambda t: C.c_void_p(t.data_ptr())
+    args = lambda D, h, hk: (p(x), p(x), p(x), p(x), p(ws), 1, 4, 4, h, hk, D, 512, 128, 128, 512, 128, 128, 512, 128, 128, 512, 128, 128, 0.1, None)
+    assert ffi.raw("gpu_int8_attn_d", *args(64, 1, 1)) == -400
+    assert ffi.raw("gpu_int8_attn_d", *args(128, 3, 2)) == -400
+    assert ffi.raw("gpu_int8_attn_d", *args(128, 1, 1)) == 0
+    torch.cuda.synchronize()
+
+
+def test_attention_dit_size_against_exact_attention():
+    """The DiT joint-attention shape (4608 tokens, 24 heads): no oracle at this size, so the check is against fp32 softmax
+    attention on the GPU, and row-stochasticity: attention over constant V returns that constant."""
+    ql, ffi = _pkg()
+    b, l, h = 1, 4608, 24
+    g = torch.Generator(device="cuda").manual_seed(3)
+    q = torch.randn(b, l, h, 128, generator=g, device="cuda").bfloat16()
+    k = (torch.randn(b, l, h, 128, generator=g, device="cuda") + 0.3).bfloat16()
+    v = torch.randn(b, l, h, 128, generator=g, device="cuda").bfloat16()
+    scale = 128 ** -0.5
+    o = ql.int8_attn(q, k, v, scale).float()
+    ex = torch.nn.functional.scaled_dot_product_attention(q.float().transpose(1, 2), k.float().transpose(1, 2),
+                                                          v.float().transpose(1, 2), scale=scale).transpose(1, 2)
+    cos = float((o * ex).sum() / torch.sqrt((o * o).sum() * (ex * ex).sum()))
+    assert cos > 0.999, cos
+    vc = torch.full_like(v, 0.75)
+    oc = ql.int8_attn(q, k, vc, scale).float()
+    assert float((oc - 0.75).abs().max()) <= 0.75 * 2 ** -7

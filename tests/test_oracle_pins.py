@@ -866,3 +866,102 @@ def test_w6_requant_invariants_and_closed_form(synth):
     c = np.float32(31 * 2.0 ** -6)
     rc, p1, r1, s1 = oracle.w6_requant(oracle.bf16_bits(np.full((1, 256), c, np.float32)), 12345)
     assert (w6_codes_of(p1, 256) == 63).all() and (r1 == 0x48).all() and s1[0] == c / np.float32(127)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# INT8 attention oracle
+# ---------------------------------------------------------------------------------------------------------------
+_ATTN_SIGNS = [0x1035997B, 0x8087F5EE, 0xEE2E4E1A, 0x71132418]
+
+
+def _attn_sign_vector():
+    return np.array([1.0 if ((_ATTN_SIGNS[(ch >> 2) >> 3] >> (((ch >> 2) & 7) * 4 + (ch & 3))) & 1) else -1.0 for ch in range(128)])
+
+
+def test_attn_rotation_is_the_signed_sylvester_hadamard():
+    """A dense Sylvester matrix from scipy, not the butterfly: a wrong stage order, sign or scale fails here."""
+    import scipy.linalg
+    H = scipy.linalg.hadamard(128).astype(np.float64) / np.sqrt(128.0)
+    sg = _attn_sign_vector()
+    rng = np.random.default_rng(11)
+    for _ in range(4):
+        x = rng.standard_normal(128).astype(np.float32)
+        assert np.abs(oracle.attn_rot128(x) - H @ (x.astype(np.float64) * sg)).max() < 2e-6
+    # exact on small integers scaled so every butterfly sum is representable: compare unscaled
+    e = np.zeros(128, np.float32)
+    e[77] = 1.0
+    col = oracle.attn_rot128(e)
+    assert np.array_equal(col, (H[:, 77] * sg[77]).astype(np.float32))
+    # orthonormal: the rotation of Q and K leaves their dot product alone
+    a, b = rng.standard_normal(128).astype(np.float32), rng.standard_normal(128).astype(np.float32)
+    assert abs(float(oracle.attn_rot128(a).astype(np.float64) @ oracle.attn_rot128(b).astype(np.float64)) - float(a.astype(np.float64) @ b.astype(np.float64))) < 1e-4
+
+
+def _attn_case(b, lq, lk, h, hk, seed, k_offset=0.0):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(b, lq, h, 128, generator=g).bfloat16()
+    k = (torch.randn(b, lk, hk, 128, generator=g) + k_offset).bfloat16()
+    v = torch.randn(b, lk, hk, 128, generator=g).bfloat16()
+    bits = lambda t: t.view(torch.int16).numpy().view(np.uint16)
+    return q, k, v, bits
+
+
+def test_attn_quantizers_scale_groups_and_half_step_bound():
+    """Dequantized codes sit within half a step of the rotated rows, the step being the group's scale; the groups are the
+    ones the layout says (rows r, r+8, .. for Q; keys with equal (key % 8) / 2 per tile for K); V per channel."""
+    import scipy.linalg
+    H = scipy.linalg.hadamard(128).astype(np.float64) / np.sqrt(128.0)
+    sg = _attn_sign_vector()
+    q, k, v, bits = _attn_case(1, 70, 150, 2, 1, seed=2)
+    z = oracle.attn_quant(oracle.BF16, bits(q), bits(k), bits(v), use_anchor=False)
+    assert z["ck"] == 64 and oracle.lib().orc_attn_cta_k(1025, 128) == 128 and oracle.lib().orc_attn_cta_k(4096, 64) == 64
+    rq = (q.double().numpy() * sg) @ H.T                                 # [1, lq, h, 128]
+    rk = (k.double().numpy() * sg) @ H.T
+    for r in range(70):
+        for hi in range(2):
+            sc = z["qs"][0, hi, (r // 32) * 8 + r % 8]
+            assert np.abs(z["qi"][0, hi, r] * np.float64(sc) - rq[0, r, hi]).max() <= 0.5 * sc * 1.0001 + 1e-6
+    for n in range(150):
+        sc = z["ks"][0, 0, (n // 64) * 4 + (n % 8) // 2]
+        assert np.abs(z["ki"][0, 0, n] * np.float64(sc) - rk[0, n, 0]).max() <= 0.5 * sc * 1.0001 + 1e-6
+    # every group's largest code reaches the ends of the int8 range: the scale is the group's abs-max / 127
+    grp = np.array([(n // 64) * 4 + (n % 8) // 2 for n in range(150)])
+    for gi in np.unique(grp):
+        assert np.abs(z["ki"][0, 0, grp == gi].astype(int)).max() in (126, 127)
+    vs = z["vs"][0, 0]
+    vf = v.float().numpy()[0, :, 0]
+    assert np.array_equal(vs, np.maximum(np.abs(vf).max(0) * np.float32(1.0 / 127.0), np.float32(1e-12)))
+    assert np.abs(z["vi"][0, 0] * vs.astype(np.float64) - vf).max() <= 0.5 * vs.max() * 1.0001
+
+
+def test_attn_anchor_switches_on_for_offset_keys_only():
+    q, k, v, bits = _attn_case(1, 8, 90, 2, 2, seed=4, k_offset=0.0)
+    assert (oracle.attn_quant(oracle.BF16, bits(q), bits(k), bits(v))["anchors"] == -1).all()
+    q, k, v, bits = _attn_case(1, 8, 90, 2, 2, seed=4, k_offset=5.0)
+    z = oracle.attn_quant(oracle.BF16, bits(q), bits(k), bits(v))
+    samples = {i * 89 // 8 for i in range(9)}
+    assert all(int(a) in samples for a in z["anchors"].ravel())
+    # the shift is softmax-invariant: attention with and without the anchor agree to quantization accuracy
+    a = oracle.bf16_to_f32(oracle.attn_int8(oracle.BF16, bits(q), bits(k), bits(v), 0.09, use_anchor=True))
+    c = oracle.bf16_to_f32(oracle.attn_int8(oracle.BF16, bits(q), bits(k), bits(v), 0.09, use_anchor=False))
+    assert np.abs(a - c).max() < 0.05
+
+
+@pytest.mark.parametrize("shape", [(1, 40, 130, 2, 1), (2, 33, 64, 2, 2), (1, 5, 1100, 1, 1)])
+def test_attn_oracle_is_attention(shape):
+    """Against exact fp64 softmax attention of the same rounded inputs: a dropped rescale, a wrong scale group or a
+    transposed operand would be far outside this."""
+    b, lq, lk, h, hk = shape
+    q, k, v, bits = _attn_case(b, lq, lk, h, hk, seed=lq + lk, k_offset=0.5)
+    scale = 128 ** -0.5
+    got = oracle.bf16_to_f32(oracle.attn_int8(oracle.BF16, bits(q), bits(k), bits(v), scale))
+    qq = q.double().permute(0, 2, 1, 3)
+    kk = k.double().permute(0, 2, 1, 3).repeat_interleave(h // hk, 1)
+    vv = v.double().permute(0, 2, 1, 3).repeat_interleave(h // hk, 1)
+    ex = (torch.softmax(qq @ kk.transpose(-1, -2) * scale, -1) @ vv).permute(0, 2, 1, 3).numpy()
+    assert np.abs(got - ex).max() < 0.03
+    assert float((got * ex).sum() / np.sqrt((got * got).sum() * (ex * ex).sum())) > 0.9997
+    # one key: the output is that key's value, whatever the scores
+    o1 = oracle.bf16_to_f32(oracle.attn_int8(oracle.BF16, bits(q), bits(k[:, :1]), bits(v[:, :1]), scale))
+    want = v[:, :1].float().numpy().repeat(h // hk, 2)
+    assert np.abs(o1 - want).max() <= np.abs(want).max() / 127.0 * 0.51 + 2 ** -8 * np.abs(want).max()
