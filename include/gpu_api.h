@@ -139,6 +139,10 @@ int gpu_int8_attn(const void* q, const void* k, const void* v, void* o, void* ws
                   int64_t q_bs, int64_t q_rs, int64_t q_hs, int64_t k_bs, int64_t k_rs, int64_t k_hs, int64_t v_bs,
                   int64_t v_rs, int64_t v_hs, int64_t o_bs, int64_t o_rs, int64_t o_hs, float scale, void* stream);
 
+/* Test hook, no reference counterpart: byte offsets of the pieces of the attention workspace and its tiling,
+ * out[0..9] = qi, ki, qs, ks, vt, vs, anchors, vsum, key tile length, key tiles. */
+int gpu_internal_attn_layout(int b, int h, int hk, int lq, int lk, int64_t* out);
+
 /* D[M,N] = Out((A[M,K] . W[N,K]^T) * xs[m] * ws[n] + bias[n]).
  * Replaces gpu_int8_gemm, src/ffi.rs:38 / csrc/gemm.cu:124-129.
  * A, W int8 row-major (K contiguous); xs f32 [M]; ws f32 [N]; bias Out[N] or null; D Out[M,N]; out_dt a DT_* code. */
