@@ -12,7 +12,9 @@
 //   * the matrix cores multiply signed bytes only: probabilities 0..255 are fed as p - 128 and the accumulator starts
 //     at 128 * (column sums of the V tile), which the V quantizer leaves in the workspace.  The integers are exact.
 // The workspace layout is private to this file.
+#include <climits>
 #include <cstdio>
+#include <type_traits>
 
 #include "common.hpp"
 
@@ -214,7 +216,11 @@ __global__ __launch_bounds__(128) void attn_quant_k_kernel(AttnArgs a) {
                     uint32_t w = 0;
 #pragma unroll
                     for (int c = 0; c < 4; ++c) w |= (uint32_t)(uint8_t)rn_s8(v[c] * inv) << (8 * c);
-                    *reinterpret_cast<uint32_t*>(a.ki + (bh * a.lk + row) * D + lane32 * 4) = w;
+                    // fragment order: [32-key block][channel step of 32][half of 16 channels][key][16 bytes], so that
+                    // the 64 lanes of the attention kernel read one contiguous KB per load
+                    const int c0 = lane32 * 4;
+                    const int64_t at = (((bh * a.nblk + row / 32) * 4 + c0 / 32) * 64 + ((c0 % 32) / 16) * 32 + row % 32) * 16 + c0 % 16;
+                    *reinterpret_cast<uint32_t*>(a.ki + at) = w;
                 }
             }
         }
@@ -266,7 +272,7 @@ __global__ __launch_bounds__(256) void attn_v_quant_kernel(AttnArgs a) {
 // The attention: a wave owns 32 query rows and walks the key tiles on its own (no LDS, no barriers); four waves per
 // workgroup share K and V tiles through the caches.
 template <int OUT_DT, int CK>
-__global__ __launch_bounds__(256) void attn_int8_kernel(AttnArgs a) {
+__global__ __launch_bounds__(256, 2) void attn_int8_kernel(AttnArgs a) {
     constexpr int NB = CK / 32;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int l32 = lane & 31, hh = lane >> 5;
@@ -297,12 +303,11 @@ __global__ __launch_bounds__(256) void attn_int8_kernel(AttnArgs a) {
         v16i S[NB];
 #pragma unroll
         for (int blk = 0; blk < NB; ++blk) {
-            const int key = key0 + blk * 32 + l32;
-            const int8_t* krow = a.ki + (kvh * a.lk + (key < a.lk ? key : a.lk - 1)) * D + hh * 16;
+            const int8_t* kp = a.ki + (((kvh * a.nblk + (t * NB + blk)) * 4) * 64 + lane) * 16;
             v16i acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
-                const v4i kf = *reinterpret_cast<const v4i*>(krow + s * 32);
+                const v4i kf = *reinterpret_cast<const v4i*>(kp + s * 1024);
                 acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf, qf[s], acc, 0, 0, 0);
             }
             S[blk] = acc;
@@ -310,44 +315,67 @@ __global__ __launch_bounds__(256) void attn_int8_kernel(AttnArgs a) {
         const float* ksc = a.ks + (kvh * a.kb + t) * 4 + hh * 2;
         const float gs0 = a.sm * (q_scale * ksc[0]), gs1 = a.sm * (q_scale * ksc[1]);
 
-        float m0 = last ? -50000.f : -3.0e38f, m1 = m0;
+        // Group maxima on the integers (exact in fp32: |score| < 2^24).  Only the last tile can hold keys past lk; its
+        // maxima start at the reference's floor of -50000.
+        int i0, i1;
+        if (!last) {
+            i0 = i1 = INT_MIN;
 #pragma unroll
-        for (int blk = 0; blk < NB; ++blk)
+            for (int blk = 0; blk < NB; ++blk)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int key = key0 + blk * 32 + (i / 4) * 8 + hh * 4 + (i % 4);
-                const float sv = (float)S[blk][i];
-                if (key < a.lk) {
-                    if ((i % 4) < 2) m0 = fmax_nn(m0, sv);
-                    else m1 = fmax_nn(m1, sv);
+                for (int i = 0; i < 16; ++i) {
+                    if ((i % 4) < 2) i0 = max(i0, S[blk][i]);
+                    else i1 = max(i1, S[blk][i]);
                 }
-            }
-        float tile_m = fmax_nn(fmaf(m0, gs0, -kU8Offset), fmaf(m1, gs1, -kU8Offset));
+        } else {
+            i0 = i1 = -50000;
+#pragma unroll
+            for (int blk = 0; blk < NB; ++blk)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int key = key0 + blk * 32 + (i / 4) * 8 + hh * 4 + (i % 4);
+                    const int sv = key < a.lk ? S[blk][i] : INT_MIN;
+                    if ((i % 4) < 2) i0 = max(i0, sv);
+                    else i1 = max(i1, sv);
+                }
+        }
+        float tile_m = fmax_nn(fmaf((float)i0, gs0, -kU8Offset), fmaf((float)i1, gs1, -kU8Offset));
         tile_m = fmax_nn(tile_m, __shfl_xor(tile_m, 32));
         const float smaller = __builtin_amdgcn_exp2f(-fabsf(m - tile_m));
         const float o_scale = m < tile_m ? smaller : 1.f, t_scale = tile_m < m ? smaller : 1.f;
         m = fmax_nn(m, tile_m);
         dsum *= o_scale;
 
+        // Probabilities: exp2 of at most the u8 offset is below 255.5, so adding 2^23 leaves round-to-nearest-even(p) in
+        // the low byte of the float's bits.  p - 128 as a signed byte is p ^ 0x80.
         v4i pf[NB];
-        int psum = 0;
+        uint32_t psum = 0;
+        auto probabilities = [&](auto masked) {
 #pragma unroll
-        for (int blk = 0; blk < NB; ++blk) {
-            uint32_t w[4] = {0u, 0u, 0u, 0u};
+            for (int blk = 0; blk < NB; ++blk) {
+                uint32_t w[4];
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int key = key0 + blk * 32 + (i / 4) * 8 + hh * 4 + (i % 4);
-                int p = 0;
-                if (key < a.lk) {
-                    float e = __builtin_amdgcn_exp2f(fmaf((float)S[blk][i], (i % 4) < 2 ? gs0 : gs1, -tile_m));
-                    e = e > 255.f ? 255.f : e;
-                    p = (int)__builtin_rintf(e);
+                for (int g4 = 0; g4 < 4; ++g4) {
+                    uint32_t u[4];
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        const float e = __builtin_amdgcn_exp2f(fmaf((float)S[blk][g4 * 4 + c], c < 2 ? gs0 : gs1, -tile_m));
+                        u[c] = f2u(e + 8388608.f);
+                        if constexpr (decltype(masked)::value) {
+                            const int key = key0 + blk * 32 + g4 * 8 + hh * 4 + c;
+                            u[c] = key < a.lk ? u[c] : 0u;
+                        }
+                    }
+                    const uint32_t packed =
+                        __builtin_amdgcn_perm(u[1], u[0], 0x0c0c0400u) | __builtin_amdgcn_perm(u[3], u[2], 0x04000c0cu);
+                    psum = __builtin_amdgcn_sad_u8(packed, 0u, psum);
+                    w[g4] = packed ^ 0x80808080u;
                 }
-                psum += p;
-                w[i / 4] |= (uint32_t)((p - 128) & 0xff) << (8 * (i % 4));
+                pf[blk] = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
             }
-            pf[blk] = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
-        }
+        };
+        if (last) probabilities(std::true_type{});
+        else probabilities(std::false_type{});
         dsum += (float)psum * t_scale;
 
 #pragma unroll
@@ -409,7 +437,7 @@ Plan plan_for(int64_t b, int64_t h, int64_t hk, int64_t lq, int64_t lk) {
     int64_t n = 0;
     auto add = [&](int64_t bytes) { const int64_t at = n; n += (bytes + 255) / 256 * 256; return at; };
     p.qi = add(b * h * lq * D);
-    p.ki = add(b * hk * lk * D);
+    p.ki = add(b * hk * (int64_t)p.nblk * 32 * D);
     p.qs = add(b * h * p.qg * 8 * 4);
     p.ks = add(b * hk * p.kb * 4 * 4);
     p.vt = add(b * hk * (int64_t)p.nblk * D * 32);

@@ -91,7 +91,11 @@ def test_attention_against_oracle(case):
     if off >= 2.0:
         assert (ref_q["anchors"] >= 0).all(), "this case is meant to exercise the anchor"
     assert np.array_equal(take(qi_o, b * h * lq * 128, np.int8).reshape(b, h, lq, 128), ref_q["qi"])
-    assert np.array_equal(take(ki_o, b * hk * lk * 128, np.int8).reshape(b, hk, lk, 128), ref_q["ki"])
+    nblk = kb * (ck // 32)
+    # K lies in fragment order: [32-key block][channel step of 32][half of 16 channels][key][16 bytes]
+    ki = take(ki_o, b * hk * nblk * 32 * 128, np.int8).reshape(b, hk, nblk, 4, 2, 32, 16)
+    ki = ki.transpose(0, 1, 2, 5, 3, 4, 6).reshape(b, hk, nblk * 32, 128)[:, :, :lk]
+    assert np.array_equal(ki, ref_q["ki"])
     qs = take(qs_o, ref_q["qs"].size, np.float32).reshape(ref_q["qs"].shape)
     # groups with no row below lq are never read; compare the groups that own a row
     own = np.zeros(ref_q["qs"].shape[-1], bool)
@@ -100,7 +104,6 @@ def test_attention_against_oracle(case):
     assert np.array_equal(qs[..., own].view(np.uint32), ref_q["qs"][..., own].view(np.uint32))
     assert np.array_equal(take(ks_o, ref_q["ks"].size, np.float32).view(np.uint32), ref_q["ks"].reshape(-1).view(np.uint32))
     assert np.array_equal(take(vs_o, b * hk * 128, np.float32).view(np.uint32), ref_q["vs"].reshape(-1).view(np.uint32))
-    nblk = kb * (ck // 32)
     vt = take(vt_o, b * hk * nblk * 128 * 32, np.int8).reshape(b, hk, nblk, 128, 32)
     pos = np.arange(32)
     key_of_pos = ((pos % 16) // 4) * 8 + (pos // 16) * 4 + pos % 4
