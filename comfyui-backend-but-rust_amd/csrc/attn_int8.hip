@@ -269,18 +269,37 @@ __global__ __launch_bounds__(256) void attn_v_quant_kernel(AttnArgs a) {
     atomicAdd(&a.vsum[(bh * a.kb + s / (a.ck / 32)) * D + d], 128 * sum);
 }
 
-// The attention: a wave owns 32 query rows and walks the key tiles on its own (no LDS, no barriers); four waves per
-// workgroup share K and V tiles through the caches.
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* glb_ptr_t;
+
+// The attention: a workgroup of four waves owns 128 query rows, a wave 32 of them.  The K tile, the V tile and the
+// tile's 128 x column sums are contiguous in the workspace, in the order the fragment reads want them, so the four waves
+// copy them global -> LDS with DMA loads (no registers) into one of two stages, a tile ahead; one barrier per tile.
 template <int OUT_DT, int CK>
 __global__ __launch_bounds__(256, 2) void attn_int8_kernel(AttnArgs a) {
-    constexpr int NB = CK / 32;
+    constexpr int NB = CK / 32, KV = CK * D, STAGE = 2 * KV + 512;
+    extern __shared__ __align__(16) uint8_t smem[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int l32 = lane & 31, hh = lane >> 5;
     const int hi = blockIdx.y, bi = blockIdx.z;
     const int row0 = blockIdx.x * 128 + wave * 32;
-    if (row0 >= a.lq) return;
     const int64_t bh = (int64_t)bi * a.h + hi, kvh = (int64_t)bi * a.hk + hi / a.rep;
+    // rows past lq are computed on a clamped row and never stored: every wave takes part in the copies and barriers
     const int r = row0 + l32, rc = r < a.lq ? r : a.lq - 1;
+
+    auto fetch = [&](int t) {
+        uint8_t* st = smem + (t & 1) * STAGE;
+        const int64_t tile = (kvh * a.nblk + (int64_t)t * NB) * 4096 + lane * 16;
+#pragma unroll
+        for (int j = 0; j < KV / 4096; ++j) {
+            const int c = wave + 4 * j;
+            __builtin_amdgcn_global_load_lds((glb_ptr_t)(a.ki + tile + c * 1024), (lds_ptr_t)(st + c * 1024), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((glb_ptr_t)(a.vt + tile + c * 1024), (lds_ptr_t)(st + KV + c * 1024), 16, 0, 0);
+        }
+        if (wave == 0 && lane < 32)
+            __builtin_amdgcn_global_load_lds((glb_ptr_t)(a.vsum + (kvh * a.kb + t) * D + lane * 4), (lds_ptr_t)(st + 2 * KV), 16, 0, 0);
+    };
+    fetch(0);
 
     v4i qf[4];
     {
@@ -296,14 +315,17 @@ __global__ __launch_bounds__(256, 2) void attn_int8_kernel(AttnArgs a) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) ro[x][i] = 0.f;
     float m = -50000.f, dsum = 1.f;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
 
     for (int t = 0; t < a.kb; ++t) {
+        const uint8_t* st = smem + (t & 1) * STAGE;
         const int key0 = t * CK;
         const bool last = t == a.kb - 1;
         v16i S[NB];
 #pragma unroll
         for (int blk = 0; blk < NB; ++blk) {
-            const int8_t* kp = a.ki + (((kvh * a.nblk + (t * NB + blk)) * 4) * 64 + lane) * 16;
+            const uint8_t* kp = st + blk * 4096 + lane * 16;
             v16i acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
@@ -312,6 +334,7 @@ __global__ __launch_bounds__(256, 2) void attn_int8_kernel(AttnArgs a) {
             }
             S[blk] = acc;
         }
+        if (t + 1 < a.kb) fetch(t + 1);   // the other stage: every wave left it at the barrier that ended the last tile
         const float* ksc = a.ks + (kvh * a.kb + t) * 4 + hh * 2;
         const float gs0 = a.sm * (q_scale * ksc[0]), gs1 = a.sm * (q_scale * ksc[1]);
 
@@ -372,6 +395,7 @@ __global__ __launch_bounds__(256, 2) void attn_int8_kernel(AttnArgs a) {
                     w[g4] = packed ^ 0x80808080u;
                 }
                 pf[blk] = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+                __builtin_amdgcn_sched_barrier(0);   // one block at a time: the converted scores die here
             }
         };
         if (last) probabilities(std::true_type{});
@@ -380,7 +404,7 @@ __global__ __launch_bounds__(256, 2) void attn_int8_kernel(AttnArgs a) {
 
 #pragma unroll
         for (int x = 0; x < 4; ++x) {
-            const int* vsp = a.vsum + (kvh * a.kb + t) * D + x * 32 + hh * 4;
+            const int* vsp = reinterpret_cast<const int*>(st + 2 * KV) + x * 32 + hh * 4;
             v16i acc;
 #pragma unroll
             for (int g4 = 0; g4 < 4; ++g4) {
@@ -392,13 +416,15 @@ __global__ __launch_bounds__(256, 2) void attn_int8_kernel(AttnArgs a) {
             }
 #pragma unroll
             for (int blk = 0; blk < NB; ++blk) {
-                const int8_t* vp = a.vt + ((kvh * a.nblk + (t * NB + blk)) * D + x * 32 + l32) * 32 + hh * 16;
+                const uint8_t* vp = st + KV + ((blk * D + x * 32 + l32) * 32 + hh * 16);
                 const v4i vf = *reinterpret_cast<const v4i*>(vp);
                 acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf, pf[blk], acc, 0, 0, 0);
             }
 #pragma unroll
             for (int i = 0; i < 16; ++i) ro[x][i] = fmaf((float)acc[i], t_scale, ro[x][i] * o_scale);
         }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wave's share of the next tile has landed
+        __syncthreads();
     }
 
     const float dtot = dsum + __shfl_xor(dsum, 32);
@@ -459,8 +485,12 @@ int run(AttnArgs a, hipStream_t st) {
     attn_v_absmax_kernel<DT><<<dim3((a.lk + 127) / 128, a.hk, a.b), 256, 0, st>>>(a);
     attn_v_quant_kernel<DT><<<dim3(a.nblk, a.hk, a.b), 256, 0, st>>>(a);
     const dim3 grid((a.lq + 127) / 128, a.h, a.b);
-    if (a.ck == 64) attn_int8_kernel<DT, 64><<<grid, 256, 0, st>>>(a);
-    else attn_int8_kernel<DT, 128><<<grid, 256, 0, st>>>(a);
+    constexpr int kLds64 = 2 * (2 * 64 * D + 512), kLds128 = 2 * (2 * 128 * D + 512);
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_int8_kernel<DT, 128>),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLds128);
+    if (attr != hipSuccess) return -401;
+    if (a.ck == 64) attn_int8_kernel<DT, 64><<<grid, 256, kLds64, st>>>(a);
+    else attn_int8_kernel<DT, 128><<<grid, 256, kLds128, st>>>(a);
     return hipGetLastError() == hipSuccess ? 0 : -401;
 }
 
