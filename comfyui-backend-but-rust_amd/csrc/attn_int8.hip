@@ -34,7 +34,7 @@ struct AttnArgs {
     int b, lq, lk, h, hk, rep, qg, kb, ck, nblk;
     int64_t q_bs, q_rs, q_hs, k_bs, k_rs, k_hs, v_bs, v_rs, v_hs, o_bs, o_rs, o_hs;
     float sm;
-    int vec_ok;
+    int vec_ok, in_vec, v_vec;
 };
 
 __device__ __forceinline__ float fmax_nn(float a, float b) { return a > b ? a : b; }
@@ -69,15 +69,20 @@ __device__ __forceinline__ void rot128(float (&v)[4], int lane32) {
     for (int c = 0; c < 4; ++c) v[c] *= 0.1767766952966369f;
 }
 
+// Four consecutive elements: one 8-byte load when the caller's strides and base allow it.
+template <int DT> __device__ __forceinline__ void ld4_dt(const void* p, int64_t i, bool vec, float (&v)[4]) {
+    if (vec) {
+        load4<DT>(p, i, v);
+    } else {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) v[c] = ld_dt<DT>(p, i + c);
+    }
+}
+
 __device__ __forceinline__ float max32(float m) {
 #pragma unroll
     for (int off = 16; off > 0; off >>= 1) m = fmax_nn(m, __shfl_xor(m, off));
     return m;
-}
-
-__global__ void attn_zero_kernel(uint32_t* p, int64_t n) {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) p[i] = 0u;
 }
 
 // One workgroup of 128 threads per (kv head, batch): thread = channel.  The shuffle trees of the reference are summed
@@ -89,6 +94,11 @@ __global__ __launch_bounds__(128) void attn_anchor_kernel(AttnArgs a) {
     __shared__ int chosen;
     const int c = threadIdx.x, hi = blockIdx.x, bi = blockIdx.y;
     const int64_t base = bi * a.k_bs + hi * a.k_hs;
+    {   // the V quantizer's accumulators for this (kv head, batch) start at zero
+        const int64_t bh = (int64_t)bi * a.hk + hi;
+        a.vmax[bh * D + c] = 0u;
+        for (int t = 0; t < a.kb; ++t) a.vsum[(bh * a.kb + t) * D + c] = 0;
+    }
     float e = 0.f, m = 0.f, sum = 0.f;
 #pragma unroll
     for (int i = 0; i < 9; ++i) {
@@ -114,12 +124,16 @@ __global__ __launch_bounds__(128) void attn_anchor_kernel(AttnArgs a) {
             for (int i = 0; i < off; ++i) t[i] += t[i + off];
         return t[0];
     };
+    __shared__ float warp_sum[11][4];   // nine candidate distances, then the two energies
+    if (c < 36) warp_sum[c / 4][c % 4] = tree(&dist[c / 4][(c % 4) * 32]);
+    else if (c < 40) warp_sum[9][c - 36] = tree(&energy[(c - 36) * 32]);
+    __syncthreads();
     if (c == 0) {
         int best = 0;
         float best_d = 3.402823466e+38F;
         for (int i = 0; i < 9; ++i) {
             float d = 0.f;
-            for (int w = 0; w < 4; ++w) d += tree(&dist[i][w * 32]);
+            for (int w = 0; w < 4; ++w) d += warp_sum[i][w];
             if (d < best_d) { best = i; best_d = d; }
         }
         chosen = best;
@@ -136,11 +150,13 @@ __global__ __launch_bounds__(128) void attn_anchor_kernel(AttnArgs a) {
     best_energy[c] = be;
     bmax[c] = bm;
     __syncthreads();
+    if (c < 4) warp_sum[10][c] = tree(&best_energy[c * 32]);
+    __syncthreads();
     if (c == 0) {
         float e0 = 0.f, e1 = 0.f, m0 = 0.f, m1 = 0.f;
         for (int w = 0; w < 4; ++w) {
-            e0 += tree(&energy[w * 32]);
-            e1 += tree(&best_energy[w * 32]);
+            e0 += warp_sum[9][w];
+            e1 += warp_sum[10][w];
         }
         for (int i = 0; i < D; ++i) {
             m0 = fmax_nn(m0, amax[i]);
@@ -162,8 +178,7 @@ __global__ __launch_bounds__(256) void attn_quant_q_kernel(AttnArgs a) {
     for (int j = 0; j < 4; ++j) {
         const int row = t * 32 + g + 8 * j;
         const int rowc = row < a.lq ? row : a.lq - 1;
-#pragma unroll
-        for (int c = 0; c < 4; ++c) v[j][c] = ld_dt<DT>(a.q, base + (int64_t)rowc * a.q_rs + c);
+        ld4_dt<DT>(a.q, base + (int64_t)rowc * a.q_rs, a.in_vec, v[j]);
         rot128(v[j], lane32);
         if (row < a.lq) {
 #pragma unroll
@@ -185,83 +200,124 @@ __global__ __launch_bounds__(256) void attn_quant_q_kernel(AttnArgs a) {
     }
 }
 
-// K: one workgroup of 128 threads per tile of ck keys; each run of 32 lanes is one scale group (keys with
-// (key % 8) / 2 == g).  Two passes over the group's rows: abs-max, then codes.
-template <int DT>
+// K: one workgroup of 128 threads per tile of CK keys; each run of 32 lanes is one scale group (keys with
+// (key % 8) / 2 == g), whose CK/4 rows stay in registers between the abs-max and the codes.
+template <int DT, int CK>
 __global__ __launch_bounds__(128) void attn_quant_k_kernel(AttnArgs a) {
+    constexpr int N = CK / 4;
     const int lane32 = threadIdx.x & 31, g = threadIdx.x >> 5;
     const int t = blockIdx.x, hi = blockIdx.y, bi = blockIdx.z;
     const int64_t bh = (int64_t)bi * a.hk + hi, base = bi * a.k_bs + hi * a.k_hs + lane32 * 4;
     const int anchor = a.anchors[bh];
     float bias[4] = {0.f, 0.f, 0.f, 0.f};
-    if (anchor >= 0) {
+    if (anchor >= 0) ld4_dt<DT>(a.k, base + (int64_t)anchor * a.k_rs, a.in_vec, bias);
+    float v[N][4];
 #pragma unroll
-        for (int c = 0; c < 4; ++c) bias[c] = ld_dt<DT>(a.k, base + (int64_t)anchor * a.k_rs + c);
+    for (int i = 0; i < N; ++i) {
+        const int row = t * CK + (i / 2) * 8 + g * 2 + (i % 2);
+        ld4_dt<DT>(a.k, base + (int64_t)(row < a.lk ? row : a.lk - 1) * a.k_rs, a.in_vec, v[i]);
     }
-    const int n = a.ck / 4;
-    float mx = 0.f, inv = 0.f;
-    for (int pass = 0; pass < 2; ++pass) {
-        for (int i = 0; i < n; ++i) {
-            const int row = t * a.ck + (i / 2) * 8 + g * 2 + (i % 2);
-            const int rowc = row < a.lk ? row : a.lk - 1;
-            float v[4];
+    float mx = 0.f;
 #pragma unroll
-            for (int c = 0; c < 4; ++c) v[c] = ld_dt<DT>(a.k, base + (int64_t)rowc * a.k_rs + c) - bias[c];
-            rot128(v, lane32);
-            if (row < a.lk) {
-                if (pass == 0) {
+    for (int i = 0; i < N; ++i) {
+        const int row = t * CK + (i / 2) * 8 + g * 2 + (i % 2);
 #pragma unroll
-                    for (int c = 0; c < 4; ++c) mx = fmax_nn(mx, fabsf(v[c]));
-                } else {
-                    uint32_t w = 0;
+        for (int c = 0; c < 4; ++c) v[i][c] -= bias[c];
+        rot128(v[i], lane32);
+        if (row < a.lk) {
 #pragma unroll
-                    for (int c = 0; c < 4; ++c) w |= (uint32_t)(uint8_t)rn_s8(v[c] * inv) << (8 * c);
-                    // fragment order: [32-key block][channel step of 32][half of 16 channels][key][16 bytes], so that
-                    // the 64 lanes of the attention kernel read one contiguous KB per load
-                    const int c0 = lane32 * 4;
-                    const int64_t at = (((bh * a.nblk + row / 32) * 4 + c0 / 32) * 64 + ((c0 % 32) / 16) * 32 + row % 32) * 16 + c0 % 16;
-                    *reinterpret_cast<uint32_t*>(a.ki + at) = w;
-                }
-            }
+            for (int c = 0; c < 4; ++c) mx = fmax_nn(mx, fabsf(v[i][c]));
         }
-        if (pass == 0) {
-            mx = max32(mx);
-            const float sc = mx / 127.f + 1e-7f;
-            inv = 1.f / sc;
-            if (lane32 == 0) a.ks[(bh * a.kb + t) * 4 + g] = sc;
+    }
+    mx = max32(mx);
+    const float sc = mx / 127.f + 1e-7f, inv = 1.f / sc;
+    if (lane32 == 0) a.ks[(bh * a.kb + t) * 4 + g] = sc;
+    // fragment order: [32-key block][channel step of 32][half of 16 channels][key][16 bytes], so that the 64 lanes of
+    // the attention kernel read one contiguous KB per load
+    const int c0 = lane32 * 4;
+    const int64_t col = (int64_t)(c0 / 32) * 1024 + ((c0 % 32) / 16) * 512 + c0 % 16;
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        const int row = t * CK + (i / 2) * 8 + g * 2 + (i % 2);
+        if (row < a.lk) {
+            uint32_t w = 0;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) w |= (uint32_t)(uint8_t)rn_s8(v[i][c] * inv) << (8 * c);
+            *reinterpret_cast<uint32_t*>(a.ki + (bh * a.nblk + row / 32) * 4096 + col + (row % 32) * 16) = w;
         }
     }
 }
 
-// V abs-max per channel: 256 threads take 128 rows of one (kv head, batch); non-negative floats order as their bits.
+// V abs-max per channel: 256 threads take 128 rows of one (kv head, batch), four channels per thread; non-negative
+// floats order as their bits, so the workgroups combine with an integer atomic max.
 template <int DT>
 __global__ __launch_bounds__(256) void attn_v_absmax_kernel(AttnArgs a) {
-    const int c = threadIdx.x & 127, half = threadIdx.x >> 7;
+    __shared__ float red[8][D];
+    const int c4 = threadIdx.x & 31, rl = threadIdx.x >> 5;
     const int hi = blockIdx.y, bi = blockIdx.z;
-    const int64_t base = bi * a.v_bs + hi * a.v_hs + c;
-    float mx = 0.f;
+    const int64_t base = bi * a.v_bs + hi * a.v_hs + c4 * 4;
+    float mx[4] = {0.f, 0.f, 0.f, 0.f};
     const int r0 = blockIdx.x * 128;
-    for (int r = r0 + half; r < r0 + 128 && r < a.lk; r += 2) mx = fmax_nn(mx, fabsf(ld_dt<DT>(a.v, base + (int64_t)r * a.v_rs)));
-    atomicMax(&a.vmax[((int64_t)bi * a.hk + hi) * D + c], f2u(mx));
+#pragma unroll 4
+    for (int i = 0; i < 16; ++i) {
+        const int r = r0 + rl + 8 * i;
+        if (r < a.lk) {
+            float x[4];
+            ld4_dt<DT>(a.v, base + (int64_t)r * a.v_rs, a.v_vec, x);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) mx[c] = fmax_nn(mx[c], fabsf(x[c]));
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < 4; ++c) red[rl][c4 * 4 + c] = mx[c];
+    __syncthreads();
+    if (threadIdx.x < D) {
+        float m = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) m = fmax_nn(m, red[i][threadIdx.x]);
+        atomicMax(&a.vmax[((int64_t)bi * a.hk + hi) * D + threadIdx.x], f2u(m));
+    }
 }
 
-// V codes: one workgroup per block of 32 keys.  vt[(kv head, block)][d][32]: position h*16 + j of a row holds key
+// V codes: one workgroup per block of 32 keys.  Rows are read as they lie (a thread takes 16 channels of one key),
+// quantized and turned through LDS.  vt[(kv head, block)][d][32]: position h*16 + j of a row holds key
 // (j/4)*8 + h*4 + j%4 of the block, which is the order a lane of the attention kernel holds its 16 scores in.  Keys past
 // lk are zeros.  128 x the column sums go to vsum[(kv head, key tile)][d] by integer atomics.
 template <int DT>
 __global__ __launch_bounds__(256) void attn_v_quant_kernel(AttnArgs a) {
-    const int d = threadIdx.x & 127, hh = threadIdx.x >> 7;
+    __shared__ float inv_s[D];
+    __shared__ __align__(16) int8_t tile[32][D];
     const int s = blockIdx.x, hi = blockIdx.y, bi = blockIdx.z;
-    const int64_t bh = (int64_t)bi * a.hk + hi, base = bi * a.v_bs + hi * a.v_hs + d;
-    const float sc = fmax_nn(u2f(a.vmax[bh * D + d]) * (1.f / 127.f), 1e-12f), inv = 1.f / sc;
-    if (s == 0 && hh == 0) a.vs[bh * D + d] = sc;
+    const int64_t bh = (int64_t)bi * a.hk + hi;
+    if (threadIdx.x < D) {
+        const float sc = fmax_nn(u2f(a.vmax[bh * D + threadIdx.x]) * (1.f / 127.f), 1e-12f);
+        if (s == 0) a.vs[bh * D + threadIdx.x] = sc;
+        inv_s[threadIdx.x] = 1.f / sc;
+    }
+    __syncthreads();
+    {
+        const int key = threadIdx.x >> 3, seg = threadIdx.x & 7;
+        const int row = s * 32 + key;
+        uint32_t w[4] = {0u, 0u, 0u, 0u};
+        if (row < a.lk) {
+            const int64_t at = bi * a.v_bs + hi * a.v_hs + (int64_t)row * a.v_rs + seg * 16;
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                float x[4];
+                ld4_dt<DT>(a.v, at + g4 * 4, a.v_vec, x);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) w[g4] |= (uint32_t)(uint8_t)rn_s8(x[c] * inv_s[seg * 16 + g4 * 4 + c]) << (8 * c);
+            }
+        }
+        *reinterpret_cast<uint4*>(&tile[key][seg * 16]) = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+    __syncthreads();
+    const int d = threadIdx.x & 127, hh = threadIdx.x >> 7;
     uint32_t w[4] = {0u, 0u, 0u, 0u};
     int sum = 0;
 #pragma unroll
     for (int j = 0; j < 16; ++j) {
-        const int key = s * 32 + (j / 4) * 8 + hh * 4 + (j % 4);
-        int q = 0;
-        if (key < a.lk) q = rn_s8(ld_dt<DT>(a.v, base + (int64_t)key * a.v_rs) * inv);
+        const int q = tile[(j / 4) * 8 + hh * 4 + (j % 4)][d];
         sum += q;
         w[j / 4] |= (uint32_t)(uint8_t)q << (8 * (j % 4));
     }
@@ -469,7 +525,7 @@ Plan plan_for(int64_t b, int64_t h, int64_t hk, int64_t lq, int64_t lk) {
     p.vt = add(b * hk * (int64_t)p.nblk * D * 32);
     p.vs = add(b * hk * D * 4);
     p.anchors = add(b * hk * 4);
-    p.vmax = add(b * hk * D * 4);                  // vmax and vsum are adjacent: one fill clears both
+    p.vmax = add(b * hk * D * 4);
     p.vsum = add(b * hk * (int64_t)p.kb * D * 4);
     p.total = n;
     return p;
@@ -477,11 +533,10 @@ Plan plan_for(int64_t b, int64_t h, int64_t hk, int64_t lq, int64_t lk) {
 
 template <int DT>
 int run(AttnArgs a, hipStream_t st) {
-    const int64_t nz = ((char*)a.vsum - (char*)a.vmax) / 4 + (int64_t)a.b * a.hk * a.kb * D;
-    attn_zero_kernel<<<dim3((unsigned)((nz + 255) / 256)), 256, 0, st>>>(a.vmax, nz);
     attn_anchor_kernel<DT><<<dim3(a.hk, a.b), 128, 0, st>>>(a);
     attn_quant_q_kernel<DT><<<dim3(a.qg, a.h, a.b), 256, 0, st>>>(a);
-    attn_quant_k_kernel<DT><<<dim3(a.kb, a.hk, a.b), 128, 0, st>>>(a);
+    if (a.ck == 64) attn_quant_k_kernel<DT, 64><<<dim3(a.kb, a.hk, a.b), 128, 0, st>>>(a);
+    else attn_quant_k_kernel<DT, 128><<<dim3(a.kb, a.hk, a.b), 128, 0, st>>>(a);
     attn_v_absmax_kernel<DT><<<dim3((a.lk + 127) / 128, a.hk, a.b), 256, 0, st>>>(a);
     attn_v_quant_kernel<DT><<<dim3(a.nblk, a.hk, a.b), 256, 0, st>>>(a);
     const dim3 grid((a.lq + 127) / 128, a.h, a.b);
@@ -520,6 +575,8 @@ int int8_attn(const void* q, const void* k, const void* v, void* o, void* ws, in
     a.v_bs = v_bs; a.v_rs = v_rs; a.v_hs = v_hs; a.o_bs = o_bs; a.o_rs = o_rs; a.o_hs = o_hs;
     a.sm = scale * 1.44269504088896340736f;
     a.vec_ok = ((o_bs | o_rs | o_hs) % 4 == 0 && ((uintptr_t)o & 7) == 0) ? 1 : 0;
+    a.v_vec = ((v_bs | v_rs | v_hs) % 4 == 0 && ((uintptr_t)v & 7) == 0) ? 1 : 0;
+    a.in_vec = ((q_bs | q_rs | q_hs | k_bs | k_rs | k_hs) % 4 == 0 && (((uintptr_t)q | (uintptr_t)k) & 7) == 0) ? 1 : 0;
     return dt == DT_F16 ? run<DT_F16>(a, (hipStream_t)stream) : run<DT_BF16>(a, (hipStream_t)stream);
 }
 
