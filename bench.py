@@ -35,6 +35,8 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-skinny", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the other linears of the model configurations and the W6A8 shapes")
+    ap.add_argument("--attention-only", action="store_true",
+                    help="time only the INT8 attention shapes and print them as one JSON line (for profiling that path alone)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 256 MiB device copy a few times: under rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE its "
@@ -178,6 +180,38 @@ def time_row_kernels(torch, ffi, steps):
     return out
 
 
+def time_attention(torch, ffi, steps):
+    """INT8 attention (quantizers + attention kernel, one call) at the image-DiT joint-attention shape, HIP events on
+    the launch stream.  ops = 4 * b * h * lq * lk * 128 (the two matrix products)."""
+    dev = "cuda:0"
+    st = torch.cuda.current_stream()
+    g = torch.Generator(device=dev).manual_seed(11)
+    out = []
+    for (name, b, l, h, hk) in (("image-dit joint attention", 1, 4608, 24, 24), ("long video attention", 2, 8192, 16, 16)):
+        q, k, v = (torch.randn(b, l, hh, 128, device=dev, generator=g).to(torch.bfloat16) for hh in (h, hk, hk))
+        o = torch.empty_like(q)
+        ws = torch.empty((ffi.lib.gpu_int8_attn_workspace_d(b, h, hk, l, l, 128),), dtype=torch.uint8, device=dev)
+        sq, sk = q.stride(), k.stride()
+        call = lambda: ffi.k("gpu_int8_attn_d", q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), ws.data_ptr(), b, l, l, h,
+                             hk, 128, sq[0], sq[1], sq[2], sk[0], sk[1], sk[2], sk[0], sk[1], sk[2], sq[0], sq[1], sq[2],
+                             128 ** -0.5, st.cuda_stream)
+        for _ in range(3):
+            call()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record(st)
+        for _ in range(steps):
+            call()
+        e1.record(st)
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / steps
+        ops = 4.0 * b * h * l * l * 128
+        out.append({"name": name, "b": b, "lq": l, "lk": l, "h": h, "hk": hk, "head_dim": 128, "kernel": "gpu_int8_attn_d",
+                    "us": round(us, 1), "TOPS": round(ops / us / 1e6, 1), "frac_int8_peak": round(ops / us / 1e6 / PEAK_INT8_TOPS, 4)})
+        del q, k, v, o, ws
+    return out
+
+
 def cpu_baseline(host, M, K, N, rotate, target_s):
     """The oracle's whole linear (quantize, int32 GEMM, epilogue) on a row sample sized for about `target_s` seconds."""
     import oracle
@@ -213,6 +247,9 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(1)
     M, K, N = (int(v) for v in a.shape.split(","))
+    if a.attention_only:
+        print(json.dumps({"attention": time_attention(torch, ffi, max(5, a.steps // 3))}))
+        return
     if a.copy_probe:
         src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda:0").random_(0, 255)
         dst = torch.empty_like(src)
@@ -282,6 +319,7 @@ def main():
                        "TOPS": round(2.0 * m * n * k / us / 1e6, 1), "frac_int8_peak": round(2.0 * m * n * k / us / 1e6 / PEAK_INT8_TOPS, 4)})
         out["w6a8"] = w6
         out["row_kernels"] = time_row_kernels(torch, ffi, few)
+        out["attention"] = time_attention(torch, ffi, few)
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(host, M, K, N, a.rotate, a.cpu_seconds)
     print(json.dumps(out))
