@@ -40,6 +40,13 @@
  *                                      row sums are fp32 in the order of its thread layout and its expf / erff /
  *                                      tanhf / rsqrtf are CUDA's 1-2 ulp routines; here sums are fp64 rounded once and
  *                                      the functions are correctly rounded (fp64 libm rounded to fp32).
+ *   orc_attn_rot128                    pinned: dense Sylvester-Hadamard matrix (scipy) with the sign diagonal, unit columns exact
+ *   orc_attn_quant_qk / orc_attn_quant_v  structure pinned: half-step bound of every code against the rotated row with the
+ *                                      scale of the group the layout names, V scales against the numpy expression, anchor on
+ *                                      for offset keys only; the anchor detector's fma is an assumption about nvcc
+ *   orc_attn_int8                      pinned as attention: exact fp64 softmax attention of the same inputs, one-key case.
+ *                                      PARITY UNPINNED against a run of the reference (its exp2 / reciprocal are PTX
+ *                                      approximations and its build may use fast math): see the section's own header
  */
 #include <math.h>
 #include <stdint.h>
