@@ -45,28 +45,69 @@ __device__ __forceinline__ int8_t rn_s8(float v) {
     return (int8_t)(r > 127.f ? 127.f : r < -128.f ? -128.f : r);
 }
 
-// Sign diagonal and normalized Walsh-Hadamard over the 128 channels of one row held by 32 consecutive lanes, four
-// adjacent channels per lane.  Same operation order as the oracle: H4 in the lane, butterflies over lane bits, scale.
-__device__ __forceinline__ void rot128(float (&v)[4], int lane32) {
-    const uint32_t signs = lane32 < 8 ? 0x1035997bu : lane32 < 16 ? 0x8087f5eeu : lane32 < 24 ? 0xee2e4e1au : 0x71132418u;
-    const int shift = (lane32 & 7) * 4;
+// Cross-lane moves inside a run of eight lanes, as data-parallel-primitive modifiers (no LDS traffic).
+template <int CTRL> __device__ __forceinline__ float dpp_mov(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float lane_xor1(float x) { return dpp_mov<0xB1>(x); }                   // quad_perm [1,0,3,2]
+__device__ __forceinline__ float lane_xor2(float x) { return dpp_mov<0x4E>(x); }                   // quad_perm [2,3,0,1]
+__device__ __forceinline__ float lane_xor4(float x) { return dpp_mov<0x1B>(dpp_mov<0x141>(x)); }   // half-row mirror (xor 7), then quad reverse (xor 3)
+
+// Sign diagonal and normalized Walsh-Hadamard over the 128 channels of one row held by eight consecutive lanes, sixteen
+// adjacent channels per lane (o8 = lane within the eight).  Same operation order as the oracle: H4 on runs of four
+// channels, radix-2 butterflies over channel bits 2..6 (two in the lane, three across lanes), one scaling.
+__device__ __forceinline__ void rot128(float (&v)[16], int o8) {
+    const uint32_t word = (o8 >> 1) == 0 ? 0x1035997bu : (o8 >> 1) == 1 ? 0x8087f5eeu : (o8 >> 1) == 2 ? 0xee2e4e1au : 0x71132418u;
+    const uint32_t keep = word >> ((o8 & 1) * 16);
 #pragma unroll
-    for (int c = 0; c < 4; ++c) v[c] = u2f(f2u(v[c]) ^ ((((signs >> (shift + c)) & 1u) ^ 1u) << 31));
-    const float a0 = v[0] + v[1], a1 = v[0] - v[1], a2 = v[2] + v[3], a3 = v[2] - v[3];
-    v[0] = (a0 + a2) * 0.5f;
-    v[1] = (a1 + a3) * 0.5f;
-    v[2] = (a0 - a2) * 0.5f;
-    v[3] = (a1 - a3) * 0.5f;
+    for (int e = 0; e < 16; ++e) v[e] = u2f(f2u(v[e]) ^ ((((keep >> e) & 1u) ^ 1u) << 31));
 #pragma unroll
-    for (int bit = 1; bit < 32; bit <<= 1) {
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            const float other = __shfl_xor(v[c], bit);
-            v[c] = (lane32 & bit) ? other - v[c] : v[c] + other;
-        }
+    for (int g = 0; g < 16; g += 4) {
+        const float a0 = v[g] + v[g + 1], a1 = v[g] - v[g + 1], a2 = v[g + 2] + v[g + 3], a3 = v[g + 2] - v[g + 3];
+        v[g] = (a0 + a2) * 0.5f;
+        v[g + 1] = (a1 + a3) * 0.5f;
+        v[g + 2] = (a0 - a2) * 0.5f;
+        v[g + 3] = (a1 - a3) * 0.5f;
     }
 #pragma unroll
-    for (int c = 0; c < 4; ++c) v[c] *= 0.1767766952966369f;
+    for (int bit = 4; bit < 16; bit <<= 1)
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+            if (!(e & bit)) {
+                const float lo = v[e], hi = v[e | bit];
+                v[e] = lo + hi;
+                v[e | bit] = lo - hi;
+            }
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+        const float other = lane_xor1(v[e]);
+        v[e] = (o8 & 1) ? other - v[e] : v[e] + other;
+    }
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+        const float other = lane_xor2(v[e]);
+        v[e] = (o8 & 2) ? other - v[e] : v[e] + other;
+    }
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+        const float other = lane_xor4(v[e]);
+        v[e] = (o8 & 4) ? other - v[e] : v[e] + other;
+    }
+#pragma unroll
+    for (int e = 0; e < 16; ++e) v[e] *= 0.1767766952966369f;
+}
+
+__device__ __forceinline__ float max8(float m) {
+    m = fmax_nn(m, lane_xor1(m));
+    m = fmax_nn(m, lane_xor2(m));
+    return fmax_nn(m, lane_xor4(m));
+}
+
+__device__ __forceinline__ uint4 codes16(const float (&v)[16], float inv) {
+    uint32_t w[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int e = 0; e < 16; ++e) w[e / 4] |= (uint32_t)(uint8_t)rn_s8(v[e] * inv) << (8 * (e % 4));
+    return make_uint4(w[0], w[1], w[2], w[3]);
 }
 
 // Four consecutive elements: one 8-byte load when the caller's strides and base allow it.
@@ -79,10 +120,14 @@ template <int DT> __device__ __forceinline__ void ld4_dt(const void* p, int64_t 
     }
 }
 
-__device__ __forceinline__ float max32(float m) {
+template <int DT> __device__ __forceinline__ void ld16_dt(const void* p, int64_t i, bool vec, float (&v)[16]) {
 #pragma unroll
-    for (int off = 16; off > 0; off >>= 1) m = fmax_nn(m, __shfl_xor(m, off));
-    return m;
+    for (int g = 0; g < 4; ++g) {
+        float x[4];
+        ld4_dt<DT>(p, i + g * 4, vec, x);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) v[g * 4 + c] = x[c];
+    }
 }
 
 // One workgroup of 128 threads per (kv head, batch): thread = channel.  The shuffle trees of the reference are summed
@@ -166,86 +211,97 @@ __global__ __launch_bounds__(128) void attn_anchor_kernel(AttnArgs a) {
     }
 }
 
-// Q: one workgroup of 256 threads per 32 rows; each run of 32 lanes is one scale group (rows g, g+8, g+16, g+24).
+// Q: a wave per 32 rows, four waves per workgroup; each run of eight lanes is one scale group (rows g, g+8, g+16, g+24),
+// a lane holding 16 channels of each of the four rows.
 template <int DT>
 __global__ __launch_bounds__(256) void attn_quant_q_kernel(AttnArgs a) {
-    const int lane32 = threadIdx.x & 31, g = threadIdx.x >> 5;
-    const int t = blockIdx.x, hi = blockIdx.y, bi = blockIdx.z;
-    const int64_t bh = (int64_t)bi * a.h + hi, base = bi * a.q_bs + hi * a.q_hs + lane32 * 4;
-    float v[4][4];
+    const int lane = threadIdx.x & 63, o8 = lane & 7, g = lane >> 3;
+    const int hi = blockIdx.x, bi = blockIdx.z;   // heads fastest: neighbours read neighbouring memory
+    const int t = blockIdx.y * 4 + (threadIdx.x >> 6);
+    if (t >= a.qg) return;
+    const int64_t bh = (int64_t)bi * a.h + hi, base = bi * a.q_bs + hi * a.q_hs + o8 * 16;
+    float v[4][16];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int row = t * 32 + g + 8 * j;
+        ld16_dt<DT>(a.q, base + (int64_t)(row < a.lq ? row : a.lq - 1) * a.q_rs, a.in_vec, v[j]);
+    }
     float mx = 0.f;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        const int row = t * 32 + g + 8 * j;
-        const int rowc = row < a.lq ? row : a.lq - 1;
-        ld4_dt<DT>(a.q, base + (int64_t)rowc * a.q_rs, a.in_vec, v[j]);
-        rot128(v[j], lane32);
-        if (row < a.lq) {
+        rot128(v[j], o8);
+        if (t * 32 + g + 8 * j < a.lq) {
 #pragma unroll
-            for (int c = 0; c < 4; ++c) mx = fmax_nn(mx, fabsf(v[j][c]));
+            for (int e = 0; e < 16; ++e) mx = fmax_nn(mx, fabsf(v[j][e]));
         }
     }
-    mx = max32(mx);
+    mx = max8(mx);
     const float sc = mx / 127.f + 1e-7f, inv = 1.f / sc;
-    if (lane32 == 0) a.qs[(bh * a.qg + t) * 8 + g] = sc;
+    if (o8 == 0) a.qs[(bh * a.qg + t) * 8 + g] = sc;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const int row = t * 32 + g + 8 * j;
-        if (row < a.lq) {
-            uint32_t w = 0;
-#pragma unroll
-            for (int c = 0; c < 4; ++c) w |= (uint32_t)(uint8_t)rn_s8(v[j][c] * inv) << (8 * c);
-            *reinterpret_cast<uint32_t*>(a.qi + (bh * a.lq + row) * D + lane32 * 4) = w;
-        }
+        if (row < a.lq) *reinterpret_cast<uint4*>(a.qi + (bh * a.lq + row) * D + o8 * 16) = codes16(v[j], inv);
     }
 }
 
-// K: one workgroup of 128 threads per tile of CK keys; each run of 32 lanes is one scale group (keys with
-// (key % 8) / 2 == g), whose CK/4 rows stay in registers between the abs-max and the codes.
+// K: one workgroup of 256 threads per tile of CK keys.  A scale group is the keys with (key % 8) / 2 == g; its CK/4 rows
+// are shared out over eight runs of eight lanes, whose maxima meet in LDS.  The tile is assembled in LDS in fragment
+// order, [32-key block][channel step of 32][half of 16 channels][key][16 bytes] (the 64 lanes of the attention kernel
+// read one contiguous KB per load), and leaves as 16-byte stores over its contiguous CK * 128 bytes; keys past lk are
+// zeros.
 template <int DT, int CK>
-__global__ __launch_bounds__(128) void attn_quant_k_kernel(AttnArgs a) {
-    constexpr int N = CK / 4;
-    const int lane32 = threadIdx.x & 31, g = threadIdx.x >> 5;
-    const int t = blockIdx.x, hi = blockIdx.y, bi = blockIdx.z;
-    const int64_t bh = (int64_t)bi * a.hk + hi, base = bi * a.k_bs + hi * a.k_hs + lane32 * 4;
+__global__ __launch_bounds__(256) void attn_quant_k_kernel(AttnArgs a) {
+    constexpr int R = CK / 32;   // rows per run of eight lanes
+    __shared__ float omax[32];
+    __shared__ __align__(16) uint8_t stage[CK * D];
+    const int o8 = threadIdx.x & 7, oct = threadIdx.x >> 3, g = oct & 3, sub = oct >> 2;
+    const int hi = blockIdx.x, t = blockIdx.y, bi = blockIdx.z;   // heads fastest: neighbours read neighbouring memory
+    const int64_t bh = (int64_t)bi * a.hk + hi, base = bi * a.k_bs + hi * a.k_hs + o8 * 16;
     const int anchor = a.anchors[bh];
-    float bias[4] = {0.f, 0.f, 0.f, 0.f};
-    if (anchor >= 0) ld4_dt<DT>(a.k, base + (int64_t)anchor * a.k_rs, a.in_vec, bias);
-    float v[N][4];
+    float bias[16];
 #pragma unroll
-    for (int i = 0; i < N; ++i) {
-        const int row = t * CK + (i / 2) * 8 + g * 2 + (i % 2);
-        ld4_dt<DT>(a.k, base + (int64_t)(row < a.lk ? row : a.lk - 1) * a.k_rs, a.in_vec, v[i]);
+    for (int e = 0; e < 16; ++e) bias[e] = 0.f;
+    if (anchor >= 0) ld16_dt<DT>(a.k, base + (int64_t)anchor * a.k_rs, a.in_vec, bias);
+    float v[R][16];
+    int rt[R];
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+        const int i = sub * R + j;                  // index within the group
+        rt[j] = (i / 2) * 8 + g * 2 + (i % 2);      // row within the tile
+        const int row = t * CK + rt[j];
+        ld16_dt<DT>(a.k, base + (int64_t)(row < a.lk ? row : a.lk - 1) * a.k_rs, a.in_vec, v[j]);
     }
     float mx = 0.f;
 #pragma unroll
-    for (int i = 0; i < N; ++i) {
-        const int row = t * CK + (i / 2) * 8 + g * 2 + (i % 2);
+    for (int j = 0; j < R; ++j) {
 #pragma unroll
-        for (int c = 0; c < 4; ++c) v[i][c] -= bias[c];
-        rot128(v[i], lane32);
-        if (row < a.lk) {
+        for (int e = 0; e < 16; ++e) v[j][e] -= bias[e];
+        rot128(v[j], o8);
+        if (t * CK + rt[j] < a.lk) {
 #pragma unroll
-            for (int c = 0; c < 4; ++c) mx = fmax_nn(mx, fabsf(v[i][c]));
+            for (int e = 0; e < 16; ++e) mx = fmax_nn(mx, fabsf(v[j][e]));
         }
     }
-    mx = max32(mx);
+    mx = max8(mx);
+    if (o8 == 0) omax[oct] = mx;
+    __syncthreads();
+    mx = 0.f;
+#pragma unroll
+    for (int x = 0; x < 8; ++x) mx = fmax_nn(mx, omax[x * 4 + g]);
     const float sc = mx / 127.f + 1e-7f, inv = 1.f / sc;
-    if (lane32 == 0) a.ks[(bh * a.kb + t) * 4 + g] = sc;
-    // fragment order: [32-key block][channel step of 32][half of 16 channels][key][16 bytes], so that the 64 lanes of
-    // the attention kernel read one contiguous KB per load
-    const int c0 = lane32 * 4;
-    const int64_t col = (int64_t)(c0 / 32) * 1024 + ((c0 % 32) / 16) * 512 + c0 % 16;
+    if (sub == 0 && o8 == 0) a.ks[(bh * a.kb + t) * 4 + g] = sc;
 #pragma unroll
-    for (int i = 0; i < N; ++i) {
-        const int row = t * CK + (i / 2) * 8 + g * 2 + (i % 2);
-        if (row < a.lk) {
-            uint32_t w = 0;
-#pragma unroll
-            for (int c = 0; c < 4; ++c) w |= (uint32_t)(uint8_t)rn_s8(v[i][c] * inv) << (8 * c);
-            *reinterpret_cast<uint32_t*>(a.ki + (bh * a.nblk + row / 32) * 4096 + col + (row % 32) * 16) = w;
-        }
+    for (int j = 0; j < R; ++j) {
+        uint4 w = make_uint4(0u, 0u, 0u, 0u);
+        if (t * CK + rt[j] < a.lk) w = codes16(v[j], inv);
+        *reinterpret_cast<uint4*>(stage + (rt[j] / 32) * 4096 + (o8 >> 1) * 1024 + (o8 & 1) * 512 + (rt[j] % 32) * 16) = w;
     }
+    __syncthreads();
+    uint4* out = reinterpret_cast<uint4*>(a.ki + (bh * a.nblk + (int64_t)t * (CK / 32)) * 4096);
+#pragma unroll
+    for (int i = 0; i < CK * D / 16 / 256; ++i)
+        out[i * 256 + threadIdx.x] = *reinterpret_cast<const uint4*>(stage + (i * 256 + threadIdx.x) * 16);
 }
 
 // V abs-max per channel: 256 threads take 128 rows of one (kv head, batch), four channels per thread; non-negative
@@ -254,10 +310,10 @@ template <int DT>
 __global__ __launch_bounds__(256) void attn_v_absmax_kernel(AttnArgs a) {
     __shared__ float red[8][D];
     const int c4 = threadIdx.x & 31, rl = threadIdx.x >> 5;
-    const int hi = blockIdx.y, bi = blockIdx.z;
+    const int hi = blockIdx.x, bi = blockIdx.z;
     const int64_t base = bi * a.v_bs + hi * a.v_hs + c4 * 4;
     float mx[4] = {0.f, 0.f, 0.f, 0.f};
-    const int r0 = blockIdx.x * 128;
+    const int r0 = blockIdx.y * 128;
 #pragma unroll 4
     for (int i = 0; i < 16; ++i) {
         const int r = r0 + rl + 8 * i;
@@ -287,7 +343,7 @@ template <int DT>
 __global__ __launch_bounds__(256) void attn_v_quant_kernel(AttnArgs a) {
     __shared__ float inv_s[D];
     __shared__ __align__(16) int8_t tile[32][D];
-    const int s = blockIdx.x, hi = blockIdx.y, bi = blockIdx.z;
+    const int hi = blockIdx.x, s = blockIdx.y, bi = blockIdx.z;
     const int64_t bh = (int64_t)bi * a.hk + hi;
     if (threadIdx.x < D) {
         const float sc = fmax_nn(u2f(a.vmax[bh * D + threadIdx.x]) * (1.f / 127.f), 1e-12f);
@@ -534,11 +590,11 @@ Plan plan_for(int64_t b, int64_t h, int64_t hk, int64_t lq, int64_t lk) {
 template <int DT>
 int run(AttnArgs a, hipStream_t st) {
     attn_anchor_kernel<DT><<<dim3(a.hk, a.b), 128, 0, st>>>(a);
-    attn_quant_q_kernel<DT><<<dim3(a.qg, a.h, a.b), 256, 0, st>>>(a);
-    if (a.ck == 64) attn_quant_k_kernel<DT, 64><<<dim3(a.kb, a.hk, a.b), 128, 0, st>>>(a);
-    else attn_quant_k_kernel<DT, 128><<<dim3(a.kb, a.hk, a.b), 128, 0, st>>>(a);
-    attn_v_absmax_kernel<DT><<<dim3((a.lk + 127) / 128, a.hk, a.b), 256, 0, st>>>(a);
-    attn_v_quant_kernel<DT><<<dim3(a.nblk, a.hk, a.b), 256, 0, st>>>(a);
+    attn_quant_q_kernel<DT><<<dim3(a.h, (a.qg + 3) / 4, a.b), 256, 0, st>>>(a);
+    if (a.ck == 64) attn_quant_k_kernel<DT, 64><<<dim3(a.hk, a.kb, a.b), 256, 0, st>>>(a);
+    else attn_quant_k_kernel<DT, 128><<<dim3(a.hk, a.kb, a.b), 256, 0, st>>>(a);
+    attn_v_absmax_kernel<DT><<<dim3(a.hk, (a.lk + 127) / 128, a.b), 256, 0, st>>>(a);
+    attn_v_quant_kernel<DT><<<dim3(a.hk, a.nblk, a.b), 256, 0, st>>>(a);
     const dim3 grid((a.lq + 127) / 128, a.h, a.b);
     constexpr int kLds64 = 2 * (2 * 64 * D + 512), kLds128 = 2 * (2 * 128 * D + 512);
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_int8_kernel<DT, 128>),
@@ -556,7 +612,7 @@ int int8_attn(const void* q, const void* k, const void* v, void* o, void* ws, in
     if (Dh != D) why = "only head dim 128 is built";
     else if (!q || !k || !v || !o || !ws) why = "null pointer";
     else if (b <= 0 || lq <= 0 || lk <= 0 || h <= 0 || hk <= 0 || h % hk != 0) why = "bad sizes";
-    else if (b > 65535 || h > 65535) why = "batch or head count beyond the grid limit";
+    else if (b > 65535 || h > 65535 || lq > (1 << 20) || lk > (1 << 20)) why = "batch, head count or length beyond the grid limits";
     else if (((uintptr_t)ws & 255) != 0) why = "workspace must be 256-byte aligned";
     if (why) {
         fprintf(stderr, "int8 attention: %s\n", why);
