@@ -430,10 +430,12 @@ __global__ __launch_bounds__(256, 2) void attn_int8_kernel(AttnArgs a) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
-    for (int t = 0; t < a.kb; ++t) {
+    // One key tile.  The last tile (the only one that can hold keys past lk) is a separate instantiation, so that the
+    // validity compares exist only there.
+    auto tile = [&](const int t, auto last_tag) {
+        constexpr bool last = decltype(last_tag)::value;
         const uint8_t* st = smem + (t & 1) * STAGE;
         const int key0 = t * CK;
-        const bool last = t == a.kb - 1;
         v16i S[NB];
 #pragma unroll
         for (int blk = 0; blk < NB; ++blk) {
@@ -446,14 +448,14 @@ __global__ __launch_bounds__(256, 2) void attn_int8_kernel(AttnArgs a) {
             }
             S[blk] = acc;
         }
-        if (t + 1 < a.kb) fetch(t + 1);   // the other stage: every wave left it at the barrier that ended the last tile
+        if constexpr (!last) fetch(t + 1);   // the other stage: every wave left it at the barrier that ended the last tile
         const float* ksc = a.ks + (kvh * a.kb + t) * 4 + hh * 2;
         const float gs0 = a.sm * (q_scale * ksc[0]), gs1 = a.sm * (q_scale * ksc[1]);
 
         // Group maxima on the integers (exact in fp32: |score| < 2^24).  Only the last tile can hold keys past lk; its
         // maxima start at the reference's floor of -50000.
         int i0, i1;
-        if (!last) {
+        if constexpr (!last) {
             i0 = i1 = INT_MIN;
 #pragma unroll
             for (int blk = 0; blk < NB; ++blk)
@@ -510,8 +512,7 @@ __global__ __launch_bounds__(256, 2) void attn_int8_kernel(AttnArgs a) {
                 __builtin_amdgcn_sched_barrier(0);   // one block at a time: the converted scores die here
             }
         };
-        if (last) probabilities(std::true_type{});
-        else probabilities(std::false_type{});
+        probabilities(last_tag);
         dsum += (float)psum * t_scale;
 
 #pragma unroll
@@ -537,7 +538,9 @@ __global__ __launch_bounds__(256, 2) void attn_int8_kernel(AttnArgs a) {
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wave's share of the next tile has landed
         __syncthreads();
-    }
+    };
+    for (int t = 0; t + 1 < a.kb; ++t) tile(t, std::false_type{});
+    tile(a.kb - 1, std::true_type{});
 
     const float dtot = dsum + __shfl_xor(dsum, 32);
     const float rcp = 1.f / dtot;
