@@ -130,14 +130,14 @@ template <int DT> __device__ __forceinline__ void ld16_dt(const void* p, int64_t
     }
 }
 
-// One workgroup of 128 threads per (kv head, batch): thread = channel.  The shuffle trees of the reference are summed
-// by thread 0 in their order.
+// The K anchor of one (kv head, batch): thread = channel (the workgroup has 256 threads; the upper half repeats the
+// lower half's work and writes the same values).  The shuffle trees of the reference are summed in their order.
 template <int DT>
-__global__ __launch_bounds__(128) void attn_anchor_kernel(AttnArgs a) {
+__device__ __forceinline__ void anchor_body(const AttnArgs& a, const int hi, const int bi) {
     __shared__ float s[9][D];
     __shared__ float energy[D], best_energy[D], amax[D], bmax[D], dist[9][D];
     __shared__ int chosen;
-    const int c = threadIdx.x, hi = blockIdx.x, bi = blockIdx.y;
+    const int c = threadIdx.x & 127, tid = threadIdx.x;
     const int64_t base = bi * a.k_bs + hi * a.k_hs;
     {   // the V quantizer's accumulators for this (kv head, batch) start at zero
         const int64_t bh = (int64_t)bi * a.hk + hi;
@@ -170,10 +170,10 @@ __global__ __launch_bounds__(128) void attn_anchor_kernel(AttnArgs a) {
         return t[0];
     };
     __shared__ float warp_sum[11][4];   // nine candidate distances, then the two energies
-    if (c < 36) warp_sum[c / 4][c % 4] = tree(&dist[c / 4][(c % 4) * 32]);
-    else if (c < 40) warp_sum[9][c - 36] = tree(&energy[(c - 36) * 32]);
+    if (tid < 36) warp_sum[tid / 4][tid % 4] = tree(&dist[tid / 4][(tid % 4) * 32]);
+    else if (tid < 40) warp_sum[9][tid - 36] = tree(&energy[(tid - 36) * 32]);
     __syncthreads();
-    if (c == 0) {
+    if (tid == 0) {
         int best = 0;
         float best_d = 3.402823466e+38F;
         for (int i = 0; i < 9; ++i) {
@@ -195,9 +195,9 @@ __global__ __launch_bounds__(128) void attn_anchor_kernel(AttnArgs a) {
     best_energy[c] = be;
     bmax[c] = bm;
     __syncthreads();
-    if (c < 4) warp_sum[10][c] = tree(&best_energy[c * 32]);
+    if (tid < 4) warp_sum[10][tid] = tree(&best_energy[tid * 32]);
     __syncthreads();
-    if (c == 0) {
+    if (tid == 0) {
         float e0 = 0.f, e1 = 0.f, m0 = 0.f, m1 = 0.f;
         for (int w = 0; w < 4; ++w) {
             e0 += warp_sum[9][w];
@@ -214,10 +214,9 @@ __global__ __launch_bounds__(128) void attn_anchor_kernel(AttnArgs a) {
 // Q: a wave per 32 rows, four waves per workgroup; each run of eight lanes is one scale group (rows g, g+8, g+16, g+24),
 // a lane holding 16 channels of each of the four rows.
 template <int DT>
-__global__ __launch_bounds__(256) void attn_quant_q_kernel(AttnArgs a) {
+__device__ __forceinline__ void quant_q_body(const AttnArgs& a, const int hi, const int ty, const int bi) {
     const int lane = threadIdx.x & 63, o8 = lane & 7, g = lane >> 3;
-    const int hi = blockIdx.x, bi = blockIdx.z;   // heads fastest: neighbours read neighbouring memory
-    const int t = blockIdx.y * 4 + (threadIdx.x >> 6);
+    const int t = ty * 4 + (threadIdx.x >> 6);
     if (t >= a.qg) return;
     const int64_t bh = (int64_t)bi * a.h + hi, base = bi * a.q_bs + hi * a.q_hs + o8 * 16;
     float v[4][16];
@@ -251,12 +250,11 @@ __global__ __launch_bounds__(256) void attn_quant_q_kernel(AttnArgs a) {
 // read one contiguous KB per load), and leaves as 16-byte stores over its contiguous CK * 128 bytes; keys past lk are
 // zeros.
 template <int DT, int CK>
-__global__ __launch_bounds__(256) void attn_quant_k_kernel(AttnArgs a) {
+__device__ __forceinline__ void quant_k_body(const AttnArgs& a, const int hi, const int t, const int bi) {
     constexpr int R = CK / 32;   // rows per run of eight lanes
     __shared__ float omax[32];
     __shared__ __align__(16) uint8_t stage[CK * D];
     const int o8 = threadIdx.x & 7, oct = threadIdx.x >> 3, g = oct & 3, sub = oct >> 2;
-    const int hi = blockIdx.x, t = blockIdx.y, bi = blockIdx.z;   // heads fastest: neighbours read neighbouring memory
     const int64_t bh = (int64_t)bi * a.hk + hi, base = bi * a.k_bs + hi * a.k_hs + o8 * 16;
     const int anchor = a.anchors[bh];
     float bias[16];
@@ -307,13 +305,12 @@ __global__ __launch_bounds__(256) void attn_quant_k_kernel(AttnArgs a) {
 // V abs-max per channel: 256 threads take 128 rows of one (kv head, batch), four channels per thread; non-negative
 // floats order as their bits, so the workgroups combine with an integer atomic max.
 template <int DT>
-__global__ __launch_bounds__(256) void attn_v_absmax_kernel(AttnArgs a) {
+__device__ __forceinline__ void v_absmax_body(const AttnArgs& a, const int hi, const int chunk, const int bi) {
     __shared__ float red[8][D];
     const int c4 = threadIdx.x & 31, rl = threadIdx.x >> 5;
-    const int hi = blockIdx.x, bi = blockIdx.z;
     const int64_t base = bi * a.v_bs + hi * a.v_hs + c4 * 4;
     float mx[4] = {0.f, 0.f, 0.f, 0.f};
-    const int r0 = blockIdx.y * 128;
+    const int r0 = chunk * 128;
 #pragma unroll 4
     for (int i = 0; i < 16; ++i) {
         const int r = r0 + rl + 8 * i;
@@ -333,6 +330,35 @@ __global__ __launch_bounds__(256) void attn_v_absmax_kernel(AttnArgs a) {
         for (int i = 0; i < 8; ++i) m = fmax_nn(m, red[i][threadIdx.x]);
         atomicMax(&a.vmax[((int64_t)bi * a.hk + hi) * D + threadIdx.x], f2u(m));
     }
+}
+
+// Two launches carry the four bodies above: work that does not depend on each other shares a launch, heads fastest so
+// that neighbouring workgroups read neighbouring memory.  Stage 1: anchors (which also clear the V accumulators) and Q.
+// Stage 2: K (needs the anchors) and the V abs-max (needs the cleared accumulators).
+template <int DT>
+__global__ __launch_bounds__(256) void attn_stage1_kernel(AttnArgs a) {
+    int id = blockIdx.x;
+    const int n_anchor = a.hk * a.b;
+    if (id < n_anchor) {
+        anchor_body<DT>(a, id % a.hk, id / a.hk);
+        return;
+    }
+    id -= n_anchor;
+    const int ny = (a.qg + 3) / 4;
+    quant_q_body<DT>(a, id % a.h, (id / a.h) % ny, id / (a.h * ny));
+}
+
+template <int DT, int CK>
+__global__ __launch_bounds__(256) void attn_stage2_kernel(AttnArgs a) {
+    int id = blockIdx.x;
+    const int n_k = a.hk * a.kb * a.b;
+    if (id < n_k) {
+        quant_k_body<DT, CK>(a, id % a.hk, (id / a.hk) % a.kb, id / (a.hk * a.kb));
+        return;
+    }
+    id -= n_k;
+    const int nc = (a.lk + 127) / 128;
+    v_absmax_body<DT>(a, id % a.hk, (id / a.hk) % nc, id / (a.hk * nc));
 }
 
 // V codes: one workgroup per block of 32 keys.  Rows are read as they lie (a thread takes 16 channels of one key),
@@ -592,11 +618,12 @@ Plan plan_for(int64_t b, int64_t h, int64_t hk, int64_t lq, int64_t lk) {
 
 template <int DT>
 int run(AttnArgs a, hipStream_t st) {
-    attn_anchor_kernel<DT><<<dim3(a.hk, a.b), 128, 0, st>>>(a);
-    attn_quant_q_kernel<DT><<<dim3(a.h, (a.qg + 3) / 4, a.b), 256, 0, st>>>(a);
-    if (a.ck == 64) attn_quant_k_kernel<DT, 64><<<dim3(a.hk, a.kb, a.b), 256, 0, st>>>(a);
-    else attn_quant_k_kernel<DT, 128><<<dim3(a.hk, a.kb, a.b), 256, 0, st>>>(a);
-    attn_v_absmax_kernel<DT><<<dim3(a.hk, (a.lk + 127) / 128, a.b), 256, 0, st>>>(a);
+    const int64_t n1 = (int64_t)a.hk * a.b + (int64_t)a.h * ((a.qg + 3) / 4) * a.b;
+    const int64_t n2 = (int64_t)a.hk * a.kb * a.b + (int64_t)a.hk * ((a.lk + 127) / 128) * a.b;
+    if (n1 > 0x7fffffff || n2 > 0x7fffffff) return -400;
+    attn_stage1_kernel<DT><<<dim3((unsigned)n1), 256, 0, st>>>(a);
+    if (a.ck == 64) attn_stage2_kernel<DT, 64><<<dim3((unsigned)n2), 256, 0, st>>>(a);
+    else attn_stage2_kernel<DT, 128><<<dim3((unsigned)n2), 256, 0, st>>>(a);
     attn_v_quant_kernel<DT><<<dim3(a.hk, a.nblk, a.b), 256, 0, st>>>(a);
     const dim3 grid((a.lq + 127) / 128, a.h, a.b);
     constexpr int kLds64 = 2 * (2 * 64 * D + 512), kLds128 = 2 * (2 * 128 * D + 512);
