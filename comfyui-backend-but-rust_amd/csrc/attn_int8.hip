@@ -37,7 +37,8 @@ struct AttnArgs {
     int vec_ok, in_vec, v_vec;
 };
 
-__device__ __forceinline__ float fmax_nn(float a, float b) { return a > b ? a : b; }
+// fmaxf as the reference's device code uses it: a NaN operand is dropped.
+__device__ __forceinline__ float fmax_nn(float a, float b) { return __builtin_fmaxf(a, b); }
 
 __device__ __forceinline__ int8_t rn_s8(float v) {
     if (v != v) return 0;
