@@ -33,8 +33,8 @@ struct AttnArgs {
     int* vsum;
     int b, lq, lk, h, hk, rep, qg, kb, ck, nblk;
     int64_t q_bs, q_rs, q_hs, k_bs, k_rs, k_hs, v_bs, v_rs, v_hs, o_bs, o_rs, o_hs;
-    float sm;
-    int vec_ok, in_vec, v_vec;
+    float sm, sink;
+    int vec_ok, in_vec, v_vec, use_anchor;
 };
 
 // fmaxf as the reference's device code uses it: a NaN operand is dropped.
@@ -208,7 +208,7 @@ __device__ __forceinline__ void anchor_body(const AttnArgs& a, const int hi, con
             m0 = fmax_nn(m0, amax[i]);
             m1 = fmax_nn(m1, bmax[i]);
         }
-        a.anchors[bi * a.hk + hi] = (e1 < e0 && m1 <= m0 * 1.125f) ? (int)((int64_t)best * (a.lk - 1) / 8) : -1;
+        a.anchors[bi * a.hk + hi] = (a.use_anchor && e1 < e0 && m1 <= m0 * 1.125f) ? (int)((int64_t)best * (a.lk - 1) / 8) : -1;
     }
 }
 
@@ -569,7 +569,9 @@ __global__ __launch_bounds__(256, 2) void attn_int8_kernel(AttnArgs a) {
     for (int t = 0; t + 1 < a.kb; ++t) tile(t, std::false_type{});
     tile(a.kb - 1, std::true_type{});
 
-    const float dtot = dsum + __shfl_xor(dsum, 32);
+    float dtot = dsum + __shfl_xor(dsum, 32);
+    // `sink` more keys of score zero and value zero: each adds exp2(0 - m) to the denominator, nothing to the output
+    if (a.sink != 0.f) dtot = fmaf(a.sink, __builtin_amdgcn_exp2f(-m), dtot);
     const float rcp = 1.f / dtot;
     if (r < a.lq) {
         const int64_t ob = bi * a.o_bs + (int64_t)r * a.o_rs + hi * a.o_hs;
@@ -638,7 +640,7 @@ int run(AttnArgs a, hipStream_t st) {
 
 int int8_attn(const void* q, const void* k, const void* v, void* o, void* ws, int b, int lq, int lk, int h, int hk, int Dh,
               int64_t q_bs, int64_t q_rs, int64_t q_hs, int64_t k_bs, int64_t k_rs, int64_t k_hs, int64_t v_bs, int64_t v_rs,
-              int64_t v_hs, int64_t o_bs, int64_t o_rs, int64_t o_hs, float scale, int dt, void* stream) {
+              int64_t v_hs, int64_t o_bs, int64_t o_rs, int64_t o_hs, float scale, int dt, void* stream, float sink = 0.f) {
     const char* why = nullptr;
     if (Dh != D) why = "only head dim 128 is built";
     else if (!q || !k || !v || !o || !ws) why = "null pointer";
@@ -661,6 +663,8 @@ int int8_attn(const void* q, const void* k, const void* v, void* o, void* ws, in
     a.q_bs = q_bs; a.q_rs = q_rs; a.q_hs = q_hs; a.k_bs = k_bs; a.k_rs = k_rs; a.k_hs = k_hs;
     a.v_bs = v_bs; a.v_rs = v_rs; a.v_hs = v_hs; a.o_bs = o_bs; a.o_rs = o_rs; a.o_hs = o_hs;
     a.sm = scale * 1.44269504088896340736f;
+    a.sink = sink;
+    a.use_anchor = sink == 0.f ? 1 : 0;   // with a sink a zero key's score must stay zero: no shift (csrc/attn_int8.cu:134-141)
     a.vec_ok = ((o_bs | o_rs | o_hs) % 4 == 0 && ((uintptr_t)o & 7) == 0) ? 1 : 0;
     a.v_vec = ((v_bs | v_rs | v_hs) % 4 == 0 && ((uintptr_t)v & 7) == 0) ? 1 : 0;
     a.in_vec = ((q_bs | q_rs | q_hs | k_bs | k_rs | k_hs) % 4 == 0 && (((uintptr_t)q | (uintptr_t)k) & 7) == 0) ? 1 : 0;
@@ -701,6 +705,19 @@ GPU_API int gpu_int8_attn(const void* q, const void* k, const void* v, void* o, 
                           void* stream) {
     return int8_attn(q, k, v, o, ws, b, lq, lk, h, hk, D, q_bs, q_rs, q_hs, k_bs, k_rs, k_hs, v_bs, v_rs, v_hs, o_bs, o_rs,
                      o_hs, scale, DT_BF16, stream);
+}
+
+GPU_API int gpu_int8_attn_sink(const void* q, const void* k, const void* v, void* o, void* ws, int b, int lq, int lk, int h,
+                               int hk, int64_t q_bs, int64_t q_rs, int64_t q_hs, int64_t k_bs, int64_t k_rs, int64_t k_hs,
+                               int64_t v_bs, int64_t v_rs, int64_t v_hs, int64_t o_bs, int64_t o_rs, int64_t o_hs, float scale,
+                               float sink, const float* qw, float eps, void* stream) {
+    (void)eps;
+    if (qw) {
+        fprintf(stderr, "int8 attention: the fused q norm of the sink form is not built\n");
+        return -400;
+    }
+    return int8_attn(q, k, v, o, ws, b, lq, lk, h, hk, D, q_bs, q_rs, q_hs, k_bs, k_rs, k_hs, v_bs, v_rs, v_hs, o_bs, o_rs,
+                     o_hs, scale, DT_BF16, stream, sink);
 }
 
 // Test hook: where the pieces of the workspace lie (byte offsets), and the tiling.  out[0..9] = qi, ki, qs, ks, vt, vs,

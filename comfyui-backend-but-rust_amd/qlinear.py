@@ -228,6 +228,20 @@ def linear_w8a8(x, W, ws, bias=None, rotate=0, out_dtype=None):
     return int8_gemm(q, W, xs, ws, bias, x.dtype if out_dtype is None else out_dtype)
 
 
+def int8_attn_sink(q, k, v, scale, sink, ws=None):
+    """int8_attn over the keys given plus `sink` zero keys with zero values (bf16), csrc/attn_int8.cu:193-202."""
+    b, lq, h, D = q.shape
+    lk, hk = k.shape[1], k.shape[2]
+    assert q.dtype == torch.bfloat16 and D == 128
+    if ws is None:
+        ws = torch.empty((ffi.lib.gpu_int8_attn_workspace(b, h, hk, lq, lk),), dtype=torch.uint8, device=q.device)
+    o = torch.empty((b, lq, h, D), dtype=q.dtype, device=q.device)
+    ffi.k("gpu_int8_attn_sink", _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(ws), b, lq, lk, h, hk, q.stride(0), q.stride(1),
+          q.stride(2), k.stride(0), k.stride(1), k.stride(2), v.stride(0), v.stride(1), v.stride(2), o.stride(0), o.stride(1),
+          o.stride(2), float(scale), float(sink), None, 0.0, _stream())
+    return o
+
+
 def int8_attn(q, k, v, scale, ws=None):
     """INT8 attention over q [b, lq, h, 128], k/v [b, lk, hk, 128] (bf16 or f16, any strides with a contiguous last
     axis): the reference's attention_int8 call pattern (csrc/attn_int8.cu:101-118).  Returns o [b, lq, h, 128]."""

@@ -123,8 +123,11 @@ int gpu_w6_requant(const void* weight, void* packed, void* s_rel, void* s_channe
  * Replaces gpu_int8_attn_workspace_d / gpu_int8_attn_workspace (csrc/attn_int8.cu:62-82), gpu_int8_attn_d (:101-108),
  * gpu_int8_attn_f16 (:111-118), gpu_int8_attn (:225-231); src/ffi.rs binds them under the same names.
  * Returns 0, -400 (argument the library refuses: message on stderr; head dims other than 128 are not built) or -401
- * (launch failure), the reference's codes.  Not built: gpu_int8_attn_norm_rope, gpu_int8_attn_sink,
- * gpu_int8_attn_key_bias (csrc/attn_int8.cu:166-223). */
+ * (launch failure), the reference's codes.
+ * gpu_int8_attn_sink (csrc/attn_int8.cu:193-202): attention over lk keys plus `sink` more whose keys and values are
+ * zero, which count in the softmax denominator only; the K anchor is off so that a zero key's score stays zero; bf16.
+ * A non-null qw (q normalized first) is not built: -400.
+ * Not built: gpu_int8_attn_norm_rope, gpu_int8_attn_key_bias (csrc/attn_int8.cu:166-191,204-223). */
 int64_t gpu_int8_attn_workspace_d(int b, int h, int hk, int lq, int lk, int head_dim);
 int64_t gpu_int8_attn_workspace(int b, int h, int hk, int lq, int lk);
 int gpu_int8_attn_d(const void* q, const void* k, const void* v, void* o, void* ws, int b, int lq, int lk, int h, int hk,
@@ -138,6 +141,11 @@ int gpu_int8_attn_f16(const void* q, const void* k, const void* v, void* o, void
 int gpu_int8_attn(const void* q, const void* k, const void* v, void* o, void* ws, int b, int lq, int lk, int h, int hk,
                   int64_t q_bs, int64_t q_rs, int64_t q_hs, int64_t k_bs, int64_t k_rs, int64_t k_hs, int64_t v_bs,
                   int64_t v_rs, int64_t v_hs, int64_t o_bs, int64_t o_rs, int64_t o_hs, float scale, void* stream);
+
+int gpu_int8_attn_sink(const void* q, const void* k, const void* v, void* o, void* ws, int b, int lq, int lk, int h, int hk,
+                       int64_t q_bs, int64_t q_rs, int64_t q_hs, int64_t k_bs, int64_t k_rs, int64_t k_hs, int64_t v_bs,
+                       int64_t v_rs, int64_t v_hs, int64_t o_bs, int64_t o_rs, int64_t o_hs, float scale, float sink,
+                       const float* qw, float eps, void* stream);
 
 /* Test hook, no reference counterpart: byte offsets of the pieces of the attention workspace and its tiling,
  * out[0..9] = qi, ki, qs, ks, vt, vs, anchors, vsum, key tile length, key tiles. */

@@ -63,7 +63,7 @@ def lib():
         L.orc_attn_quant_qk.argtypes = [i32, vp, vp, i32, i32, i32, i32, i32, i64, i64, i64, i64, i64, i64, i32, i32, vp, vp, vp, vp, vp]
         L.orc_attn_quant_v.restype = i32; L.orc_attn_quant_v.argtypes = [i32, vp, i32, i32, i32, i64, i64, i64, vp, vp]
         L.orc_attn_int8.restype = i32
-        L.orc_attn_int8.argtypes = [i32, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, vp, i64, i64, i64]
+        L.orc_attn_int8.argtypes = [i32, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, f32, vp, i64, i64, i64]
         L.orc_attn_cta_k.restype = i32; L.orc_attn_cta_k.argtypes = [i32, i32]
         _lib = L
     return _lib
@@ -365,13 +365,14 @@ def attn_quant(dt, q, k, v, use_anchor=True):
     return out
 
 
-def attn_int8(dt, q, k, v, scale, use_anchor=True, quant=None):
-    """The whole int8 attention: o [b,lq,h,128] in dtype dt (uint16 bits for bf16/f16)."""
+def attn_int8(dt, q, k, v, scale, use_anchor=True, quant=None, sink=0.0):
+    """The whole int8 attention: o [b,lq,h,128] in dtype dt (uint16 bits for bf16/f16).  sink: that many more keys of
+    score zero and value zero in the denominator (callers pass use_anchor=False with it, as the reference does)."""
     b, lq, h, D = q.shape
     lk, hk = k.shape[1], k.shape[2]
     z = quant if quant is not None else attn_quant(dt, q, k, v, use_anchor)
     o = np.zeros((b, lq, h, D), np.float32 if dt == F32 else np.uint16)
     rc = lib().orc_attn_int8(dt, _p(z["qi"]), _p(z["ki"]), _p(z["vi"]), _p(z["qs"]), _p(z["ks"]), _p(z["vs"]), b, lq, lk,
-                             h, hk, z["ck"], float(scale), _p(o), lq * h * D, h * D, D)
+                             h, hk, z["ck"], float(scale), float(sink), _p(o), lq * h * D, h * D, D)
     assert rc == 0
     return o

@@ -950,7 +950,7 @@ static inline float attn_exp2(float x) { return (float)exp2((double)x); }
  * per row in key order; the reference keeps four per-thread partials. */
 ORC_API int orc_attn_int8(int out_dt, const int8_t* qi, const int8_t* ki, const int8_t* vi, const float* qs,
                           const float* ks, const float* vs, int b, int lq, int lk, int h, int hk, int ck, float scale,
-                          void* o, int64_t o_bs, int64_t o_rs, int64_t o_hs) {
+                          float sink, void* o, int64_t o_bs, int64_t o_rs, int64_t o_hs) {
     if ((ck != 64 && ck != 128) || hk <= 0 || h % hk != 0) return -1;
     const int qg = (lq + 127) / 128 * 4, kb = (lk + ck - 1) / ck, rep = h / hk;
     const float sm = scale * 1.44269504088896340736f;
@@ -1002,6 +1002,9 @@ ORC_API int orc_attn_int8(int out_dt, const int8_t* qi, const int8_t* ki, const 
                 d += (float)psum * t_scale;
                 for (int c = 0; c < ATTN_D; ++c) ro[c] = fmaf((float)pv[c], t_scale, ro[c] * o_scale);
             }
+            /* `sink` more keys of score zero and value zero: each adds exp2(0 - m) to the denominator and nothing to
+             * the output (attn_utils.cuh:1122-1130, csrc/attn_int8.cu:193-197) */
+            if (sink != 0.f) d = fmaf(sink, attn_exp2(-m), d);
             const float rcp = 1.f / d;
             for (int c = 0; c < ATTN_D; ++c)
                 st_t(out_dt, o, bi * o_bs + (int64_t)r * o_rs + hi * o_hs + c, ro[c] * rcp * vs[kvh * ATTN_D + c]);

@@ -143,6 +143,39 @@ def test_attention_strided_views_match_contiguous():
     assert torch.equal(a, c)
 
 
+@pytest.mark.parametrize("shape", [(1, 70, 200, 2, 2, 56.0), (1, 40, 1100, 2, 1, 180.0)])
+def test_attention_with_sink_keys(shape):
+    """gpu_int8_attn_sink: against the oracle (anchor off, denominator + sink * exp2(-m)) and against exact attention over
+    the keys plus that many zero keys with zero values."""
+    ql, ffi = _pkg()
+    b, lq, lk, h, hk, sink = shape
+    q, k, v = _inputs(b, lq, lk, h, hk, torch.bfloat16, seed=17, k_offset=3.0)
+    scale = 128 ** -0.5
+    ref = _to_f32(oracle.attn_int8(oracle.BF16, _bits(q), _bits(k), _bits(v), scale, use_anchor=False, sink=sink), oracle.BF16)
+    ws = torch.zeros((ffi.lib.gpu_int8_attn_workspace(b, h, hk, lq, lk),), dtype=torch.uint8, device="cuda")
+    o = ql.int8_attn_sink(q.cuda(), k.cuda(), v.cuda(), scale, sink, ws=ws)
+    torch.cuda.synchronize()
+    an_o = _layout(ffi, b, h, hk, lq, lk)[6]
+    assert (ws.cpu().numpy()[an_o:an_o + 4 * b * hk].view(np.int32) == -1).all(), "the anchor must be off with a sink"
+    got = _to_f32(_bits(o), oracle.BF16)
+    vmax = float(v.float().abs().max())
+    tol = 2 * vmax / 255.0 + 2 * 2.0 ** -8 * np.abs(ref)
+    assert (np.abs(got - ref) <= tol).all()
+    n = int(sink)
+    kz = torch.cat([k, torch.zeros(b, n, hk, 128, dtype=k.dtype)], 1)
+    vz = torch.cat([v, torch.zeros(b, n, hk, 128, dtype=v.dtype)], 1)
+    ex = _exact(q, kz, vz, scale)
+    cos = float((got * ex).sum() / np.sqrt((got * got).sum() * (ex * ex).sum()))
+    assert cos > 0.9995, cos
+    assert np.abs(got - ex).max() < 0.03
+    # the fused q norm of this form is not built
+    p = lambda t: C.c_void_p(t.data_ptr())
+    x = torch.zeros(1, 4, 1, 128, dtype=torch.bfloat16, device="cuda")
+    qw = torch.ones(128, device="cuda")
+    assert ffi.raw("gpu_int8_attn_sink", p(x), p(x), p(x), p(x), p(ws), 1, 4, 4, 1, 1, 512, 128, 128, 512, 128, 128, 512, 128,
+                   128, 512, 128, 128, 0.1, 4.0, p(qw), 1e-6, None) == -400
+
+
 def test_attention_refuses_what_it_does_not_build():
     ql, ffi = _pkg()
     x = torch.zeros(1, 4, 1, 128, dtype=torch.bfloat16, device="cuda")

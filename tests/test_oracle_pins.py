@@ -965,3 +965,21 @@ def test_attn_oracle_is_attention(shape):
     o1 = oracle.bf16_to_f32(oracle.attn_int8(oracle.BF16, bits(q), bits(k[:, :1]), bits(v[:, :1]), scale))
     want = v[:, :1].float().numpy().repeat(h // hk, 2)
     assert np.abs(o1 - want).max() <= np.abs(want).max() / 127.0 * 0.51 + 2 ** -8 * np.abs(want).max()
+
+
+def test_attn_oracle_sink_equals_zero_keys_appended():
+    """`sink` zero keys with zero values, counted in the denominator only: exact attention over the padded tensors."""
+    q, k, v, bits = _attn_case(1, 24, 140, 2, 1, seed=9, k_offset=2.0)
+    scale = 128 ** -0.5
+    got = oracle.bf16_to_f32(oracle.attn_int8(oracle.BF16, bits(q), bits(k), bits(v), scale, use_anchor=False, sink=40.0))
+    kz = torch.cat([k, torch.zeros(1, 40, 1, 128, dtype=k.dtype)], 1)
+    vz = torch.cat([v, torch.zeros(1, 40, 1, 128, dtype=v.dtype)], 1)
+    qq = q.double().permute(0, 2, 1, 3)
+    kk = kz.double().permute(0, 2, 1, 3).repeat_interleave(2, 1)
+    vv = vz.double().permute(0, 2, 1, 3).repeat_interleave(2, 1)
+    ex = (torch.softmax(qq @ kk.transpose(-1, -2) * scale, -1) @ vv).permute(0, 2, 1, 3).numpy()
+    assert np.abs(got - ex).max() < 0.03
+    assert float((got * ex).sum() / np.sqrt((got * got).sum() * (ex * ex).sum())) > 0.9995
+    # and it is not the plain attention: the sink takes a visible share of the weight
+    plain = oracle.bf16_to_f32(oracle.attn_int8(oracle.BF16, bits(q), bits(k), bits(v), scale, use_anchor=False))
+    assert np.abs(plain - got).max() > 0.01
