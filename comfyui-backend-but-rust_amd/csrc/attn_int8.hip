@@ -630,9 +630,16 @@ int run(AttnArgs a, hipStream_t st) {
     attn_v_quant_kernel<DT><<<dim3(a.hk, a.nblk, a.b), 256, 0, st>>>(a);
     const dim3 grid((a.lq + 127) / 128, a.h, a.b);
     constexpr int kLds64 = 2 * (2 * 64 * D + 512), kLds128 = 2 * (2 * 128 * D + 512);
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_int8_kernel<DT, 128>),
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLds128);
-    if (attr != hipSuccess) return -401;
+    // more than 64 KB of dynamic LDS has to be allowed once per device; a repeated set is harmless if two threads race
+    static bool allowed[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return -401;
+    if (!allowed[dev]) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_int8_kernel<DT, 128>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kLds128) != hipSuccess)
+            return -401;
+        allowed[dev] = true;
+    }
     if (a.ck == 64) attn_int8_kernel<DT, 64><<<grid, 256, kLds64, st>>>(a);
     else attn_int8_kernel<DT, 128><<<grid, 256, kLds128, st>>>(a);
     return hipGetLastError() == hipSuccess ? 0 : -401;
