@@ -176,6 +176,34 @@ def test_attention_with_sink_keys(shape):
                    128, 512, 128, 128, 0.1, 4.0, p(qw), 1e-6, None) == -400
 
 
+def test_attention_unaligned_views_take_the_scalar_paths():
+    """Rows that start on odd element offsets with strides that are not multiples of four: the 8-byte vector accesses
+    are off for inputs and output, and the result is the same bits as for contiguous tensors."""
+    ql, ffi = _pkg()
+    b, lq, lk, h, hk = 1, 45, 130, 2, 1
+    q, k, v = (t.cuda() for t in _inputs(b, lq, lk, h, hk, torch.float16, seed=23))
+    scale = 0.09
+    want = ql.int8_attn(q, k, v, scale)
+
+    def odd_view(t):
+        bb, l, hh, d = t.shape
+        row = hh * d + 2
+        base = torch.zeros(bb * l * row + 1, dtype=t.dtype, device=t.device)
+        view = base.as_strided((bb, l, hh, d), (l * row, row, d, 1), 1)
+        view.copy_(t)
+        return view
+
+    qo, ko, vo = odd_view(q), odd_view(k), odd_view(v)
+    oo = odd_view(torch.zeros_like(q))
+    ws = torch.zeros((ffi.lib.gpu_int8_attn_workspace_d(b, h, hk, lq, lk, 128),), dtype=torch.uint8, device="cuda")
+    P = lambda t: C.c_void_p(t.data_ptr())
+    assert qo.data_ptr() % 4 == 2 and qo.stride(1) % 4 == 2
+    ffi.k("gpu_int8_attn_f16", P(qo), P(ko), P(vo), P(oo), P(ws), b, lq, lk, h, hk, 128, *qo.stride()[:3], *ko.stride()[:3],
+          *vo.stride()[:3], *oo.stride()[:3], scale, None)
+    torch.cuda.synchronize()
+    assert torch.equal(oo, want)
+
+
 def test_attention_refuses_what_it_does_not_build():
     ql, ffi = _pkg()
     x = torch.zeros(1, 4, 1, 128, dtype=torch.bfloat16, device="cuda")
