@@ -510,8 +510,8 @@ __global__ __launch_bounds__(256, 2) void attn_int8_kernel(AttnArgs a) {
         m = fmax_nn(m, tile_m);
         dsum *= o_scale;
 
-        // Probabilities: exp2 of at most the u8 offset is below 255.5, so adding 2^23 leaves round-to-nearest-even(p) in
-        // the low byte of the float's bits.  p - 128 as a signed byte is p ^ 0x80.
+        // Probabilities: v_cvt_pk_u8_f32 rounds to nearest even, saturates to 0..255 and writes one byte of a dword, which
+        // is the reference's cvt.rni.sat.u8 plus the packing.  p - 128 as a signed byte is p ^ 0x80.
         v4i pf[NB];
         uint32_t psum = 0;
         auto probabilities = [&](auto masked) {
@@ -520,18 +520,16 @@ __global__ __launch_bounds__(256, 2) void attn_int8_kernel(AttnArgs a) {
                 uint32_t w[4];
 #pragma unroll
                 for (int g4 = 0; g4 < 4; ++g4) {
-                    uint32_t u[4];
+                    uint32_t packed = 0u;
 #pragma unroll
                     for (int c = 0; c < 4; ++c) {
-                        const float e = __builtin_amdgcn_exp2f(fmaf((float)S[blk][g4 * 4 + c], c < 2 ? gs0 : gs1, -tile_m));
-                        u[c] = f2u(e + 8388608.f);
+                        float e = __builtin_amdgcn_exp2f(fmaf((float)S[blk][g4 * 4 + c], c < 2 ? gs0 : gs1, -tile_m));
                         if constexpr (decltype(masked)::value) {
                             const int key = key0 + blk * 32 + g4 * 8 + hh * 4 + c;
-                            u[c] = key < a.lk ? u[c] : 0u;
+                            e = key < a.lk ? e : 0.f;
                         }
+                        packed = __builtin_amdgcn_cvt_pk_u8_f32(e, c, packed);
                     }
-                    const uint32_t packed =
-                        __builtin_amdgcn_perm(u[1], u[0], 0x0c0c0400u) | __builtin_amdgcn_perm(u[3], u[2], 0x04000c0cu);
                     psum = __builtin_amdgcn_sad_u8(packed, 0u, psum);
                     w[g4] = packed ^ 0x80808080u;
                 }
@@ -725,6 +723,20 @@ GPU_API int gpu_int8_attn_sink(const void* q, const void* k, const void* v, void
     }
     return int8_attn(q, k, v, o, ws, b, lq, lk, h, hk, D, q_bs, q_rs, q_hs, k_bs, k_rs, k_hs, v_bs, v_rs, v_hs, o_bs, o_rs,
                      o_hs, scale, DT_BF16, stream, sink);
+}
+
+// Test hook: y[i] = v_cvt_pk_u8_f32(x[i]) into byte 0 of zero, so that a test can hold the instruction to
+// round-to-nearest-even with saturation, which the probabilities rely on.
+namespace {
+__global__ void cvt_pk_u8_probe_kernel(const float* x, uint32_t* y, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) y[i] = __builtin_amdgcn_cvt_pk_u8_f32(x[i], 0, 0u);
+}
+}  // namespace
+GPU_API int gpu_internal_cvt_pk_u8_probe(const float* x, uint32_t* y, int n, void* stream) {
+    if (!x || !y || n <= 0) return -400;
+    cvt_pk_u8_probe_kernel<<<dim3((n + 255) / 256), 256, 0, (hipStream_t)stream>>>(x, y, n);
+    return hipGetLastError() == hipSuccess ? 0 : -401;
 }
 
 // Test hook: where the pieces of the workspace lie (byte offsets), and the tiling.  out[0..9] = qi, ki, qs, ks, vt, vs,

@@ -147,6 +147,10 @@ int gpu_int8_attn_sink(const void* q, const void* k, const void* v, void* o, voi
                        int64_t v_rs, int64_t v_hs, int64_t o_bs, int64_t o_rs, int64_t o_hs, float scale, float sink,
                        const float* qw, float eps, void* stream);
 
+/* Test hook, no reference counterpart: y[i] = the gfx950 float -> u8 pack conversion of x[i] (byte 0), which the attention
+ * kernel's probabilities rely on being round-to-nearest-even with saturation to 0..255. */
+int gpu_internal_cvt_pk_u8_probe(const float* x, uint32_t* y, int n, void* stream);
+
 /* Test hook, no reference counterpart: byte offsets of the pieces of the attention workspace and its tiling,
  * out[0..9] = qi, ki, qs, ks, vt, vs, anchors, vsum, key tile length, key tiles. */
 int gpu_internal_attn_layout(int b, int h, int hk, int lq, int lk, int64_t* out);

@@ -204,6 +204,22 @@ def test_attention_unaligned_views_take_the_scalar_paths():
     assert torch.equal(oo, want)
 
 
+def test_u8_pack_conversion_rounds_to_nearest_even_and_saturates():
+    """The probabilities are rounded by the hardware's float -> u8 pack conversion; the reference rounds with
+    cvt.rni.sat.u8 and the oracle with clamp + rint.  Every integer 0..255 with fractions either side of one half, the
+    exact halves, and values outside the range."""
+    ql, ffi = _pkg()
+    fr = np.array([0.0, 0.25, 0.4999, 0.5, 0.5001, 0.75, 0.999, np.float32(0.49999997)], np.float32)
+    x = (np.arange(256, dtype=np.float32)[:, None] + fr[None, :]).reshape(-1)
+    x = np.concatenate([x, np.array([255.4, 255.5, 255.6, 256.0, 300.0, 1e9, -0.4, -0.5, -1.0, -1e9, np.nan], np.float32)])
+    xd = torch.from_numpy(x).cuda()
+    yd = torch.zeros(x.size, dtype=torch.int32, device="cuda")
+    ffi.k("gpu_internal_cvt_pk_u8_probe", C.c_void_p(xd.data_ptr()), C.c_void_p(yd.data_ptr()), x.size, None)
+    torch.cuda.synchronize()
+    want = np.rint(np.clip(np.nan_to_num(x, nan=0.0), 0.0, 255.0)).astype(np.int32)
+    assert np.array_equal(yd.cpu().numpy(), want)
+
+
 def test_attention_refuses_what_it_does_not_build():
     ql, ffi = _pkg()
     x = torch.zeros(1, 4, 1, 128, dtype=torch.bfloat16, device="cuda")
