@@ -463,18 +463,18 @@ __global__ __launch_bounds__(256, 2) void attn_int8_kernel(AttnArgs a) {
         constexpr bool last = decltype(last_tag)::value;
         const uint8_t* st = smem + (t & 1) * STAGE;
         const int key0 = t * CK;
+        // Channel steps outside, key blocks inside: consecutive MFMAs write different accumulators, so none waits for
+        // the one before it.
         v16i S[NB];
 #pragma unroll
-        for (int blk = 0; blk < NB; ++blk) {
-            const uint8_t* kp = st + blk * 4096 + lane * 16;
-            v16i acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        for (int blk = 0; blk < NB; ++blk) S[blk] = v16i{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                const v4i kf = *reinterpret_cast<const v4i*>(kp + s * 1024);
-                acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf, qf[s], acc, 0, 0, 0);
+        for (int s = 0; s < 4; ++s)
+#pragma unroll
+            for (int blk = 0; blk < NB; ++blk) {
+                const v4i kf = *reinterpret_cast<const v4i*>(st + blk * 4096 + s * 1024 + lane * 16);
+                S[blk] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf, qf[s], S[blk], 0, 0, 0);
             }
-            S[blk] = acc;
-        }
         if constexpr (!last) fetch(t + 1);   // the other stage: every wave left it at the barrier that ended the last tile
         const float* ksc = a.ks + (kvh * a.kb + t) * 4 + hh * 2;
         const float gs0 = a.sm * (q_scale * ksc[0]), gs1 = a.sm * (q_scale * ksc[1]);
@@ -540,27 +540,32 @@ __global__ __launch_bounds__(256, 2) void attn_int8_kernel(AttnArgs a) {
         probabilities(last_tag);
         dsum += (float)psum * t_scale;
 
+        // P.V: the four 32-channel blocks of the output keep their own accumulators (the scores are dead by now), key
+        // blocks outside, so that consecutive MFMAs are independent here too.
+        v16i acc[4];
 #pragma unroll
         for (int x = 0; x < 4; ++x) {
             const int* vsp = reinterpret_cast<const int*>(st + 2 * KV) + x * 32 + hh * 4;
-            v16i acc;
 #pragma unroll
             for (int g4 = 0; g4 < 4; ++g4) {
                 const v4i c4 = *reinterpret_cast<const v4i*>(vsp + g4 * 8);
-                acc[g4 * 4 + 0] = c4[0];
-                acc[g4 * 4 + 1] = c4[1];
-                acc[g4 * 4 + 2] = c4[2];
-                acc[g4 * 4 + 3] = c4[3];
+                acc[x][g4 * 4 + 0] = c4[0];
+                acc[x][g4 * 4 + 1] = c4[1];
+                acc[x][g4 * 4 + 2] = c4[2];
+                acc[x][g4 * 4 + 3] = c4[3];
             }
-#pragma unroll
-            for (int blk = 0; blk < NB; ++blk) {
-                const uint8_t* vp = st + KV + ((blk * D + x * 32 + l32) * 32 + hh * 16);
-                const v4i vf = *reinterpret_cast<const v4i*>(vp);
-                acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf, pf[blk], acc, 0, 0, 0);
-            }
-#pragma unroll
-            for (int i = 0; i < 16; ++i) ro[x][i] = fmaf((float)acc[i], t_scale, ro[x][i] * o_scale);
         }
+#pragma unroll
+        for (int blk = 0; blk < NB; ++blk)
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                const v4i vf = *reinterpret_cast<const v4i*>(st + KV + ((blk * D + x * 32 + l32) * 32 + hh * 16));
+                acc[x] = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf, pf[blk], acc[x], 0, 0, 0);
+            }
+#pragma unroll
+        for (int x = 0; x < 4; ++x)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) ro[x][i] = fmaf((float)acc[x][i], t_scale, ro[x][i] * o_scale);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wave's share of the next tile has landed
         __syncthreads();
     };
