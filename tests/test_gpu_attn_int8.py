@@ -220,6 +220,40 @@ def test_u8_pack_conversion_rounds_to_nearest_even_and_saturates():
     assert np.array_equal(yd.cpu().numpy(), want)
 
 
+def test_attention_replays_from_a_captured_graph():
+    """The call allocates nothing and clears its accumulators with kernels, so it can be captured (after one eager call
+    on the device, which sets the kernel's LDS limit).  Three replays with eager work and new inputs between them, each
+    against the eager result for the same inputs."""
+    ql, ffi = _pkg()
+    b, lq, lk, h, hk = 1, 200, 1300, 2, 2
+    q, k, v = (t.cuda() for t in _inputs(b, lq, lk, h, hk, torch.bfloat16, seed=31))
+    ws = torch.zeros((ffi.lib.gpu_int8_attn_workspace(b, h, hk, lq, lk),), dtype=torch.uint8, device="cuda")
+    o = torch.empty_like(q)
+    P = lambda t: C.c_void_p(t.data_ptr())
+
+    def call():
+        ffi.k("gpu_int8_attn", P(q), P(k), P(v), P(o), P(ws), b, lq, lk, h, hk, *q.stride()[:3], *k.stride()[:3],
+              *v.stride()[:3], *o.stride()[:3], 0.088, C.c_void_p(torch.cuda.current_stream().cuda_stream))
+
+    call()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()
+    g = torch.Generator(device="cuda").manual_seed(5)
+    for rep in range(3):
+        q.copy_(torch.randn(q.shape, device="cuda", generator=g).to(q.dtype))
+        k.copy_((torch.randn(k.shape, device="cuda", generator=g) + rep).to(k.dtype))
+        v.copy_(torch.randn(v.shape, device="cuda", generator=g).to(v.dtype))
+        o.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = o.clone()
+        want = ql.int8_attn(q, k, v, 0.088)      # eager, its own workspace
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), "replay %d differs from the eager call" % rep
+
+
 def test_attention_refuses_what_it_does_not_build():
     ql, ffi = _pkg()
     x = torch.zeros(1, 4, 1, 128, dtype=torch.bfloat16, device="cuda")
