@@ -6,7 +6,7 @@
 // one row), so tiles go global -> LDS as 16-byte chunks with an XOR swizzle and come back as ds_read_b128 fragments.
 // W rides in src0 and A in src1, which leaves every lane holding runs of four consecutive n for one m: the epilogue
 // stores 8-byte (bf16/f16) or 16-byte (f32) vectors straight from the accumulators.
-#include <cstdlib>
+#include <atomic>
 
 #include "common.hpp"
 
@@ -31,9 +31,6 @@ struct GemmArgs {
     int M, N, K;
     int tiles_m, tiles_n;
     int kslice;   // ring kernel only: K elements per split-K slice (a multiple of 128), 0 = no split
-#ifdef GEMM_TRACE
-    long long* trace;   // [workgroup][16] shader-clock stamps: start, then (K loop end, epilogue end) per tile
-#endif
 };
 
 template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int OCC_>
@@ -156,17 +153,6 @@ __device__ __forceinline__ void epilogue_shuffle(const GemmArgs& p, v16i (&acc)[
     // the stores, each behind a full memory wait.  Making the lane number opaque here keeps the address arithmetic local.
     asm volatile("" : "+v"(lane));
     const int frow = lane & 31, fhalf = lane >> 5;
-#ifdef GEMM_TRACE
-    int estamp = 8;
-    auto stamp_e = [&]() {
-        if (p.trace && threadIdx.x == 0 && estamp < 15 && p.trace[blockIdx.x * 16 + 8 + 6] == 0)
-            p.trace[blockIdx.x * 16 + estamp] = (long long)__builtin_readcyclecounter();
-        ++estamp;
-    };
-    stamp_e();
-#else
-    auto stamp_e = [&]() {};
-#endif
 
     // per-lane column constants, loaded once and in one batch (no branches between the loads, so a single wait covers
     // them): ws and the raw bias words for the 4 n of every (in, rb).  Columns past N read the last valid vector.
@@ -515,20 +501,6 @@ __global__ void __launch_bounds__(C::NT, C::OCC) int8_gemm_kernel(GemmArgs p) {
     epilogue<C::TM, C::TN, OUT_DT, EPI>(p, acc, m0 + wm * C::WTM, n0 + wn * C::WTN, lane, wave, smem);
 }
 
-// ---------------------------------------------------------------------------------------------------------------
-// The large-shape kernel: tiles stream global -> LDS with global_load_lds_dwordx4 (no register staging) into a ring of
-// NS stages, and the MFMA loop is software-pipelined by hand: while the 16 (TN*TM) MFMAs of one 32-deep K sub-step
-// issue, the ds_read_b128 fragment loads of the next sub-step and the DMA loads of a tile NS-1 ahead are interleaved
-// between them, pinned in that order with scheduling barriers.
-//
-// One 64-lane DMA instruction fills 1 KB of LDS (lane l -> bytes 16*l..16*l+15): 16 tile rows of 64 bytes.  The XOR
-// swizzle is applied on the global side: lane l fetches chunk (l%4) ^ swizzle(row) of row l/4, so the chunk lands in its
-// swizzled slot.  Requires K % 64 == 0.
-// ---------------------------------------------------------------------------------------------------------------
-typedef __attribute__((address_space(3))) void* lds_ptr_t;
-typedef const __attribute__((address_space(1))) void* glb_ptr_t;
-
-
 // 16-byte global store the compiler's wait-count bookkeeping does not see (see the ring kernel's epilogue)
 __device__ __forceinline__ void store16_untracked(void* ptr, uint4 v) {
     const v4i d = v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w};
@@ -538,311 +510,8 @@ __device__ __forceinline__ void store16_untracked(void* ptr, uint4 v) {
 }
 
 template <int N> __device__ __forceinline__ void wait_vmcnt() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
-// vmcnt wait whose count is only known at run time (a multiple of a tile's DMA count): pick the immediate by switch
-__device__ __forceinline__ void wait_vmcnt_n(int n) {
-    switch (n) {
-        case 4: wait_vmcnt<4>(); break;
-        case 6: wait_vmcnt<6>(); break;
-        case 8: wait_vmcnt<8>(); break;
-        case 12: wait_vmcnt<12>(); break;
-        case 16: wait_vmcnt<16>(); break;
-        case 24: wait_vmcnt<24>(); break;
-        case 32: wait_vmcnt<32>(); break;
-        default: wait_vmcnt<0>(); break;
-    }
-}
 __device__ __forceinline__ void wg_barrier() { asm volatile("s_barrier" ::: "memory"); }
-
-template <int BM_, int BN_, int WGM_, int WGN_, int NS_>
-struct DmaCfg {
-    static constexpr int BM = BM_, BN = BN_, BK = 64, WGM = WGM_, WGN = WGN_, NS = NS_;
-    static constexpr int NT = 256;
-    static constexpr int WTM = BM / WGM, WTN = BN / WGN, TM = WTM / 32, TN = WTN / 32;
-    static constexpr int A_LD = BM / 64, W_LD = BN / 64;   // DMA instructions per wave per K tile (16 rows each, 4 waves)
-    static constexpr int LD = A_LD + W_LD;
-    static constexpr int STAGE = (BM + BN) * BK;
-    static constexpr int SMEM = NS * STAGE;
-    static_assert(WGM * WGN == 4, "four waves");
-    static_assert(BM % (32 * WGM) == 0 && BN % (32 * WGN) == 0 && BM % 64 == 0 && BN % 64 == 0, "tile shape");
-    static_assert(NS >= 3 && (NS - 1) * LD < 64, "vmcnt is a 6-bit counter");
-};
-
-template <bool V> struct flag { static constexpr bool value = V; };
-
-template <class C, int OUT_DT, int EPI>
-__device__ __forceinline__ void dma_gemm_tile(const GemmArgs& p, uint8_t* smem, int m0, int n0) {
-    constexpr int BM = C::BM, BN = C::BN, BK = C::BK, NS = C::NS, TM = C::TM, TN = C::TN, LD = C::LD;
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar: LDS destinations of the DMA go through M0
-    const int wm = wave / C::WGN, wn = wave % C::WGN;
-    const int K = p.K, nk = K / BK;
-
-    // DMA sources: wave w owns 16-row blocks w, w+4, ... of the A tile and of the W tile.  Per-lane 32-bit offsets from
-    // the tile bases (the launcher guarantees M*K and N*K fit), so an instruction is scalar base + vector offset.
-    uint32_t ga[C::A_LD], gw[C::W_LD];
-    const int lrow = lane >> 2, lch = (lane & 3) ^ ((lrow >> 2) & 3);   // rows come in blocks of 16: swz<64> of the row
-#pragma unroll
-    for (int i = 0; i < C::A_LD; ++i) {
-        const int row = (wave + 4 * i) * 16 + lrow;
-        const int gr = m0 + row < p.M ? m0 + row : p.M - 1;
-        ga[i] = (uint32_t)gr * (uint32_t)K + lch * 16;
-    }
-#pragma unroll
-    for (int i = 0; i < C::W_LD; ++i) {
-        const int row = (wave + 4 * i) * 16 + lrow;
-        const int gr = n0 + row < p.N ? n0 + row : p.N - 1;
-        gw[i] = (uint32_t)gr * (uint32_t)K + lch * 16;
-    }
-    // One DMA instruction of ring slot t (K tile min(t, nk-1): slots past the last tile re-fetch it into a stage that
-    // nothing reads again, which keeps the loop body and its vmcnt bookkeeping free of branches).
-    auto dma = [&](int t, int j) {
-        const int kt = t < nk ? t : nk - 1;
-        uint8_t* s = smem + (t % NS) * C::STAGE;
-        if (j < C::A_LD)
-            __builtin_amdgcn_global_load_lds((glb_ptr_t)(p.A + (int64_t)kt * BK + ga[j]), (lds_ptr_t)(s + (wave + 4 * j) * 1024), 16, 0, 0);
-        else
-            __builtin_amdgcn_global_load_lds((glb_ptr_t)(p.W + (int64_t)kt * BK + gw[j - C::A_LD]),
-                                             (lds_ptr_t)(s + BM * BK + (wave + 4 * (j - C::A_LD)) * 1024), 16, 0, 0);
-    };
-
-    // fragment addresses: row r of a tile at r*64, chunk c at slot c ^ ((r>>1)&3); K sub-step kk flips address bit 5
-    const int frow = lane & 31, fhalf = lane >> 5;
-    const int fsw = (fhalf ^ ((frow >> 2) & 3)) << 4;
-    int aoff[2], woff[2];
-    aoff[0] = (wm * C::WTM + frow) * BK + fsw;
-    woff[0] = BM * BK + (wn * C::WTN + frow) * BK + fsw;
-    aoff[1] = aoff[0] ^ 32;
-    woff[1] = woff[0] ^ 32;
-    // fragment j of sub-step kk of the stage at s: j < TM are A fragments, the rest W fragments
-    auto frag = [&](const uint8_t* s, int kk, int j) -> v4i {
-        if (j < TM) return *reinterpret_cast<const v4i*>(s + aoff[kk] + j * 32 * BK);
-        return *reinterpret_cast<const v4i*>(s + woff[kk] + (j - TM) * 32 * BK);
-    };
-
-    v16i acc[TN][TM];
-#pragma unroll
-    for (int in = 0; in < TN; ++in)
-#pragma unroll
-        for (int im = 0; im < TM; ++im)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[in][im][r] = 0;
-
-    v4i f0[TM + TN], f1[TM + TN];   // fragments of the two sub-steps in flight
-
-    // One sub-step: TN*TM MFMAs on `cur`; between them, optionally the fragment loads of the next sub-step into `nxt`
-    // and the DMA instructions of ring slot t_dma.
-    auto substep = [&](auto LOAD, auto DMA, v4i* cur, v4i* nxt, const uint8_t* s_nxt, int kk_nxt, int t_dma) {
-        constexpr int NM = TN * TM, NF = TM + TN, EVERY = 1;   // fragment loads ride behind the first NF MFMAs
-        static_assert(NF <= NM, "more fragments than MFMAs");
-#pragma unroll
-        for (int i = 0; i < NM; ++i) {
-            const int in = i / TM, im = i % TM;
-            acc[in][im] = __builtin_amdgcn_mfma_i32_32x32x32_i8(cur[TM + in], cur[im], acc[in][im], 0, 0, 0);
-            SCHED_FENCE();
-            if constexpr (decltype(DMA)::value) {
-                if (i < LD) { dma(t_dma, i); SCHED_FENCE(); }
-            }
-            if constexpr (decltype(LOAD)::value) {
-                if (i % EVERY == 0 && i / EVERY < NF) { nxt[i / EVERY] = frag(s_nxt, kk_nxt, i / EVERY); SCHED_FENCE(); }
-            }
-        }
-    };
-
-    // prologue: ring slots 0..NS-2 in flight, wait for slot 0
-#pragma unroll
-    for (int t = 0; t < NS - 1; ++t)
-#pragma unroll
-        for (int j = 0; j < LD; ++j) dma(t, j);
-    wait_vmcnt<(NS - 2) * LD>();
-    wg_barrier();
-#pragma unroll
-    for (int j = 0; j < TM + TN; ++j) f0[j] = frag(smem, 0, j);
-
-    for (int kt = 0; kt + 1 < nk; ++kt) {
-        const uint8_t* s_cur = smem + (kt % NS) * C::STAGE;
-        const uint8_t* s_nxt = smem + ((kt + 1) % NS) * C::STAGE;
-        // first half: MFMAs of sub-step 0; fragment loads of sub-step 1 of the same tile
-        substep(flag<true>{}, flag<false>{}, f0, f1, s_cur, 1, 0);
-        // slot kt+1 must have landed for every wave (the NS-3 slots issued after it may stay in flight), and every wave
-        // must be done reading slot kt-1 before its stage is refilled
-        wait_vmcnt<(NS - 3) * LD>();
-        wg_barrier();
-        // second half: MFMAs of sub-step 1; DMA of slot kt+NS-1; fragment loads of sub-step 0 of tile kt+1
-        substep(flag<true>{}, flag<true>{}, f1, f0, s_nxt, 0, kt + NS - 1);
-    }
-    {
-        const uint8_t* s_cur = smem + ((nk - 1) % NS) * C::STAGE;
-        substep(flag<true>{}, flag<false>{}, f0, f1, s_cur, 1, 0);
-        substep(flag<false>{}, flag<false>{}, f1, f0, s_cur, 0, 0);
-    }
-    wait_vmcnt<0>();   // drain the re-fetches of the last slots before the LDS is reused
-    epilogue<TM, TN, OUT_DT, EPI>(p, acc, m0 + wm * C::WTM, n0 + wn * C::WTN, lane, wave, smem);
-}
-
-template <class C, int OUT_DT, int EPI>
-__global__ void __launch_bounds__(256, 1) int8_gemm_dma_kernel(GemmArgs p) {
-    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    int tm, tn;
-    tile_of_block(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, tm, tn);
-    dma_gemm_tile<C, OUT_DT, EPI>(p, smem, tm * C::BM, tn * C::BN);
-}
-
-// ---------------------------------------------------------------------------------------------------------------
-// Variant with 128-byte tile rows (BK = 128) and two LDS stages: every DMA lane group fetches whole 128-byte cache
-// lines (8 rows per 1 KB instruction), which halves the number of L2 requests per byte compared with 64-byte rows.
-// A K tile is four 32-deep sub-steps.  Two workgroup barriers per tile: X, after which the other stage is free and the
-// DMA of the next tile is issued (it then has three sub-steps of MFMAs to land), and Y, before the last sub-step, after
-// which the next tile is visible and its first fragments are prefetched.
-// ---------------------------------------------------------------------------------------------------------------
-template <int BM_, int BN_, int WGM_, int WGN_>
-struct Dma2Cfg {
-    static constexpr int BM = BM_, BN = BN_, BK = 128, WGM = WGM_, WGN = WGN_, NS = 2;
-    static constexpr int NT = 256;
-    static constexpr int WTM = BM / WGM, WTN = BN / WGN, TM = WTM / 32, TN = WTN / 32;
-    static constexpr int A_LD = BM / 32, W_LD = BN / 32;   // DMA instructions per wave per K tile (8 rows each, 4 waves)
-    static constexpr int LD = A_LD + W_LD;
-    static constexpr int STAGE = (BM + BN) * BK;
-    static constexpr int SMEM = NS * STAGE;
-    static_assert(WGM * WGN == 4, "four waves");
-    static_assert(BM % (32 * WGM) == 0 && BN % (32 * WGN) == 0, "tile shape");
-};
-
-template <class C, int OUT_DT, int EPI>
-__device__ __forceinline__ void dma2_gemm_tile(const GemmArgs& p, uint8_t* smem, int m0, int n0) {
-    constexpr int BM = C::BM, BN = C::BN, BK = C::BK, TM = C::TM, TN = C::TN, LD = C::LD;
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar: LDS destinations of the DMA go through M0
-    const int wm = wave / C::WGN, wn = wave % C::WGN;
-    const int K = p.K, nk = K / BK;
-
-    // DMA sources: wave w owns 8-row blocks w, w+4, ... of the A tile and of the W tile, as 32-bit lane offsets
-    uint32_t ga[C::A_LD], gw[C::W_LD];
-    // rows come in blocks of 8 (block index wave + 4i has the parity of wave): swz<128> of the row
-    const int lrow = lane >> 3, lch = (lane & 7) ^ (((wave & 1) << 2) | (lrow >> 1));
-#pragma unroll
-    for (int i = 0; i < C::A_LD; ++i) {
-        const int row = (wave + 4 * i) * 8 + lrow;
-        const int gr = m0 + row < p.M ? m0 + row : p.M - 1;
-        ga[i] = (uint32_t)gr * (uint32_t)K + lch * 16;
-    }
-#pragma unroll
-    for (int i = 0; i < C::W_LD; ++i) {
-        const int row = (wave + 4 * i) * 8 + lrow;
-        const int gr = n0 + row < p.N ? n0 + row : p.N - 1;
-        gw[i] = (uint32_t)gr * (uint32_t)K + lch * 16;
-    }
-    // One DMA instruction of K tile min(t, nk-1) into stage t&1 (a tile index past the end re-fetches the last tile
-    // into the stage nothing reads again, which keeps the loop body free of branches).
-    auto dma = [&](int t, int j) {
-        const int kt = t < nk ? t : nk - 1;
-        uint8_t* s = smem + (t & 1) * C::STAGE;
-        if (j < C::A_LD)
-            __builtin_amdgcn_global_load_lds((glb_ptr_t)(p.A + (int64_t)kt * BK + ga[j]), (lds_ptr_t)(s + (wave + 4 * j) * 1024), 16, 0, 0);
-        else
-            __builtin_amdgcn_global_load_lds((glb_ptr_t)(p.W + (int64_t)kt * BK + gw[j - C::A_LD]),
-                                             (lds_ptr_t)(s + BM * BK + (wave + 4 * (j - C::A_LD)) * 1024), 16, 0, 0);
-    };
-
-    // fragment addresses: row r at r*128, chunk c at slot c ^ ((r>>1)&7); K sub-step kk flips address bits 5 and 6
-    const int frow = lane & 31, fhalf = lane >> 5;
-    const int fsw = (fhalf ^ ((frow >> 1) & 7)) << 4;
-    int aoff[4], woff[4];
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
-        aoff[kk] = ((wm * C::WTM + frow) * BK + fsw) ^ (kk << 5);
-        woff[kk] = (BM * BK + (wn * C::WTN + frow) * BK + fsw) ^ (kk << 5);
-    }
-    auto frag = [&](const uint8_t* s, int kk, int j) -> v4i {
-        if (j < TM) return *reinterpret_cast<const v4i*>(s + aoff[kk] + j * 32 * BK);
-        return *reinterpret_cast<const v4i*>(s + woff[kk] + (j - TM) * 32 * BK);
-    };
-
-    v16i acc[TN][TM];
-#pragma unroll
-    for (int in = 0; in < TN; ++in)
-#pragma unroll
-        for (int im = 0; im < TM; ++im)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[in][im][r] = 0;
-
-    v4i f0[TM + TN], f1[TM + TN];
-
-    // One sub-step: TN*TM MFMAs on `cur`, with the fragment loads of the next sub-step into `nxt` behind the first
-    // MFMAs, and one DMA instruction of tile t_dma after every DMA_EVERY-th MFMA of the tile (this sub-step's MFMAs
-    // are numbers mfma_base .. mfma_base + TN*TM - 1 of the tile).  The
-    // texture-address unit takes about 16 cycles per 1 KB DMA instruction and serves all four waves, so the DMA of a
-    // tile is spread over three sub-steps instead of being bunched: bunched, the waves stall at issue and the MFMA
-    // pipe drains.
-    constexpr int DMA_EVERY = 3;
-    auto substep = [&](auto DMA, v4i* cur, v4i* nxt, const uint8_t* s_nxt, int kk_nxt, int t_dma, int mfma_base) {
-        constexpr int NM = TN * TM, NF = TM + TN;
-        static_assert(NF <= NM, "more fragment loads than MFMAs to hide them behind");
-#pragma unroll
-        for (int i = 0; i < NM; ++i) {
-            const int in = i / TM, im = i % TM;
-            acc[in][im] = __builtin_amdgcn_mfma_i32_32x32x32_i8(cur[TM + in], cur[im], acc[in][im], 0, 0, 0);
-            SCHED_FENCE();
-            if constexpr (decltype(DMA)::value) {
-                if ((mfma_base + i) % DMA_EVERY == 0 && (mfma_base + i) / DMA_EVERY < LD) {
-                    dma(t_dma, (mfma_base + i) / DMA_EVERY);
-                    SCHED_FENCE();
-                }
-            }
-            if (i < NF) { nxt[i] = frag(s_nxt, kk_nxt, i); SCHED_FENCE(); }
-        }
-    };
-    static_assert((LD - 1) * DMA_EVERY < 3 * TN * TM, "the DMA of a tile must fit in three sub-steps");
-
-#pragma unroll
-    for (int j = 0; j < LD; ++j) dma(0, j);
-    wait_vmcnt<0>();
-    wg_barrier();
-#pragma unroll
-    for (int j = 0; j < TM + TN; ++j) f0[j] = frag(smem, 0, j);
-
-    for (int kt = 0; kt < nk; ++kt) {
-        const uint8_t* s_cur = smem + (kt & 1) * C::STAGE;
-        const uint8_t* s_nxt = smem + ((kt + 1) & 1) * C::STAGE;
-        wg_barrier();                                              // X: every wave is done with tile kt-1
-        substep(flag<true>{}, f0, f1, s_cur, 1, kt + 1, 0);
-        substep(flag<true>{}, f1, f0, s_cur, 2, kt + 1, TN * TM);
-        substep(flag<true>{}, f0, f1, s_cur, 3, kt + 1, 2 * TN * TM);
-        wait_vmcnt<0>();
-        wg_barrier();                                              // Y: tile kt+1 has landed for every wave
-        substep(flag<false>{}, f1, f0, s_nxt, 0, 0, 0);
-    }
-    epilogue<TM, TN, OUT_DT, EPI>(p, acc, m0 + wm * C::WTM, n0 + wn * C::WTN, lane, wave, smem);
-}
-
-template <class C, int OUT_DT, int EPI>
-__global__ void __launch_bounds__(256, 1) int8_gemm_dma2_kernel(GemmArgs p) {
-    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    int tm, tn;
-    tile_of_block(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, tm, tn);
-    dma2_gemm_tile<C, OUT_DT, EPI>(p, smem, tm * C::BM, tn * C::BN);
-}
-
-using Dma2L = Dma2Cfg<256, 256, 2, 2>;
-
-using DmaL = DmaCfg<256, 256, 2, 2, 4>;
-
-template <class C, int OUT_DT, int EPI>
-int launch_dma(GemmArgs a, hipStream_t st) {
-    a.tiles_m = (a.M + C::BM - 1) / C::BM;
-    a.tiles_n = (a.N + C::BN - 1) / C::BN;
-    const int64_t nblocks = (int64_t)a.tiles_m * a.tiles_n;
-    if (nblocks > 0x7fffffff) return -1;
-    auto kern = int8_gemm_dma_kernel<C, OUT_DT, EPI>;
-    static bool once = false;  // benign race: the attribute is idempotent
-    if (!once) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
-        if (e != hipSuccess) return (int)e;
-        once = true;
-    }
-    hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(C::NT), C::SMEM, st, a);
-    KCHECK();
-    return 0;
-}
+__device__ __forceinline__ void wait_lgkmcnt0() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 
 // ---------------------------------------------------------------------------------------------------------------
 // The persistent ring kernel: one workgroup per CU walks its share of the 256x256 output tiles and keeps ONE
@@ -860,25 +529,29 @@ int launch_dma(GemmArgs a, hipStream_t st) {
 // ---------------------------------------------------------------------------------------------------------------
 template <int V> struct ic { static constexpr int value = V; };
 
-// BN: tile width; WGM x WGN: wave grid (four waves); NSA: LDS stages of A (2 for the 256-wide tile, where 160 KB of LDS
-// leave no room for a third; 3 where a narrower tile leaves room).  W always has three stages.
+// BN: tile width; WGM x WGN: wave grid, four waves (one per SIMD, 128x128 wave tiles, up to 512 registers each) or eight
+// (two per SIMD, 256 registers each: while one wave of a SIMD issues DMA, waits at a barrier or runs the epilogue's vector
+// arithmetic, the other's MFMAs keep the matrix pipe busy); NSA: LDS stages of A (2 for the 256-wide tile, where 160 KB
+// of LDS leave no room for a third; 3 where a narrower tile leaves room).  W always has three stages.
 template <int BN_, int WGM_, int WGN_, int NSA_, int BM_ = 256>
 struct RingCfg {
-    static constexpr int BM = BM_, BN = BN_, BK = 128, WGM = WGM_, WGN = WGN_, NT = 256, NSA = NSA_, NSW = 3;
+    static constexpr int BM = BM_, BN = BN_, BK = 128, WGM = WGM_, WGN = WGN_, NW = WGM * WGN, NT = 64 * NW, NSA = NSA_, NSW = 3;
     static constexpr int WTM = BM / WGM, WTN = BN / WGN, TM = WTM / 32, TN = WTN / 32;
-    static constexpr int A_LD = BM / 32, W_LD = BN / 32;     // DMA instructions per wave per stage (8 rows each)
+    static constexpr int A_LD = BM / (8 * NW), W_LD = BN / (8 * NW);   // DMA instructions per wave per stage (8 rows each)
     static constexpr int NDMA = A_LD + W_LD, NM = TM * TN, NF = TM + TN;
     static constexpr int A_STAGE = BM * BK, W_STAGE = BN * BK;
     static constexpr int W_BASE = NSA * A_STAGE;
     static constexpr int SMEM = NSA * A_STAGE + NSW * W_STAGE;
-    static_assert(WGM * WGN == 4 && BM % (32 * WGM) == 0 && BN % (32 * WGN) == 0 && BN % 32 == 0, "tile shape");
+    static_assert((NW == 4 || NW == 8) && BM % (32 * WGM) == 0 && BN % (32 * WGN) == 0 && BN % 32 == 0, "tile shape");
+    static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "whole DMA blocks per wave");
     static_assert(NF <= NM && SMEM <= 160 * 1024, "fragment loads hide behind MFMAs; LDS fits");
     // Slot of the d-th DMA instruction of an iteration (A first, then W), as the number of the MFMA it follows; an
     // iteration has 4*NM MFMAs and barrier Y sits after MFMA 3*NM - 1.  With two A stages the A DMA is needed by this
-    // iteration's barrier Y, so it goes first and dense; with three, everything has an iteration of slack and is
-    // spread evenly.
+    // iteration's barrier Y, so it goes first and dense (inside the first one and a half sub-steps); with three,
+    // everything has an iteration of slack and is spread evenly.
     static constexpr int slot(int d) {
-        return NSA == 2 ? (d < A_LD ? d * 3 : 24 + (d - A_LD) * 4) : (d * 4 * NM) / NDMA;
+        return NSA == 2 ? (d < A_LD ? d * ((3 * NM) / (2 * A_LD)) : (3 * NM) / 2 + (d - A_LD) * ((4 * NM - (3 * NM) / 2 - 1) / W_LD))
+                        : (d * 4 * NM) / NDMA;
     }
     // DMA instructions of this iteration that may still be in flight at barrier Y
     static constexpr int in_flight_at_y() {
@@ -899,15 +572,19 @@ struct RingCfg {
     // per lane in flight between the read and the store half of a piece) where the wave tile's width allows
     static constexpr int piece_cols(int sz) { return WTN % (128 / sz) == 0 ? 128 / sz : 32; }
     // Epilogue scratch of one wave inside a stage that was just multiplied: a shuffle piece in each of an A and a W
-    // stage, and the wave's column constants (2 x WTN floats) behind the piece in the W stage.
-    static constexpr int A_REGION = A_STAGE / 4, W_REGION = W_STAGE / 4;
+    // stage.  With four waves (128 columns each) the wave's column constants (2 x WTN floats) sit behind the piece in the
+    // W stage; with eight (64 columns each) they fit in registers.
+    static constexpr bool STAGED = NW == 4;
+    static constexpr int A_REGION = A_STAGE / NW, W_REGION = W_STAGE / NW;
     static constexpr int piece_bytes(int sz) { return 32 * piece_cols(sz) * sz; }
-    static constexpr bool scratch_ok(int sz) { return piece_bytes(sz) <= A_REGION && piece_bytes(sz) + 2 * WTN * 4 <= W_REGION; }
+    static constexpr bool scratch_ok(int sz) {
+        return piece_bytes(sz) <= A_REGION && piece_bytes(sz) + (STAGED ? 2 * WTN * 4 : 0) <= W_REGION;
+    }
     static_assert(scratch_ok(2) && scratch_ok(4), "epilogue scratch fits the stages");
 };
 
 template <class C, int OUT_DT, int EPI>
-__global__ void __launch_bounds__(256, 1) int8_gemm_ring_kernel(GemmArgs p) {
+__global__ void __launch_bounds__(C::NT, 1) int8_gemm_ring_kernel(GemmArgs p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     constexpr int BK = C::BK, TM = C::TM, TN = C::TN, NM = C::NM, NF = C::NF, NSA = C::NSA;
     const int tid = threadIdx.x, lane = tid & 63;
@@ -933,7 +610,7 @@ __global__ void __launch_bounds__(256, 1) int8_gemm_ring_kernel(GemmArgs p) {
 
     // DMA streams.  Each walks (tile, K tile) pairs in the order the MFMAs will consume them and stops on the last one
     // (re-fetching it into a stage nothing reads again keeps the loop free of branches around the DMA slots).
-    // rows come in blocks of 8 (block index wave + 4j has the parity of wave): swz<128> of the row
+    // rows come in blocks of 8 (block index wave + NW*j has the parity of wave): swz<128> of the row
     uint32_t ga[C::A_LD], gw[C::W_LD];
     int a_tile = 0, a_kt = 0, a_stage = 0, w_tile = 0, w_kt = 0, w_stage = 0;
     // The row and chunk of a lane are recomputed from the hardware lane number each time a stream moves to its next
@@ -946,7 +623,7 @@ __global__ void __launch_bounds__(256, 1) int8_gemm_ring_kernel(GemmArgs p) {
         const int lr = l >> 3, lc = ((l & 7) ^ (((wave & 1) << 2) | (lr >> 1))) * 16;
 #pragma unroll
         for (int j = 0; j < C::A_LD; ++j) {
-            const int row = (wave + 4 * j) * 8 + lr;
+            const int row = (wave + C::NW * j) * 8 + lr;
             const int gr = m0 + row < p.M ? m0 + row : p.M - 1;
             ga[j] = (uint32_t)gr * (uint32_t)ld + lc;
         }
@@ -958,7 +635,7 @@ __global__ void __launch_bounds__(256, 1) int8_gemm_ring_kernel(GemmArgs p) {
         const int lr = l >> 3, lc = ((l & 7) ^ (((wave & 1) << 2) | (lr >> 1))) * 16;
 #pragma unroll
         for (int j = 0; j < C::W_LD; ++j) {
-            const int row = (wave + 4 * j) * 8 + lr;
+            const int row = (wave + C::NW * j) * 8 + lr;
             const int gr = n0 + row < p.N ? n0 + row : p.N - 1;
             gw[j] = (uint32_t)gr * (uint32_t)ld + lc;
         }
@@ -969,12 +646,12 @@ __global__ void __launch_bounds__(256, 1) int8_gemm_ring_kernel(GemmArgs p) {
     const uint32_t lds_base = (uint32_t)(uintptr_t)smem;   // LDS byte address of the dynamic segment
     auto dma_a = [&](int j) {
         const int8_t* base = Ab + (int64_t)a_kt * BK;
-        const uint32_t dst = lds_base + a_stage * C::A_STAGE + (wave + 4 * j) * 1024;
+        const uint32_t dst = lds_base + a_stage * C::A_STAGE + (wave + C::NW * j) * 1024;
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(ga[j]), "s"(base) : "memory", "m0");
     };
     auto dma_w = [&](int j) {
         const int8_t* base = Wb + (int64_t)w_kt * BK;
-        const uint32_t dst = lds_base + C::W_BASE + w_stage * C::W_STAGE + (wave + 4 * j) * 1024;
+        const uint32_t dst = lds_base + C::W_BASE + w_stage * C::W_STAGE + (wave + C::NW * j) * 1024;
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(gw[j]), "s"(base) : "memory", "m0");
     };
     auto advance_a = [&]() {
@@ -1025,12 +702,6 @@ __global__ void __launch_bounds__(256, 1) int8_gemm_ring_kernel(GemmArgs p) {
         }
     };
 
-#ifdef GEMM_TRACE
-    auto stamp = [&](int i) { if (p.trace && tid == 0 && i < 16) p.trace[blockIdx.x * 16 + i] = (long long)__builtin_readcyclecounter(); };
-    stamp(0);
-#else
-    auto stamp = [&](int) {};
-#endif
     // prologue: A(0), W(0), [A(1),] W(1) in flight; A(0) and W(0) must land
     set_a(0);
     set_w(0);
@@ -1053,9 +724,6 @@ __global__ void __launch_bounds__(256, 1) int8_gemm_ring_kernel(GemmArgs p) {
 #pragma unroll
     for (int j = 0; j < NF; ++j) f0[j] = frag(smem, smem + C::W_BASE, 0, j);
 
-#ifdef GEMM_TRACE
-    long long qs[5] = {0, 0, 0, 0, 0};
-#endif
     int ca = 0, cw = 0;   // stages of the iteration being multiplied
     for (int ti = 0; ti < nt_b; ++ti) {
 #pragma unroll
@@ -1074,32 +742,13 @@ __global__ void __launch_bounds__(256, 1) int8_gemm_ring_kernel(GemmArgs p) {
             const uint8_t* sa = smem + ca * C::A_STAGE;
             const uint8_t* sw = smem + C::W_BASE + cw * C::W_STAGE;
             const int na = ca == NSA - 1 ? 0 : ca + 1, nw = cw == C::NSW - 1 ? 0 : cw + 1;
-#ifdef GEMM_TRACE
-            const long long q0 = (long long)__builtin_readcyclecounter();
-#endif
             wg_barrier();                                                   // X
-#ifdef GEMM_TRACE
-            const long long q1 = (long long)__builtin_readcyclecounter();
-#endif
             substep(ic<0>{}, f0, f1, sa, sw, 1);
             substep(ic<NM>{}, f1, f0, sa, sw, 2);
             substep(ic<2 * NM>{}, f0, f1, sa, sw, 3);
-#ifdef GEMM_TRACE
-            const long long q2 = (long long)__builtin_readcyclecounter();
-#endif
             wait_vmcnt<C::in_flight_at_y()>();
-#ifdef GEMM_TRACE
-            const long long q3 = (long long)__builtin_readcyclecounter();
-#endif
             wg_barrier();                                                   // Y
-#ifdef GEMM_TRACE
-            const long long q4 = (long long)__builtin_readcyclecounter();
-#endif
             substep(ic<3 * NM>{}, f1, f0, smem + na * C::A_STAGE, smem + C::W_BASE + nw * C::W_STAGE, 0);
-#ifdef GEMM_TRACE
-            const long long q5 = (long long)__builtin_readcyclecounter();
-            qs[0] += q1 - q0; qs[1] += q2 - q1; qs[2] += q3 - q2; qs[3] += q4 - q3; qs[4] += q5 - q4;
-#endif
             advance_a();
             advance_w();
             pa = ca;
@@ -1112,7 +761,6 @@ __global__ void __launch_bounds__(256, 1) int8_gemm_ring_kernel(GemmArgs p) {
         // (The launcher only picks this kernel when the coalesced epilogue's alignment conditions hold.)
         int m0, n0;
         tile_origin(ti, m0, n0);
-        stamp(1 + 2 * ti);
         __syncthreads();   // every wave is done reading that stage
         constexpr int SZ = (EPI == EPI_ACC || OUT_DT == DT_F32) ? 4 : 2;
         constexpr int PW = C::piece_cols(SZ);
@@ -1120,20 +768,223 @@ __global__ void __launch_bounds__(256, 1) int8_gemm_ring_kernel(GemmArgs p) {
         // flight fills the other stages; the next write into these two is issued inside the next iteration).
         uint8_t* ra = smem + pa * C::A_STAGE + wave * C::A_REGION;
         uint8_t* rw = smem + C::W_BASE + pw * C::W_STAGE + wave * C::W_REGION;
-        epilogue_shuffle<TM, TN, OUT_DT, EPI, PW, true, true>(p, acc, m0 + wm * C::WTM, n0 + wn * C::WTN, hw_lane(), ra, rw,
+        epilogue_shuffle<TM, TN, OUT_DT, EPI, PW, true, C::STAGED>(p, acc, m0 + wm * C::WTM, n0 + wn * C::WTN, hw_lane(), ra, rw,
                                                                reinterpret_cast<float*>(rw + C::piece_bytes(SZ)));
         // The first fragments of the next tile were prefetched by the last sub-step; fetching them again here instead of
         // carrying 32 registers across the epilogue keeps the epilogue free of spills.
 #pragma unroll
         for (int j = 0; j < NF; ++j) f0[j] = frag(smem + ca * C::A_STAGE, smem + C::W_BASE + cw * C::W_STAGE, 0, j);
-        stamp(2 + 2 * ti);
     }
     wait_vmcnt<0>();   // no DMA may still be writing this workgroup's LDS when it retires
-    stamp(15);
-#ifdef GEMM_TRACE
-    if (p.trace && lane == 0 && wave < 2)
-        for (int i = 0; i < 5; ++i) p.trace[4096 + (blockIdx.x * 2 + wave) * 5 + i] = qs[i];
-#endif
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// The two-group persistent kernel for large shapes.  A global_load_lds_dwordx4 keeps the wave that issues it busy for
+// about 68 cycles (measured: one wave alone, 16 of them back to back, 1088 cycles), twice the 32 cycles of a
+// v_mfma_i32_32x32x32_i8, so a wave that issues its own DMA between its MFMAs leaves the matrix pipe of its SIMD idle
+// for part of each one.  Here a workgroup has eight waves, two per SIMD, in two groups of four: group g owns rows
+// 128g..128g+127 of a 256x256 tile (wave tiles 128x64).  The groups alternate between two kinds of phase, with one
+// workgroup barrier between phases:
+//   compute: the 32 MFMAs of one 128-deep K step, on fragments already in registers, and nothing else;
+//   memory:  the 24 fragment reads of the group's next K step and 8 DMA instructions per wave.
+// While one wave of a SIMD is in its memory phase the other is in its compute phase, so the matrix pipe always has an
+// MFMA to run and no MFMA waits behind a DMA.
+//
+// LDS (160 KB): three 32 KB stages of W (both groups read them) and two 16 KB stages of A for each group.  With global
+// step s = tile * nk + k tile, group 0 computes step s in phase 2s and group 1 in phase 2s + 1.  Group 0's memory phase
+// before step s fetches A of group 1 for step s + 1 and rows 0..127 of W for step s + 2; group 1's fetches A of group 0
+// and rows 128..255 of W, both for step s + 2.  Every memory phase ends with a wait that leaves only its own 8 DMA
+// instructions in flight, so what a phase fetches is visible to everybody two phases later, and each stage is refilled
+// only after the barrier that follows its last reader.  Steps run straight through tile boundaries.
+//
+// End of a tile: group 0 runs its epilogue while group 1 multiplies its last step and then runs its own; the shuffle
+// scratch is the W stage of that step (4 KB per wave), which no DMA in flight targets.  One barrier, then group 0's
+// first memory phase of the next tile (group 1 has nothing to do in it), and the alternation resumes.
+// Requires K % 128 == 0, M*K and N*K < 2^32, and the coalesced epilogue's alignment.
+// ---------------------------------------------------------------------------------------------------------------
+struct PpCfg {
+    static constexpr int BM = 256, BN = 256, BK = 128, NT = 512, GM = 128;         // GM: rows of a group
+    static constexpr int TM = 4, TN = 2, WTN = 64;                                  // wave tile 128 x 64
+    static constexpr int W_STAGE = BN * BK, A_STAGE = GM * BK, NSW = 3, NSA = 2;
+    static constexpr int A_BASE = NSW * W_STAGE;                                    // group g's A ring at A_BASE + g*NSA*A_STAGE
+    static constexpr int SMEM = NSW * W_STAGE + 2 * NSA * A_STAGE;
+    static constexpr int NLD = 4;                                                   // DMA instructions per wave and 128-row block set
+    static_assert(SMEM <= 160 * 1024, "LDS fits");
+    static constexpr int piece_cols(int sz) { return sz == 2 ? 64 : 32; }           // 4 KB shuffle pieces
+};
+
+template <int OUT_DT, int EPI>
+__global__ void __launch_bounds__(PpCfg::NT, 1) int8_gemm_pp_kernel(GemmArgs p) {
+    using C = PpCfg;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    constexpr int BK = C::BK, TM = C::TM, TN = C::TN;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int grp = wave >> 2, wq = wave & 3;            // group; wave within the group = its column quarter
+    const int ld = p.K, nk = p.K / BK;
+    const int G = gridDim.x, ntiles = p.tiles_m * p.tiles_n;
+    const int nt_b = (ntiles - (int)blockIdx.x + G - 1) / G;   // tiles of this workgroup: blockIdx, blockIdx + G, ...
+    const int S = nt_b * nk;                             // steps of this workgroup
+    auto tile_origin = [&](int i, int& m0, int& n0) {
+        int tm, tn;
+        tile_of_block((int)blockIdx.x + i * G, ntiles, p.tiles_m, p.tiles_n, tm, tn);
+        m0 = tm * C::BM;
+        n0 = tn * C::BN;
+    };
+    const uint32_t lds_base = (uint32_t)(uintptr_t)smem;
+    auto dma = [&](uint32_t dst, uint32_t off, const int8_t* base) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(off), "s"(base) : "memory", "m0");
+    };
+
+    // DMA streams of this wave.  A wave fetches 8-row blocks wq, wq + 4, wq + 8, wq + 12 of a 128-row half: of the
+    // OTHER group's A tile and of its own half of the W tile (group 0: rows 0..127, group 1: rows 128..255).
+    // Lane offsets carry the chunk swizzle (bits 1..3 of the row) on the global side, as in the ring kernel.
+    uint32_t ga[C::NLD], gw[C::NLD];
+    // a stream's position: the (tile, k tile) it fetches next and the stage that goes to.  A stream stops on the last step
+    // and keeps re-fetching it, into the stage it would have used, which nothing reads again.
+    int a_tile, a_kt, a_stage, w_tile = 0, w_kt = 0, w_stage = 0;
+    auto set_rows = [&](uint32_t* g, int origin, int limit) {
+        const int l = hw_lane();
+        const int lr = l >> 3, lc = ((l & 7) ^ (((wq & 1) << 2) | (lr >> 1))) * 16;
+#pragma unroll
+        for (int j = 0; j < C::NLD; ++j) {
+            const int row = origin + (wq + 4 * j) * 8 + lr;
+            g[j] = (uint32_t)(row < limit ? row : limit - 1) * (uint32_t)ld + lc;
+        }
+    };
+    auto set_a = [&](int tile) { int m0, n0; tile_origin(tile, m0, n0); set_rows(ga, m0 + (grp ^ 1) * C::GM, p.M); };
+    auto set_w = [&](int tile) { int m0, n0; tile_origin(tile, m0, n0); set_rows(gw, n0 + grp * C::GM, p.N); };
+    auto fetch_a = [&]() {
+        const int8_t* base = p.A + (int64_t)a_kt * BK;
+        const uint32_t dst = lds_base + C::A_BASE + ((grp ^ 1) * C::NSA + a_stage) * C::A_STAGE + wq * 1024;
+#pragma unroll
+        for (int j = 0; j < C::NLD; ++j) dma(dst + j * 4096, ga[j], base);
+        a_stage = a_stage == C::NSA - 1 ? 0 : a_stage + 1;
+        if (a_tile == nt_b - 1 && a_kt == nk - 1) return;
+        if (++a_kt == nk) { a_kt = 0; set_a(++a_tile); }
+    };
+    auto fetch_w = [&]() {
+        const int8_t* base = p.W + (int64_t)w_kt * BK;
+        const uint32_t dst = lds_base + w_stage * C::W_STAGE + grp * C::GM * BK + wq * 1024;
+#pragma unroll
+        for (int j = 0; j < C::NLD; ++j) dma(dst + j * 4096, gw[j], base);
+        w_stage = w_stage == C::NSW - 1 ? 0 : w_stage + 1;
+        if (w_tile == nt_b - 1 && w_kt == nk - 1) return;
+        if (++w_kt == nk) { w_kt = 0; set_w(++w_tile); }
+    };
+
+    // fragment addresses inside a stage: row r at r*128, chunk c at slot c ^ ((r>>1)&7); K sub-step kk flips bits 5 and 6
+    v16i acc[TN][TM];
+    v4i f[4][TM + TN];
+    int ra_stage = 0, rw_stage = 0;   // stages this group's next fragments come from
+    auto load_frags = [&]() {
+        const int l = hw_lane();
+        const int frow = l & 31, fhalf = l >> 5;
+        const int x = frow * BK + ((fhalf ^ ((frow >> 1) & 7)) << 4);
+        const uint8_t* sa = smem + C::A_BASE + (grp * C::NSA + ra_stage) * C::A_STAGE;
+        const uint8_t* sw = smem + rw_stage * C::W_STAGE + wq * C::WTN * BK;
+        ra_stage = ra_stage == C::NSA - 1 ? 0 : ra_stage + 1;
+        rw_stage = rw_stage == C::NSW - 1 ? 0 : rw_stage + 1;
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+#pragma unroll
+            for (int j = 0; j < TM; ++j) f[kk][j] = *reinterpret_cast<const v4i*>(sa + (x ^ (kk << 5)) + j * 32 * BK);
+#pragma unroll
+            for (int j = 0; j < TN; ++j) f[kk][TM + j] = *reinterpret_cast<const v4i*>(sw + (x ^ (kk << 5)) + j * 32 * BK);
+        }
+    };
+    auto compute = [&](bool first) {
+        __builtin_amdgcn_s_setprio(1);
+        if (first) {
+#pragma unroll
+            for (int in = 0; in < TN; ++in)
+#pragma unroll
+                for (int im = 0; im < TM; ++im) {
+                    v16i z;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) z[r] = 0;
+                    acc[in][im] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f[0][TM + in], f[0][im], z, 0, 0, 0);
+                    SCHED_FENCE();
+                }
+        }
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+            if (first && kk == 0) continue;
+#pragma unroll
+            for (int in = 0; in < TN; ++in)
+#pragma unroll
+                for (int im = 0; im < TM; ++im) {
+                    acc[in][im] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f[kk][TM + in], f[kk][im], acc[in][im], 0, 0, 0);
+                    SCHED_FENCE();
+                }
+        }
+        __builtin_amdgcn_s_setprio(0);
+    };
+    // memory phase before this group's next step
+    auto memory = [&]() {
+        load_frags();
+        SCHED_FENCE();
+        fetch_a();
+        fetch_w();
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * C::NLD) : "memory");   // everything but this phase's own DMA has landed
+    };
+
+    // prologue: every group fetches its OWN A for step 0 (group 0 also for step 1: group 1's first memory phase fetches
+    // A0 of step 2) and its half of W for steps 0 and 1; then the streams move to where the memory phases expect them
+    {
+        int m0, n0;
+        const int own_a = C::A_BASE + grp * C::NSA * C::A_STAGE;
+        const int t1 = (nk == 1 && nt_b > 1) ? 1 : 0, k1 = nk > 1 ? 1 : 0;   // step 1 as (tile, k tile); step 0 again if S == 1
+        tile_origin(0, m0, n0);
+        set_rows(ga, m0 + grp * C::GM, p.M);
+#pragma unroll
+        for (int j = 0; j < C::NLD; ++j) dma(lds_base + own_a + (wq + 4 * j) * 1024, ga[j], p.A);
+        if (grp == 0) {
+            if (t1) { tile_origin(1, m0, n0); set_rows(ga, m0, p.M); }
+#pragma unroll
+            for (int j = 0; j < C::NLD; ++j) dma(lds_base + own_a + C::A_STAGE + (wq + 4 * j) * 1024, ga[j], p.A + (int64_t)k1 * BK);
+        }
+        set_w(0);
+        fetch_w();
+        fetch_w();
+        // the A stream of the OTHER group's tile: group 0 starts at step 1, group 1 at step 2 (clamped to the last step)
+        int st = grp == 0 ? 1 : 2;
+        a_stage = st % C::NSA;
+        if (st > S - 1) st = S - 1;
+        a_tile = st / nk;
+        a_kt = st - a_tile * nk;
+        set_a(a_tile);
+        wait_vmcnt<0>();
+        wg_barrier();
+    }
+
+    constexpr int SZ = (EPI == EPI_ACC || OUT_DT == DT_F32) ? 4 : 2;
+    constexpr int PW = C::piece_cols(SZ);
+    auto run_epilogue = [&](int ti, int s_last) {
+        int m0, n0;
+        tile_origin(ti, m0, n0);
+        uint8_t* scratch = smem + (s_last % C::NSW) * C::W_STAGE + wave * 4096;
+        epilogue_shuffle<TM, TN, OUT_DT, EPI, PW, true, false>(p, acc, m0 + grp * C::GM, n0 + wq * C::WTN, hw_lane(), scratch);
+    };
+
+    // Both groups run the same loop; group 1 is one phase behind (the barrier in front), multiplies its last step of a
+    // tile in the phase in which group 0 already runs its epilogue, and has nothing to do while group 0 reads the first
+    // fragments of the next tile (the second barrier after its epilogue).
+    if (grp == 1) wg_barrier();
+    int s = 0;
+    for (int ti = 0; ti < nt_b; ++ti) {
+        for (int kt = 0; kt < nk; ++kt, ++s) {
+            memory();
+            wait_lgkmcnt0();
+            wg_barrier();
+            compute(kt == 0);
+            if (grp == 0 || kt + 1 < nk) wg_barrier();
+        }
+        run_epilogue(ti, s - 1);
+        wg_barrier();
+        if (grp == 1 && ti + 1 < nt_b) wg_barrier();
+    }
+    wait_vmcnt<0>();   // no DMA may still be writing this workgroup's LDS when it retires
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -1310,9 +1161,6 @@ __global__ void __launch_bounds__(StreamCfg::NT, 1) int8_gemm_stream_kernel(Gemm
     wg_barrier();   // A(0) and W(0) have landed
 #pragma unroll
     for (int j = 0; j < NF; ++j) f0[j] = frag(smem, smem + C::W_BASE, 0, j);
-#ifdef GEMM_TRACE
-    long long qs[5] = {0, 0, 0, 0, 0};
-#endif
     int ca = 0, cw = 0;   // stages of the iteration being multiplied
     for (int ti = 0; ti < nt_b; ++ti) {
 #pragma unroll
@@ -1373,9 +1221,8 @@ __global__ void __launch_bounds__(256) splitk_epilogue_kernel(GemmArgs p, const 
     }
 }
 
-// Tile shapes.  L: the large-shape workhorse, one workgroup per CU, each of 4 waves owns a 128x128 accumulator tile
-// (256 accumulator registers).  M: 128x128 for mid-size problems and better wave quantization.  S: 64x64 for small M or N.
-using CfgL = Cfg<256, 256, 64, 2, 2, 1>;
+// Tile shapes of the register-staged kernel, the fallback for K % 128 != 0, unaligned outputs and small problems.
+// M: 128x128, two workgroups per CU.  S: 64x64 for small M or N.
 using CfgM = Cfg<128, 128, 64, 2, 2, 2>;
 using CfgS = Cfg<64, 64, 64, 2, 2, 4>;
 
@@ -1427,18 +1274,13 @@ int launch_ring_cfg(GemmArgs a, int slices, hipStream_t st) {
     const int num_cu = device_cu_count();
     const int64_t per_slice = slices > 1 ? (num_cu / slices > 0 ? num_cu / slices : 1) : num_cu;
     const unsigned grid = (unsigned)(ntiles < per_slice ? ntiles : per_slice);
-#ifdef GEMM_TRACE
-    {
-        const char* tp = getenv("GEMM_TRACE_PTR");
-        a.trace = tp ? (long long*)strtoull(tp, nullptr, 0) : nullptr;
-    }
-#endif
     hipLaunchKernelGGL(kern, dim3(grid, (unsigned)slices), dim3(C::NT), C::SMEM, st, a);
     KCHECK();
     return 0;
 }
 
 using RingL = RingCfg<256, 2, 2, 2>;         // 256x256, waves 2x2 of 128x128: the compute-bound workhorse
+using RingL8 = RingCfg<256, 2, 4, 2>;        // 256x256, waves 2x4 of 128x64, two per SIMD
 using RingS = RingCfg<192, 2, 2, 3, 128>;    // 128x192, waves 2x2 of 64x96: re-tiles what the last round of RingL leaves
 
 // Rows [row0, row0 + rows) of the problem as a problem of its own.
@@ -1462,7 +1304,7 @@ template <int OUT_DT, int EPI>
 int launch_ring(GemmArgs a, hipStream_t st) {
     bool vec_ok, aligned;
     epilogue_alignment<OUT_DT, EPI>(a, vec_ok, aligned);
-    if (!aligned) return launch_cfg<CfgL, OUT_DT, EPI>(a, st);   // the ring kernel has only the coalesced epilogue
+    if (!aligned) return launch_cfg<CfgM, OUT_DT, EPI>(a, st);   // the ring kernel has only the coalesced epilogue
     const int64_t G = device_cu_count();
     const int64_t tm = (a.M + RingL::BM - 1) / RingL::BM, tn = (a.N + RingL::BN - 1) / RingL::BN;
     const int64_t full = tm * tn / G, rem = tm * tn % G;
@@ -1479,6 +1321,40 @@ int launch_ring(GemmArgs a, hipStream_t st) {
         }
     }
     return launch_ring_cfg<RingL, OUT_DT, EPI>(a, 1, st);
+}
+
+// The eight-wave 256x256 ring kernel on the whole problem.
+template <int OUT_DT, int EPI>
+int launch_ring8(GemmArgs a, hipStream_t st) {
+    bool vec_ok, aligned;
+    epilogue_alignment<OUT_DT, EPI>(a, vec_ok, aligned);
+    if (!aligned) return launch_cfg<CfgM, OUT_DT, EPI>(a, st);
+    return launch_ring_cfg<RingL8, OUT_DT, EPI>(a, 1, st);
+}
+
+// The two-group 256x256 kernel on the whole problem.
+template <int OUT_DT, int EPI>
+int launch_pp(GemmArgs a, hipStream_t st) {
+    using C = PpCfg;
+    bool vec_ok, aligned;
+    epilogue_alignment<OUT_DT, EPI>(a, vec_ok, aligned);
+    if (!aligned) return launch_cfg<CfgM, OUT_DT, EPI>(a, st);
+    a.tiles_m = (a.M + C::BM - 1) / C::BM;
+    a.tiles_n = (a.N + C::BN - 1) / C::BN;
+    const int64_t ntiles = (int64_t)a.tiles_m * a.tiles_n;
+    if (ntiles > 0x7fffffff) return -1;
+    auto kern = int8_gemm_pp_kernel<OUT_DT, EPI>;
+    static bool once = false;  // benign race: the attribute is idempotent
+    if (!once) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
+        if (e != hipSuccess) return (int)e;
+        once = true;
+    }
+    const int num_cu = device_cu_count();
+    const unsigned grid = (unsigned)(ntiles < num_cu ? ntiles : num_cu);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(C::NT), C::SMEM, st, a);
+    KCHECK();
+    return 0;
 }
 
 // The 128x192 ring kernel on the whole problem: shapes with too few 256x256 tiles to fill the CUs.
@@ -1523,12 +1399,6 @@ int launch_stream(GemmArgs a, int slices, hipStream_t st) {
     const int num_cu = device_cu_count();
     const int64_t per_slice = slices > 1 ? (num_cu / slices > 0 ? num_cu / slices : 1) : num_cu;
     const unsigned grid = (unsigned)(ntiles < per_slice ? ntiles : per_slice);
-#ifdef GEMM_TRACE
-    {
-        const char* tp = getenv("GEMM_TRACE_PTR");
-        a.trace = tp ? (long long*)strtoull(tp, nullptr, 0) : nullptr;
-    }
-#endif
     hipLaunchKernelGGL(kern, dim3(grid, (unsigned)slices), dim3(C::NT), C::SMEM, st, a);
     KCHECK();
     return 0;
@@ -1573,35 +1443,18 @@ int launch_skinny(GemmArgs a, hipStream_t st) {
     return rc;
 }
 
-template <class C, int OUT_DT, int EPI>
-int launch_dma2(GemmArgs a, hipStream_t st) {
-    a.tiles_m = (a.M + C::BM - 1) / C::BM;
-    a.tiles_n = (a.N + C::BN - 1) / C::BN;
-    const int64_t nblocks = (int64_t)a.tiles_m * a.tiles_n;
-    if (nblocks > 0x7fffffff) return -1;
-    auto kern = int8_gemm_dma2_kernel<C, OUT_DT, EPI>;
-    static bool once = false;  // benign race: the attribute is idempotent
-    if (!once) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
-        if (e != hipSuccess) return (int)e;
-        once = true;
-    }
-    hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(C::NT), C::SMEM, st, a);
-    KCHECK();
-    return 0;
-}
-
-// 0 = L, 1 = M, 2 = S; -1 = choose by shape.
-int g_force_cfg = -1;
+// Kernel family forced by the test hook (-1 = choose by shape).  Process-wide and only meant for tests and benchmarks:
+// relaxed atomic, so a concurrent call sees either the old or the new value, never a torn one.
+std::atomic<int> g_force_cfg{-1};
 
 int choose_cfg(int64_t M, int64_t N, int64_t K) {
+    const int force = g_force_cfg.load(std::memory_order_relaxed);
     const bool dma_ok = M * K < ((int64_t)1 << 32) && N * K < ((int64_t)1 << 32);   // 32-bit lane offsets
-    if (!dma_ok && g_force_cfg >= 3) return 0;
-    if (g_force_cfg >= 4) return (K % 128) == 0 ? g_force_cfg : 0;
-    if (g_force_cfg >= 0) return (g_force_cfg == 3 && (K % 64) != 0) ? 0 : g_force_cfg;
+    if (force >= 5 && force <= 9) return (dma_ok && (K % 128) == 0) ? force : 1;
+    if (force == 1 || force == 2) return force;
     if (M <= 256 && N >= 1024 && (K % 128) == 0 && K >= 512 && dma_ok) return 6;
     const int64_t tiles_l = ((M + 255) / 256) * ((N + 255) / 256);
-    if (M >= 512 && N >= 512 && tiles_l >= 192) return !dma_ok ? 0 : (K % 128) == 0 ? 5 : (K % 64) == 0 ? 3 : 0;
+    if (M >= 512 && N >= 512 && tiles_l >= 192) return (dma_ok && (K % 128) == 0) ? 5 : 1;
     // too few 256x256 tiles for the CUs: the persistent kernel on 128x192 tiles, where those fill at least a third of them
     const int64_t tiles_s = ((M + 127) / 128) * ((N + 191) / 192);
     if (dma_ok && (K % 128) == 0 && M > 128 && N >= 192 && tiles_s >= 96) return 7;
@@ -1613,12 +1466,11 @@ int choose_cfg(int64_t M, int64_t N, int64_t K) {
 template <int OUT_DT, int EPI>
 int dispatch_cfg(const GemmArgs& a, hipStream_t st) {
     switch (choose_cfg(a.M, a.N, a.K)) {
-        case 3: return launch_dma<DmaL, OUT_DT, EPI>(a, st);
-        case 4: return launch_dma2<Dma2L, OUT_DT, EPI>(a, st);
         case 5: return launch_ring<OUT_DT, EPI>(a, st);
         case 6: return launch_skinny<OUT_DT, EPI>(a, st);
         case 7: return launch_ring_small<OUT_DT, EPI>(a, st);
-        case 0: return launch_cfg<CfgL, OUT_DT, EPI>(a, st);
+        case 8: return launch_ring8<OUT_DT, EPI>(a, st);
+        case 9: return launch_pp<OUT_DT, EPI>(a, st);
         case 1: return launch_cfg<CfgM, OUT_DT, EPI>(a, st);
         default: return launch_cfg<CfgS, OUT_DT, EPI>(a, st);
     }
@@ -1682,10 +1534,10 @@ GPU_API int gpu_int8_gemm_acc(const int8_t* A, const int8_t* W, int32_t* acc, in
     return rc < 0 ? -200 : rc;
 }
 
-// Test hook: force a kernel family (0 = 256x256, 1 = 128x128, 2 = 64x64 register-staged tiles; 3, 4 = the earlier
-// direct-to-LDS kernels; 5 = persistent ring, 256x256; 6 = weight streaming; 7 = persistent ring, 128x192; -1 = automatic).
+// Test hook: force a kernel family (1 = 128x128, 2 = 64x64 register-staged tiles; 5 = persistent ring, 256x256;
+// 6 = weight streaming; 7 = persistent ring, 128x192; -1 or anything else = automatic).
 GPU_API int gpu_int8_gemm_force_config(int cfg) {
-    g_force_cfg = cfg;
+    g_force_cfg.store(cfg, std::memory_order_relaxed);
     return 0;
 }
 

@@ -645,7 +645,7 @@ ACC_CASES = [(1, 96, 256), (3, 32, 16), (64, 64, 64), (65, 72, 48), (100, 104, 3
              (77, 4096, 1280), (250, 25000, 128)]
 
 
-@pytest.mark.parametrize("cfg", [2, 1, 0, 3, 4, 5, 6, 7])
+@pytest.mark.parametrize("cfg", [2, 1, 5, 6, 7, 8, 9])
 @pytest.mark.parametrize("M,N,K", ACC_CASES)
 def test_int8_gemm_acc_bit_exact(M, N, K, cfg):
     say("gemm_acc", M, N, K, "cfg", cfg)
@@ -712,7 +712,7 @@ def test_int8_gemm_epilogue(M, N, K, with_bias, out_dt):
     bias = tob(synth.normal(2, 5, N) * np.float32(0.02)) if with_bias else None
     want = oracle.int8_gemm(A, W, xs, ws, bias, out_dt, fma=1)
     loose = oracle.int8_gemm(A, W, xs, ws, bias, out_dt, fma=0)
-    for cfg in (-1, 0, 1, 2, 3, 4, 5, 6):
+    for cfg in (-1, 1, 2, 5, 6, 7, 8, 9):
         ffi.raw("gpu_int8_gemm_force_config", cfg)
         try:
             got = ql.int8_gemm(dev(A), dev(W), dev(xs), dev(ws), None if bias is None else dev_bits(bias, out_dt), TDT[out_dt])
@@ -894,7 +894,7 @@ def test_full_size_linear_rows_against_oracle(name, M, K, N, rotate, kind):
     got_rowsum = acc.to(torch.int64).sum(dim=1).cpu().numpy()
     assert np.array_equal(got_rowsum, want_rowsum)
     # every kernel family that can run the shape gives the same bits
-    for cfg in (0, 3, 5) if M > 256 else (6, 1):
+    for cfg in (1, 5, 8, 9) if M > 256 else (6, 1):
         ffi.raw("gpu_int8_gemm_force_config", cfg)
         try:
             d2 = ql.int8_gemm(qd, Wd, xsd, wsd, bd, torch.bfloat16)
