@@ -802,32 +802,37 @@ __global__ void __launch_bounds__(C::NT, 1) int8_gemm_ring_kernel(GemmArgs p) {
 // first memory phase of the next tile (group 1 has nothing to do in it), and the alternation resumes.
 // Requires K % 128 == 0, M*K and N*K < 2^32, and the coalesced epilogue's alignment.
 // ---------------------------------------------------------------------------------------------------------------
+// GM: rows of a group.  128 gives the 256x256 tile (wave tiles 128x64); 64 gives a 128x256 tile (wave tiles 64x64) for
+// the rows a whole number of rounds of the large tile leaves over: half the work per tile, so the last, partly filled
+// round costs half as much, at a step that is bound by its 6 DMA instructions per wave rather than by its 16 MFMAs.
+template <int GM_>
 struct PpCfg {
-    static constexpr int BM = 256, BN = 256, BK = 128, NT = 512, GM = 128;         // GM: rows of a group
-    static constexpr int TM = 4, TN = 2, WTN = 64;                                  // wave tile 128 x 64
+    static constexpr int GM = GM_, BM = 2 * GM, BN = 256, BK = 128, NT = 512;
+    static constexpr int TM = GM / 32, TN = 2, WTN = 64;                            // wave tile GM x 64
     static constexpr int W_STAGE = BN * BK, A_STAGE = GM * BK, NSW = 3, NSA = 2;
     static constexpr int A_BASE = NSW * W_STAGE;                                    // group g's A ring at A_BASE + g*NSA*A_STAGE
     static constexpr int SMEM = NSW * W_STAGE + 2 * NSA * A_STAGE;
-    static constexpr int NLD = 4;                                                   // DMA instructions per wave and 128-row block set
-    static_assert(SMEM <= 160 * 1024, "LDS fits");
+    static constexpr int NLA = GM / 32, NLW = 4;       // DMA instructions per wave for a group's A half / a 128-row W half
+    static_assert(GM % 32 == 0 && SMEM <= 160 * 1024, "tile shape; LDS fits");
     static constexpr int piece_cols(int sz) { return sz == 2 ? 64 : 32; }           // 4 KB shuffle pieces
 };
+using PpL = PpCfg<128>;
+using PpS = PpCfg<64>;
 
-template <int OUT_DT, int EPI>
-__global__ void __launch_bounds__(PpCfg::NT, 1) int8_gemm_pp_kernel(GemmArgs p) {
-    using C = PpCfg;
-    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+// The work of workgroup `bid` of `G` on problem p.
+template <class C, int OUT_DT, int EPI>
+__device__ __forceinline__ void pp_gemm_tiles(const GemmArgs& p, uint8_t* smem, const int bid, const int G) {
     constexpr int BK = C::BK, TM = C::TM, TN = C::TN;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int grp = wave >> 2, wq = wave & 3;            // group; wave within the group = its column quarter
     const int ld = p.K, nk = p.K / BK;
-    const int G = gridDim.x, ntiles = p.tiles_m * p.tiles_n;
-    const int nt_b = (ntiles - (int)blockIdx.x + G - 1) / G;   // tiles of this workgroup: blockIdx, blockIdx + G, ...
+    const int ntiles = p.tiles_m * p.tiles_n;
+    const int nt_b = (ntiles - bid + G - 1) / G;         // tiles of this workgroup: bid, bid + G, ...
     const int S = nt_b * nk;                             // steps of this workgroup
     auto tile_origin = [&](int i, int& m0, int& n0) {
         int tm, tn;
-        tile_of_block((int)blockIdx.x + i * G, ntiles, p.tiles_m, p.tiles_n, tm, tn);
+        tile_of_block(bid + i * G, ntiles, p.tiles_m, p.tiles_n, tm, tn);
         m0 = tm * C::BM;
         n0 = tn * C::BN;
     };
@@ -836,38 +841,38 @@ __global__ void __launch_bounds__(PpCfg::NT, 1) int8_gemm_pp_kernel(GemmArgs p) 
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(off), "s"(base) : "memory", "m0");
     };
 
-    // DMA streams of this wave.  A wave fetches 8-row blocks wq, wq + 4, wq + 8, wq + 12 of a 128-row half: of the
-    // OTHER group's A tile and of its own half of the W tile (group 0: rows 0..127, group 1: rows 128..255).
+    // DMA streams of this wave.  A wave fetches 8-row blocks wq, wq + 4, ... of the OTHER group's A rows and of its own
+    // half of the W tile (group 0: rows 0..127, group 1: rows 128..255).
     // Lane offsets carry the chunk swizzle (bits 1..3 of the row) on the global side, as in the ring kernel.
-    uint32_t ga[C::NLD], gw[C::NLD];
+    uint32_t ga[C::NLA], gw[C::NLW];
     // a stream's position: the (tile, k tile) it fetches next and the stage that goes to.  A stream stops on the last step
     // and keeps re-fetching it, into the stage it would have used, which nothing reads again.
     int a_tile, a_kt, a_stage, w_tile = 0, w_kt = 0, w_stage = 0;
-    auto set_rows = [&](uint32_t* g, int origin, int limit) {
+    auto set_rows = [&](uint32_t* g, auto n, int origin, int limit) {
         const int l = hw_lane();
         const int lr = l >> 3, lc = ((l & 7) ^ (((wq & 1) << 2) | (lr >> 1))) * 16;
 #pragma unroll
-        for (int j = 0; j < C::NLD; ++j) {
+        for (int j = 0; j < decltype(n)::value; ++j) {
             const int row = origin + (wq + 4 * j) * 8 + lr;
             g[j] = (uint32_t)(row < limit ? row : limit - 1) * (uint32_t)ld + lc;
         }
     };
-    auto set_a = [&](int tile) { int m0, n0; tile_origin(tile, m0, n0); set_rows(ga, m0 + (grp ^ 1) * C::GM, p.M); };
-    auto set_w = [&](int tile) { int m0, n0; tile_origin(tile, m0, n0); set_rows(gw, n0 + grp * C::GM, p.N); };
+    auto set_a = [&](int tile) { int m0, n0; tile_origin(tile, m0, n0); set_rows(ga, ic<C::NLA>{}, m0 + (grp ^ 1) * C::GM, p.M); };
+    auto set_w = [&](int tile) { int m0, n0; tile_origin(tile, m0, n0); set_rows(gw, ic<C::NLW>{}, n0 + grp * 128, p.N); };
     auto fetch_a = [&]() {
         const int8_t* base = p.A + (int64_t)a_kt * BK;
         const uint32_t dst = lds_base + C::A_BASE + ((grp ^ 1) * C::NSA + a_stage) * C::A_STAGE + wq * 1024;
 #pragma unroll
-        for (int j = 0; j < C::NLD; ++j) dma(dst + j * 4096, ga[j], base);
+        for (int j = 0; j < C::NLA; ++j) dma(dst + j * 4096, ga[j], base);
         a_stage = a_stage == C::NSA - 1 ? 0 : a_stage + 1;
         if (a_tile == nt_b - 1 && a_kt == nk - 1) return;
         if (++a_kt == nk) { a_kt = 0; set_a(++a_tile); }
     };
     auto fetch_w = [&]() {
         const int8_t* base = p.W + (int64_t)w_kt * BK;
-        const uint32_t dst = lds_base + w_stage * C::W_STAGE + grp * C::GM * BK + wq * 1024;
+        const uint32_t dst = lds_base + w_stage * C::W_STAGE + grp * 128 * BK + wq * 1024;
 #pragma unroll
-        for (int j = 0; j < C::NLD; ++j) dma(dst + j * 4096, gw[j], base);
+        for (int j = 0; j < C::NLW; ++j) dma(dst + j * 4096, gw[j], base);
         w_stage = w_stage == C::NSW - 1 ? 0 : w_stage + 1;
         if (w_tile == nt_b - 1 && w_kt == nk - 1) return;
         if (++w_kt == nk) { w_kt = 0; set_w(++w_tile); }
@@ -926,7 +931,7 @@ __global__ void __launch_bounds__(PpCfg::NT, 1) int8_gemm_pp_kernel(GemmArgs p) 
         SCHED_FENCE();
         fetch_a();
         fetch_w();
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * C::NLD) : "memory");   // everything but this phase's own DMA has landed
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(C::NLA + C::NLW) : "memory");   // everything but this phase's own DMA has landed
     };
 
     // prologue: every group fetches its OWN A for step 0 (group 0 also for step 1: group 1's first memory phase fetches
@@ -936,13 +941,13 @@ __global__ void __launch_bounds__(PpCfg::NT, 1) int8_gemm_pp_kernel(GemmArgs p) 
         const int own_a = C::A_BASE + grp * C::NSA * C::A_STAGE;
         const int t1 = (nk == 1 && nt_b > 1) ? 1 : 0, k1 = nk > 1 ? 1 : 0;   // step 1 as (tile, k tile); step 0 again if S == 1
         tile_origin(0, m0, n0);
-        set_rows(ga, m0 + grp * C::GM, p.M);
+        set_rows(ga, ic<C::NLA>{}, m0 + grp * C::GM, p.M);
 #pragma unroll
-        for (int j = 0; j < C::NLD; ++j) dma(lds_base + own_a + (wq + 4 * j) * 1024, ga[j], p.A);
+        for (int j = 0; j < C::NLA; ++j) dma(lds_base + own_a + (wq + 4 * j) * 1024, ga[j], p.A);
         if (grp == 0) {
-            if (t1) { tile_origin(1, m0, n0); set_rows(ga, m0, p.M); }
+            if (t1) { tile_origin(1, m0, n0); set_rows(ga, ic<C::NLA>{}, m0, p.M); }
 #pragma unroll
-            for (int j = 0; j < C::NLD; ++j) dma(lds_base + own_a + C::A_STAGE + (wq + 4 * j) * 1024, ga[j], p.A + (int64_t)k1 * BK);
+            for (int j = 0; j < C::NLA; ++j) dma(lds_base + own_a + C::A_STAGE + (wq + 4 * j) * 1024, ga[j], p.A + (int64_t)k1 * BK);
         }
         set_w(0);
         fetch_w();
@@ -985,6 +990,17 @@ __global__ void __launch_bounds__(PpCfg::NT, 1) int8_gemm_pp_kernel(GemmArgs p) 
         if (grp == 1 && ti + 1 < nt_b) wg_barrier();
     }
     wait_vmcnt<0>();   // no DMA may still be writing this workgroup's LDS when it retires
+}
+
+// Workgroups 0 .. g_main-1 walk the 256x256 tiles of `main`; the rest walk the 128x256 tiles of `rest` (the rows that
+// whole rounds of large tiles leave over, or nothing).  One launch: the hardware starts a workgroup of the second kind
+// on each CU as its workgroup of the first kind retires, with no gap between two launches.
+template <int OUT_DT, int EPI>
+__global__ void __launch_bounds__(PpL::NT, 1) int8_gemm_pp_kernel(GemmArgs main, GemmArgs rest, int g_main) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int bid = (int)blockIdx.x;
+    if (bid < g_main) pp_gemm_tiles<PpL, OUT_DT, EPI>(main, smem, bid, g_main);
+    else pp_gemm_tiles<PpS, OUT_DT, EPI>(rest, smem, bid - g_main, (int)gridDim.x - g_main);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -1296,6 +1312,52 @@ GemmArgs row_band(const GemmArgs& a, int64_t row0, int64_t rows) {
     return b;
 }
 
+// Large shapes on the two-group kernel.  Every CU gets whole 256x256 tiles; when the tile count is not a multiple of the
+// CU count, the last round would keep only some CUs busy for a full tile's time (864 tiles on 256 CUs: 96 busy, 160
+// idle, a sixth of the run).  The tile rows that fill whole rounds are then run as 256x256 tiles and the rows left over
+// as 128x256 tiles by further workgroups of the same launch, when that is estimated to be shorter (a small tile costs
+// about 0.6 of a large one).
+template <int OUT_DT, int EPI>
+int launch_pp(GemmArgs a, hipStream_t st) {
+    bool vec_ok, aligned;
+    epilogue_alignment<OUT_DT, EPI>(a, vec_ok, aligned);
+    if (!aligned) return launch_cfg<CfgM, OUT_DT, EPI>(a, st);   // this kernel has only the coalesced epilogue
+    const int64_t G = device_cu_count();
+    const int64_t tm = (a.M + PpL::BM - 1) / PpL::BM, tn = (a.N + PpL::BN - 1) / PpL::BN;
+    const int64_t full = tm * tn / G, rem = tm * tn % G;
+    GemmArgs main = a, rest = a;
+    int64_t n_main = tm * tn, n_rest = 0;
+    if (full >= 1 && rem > 0 && tm > 1) {
+        int64_t main_rows = full * G / tn;
+        if (main_rows >= tm) main_rows = tm - 1;
+        const int64_t m_main = main_rows * PpL::BM, m_rest = a.M - m_main;
+        const int64_t small = ((m_rest + PpS::BM - 1) / PpS::BM) * tn;
+        const double split_cost = (double)((main_rows * tn + G - 1) / G) + 0.6 * (double)((small + G - 1) / G);
+        if (main_rows > 0 && split_cost < (double)(full + 1) - 0.1) {
+            main = row_band<OUT_DT, EPI>(a, 0, m_main);
+            rest = row_band<OUT_DT, EPI>(a, m_main, m_rest);
+            n_main = main_rows * tn;
+            n_rest = small;
+        }
+    }
+    if (n_main > 0x7fffffff) return -1;
+    main.tiles_m = (main.M + PpL::BM - 1) / PpL::BM;
+    main.tiles_n = (int)tn;
+    rest.tiles_m = (rest.M + PpS::BM - 1) / PpS::BM;
+    rest.tiles_n = (int)tn;
+    const int g_main = (int)(n_main < G ? n_main : G), g_rest = (int)(n_rest < G ? n_rest : G);
+    auto kern = int8_gemm_pp_kernel<OUT_DT, EPI>;
+    static bool once = false;  // benign race: the attribute is idempotent
+    if (!once) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, PpL::SMEM);
+        if (e != hipSuccess) return (int)e;
+        once = true;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)(g_main + g_rest)), dim3(PpL::NT), PpL::SMEM, st, main, rest, g_main);
+    KCHECK();
+    return 0;
+}
+
 // The persistent kernel gives every CU whole 256x256 tiles: when the tile count is not a multiple of the CU count, the
 // last round keeps only some CUs busy for a full tile's time (864 tiles on 256 CUs: 96 busy, 160 idle, a sixth of the
 // launch).  The tile rows that fill whole rounds go to the 256x256 kernel; the rows left over are re-tiled 128x192 and
@@ -1330,31 +1392,6 @@ int launch_ring8(GemmArgs a, hipStream_t st) {
     epilogue_alignment<OUT_DT, EPI>(a, vec_ok, aligned);
     if (!aligned) return launch_cfg<CfgM, OUT_DT, EPI>(a, st);
     return launch_ring_cfg<RingL8, OUT_DT, EPI>(a, 1, st);
-}
-
-// The two-group 256x256 kernel on the whole problem.
-template <int OUT_DT, int EPI>
-int launch_pp(GemmArgs a, hipStream_t st) {
-    using C = PpCfg;
-    bool vec_ok, aligned;
-    epilogue_alignment<OUT_DT, EPI>(a, vec_ok, aligned);
-    if (!aligned) return launch_cfg<CfgM, OUT_DT, EPI>(a, st);
-    a.tiles_m = (a.M + C::BM - 1) / C::BM;
-    a.tiles_n = (a.N + C::BN - 1) / C::BN;
-    const int64_t ntiles = (int64_t)a.tiles_m * a.tiles_n;
-    if (ntiles > 0x7fffffff) return -1;
-    auto kern = int8_gemm_pp_kernel<OUT_DT, EPI>;
-    static bool once = false;  // benign race: the attribute is idempotent
-    if (!once) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
-        if (e != hipSuccess) return (int)e;
-        once = true;
-    }
-    const int num_cu = device_cu_count();
-    const unsigned grid = (unsigned)(ntiles < num_cu ? ntiles : num_cu);
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(C::NT), C::SMEM, st, a);
-    KCHECK();
-    return 0;
 }
 
 // The 128x192 ring kernel on the whole problem: shapes with too few 256x256 tiles to fill the CUs.
@@ -1454,7 +1491,7 @@ int choose_cfg(int64_t M, int64_t N, int64_t K) {
     if (force == 1 || force == 2) return force;
     if (M <= 256 && N >= 1024 && (K % 128) == 0 && K >= 512 && dma_ok) return 6;
     const int64_t tiles_l = ((M + 255) / 256) * ((N + 255) / 256);
-    if (M >= 512 && N >= 512 && tiles_l >= 192) return (dma_ok && (K % 128) == 0) ? 5 : 1;
+    if (M >= 512 && N >= 512 && tiles_l >= 192) return (dma_ok && (K % 128) == 0) ? 9 : 1;
     // too few 256x256 tiles for the CUs: the persistent kernel on 128x192 tiles, where those fill at least a third of them
     const int64_t tiles_s = ((M + 127) / 128) * ((N + 191) / 192);
     if (dma_ok && (K % 128) == 0 && M > 128 && N >= 192 && tiles_s >= 96) return 7;
