@@ -1049,6 +1049,11 @@ __global__ void __launch_bounds__(StreamCfg::NT, 1) int8_gemm_stream_kernel(Gemm
         m0 = tm * C::BM;
         n0 = tn * C::BN;
     };
+    // The K tiles of a slice are walked from a start that differs between the workgroups of an XCD (the int32 sums do
+    // not depend on the order): otherwise all 32 of them ask that XCD's L2 for the same 256 lines of A at the same
+    // moment, and every weight stream sits at the same offset inside its 4 KB-apart rows.
+    const int rot = (int)(((blockIdx.x >> 3) & 31) * (unsigned)nk) >> 5;
+    auto rk = [&](int kt) { return kt + rot < nk ? kt + rot : kt + rot - nk; };
     const uint32_t lds_base = (uint32_t)(uintptr_t)smem;
     const int lrow = lane >> 3;
     auto dma = [&](uint32_t dst, uint32_t off, const int8_t* base) {
@@ -1071,7 +1076,7 @@ __global__ void __launch_bounds__(StreamCfg::NT, 1) int8_gemm_stream_kernel(Gemm
         };
         // blocks [j0, j1) of the stream's current K tile into the current stage
         auto fetch_w = [&](int j0, int j1) {
-            const int8_t* base = p.W + k_lo + (int64_t)w_kt * BK;
+            const int8_t* base = p.W + k_lo + (int64_t)rk(w_kt) * BK;
 #pragma unroll
             for (int j = 0; j < C::W_BLK; ++j)
                 if (j >= j0 && j < j1) dma(lds_base + C::W_BASE + w_stage * C::W_STAGE + j * 1024, gw[j], base);
@@ -1117,7 +1122,7 @@ __global__ void __launch_bounds__(StreamCfg::NT, 1) int8_gemm_stream_kernel(Gemm
             }
         };
         auto fetch_a = [&](int j0, int j1) {
-            const int8_t* base = p.A + k_lo + (int64_t)a_kt * BK;
+            const int8_t* base = p.A + k_lo + (int64_t)rk(a_kt) * BK;
 #pragma unroll
             for (int j = 0; j < C::A_PER; ++j)
                 if (j >= j0 && j < j1 && ap + 3 * j < C::A_BLK) dma(lds_base + a_stage * C::A_STAGE + (ap + 3 * j) * 1024, ga[j], base);
