@@ -7,6 +7,7 @@
 // W rides in src0 and A in src1, which leaves every lane holding runs of four consecutive n for one m: the epilogue
 // stores 8-byte (bf16/f16) or 16-byte (f32) vectors straight from the accumulators.
 #include <atomic>
+#include <cstdio>
 
 #include "common.hpp"
 
@@ -1191,6 +1192,8 @@ __global__ void __launch_bounds__(StreamCfg::NT, 1) int8_gemm_stream_kernel(Gemm
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc[in][im][r] = 0;
         int pa = 0, pw = 0;
+        int m0, n0;
+        tile_origin(ti, m0, n0);
         for (int kt = 0; kt < nk; ++kt) {
             const uint8_t* sa = smem + ca * C::A_STAGE;
             const uint8_t* sw = smem + C::W_BASE + cw * C::W_STAGE;
@@ -1206,8 +1209,6 @@ __global__ void __launch_bounds__(StreamCfg::NT, 1) int8_gemm_stream_kernel(Gemm
             ca = na;
             cw = nw;
         }
-        int m0, n0;
-        tile_origin(ti, m0, n0);
         __syncthreads();   // every wave is done with the stage that becomes the shuffle scratch (8 KB per wave)
         constexpr int SZ = (EPI == EPI_ACC || OUT_DT == DT_F32) ? 4 : 2;
         // (The stage of A(g) is refilled with A(g+3), issued after barrier X of the next iteration: behind this epilogue.)
@@ -1408,6 +1409,40 @@ int launch_ring_small(GemmArgs a, hipStream_t st) {
     return launch_ring_cfg<RingS, OUT_DT, EPI>(a, 1, st);
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// Scratch of the entry point that allocates nothing (gpu_int8_gemm_static): the int32 planes of a split-K run live in
+// this file-scope device array instead of a stream-ordered allocation.  Every GPU the library runs on holds its own
+// copy at its own address until the process ends; the array's name is only a host-side handle, so the device address
+// is looked up once per device and host code uses that pointer from then on.  24 MiB covers every shape the skinny
+// path splits on a GPU with up to 256 CUs: slices * N <= 256 * 96 columns and M <= 256 rows of int32.
+// ---------------------------------------------------------------------------------------------------------------
+constexpr size_t kStaticScratchBytes = (size_t)24 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];   // device address of `scratch` on each device, null until looked up
+
+// Device address of the scratch array on the current device; 0 and a hipError_t / -210 in *rc on failure.
+void* static_scratch(int* rc) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) { *rc = (int)e; return nullptr; }
+    if (dev < 0 || dev >= kMaxDevices) { *rc = -210; return nullptr; }
+    void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!ptr) {
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));   // the current device's copy
+        if (e != hipSuccess || !ptr) { *rc = e != hipSuccess ? (int)e : -210; return nullptr; }
+        g_scratch_ptr[dev].store(ptr, std::memory_order_release);   // every thread finds the same address
+    }
+    *rc = 0;
+    return ptr;
+}
+
+// Set by gpu_int8_gemm_static around its dispatch: split-K planes go to this buffer instead of a stream-ordered
+// allocation.  Thread-local, so calls from other threads through the other entry points are not affected.
+thread_local void* tl_scratch = nullptr;
+thread_local size_t tl_scratch_bytes = 0;
+
 // Keep freed scratch in the device's default pool instead of returning it to the driver at every synchronization, as
 // the reference's runtime layer does at start-up (src/cuda.rs:88-97): otherwise each call that needs scratch pays a
 // fresh allocation.
@@ -1465,10 +1500,21 @@ int launch_skinny(GemmArgs a, hipStream_t st) {
     }
     if (slices <= 1) return launch_stream<OUT_DT, EPI>(a, 1, st);
     const int per = (nk + slices - 1) / slices;
-    retain_pool_memory();
+    const size_t need = (size_t)slices * a.M * a.N * sizeof(int);
     int* planes = nullptr;
-    hipError_t e = hipMallocAsync((void**)&planes, (size_t)slices * a.M * a.N * sizeof(int), st);
-    if (e != hipSuccess) return (int)e;
+    const bool own = tl_scratch == nullptr;
+    if (own) {
+        retain_pool_memory();
+        hipError_t e = hipMallocAsync((void**)&planes, need, st);
+        if (e != hipSuccess) return (int)e;
+    } else {
+        if (need > tl_scratch_bytes) {
+            fprintf(stderr, "gpu_int8_gemm_static: M=%d N=%d K=%d needs %zu bytes of split-K scratch, the static buffer has %zu\n",
+                    a.M, a.N, a.K, need, tl_scratch_bytes);
+            return -210;
+        }
+        planes = (int*)tl_scratch;   // every plane element is written before it is read: nothing to clear
+    }
     GemmArgs pa = a;
     pa.D = planes;
     pa.kslice = per * 128;
@@ -1480,8 +1526,10 @@ int launch_skinny(GemmArgs a, hipStream_t st) {
         hipError_t le = hipGetLastError();
         if (le != hipSuccess) rc = (int)le;
     }
-    e = hipFreeAsync(planes, st);
-    if (rc == 0 && e != hipSuccess) rc = (int)e;
+    if (own) {
+        hipError_t e = hipFreeAsync(planes, st);
+        if (rc == 0 && e != hipSuccess) rc = (int)e;
+    }
     return rc;
 }
 
@@ -1567,6 +1615,24 @@ GPU_API int gpu_int8_gemm_residual(const int8_t* A, const int8_t* W, const float
     const int rc = dispatch_dt<EPI_RESID>(a, out_dt, (hipStream_t)stream);
     return rc < 0 ? -201 : rc;
 }
+
+GPU_API int gpu_int8_gemm_static(const int8_t* A, const int8_t* W, const float* xs, const float* ws, const void* bias, void* D,
+                                 int64_t M, int64_t N, int64_t K, int out_dt, void* stream) {
+    if (M == 0 || N == 0 || K == 0) return 0;
+    if (out_dt < DT_F32 || out_dt > DT_BF16 || M < 0 || N < 0 || K < 0 || !shape_ok(M, N, K)) return -200;
+    int rc = 0;
+    void* ptr = static_scratch(&rc);
+    if (!ptr) return rc;
+    GemmArgs a{A, W, xs, ws, bias, nullptr, nullptr, D, (int)M, (int)N, (int)K, 0, 0, 0};
+    tl_scratch = ptr;
+    tl_scratch_bytes = kStaticScratchBytes;
+    rc = dispatch_dt<EPI_PLAIN>(a, out_dt, (hipStream_t)stream);
+    tl_scratch = nullptr;
+    tl_scratch_bytes = 0;
+    return rc == -210 ? -210 : rc < 0 ? -200 : rc;
+}
+
+GPU_API int64_t gpu_int8_gemm_static_limit(void) { return (int64_t)kStaticScratchBytes; }
 
 GPU_API int gpu_int8_gemm_acc(const int8_t* A, const int8_t* W, int32_t* acc, int64_t M, int64_t N, int64_t K, void* stream) {
     if (M == 0 || N == 0 || K == 0) return 0;

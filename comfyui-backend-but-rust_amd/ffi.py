@@ -37,6 +37,7 @@ SIGNATURES = {
     "gpu_int8_gemm_residual": [_P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I32, _P],
     "gpu_w6_decode": [_P, _P, _P, _I64, _I32, _I32, _P],
     "gpu_int8_gemm_acc": [_P, _P, _P, _I64, _I64, _I64, _P],
+    "gpu_int8_gemm_static": [_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I32, _P],
     "gpu_w6a8_gemm": [_P, _P, _P, _I32, _P, _P, _P, _P, _I64, _I64, _I64, _I32, _P],
     "gpu_w6a8_group_gemm": [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I32, _P],
     "gpu_int8_attn_d": [_P, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _I32, _I32] + [_I64] * 12 + [_F32, _P],
@@ -63,6 +64,8 @@ def _load():
     lib.gpu_int8_attn_workspace_d.restype = _I64
     lib.gpu_int8_attn_workspace.argtypes = [_I32] * 5
     lib.gpu_int8_attn_workspace.restype = _I64
+    lib.gpu_int8_gemm_static_limit.argtypes = []
+    lib.gpu_int8_gemm_static_limit.restype = _I64
     lib.gpu_kernels_build_info.restype = C.c_char_p
     lib.gpu_kernels_build_info.argtypes = []
     return lib

@@ -178,6 +178,18 @@ int gpu_w6_decode(const void* q, const void* s_rel, void* out, int64_t N, int K,
 /* The int32 accumulators of gpu_int8_gemm, before the epilogue: acc[M,N] = A . W^T.  For bit-exact checks. */
 int gpu_int8_gemm_acc(const int8_t* A, const int8_t* W, int32_t* acc, int64_t M, int64_t N, int64_t K, void* stream);
 
+/* gpu_int8_gemm for callers that cannot allocate device memory (code under HIP graph capture, serving loops and
+ * harnesses that forbid hipMalloc): same arguments, same results bit for bit, but the int32 planes of a split-K run
+ * (M <= 256 with a narrow N) live in a fixed 24 MiB device array inside the library instead of a stream-ordered
+ * allocation, and the call makes no hipMalloc / hipFree of any kind.  No counterpart in the reference.
+ * Every call on one GPU shares that GPU's array: calls that overlap in time on one GPU (two streams, two threads) race
+ * on it and must be serialized by the caller.  Nothing in the array needs clearing between calls (every plane element
+ * is written before it is read).  A shape whose planes would not fit returns -210 with a message on stderr;
+ * gpu_int8_gemm_static_limit() returns the array's size in bytes.  Other return codes as gpu_int8_gemm. */
+int gpu_int8_gemm_static(const int8_t* A, const int8_t* W, const float* xs, const float* ws, const void* bias, void* D,
+                         int64_t M, int64_t N, int64_t K, int out_dt, void* stream);
+int64_t gpu_int8_gemm_static_limit(void);
+
 /* One W6A8 linear in a single call: gpu_w6_decode into a stream-ordered scratch buffer, then gpu_int8_gemm with
  * ws = s_channel (the call pattern of src/h3.rs:1208-1216,1251).  Returns -1 for K % 32 or G % 16, otherwise as
  * gpu_int8_gemm. */
