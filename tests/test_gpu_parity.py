@@ -755,6 +755,43 @@ def test_int8_gemm_residual_in_place(out_dt):
     assert np.array_equal(host_bits(got2).view(view), want2.view(view))
 
 
+RESID_CASES = [  # (M, N, K, kernel families that can run the shape)
+    (200, 1024, 4096, (-1, 6, 1, 2)),          # skinny: split K, planes summed by the reduce kernel
+    (256, 2400, 1024, (-1, 6, 1)),             # skinny: one K slice, the streaming kernel's own epilogue
+    (600, 768, 512, (-1, 1, 2, 5, 7, 8, 9)),   # tile kernels and every persistent kernel
+]
+
+
+@pytest.mark.parametrize("out_dt", [BF16, F16, F32])
+@pytest.mark.parametrize("M,N,K,cfgs", RESID_CASES)
+def test_int8_gemm_residual_in_place_every_kernel_family(M, N, K, cfgs, out_dt):
+    """gpu_int8_gemm_residual with D aliasing resid (the down-projection pattern of src/dit.rs:592) through every kernel
+    family: the streaming kernel's residual epilogue, the split-K reduce kernel's, the persistent kernels' and the
+    tile kernels', bit-exact against the oracle."""
+    say("gemm_residual", M, N, K, out_dt)
+    A = rand_i8(13, 1, M, K, -127, 127)
+    W = rand_i8(13, 2, N, K, -127, 127)
+    xs = synth.uniform(13, 3, M, 0.005, 0.2)
+    ws = synth.uniform(13, 4, N, 1e-3, 1e-2)
+    tob = {BF16: oracle.bf16_bits, F16: oracle.f16_bits, F32: lambda a: a.astype(np.float32)}[out_dt]
+    bias = tob(synth.normal(13, 5, N) * np.float32(0.02))
+    rscale = tob(synth.normal(13, 6, N))
+    resid = tob(synth.normal(13, 7, M * N).reshape(M, N))
+    want = oracle.int8_gemm_residual(A, W, xs, ws, bias, rscale, resid, out_dt, fma=1)
+    view = np.uint32 if out_dt == F32 else np.uint16
+    Ad, Wd, xsd, wsd = dev(A), dev(W), dev(xs), dev(ws)
+    bd, rsd = dev_bits(bias, out_dt), dev_bits(rscale, out_dt)
+    for cfg in cfgs:
+        x = dev_bits(resid, out_dt)
+        ffi.raw("gpu_int8_gemm_force_config", cfg)
+        try:
+            ql.int8_gemm_residual(Ad, Wd, xsd, wsd, bd, rsd, x, D=x)
+            torch.cuda.synchronize()
+        finally:
+            ffi.raw("gpu_int8_gemm_force_config", -1)
+        assert np.array_equal(host_bits(x).view(view), want.view(view)), cfg
+
+
 def test_config0_end_to_end_matches_golden_fixture():
     g = json.load(open(os.path.join(ROOT, "tests", "golden", "config0_w8a8.json")))
     c = synth.config0(0)
@@ -865,6 +902,10 @@ FULL = [  # (name, M, K, N, rotate, kind)
     ("skinny gate+up", 256, 4096, 24576, 128, "normal"),
     ("skinny down", 256, 12288, 4096, 1, "normal"),
     ("sdxl geglu", 8192, 640, 5120, 0, "normal"),
+    ("dit qkv", 4608, 3072, 9216, 128, "t3"),
+    ("dit out-proj", 4608, 3072, 3072, 128, "t3"),
+    ("sdxl attn proj", 8192, 640, 640, 0, "normal"),
+    ("sdxl down", 8192, 2560, 640, 0, "normal"),
 ]
 
 
@@ -894,7 +935,7 @@ def test_full_size_linear_rows_against_oracle(name, M, K, N, rotate, kind):
     got_rowsum = acc.to(torch.int64).sum(dim=1).cpu().numpy()
     assert np.array_equal(got_rowsum, want_rowsum)
     # every kernel family that can run the shape gives the same bits
-    for cfg in (1, 5, 8, 9) if M > 256 else (6, 1):
+    for cfg in (1, 5, 8, 9) if M > 256 and M * N < 8192 * 5120 else (1,) if M > 256 else (6, 1):
         ffi.raw("gpu_int8_gemm_force_config", cfg)
         try:
             d2 = ql.int8_gemm(qd, Wd, xsd, wsd, bd, torch.bfloat16)
@@ -902,3 +943,68 @@ def test_full_size_linear_rows_against_oracle(name, M, K, N, rotate, kind):
         finally:
             ffi.raw("gpu_int8_gemm_force_config", -1)
         assert torch.equal(d2.view(torch.int16), d.view(torch.int16)), cfg
+
+
+SD_FULL = [("sdxl attn proj", 8192, 640, 640, 64), ("sdxl geglu", 8192, 640, 5120, 64), ("sdxl down", 8192, 2560, 640, 256)]
+
+
+@pytest.mark.parametrize("name,M,K,N,rotate", SD_FULL)
+def test_full_size_sd_linear_rows_against_oracle(name, M, K, N, rotate):
+    """The SD UNet reading of the SDXL-level shapes (src/unet.rs:367-456): fp16 activations through gpu_sd_quant_rows with
+    the widest rotation that divides K, fp16 bias and output.  Quantizer on every row, GEMM on a spread of rows,
+    checksum identity over the whole int32 result."""
+    say("full size sd", name, M, K, N, rotate)
+    xh = oracle.f16_bits(synth.activations(17, M, K, "normal", synth.outlier_columns(17, K, 0.001)))
+    W, ws, bias32 = synth.w8_weights(17, N, K)
+    bias = oracle.f16_bits(bias32)
+    rc, q, xs = oracle.sd_quant_rows(xh, K, rotate)
+    assert rc == 0
+    qd, xsd = ql.sd_quant_rows(dev_bits(xh, F16), rotate)
+    Wd = dev(W)
+    d = ql.int8_gemm(qd, Wd, xsd, dev(ws), dev_bits(bias, F16), torch.float16)
+    acc = ql.int8_gemm_acc(qd, Wd)
+    torch.cuda.synchronize()
+    assert np.array_equal(qd.cpu().numpy(), q) and np.array_equal(xsd.cpu().numpy(), xs)
+    rows = sorted(set([0, 1, 127, 128, 255, M // 2, M - 2, M - 1] + list(range(5, M, 256))))
+    want = oracle.int8_gemm(q[rows], W, xs[rows], ws, bias, F16, fma=1)
+    assert np.array_equal(host_bits(d[torch.tensor(rows, device=DEV)]), want.view(np.uint16))
+    want_rowsum = q.astype(np.int64) @ W.astype(np.int64).sum(axis=0)
+    assert np.array_equal(acc.to(torch.int64).sum(dim=1).cpu().numpy(), want_rowsum)
+
+
+W6G_FULL = [("video-dit ffn up", 8192, 5120, 13824), ("video-dit ffn down", 8192, 13824, 5120)]
+
+
+@pytest.mark.parametrize("name,M,K,N", W6G_FULL)
+def test_full_size_w6a8_group_gemm(name, M, K, N):
+    """The fused-unpack W6A8 kernel at the video-DiT sizes (40 and 108 scale groups, 3456 and 1280 tiles): a spread of
+    rows (one per tile row and the edges) bit-exact against the oracle; every int32 group partial of a 160-row band
+    bit-exact and equal, summed over n, to A[m, group] . sum_n codes[n, group]; outputs of that band equal the full run's."""
+    say("full size w6a8", name, M, K, N)
+    g = torch.Generator().manual_seed(K)
+    A = torch.randint(-127, 128, (M, K), dtype=torch.int8, generator=g).numpy()
+    A[0, :] = -128
+    qv = synth.w6_codes(21, N, K)
+    qv[0, :] = -32
+    packed = oracle.w6_pack_words(qv)
+    xs = synth.uniform(21, 3, M, 0.005, 0.2)
+    sw = synth.w6_group_scales(21, N, K)
+    bias = oracle.bf16_bits(synth.normal(21, 5, N) * np.float32(0.02))
+    Ad, pd, xsd, swd, bd = dev(A), dev(packed), dev(xs), dev(sw), dev_bits(bias, BF16)
+    got = ql.w6a8_group_gemm(Ad, pd, xsd, swd, bd, torch.bfloat16)
+    torch.cuda.synchronize()
+    rows = sorted(set([0, 1, 255, 256, M // 2, M - 1] + list(range(7, M, 256))))
+    rc, want, _ = oracle.w6a8_group_gemm(A[rows], packed, xs[rows], sw, bias, BF16)
+    assert rc == 0
+    assert np.array_equal(host_bits(got[torch.tensor(rows, device=DEV)]), want.view(np.uint16))
+    # a band of rows that straddles a tile boundary, with the partials dumped
+    r0, nr = 3 * 256 - 80, 160
+    band, part = ql.w6a8_group_gemm(Ad[r0:r0 + nr].contiguous(), pd, xsd[r0:r0 + nr].contiguous(), swd, bd, torch.bfloat16, want_partials=True)
+    torch.cuda.synchronize()
+    assert torch.equal(band.view(torch.int16), got[r0:r0 + nr].view(torch.int16))
+    part = part.cpu().numpy().astype(np.int64).reshape(nr, N, K // 128)
+    colsum = qv.astype(np.int64).reshape(N, K // 128, 128).sum(axis=0)             # [group, 128]
+    want_sum = np.einsum("mgk,gk->mg", A[r0:r0 + nr].astype(np.int64).reshape(nr, K // 128, 128), colsum)
+    assert np.array_equal(part.sum(axis=1), want_sum)
+    rc, _, want_part = oracle.w6a8_group_gemm(A[r0:r0 + 4], packed, xs[r0:r0 + 4], sw, bias, BF16, want_partials=True)
+    assert np.array_equal(part[:4].reshape(want_part.shape), want_part)

@@ -109,6 +109,42 @@ def test_fht_association_order_is_left_to_right():
         assert np.array_equal(y.astype(np.float64), want)
 
 
+def _staged_h4(x, strides):
+    """Radix-4 stages over the digits of the index in the given stride order, float32 throughout, every output
+    0.5 * (three adds evaluated left to right) as csrc/common.cuh:99-106 writes them; numpy slices instead of the
+    reference's butterfly index arithmetic."""
+    x = x.astype(np.float32).copy()
+    h = np.float32(0.5)
+    for s in strides:
+        v = x.reshape(-1, 4, s)                                       # digit of this stage in the middle axis
+        x0, x1, x2, x3 = (v[:, j, :].copy() for j in range(4))
+        v[:, 0, :] = h * (((x0 + x1) + x2) - x3)
+        v[:, 1, :] = h * (((x0 + x1) - x2) + x3)
+        v[:, 2, :] = h * (((x0 - x1) + x2) + x3)
+        v[:, 3, :] = h * (((-x0 + x1) + x2) + x3)
+        x = v.reshape(-1)
+    return x
+
+
+def test_fht_stage_order_is_stride_1_first():
+    """Non-dyadic values in every digit position: the stages commute in exact arithmetic but not in float32, so the
+    bits tell the order.  The oracle must equal the hand-staged evaluation with strides 1, 4, 16, 64
+    (csrc/common.cuh:110-126 runs `for s = 1; s < 256; s *= 4`) and must differ from the reversed order."""
+    rng = np.random.default_rng(20251)
+    for g, strides in ((256, (1, 4, 16, 64)), (64, (1, 4, 16))):
+        differs = 0
+        for trial in range(8):
+            x = (rng.normal(0, 1, g) * rng.choice([1e-3, 1.0, 37.0], g) + rng.normal(0, 1e-4, g)).astype(np.float32)
+            y = oracle.fht(x, g)
+            fwd = _staged_h4(x, strides)
+            rev = _staged_h4(x, strides[::-1])
+            assert np.array_equal(y.view(np.uint32), fwd.view(np.uint32)), (g, trial)
+            # both orders are the same transform up to rounding
+            assert np.allclose(fwd, rev, rtol=0, atol=1e-4 * np.abs(x).max())
+            differs += int(not np.array_equal(fwd.view(np.uint32), rev.view(np.uint32)))
+        assert differs == 8, "reversed stage order should change bits on general floats"
+
+
 def test_fht128_is_orthonormal_h2_kron_h64():
     H2 = np.array([[1, 1], [1, -1]], np.float64) / np.sqrt(2.0)
     H = np.kron(H2, kron_h(3))
