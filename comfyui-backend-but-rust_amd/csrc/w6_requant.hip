@@ -154,11 +154,12 @@ GPU_API int gpu_w6_requant(const void* weight, void* packed, void* s_rel, void* 
     if (N <= 0) return 0;
     static bool once = false;   // benign race: the attribute is idempotent
     if (!once) {
-        if (hipFuncSetAttribute((const void*)w6_requant_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxDynamic) != hipSuccess)
-            return -2;
+        const hipError_t e = hipFuncSetAttribute((const void*)w6_requant_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxDynamic);
+        if (e != hipSuccess) return (int)e;
         once = true;
     }
     hipLaunchKernelGGL(w6_requant_kernel, dim3((unsigned)N), dim3(256), smem, (hipStream_t)stream, (const uint16_t*)weight,
                        (uint8_t*)packed, (uint8_t*)s_rel, (float*)s_channel, K, seed);
-    return hipGetLastError() == hipSuccess ? 0 : -3;
+    KCHECK();
+    return 0;
 }
