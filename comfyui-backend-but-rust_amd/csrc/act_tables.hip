@@ -24,21 +24,25 @@ __global__ void __launch_bounds__(256) fill_tables_kernel(uint16_t* h16, float* 
 constexpr int kMaxDevices = 16;
 std::mutex g_mu;
 ActTables g_tables[kMaxDevices];
-int g_state[kMaxDevices];   // 0 not tried, 1 built, -1 failed
+int g_state[kMaxDevices];   // 0 not built (yet), 1 built
 
 }  // namespace
 
-const ActTables* act_tables() {
+const ActTables* act_tables(hipStream_t stream) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
     std::lock_guard<std::mutex> hold(g_mu);
     if (g_state[dev] == 1) return &g_tables[dev];
-    if (g_state[dev] == -1) return nullptr;
-    g_state[dev] = -1;
+    // Building allocates, launches on the null stream and synchronizes, none of which a stream capture survives: a
+    // call made while `stream` is being captured evaluates per element instead, and a later call builds the tables.
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (stream && (hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone)) return nullptr;
+    // A failure (a transient out-of-memory, say) leaves the state at "not built", so that the next call tries again.
     uint16_t* h16 = nullptr;
     float* f32 = nullptr;
-    if (hipMalloc(&h16, 5 * 65536 * sizeof(uint16_t)) != hipSuccess) return nullptr;
+    if (hipMalloc(&h16, 5 * 65536 * sizeof(uint16_t)) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
     if (hipMalloc(&f32, 2 * 65536 * sizeof(float)) != hipSuccess) {
+        (void)hipGetLastError();
         (void)hipFree(h16);
         return nullptr;
     }
@@ -52,3 +56,6 @@ const ActTables* act_tables() {
     g_state[dev] = 1;
     return &g_tables[dev];
 }
+
+// Explicit warm-up for callers that capture graphs or want the first prologue call to be asynchronous like the rest.
+GPU_API int gpu_act_tables_init(void) { return act_tables(nullptr) ? 0 : -1; }

@@ -169,7 +169,7 @@ template <int DT>
 int dispatch(int prologue, ProArgs p, int M, hipStream_t st, bool b_variant) {
     if (DT == DT_BF16 && M > 0 &&
         (prologue == PRO_GATE || prologue == PRO_SWIGLU || prologue == PRO_SILU || prologue == PRO_GELU || prologue == PRO_GELU_TANH))
-        if (const ActTables* t = act_tables()) p.tab = *t;
+        if (const ActTables* t = act_tables(st)) p.tab = *t;
     switch (prologue) {
         case PRO_PLAIN: return launch<DT, PRO_PLAIN>(p, M, st);
         case PRO_RMS: return b_variant ? -3 : launch<DT, PRO_RMS>(p, M, st);

@@ -415,11 +415,11 @@ int run_quant(QuantArgs a, int g, hipStream_t st) {
 }
 
 // The activation tables, for the prologues that evaluate exp / erf / tanh on a 16-bit row.
-void attach_tables(QuantArgs& a) {
+void attach_tables(QuantArgs& a, hipStream_t st) {
     const int p = a.pro;
     if (p == PRO_GATE || p == PRO_SWIGLU || p == PRO_SITU || p == PRO_SITU_FAST || p == PRO_SILU || p == PRO_GELU || p == PRO_GELU_TANH ||
         p == PRO_SD_GEGLU)
-        if (const ActTables* t = act_tables()) a.tab = *t;
+        if (const ActTables* t = act_tables(st)) a.tab = *t;
 }
 
 int rotate_group(int rotate) { return rotate == 0 ? 0 : (rotate == 64 || rotate == 128) ? rotate : 256; }
@@ -439,7 +439,7 @@ GPU_API int gpu_quant_rows(int dtype, int prologue, const void* x, int64_t x_str
     if (K > 32768) return -2;
     QuantArgs a{x, x_stride, q, scales, nullptr, M, K, 1, 1, 0, prologue, g, g_stride, up_offset, norm_w, nullptr, eps, mod_scale,
                 mod_shift};
-    if (dtype == DT_BF16 && M > 0) attach_tables(a);
+    if (dtype == DT_BF16 && M > 0) attach_tables(a, (hipStream_t)stream);
     return dtype == DT_BF16 ? run_quant<MODE_BF16>(a, grp, (hipStream_t)stream) : run_quant<MODE_F32>(a, grp, (hipStream_t)stream);
 }
 
@@ -484,7 +484,7 @@ int sd_fused(QuantArgs a, int rotate, hipStream_t st) {
     if (a.K <= 0 || (a.K % 16) != 0) return -1;
     if (a.K > 32768) return -2;
     if (a.M <= 0) return 0;
-    attach_tables(a);
+    attach_tables(a, st);
     return run_quant<MODE_SD_F16>(a, rotate, st);
 }
 }  // namespace

@@ -47,6 +47,7 @@ SIGNATURES = {
     "gpu_internal_cvt_pk_u8_probe": [_P, _P, _I32, _P],
     "gpu_internal_attn_layout": [_I32, _I32, _I32, _I32, _I32, _P],
     "gpu_int8_gemm_force_config": [_I32],
+    "gpu_act_tables_init": [],
     "gpu_mfma_layout_probe": [_P, _P],
 }
 

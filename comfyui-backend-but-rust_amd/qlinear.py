@@ -18,12 +18,38 @@ def _ptr(t):
     return 0 if t is None else t.data_ptr()
 
 
+def _dense(*ts):
+    """The kernels read these operands as dense row-major device arrays: a view with other strides would be read as if
+    it were dense and give wrong results without an error, so it is refused here."""
+    for t in ts:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise ValueError("expected a CUDA tensor")
+        if not t.is_contiguous():
+            raise ValueError("expected a contiguous tensor, got strides %s for shape %s" % (t.stride(), tuple(t.shape)))
+
+
+def _rows(t):
+    """Row operands may have a row stride; their last axis must be dense."""
+    if not t.is_cuda or t.dim() != 2 or t.stride(1) != 1:
+        raise ValueError("expected a 2-D CUDA tensor with a dense last axis, got strides %s" % (t.stride(),))
+
+
+def _want(t, dtype, what):
+    if t is not None and t.dtype != dtype:
+        raise ValueError("%s must be %s, got %s" % (what, dtype, t.dtype))
+
+
 def quant_rows(x, rotate=0, K=None, q=None, scales=None):
     """x: [M, x_stride] bf16 or f32 CUDA tensor -> (q int8 [M,K], scales f32 [M])."""
+    _rows(x)
     M, x_stride = x.shape
     K = x_stride if K is None else K
     q = torch.empty((M, K), dtype=torch.int8, device=x.device) if q is None else q
     scales = torch.empty((M,), dtype=torch.float32, device=x.device) if scales is None else scales
+    _dense(q, scales)
+    _want(q, torch.int8, "q"); _want(scales, torch.float32, "scales")
     ffi.k("gpu_quant_rows", _TORCH_DT[x.dtype], ffi.PRO_PLAIN, _ptr(x), x.stride(0), 0, 0, 0, 0, 0.0, 0, 0, _ptr(q),
           _ptr(scales), M, K, rotate, _stream())
     return q, scales
@@ -167,10 +193,20 @@ def rotate_rows_f32(x, K=None, prologue=ffi.PRO_PLAIN, up_offset=0, norm_w=None,
     return out
 
 
+def _gemm_operands(A, W, xs, ws):
+    _dense(A, W, xs, ws)
+    _want(A, torch.int8, "A"); _want(W, torch.int8, "W"); _want(xs, torch.float32, "xs"); _want(ws, torch.float32, "ws")
+    if A.dim() != 2 or W.dim() != 2 or A.shape[1] != W.shape[1]:
+        raise ValueError("A [M,K] and W [N,K] must share K, got %s and %s" % (tuple(A.shape), tuple(W.shape)))
+
+
 def int8_gemm(A, W, xs, ws, bias=None, out_dtype=torch.bfloat16, D=None):
+    _gemm_operands(A, W, xs, ws)
     M, K = A.shape
     N = W.shape[0]
     D = torch.empty((M, N), dtype=out_dtype, device=A.device) if D is None else D
+    _dense(bias, D)
+    _want(bias, out_dtype, "bias"); _want(D, out_dtype, "D")
     ffi.k("gpu_int8_gemm", _ptr(A), _ptr(W), _ptr(xs), _ptr(ws), _ptr(bias), _ptr(D), M, N, K, _TORCH_DT[out_dtype],
           _stream())
     return D
@@ -178,15 +214,21 @@ def int8_gemm(A, W, xs, ws, bias=None, out_dtype=torch.bfloat16, D=None):
 
 def int8_gemm_residual(A, W, xs, ws, bias, rscale, resid, D=None):
     """D = resid + rscale * (...); pass D=resid for the in-place form the DiT block uses."""
+    _gemm_operands(A, W, xs, ws)
     M, K = A.shape
     N = W.shape[0]
     D = torch.empty_like(resid) if D is None else D
+    _dense(bias, rscale, resid, D)
+    for t_, what in ((bias, "bias"), (rscale, "rscale"), (D, "D")):
+        _want(t_, resid.dtype, what)
     ffi.k("gpu_int8_gemm_residual", _ptr(A), _ptr(W), _ptr(xs), _ptr(ws), _ptr(bias), _ptr(rscale), _ptr(resid), _ptr(D),
           M, N, K, _TORCH_DT[resid.dtype], _stream())
     return D
 
 
 def int8_gemm_acc(A, W):
+    _dense(A, W)
+    _want(A, torch.int8, "A"); _want(W, torch.int8, "W")
     M, K = A.shape
     N = W.shape[0]
     acc = torch.empty((M, N), dtype=torch.int32, device=A.device)
@@ -195,6 +237,7 @@ def int8_gemm_acc(A, W):
 
 
 def w6_decode(wq, s_rel, N, K, G):
+    _dense(wq, s_rel)
     out = torch.empty((N, K), dtype=torch.int8, device=wq.device)
     ffi.k("gpu_w6_decode", _ptr(wq), _ptr(s_rel), _ptr(out), N, K, G, _stream())
     return out
@@ -202,6 +245,8 @@ def w6_decode(wq, s_rel, N, K, G):
 
 def w6a8_gemm(A, wq, s_rel, G, xs, s_channel, bias=None, out_dtype=torch.bfloat16):
     """W6A8 linear on already-quantized rows: packed two-plane weights wq [N, 3K/4], e4m3 s_rel [N, K/G], f32 s_channel."""
+    _dense(A, wq, s_rel, xs, s_channel, bias)
+    _want(A, torch.int8, "A"); _want(xs, torch.float32, "xs"); _want(s_channel, torch.float32, "s_channel")
     M, K = A.shape
     N = wq.shape[0]
     D = torch.empty((M, N), dtype=out_dtype, device=A.device)
@@ -213,6 +258,8 @@ def w6a8_gemm(A, wq, s_rel, G, xs, s_channel, bias=None, out_dtype=torch.bfloat1
 def w6a8_group_gemm(A, packed, xs, sw, bias=None, out_dtype=torch.bfloat16, want_partials=False):
     """W6A8 linear on already-quantized rows with the library's own weight format: 24-bit words of four 6-bit codes,
     packed [N, 3K/4], and f32 group scales sw [N, K/128].  Returns D, or (D, partials [M, N, K/128]) on request."""
+    _dense(A, packed, xs, sw, bias)
+    _want(A, torch.int8, "A"); _want(xs, torch.float32, "xs"); _want(sw, torch.float32, "sw")
     M, K = A.shape
     N = packed.shape[0]
     D = torch.empty((M, N), dtype=out_dtype, device=A.device)

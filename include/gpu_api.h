@@ -4,8 +4,10 @@
  * The first block of entry points has the reference's names, argument order and C types, so the reference's Rust
  * declarations (src/ffi.rs) bind to this library unchanged; each prototype cites the declaration it replaces.
  * All pointers are device pointers unless stated; `stream` is a hipStream_t passed as void* (null = default stream).
- * Every call is asynchronous on `stream`, allocates nothing that outlives it, keeps no state between calls and
- * never throws.
+ * Every call is asynchronous on `stream`, allocates nothing that outlives it and never throws.  State kept between
+ * calls: cached device attributes; per device, the lookup tables of the prologue activations (see
+ * gpu_act_tables_init); the kernel family forced by the test hook gpu_int8_gemm_force_config; the static scratch of
+ * gpu_int8_gemm_static.
  *
  * Return convention (src/ffi.rs:336-344, csrc/common.cuh:128): 0 = ok; > 0 = a hipError_t from the launch
  * (hipGetErrorString names it); < 0 = the launcher refused the arguments, with the reference's codes:
@@ -174,6 +176,15 @@ int gpu_w6_decode(const void* q, const void* s_rel, void* out, int64_t N, int K,
 /* ---------------------------------------------------------------------------------------------------------------
  * Additions with no counterpart in the reference.
  * ------------------------------------------------------------------------------------------------------------- */
+
+/* Builds, for the current device, the lookup tables that the prologues GATE / SWIGLU / SILU / GELU / GELU_TANH / SITU and
+ * the SD GEGLU source use on 16-bit rows (all 65536 inputs of each activation, about 1.2 MB, held until the process
+ * ends).  Optional: the first call with such a prologue builds them itself, with two device allocations, a launch on
+ * the null stream and a device synchronization -- unless its stream is being captured, in which case that call
+ * evaluates the activations per element (same bits, slower) and a later call builds the tables.  Call this once at
+ * start-up to keep every quantizer call asynchronous and capturable.  Returns 0, or -1 if the tables could not be
+ * built (calls then evaluate per element, and a later call tries again). */
+int gpu_act_tables_init(void);
 
 /* The int32 accumulators of gpu_int8_gemm, before the epilogue: acc[M,N] = A . W^T.  For bit-exact checks. */
 int gpu_int8_gemm_acc(const int8_t* A, const int8_t* W, int32_t* acc, int64_t M, int64_t N, int64_t K, void* stream);

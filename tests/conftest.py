@@ -20,6 +20,21 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 
 
+def pytest_collection_modifyitems(config, items):
+    """Without a GPU the `gpu` tests are skipped rather than failing in their first device call."""
+    try:
+        import torch
+        have = torch.cuda.is_available()
+    except ImportError:
+        have = False
+    if have:
+        return
+    skip = pytest.mark.skip(reason="needs a GPU")
+    for item in items:
+        if "gpu" in item.keywords:
+            item.add_marker(skip)
+
+
 @pytest.fixture(scope="session")
 def synth():
     return pkg("synth")
