@@ -122,6 +122,70 @@ def time_w6a8(torch, ffi, M, K, N, steps, warmup):
     return e0.elapsed_time(e1) / steps * 1e3
 
 
+def time_w6_reference_format(torch, ffi, M, K, N, steps, warmup):
+    """The reference's own W6 format (two planes + e4m3 scale per 32 + f32 row scale) at an H3 linear's shape:
+    gpu_w6_decode alone, and gpu_w6a8_gemm (decode into a stream-ordered buffer, then the int8 GEMM), in microseconds."""
+    dev = "cuda:0"
+    g = torch.Generator(device=dev).manual_seed(5)
+    wq = torch.randint(0, 256, (N, K // 4 * 3), dtype=torch.uint8, device=dev, generator=g)
+    # e4m3 bytes with exponent field 6..8 and any mantissa: scales in [0.5, 3.75]
+    s_rel = (torch.randint(6, 9, (N, K // 32), device=dev, generator=g) * 8 + torch.randint(0, 8, (N, K // 32), device=dev, generator=g)).to(torch.uint8)
+    s_ch = torch.rand(N, device=dev, generator=g) * 9e-3 + 1e-3
+    A = torch.randint(-127, 128, (M, K), dtype=torch.int8, device=dev, generator=g)
+    xs = torch.rand(M, device=dev, generator=g) * 0.1 + 0.01
+    w8 = torch.empty((N, K), dtype=torch.int8, device=dev)
+    D = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+    st = torch.cuda.current_stream()
+    s = st.cuda_stream
+
+    def timed(fn):
+        for _ in range(warmup):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record(st)
+        for _ in range(steps):
+            fn()
+        e1.record(st)
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps * 1e3
+
+    dec = timed(lambda: ffi.k("gpu_w6_decode", wq.data_ptr(), s_rel.data_ptr(), w8.data_ptr(), N, K, 32, s))
+    lin = timed(lambda: ffi.k("gpu_w6a8_gemm", A.data_ptr(), wq.data_ptr(), s_rel.data_ptr(), 32, xs.data_ptr(), s_ch.data_ptr(), 0,
+                              D.data_ptr(), M, N, K, ffi.DT_BF16, s))
+    return dec, lin
+
+
+def time_mfma_ceiling(torch, ffi):
+    """The matrix pipes alone: four waves per CU issuing nothing but v_mfma_i32_32x32x32_i8 on register operands, with
+    pseudo-random and with all-zero bits.  The chip's power management sets the clock by what the operands toggle, so
+    this is the ceiling any int8 GEMM on this part runs under; the kernel's own shader-clock counts give that clock."""
+    dev = "cuda:0"
+    cu = torch.cuda.get_device_properties(0).multi_processor_count
+    cyc = torch.zeros(cu, dtype=torch.int64, device=dev)
+    sink = torch.zeros(1, dtype=torch.int32, device=dev)
+    st = torch.cuda.current_stream()
+    iters, reps = 600, 10
+    out = {"kernel": "gpu_mfma_ceiling_probe: %d workgroups x 4 waves x %d x 64 MFMA" % (cu, iters)}
+    for name, rnd in (("random_bits", 1), ("zero_bits", 0)):
+        run = lambda: ffi.k("gpu_mfma_ceiling_probe", iters, rnd, cyc.data_ptr(), sink.data_ptr(), st.cuda_stream)
+        for _ in range(20):   # the clock takes a few launches to settle
+            run()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record(st)
+        for _ in range(reps):
+            run()
+        e1.record(st)
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / reps
+        ops = cu * 4.0 * iters * 64 * 65536
+        cycles = float(cyc.double().mean().item())
+        out[name] = {"TOPS": round(ops / ms / 1e9, 1), "frac_peak": round(ops / ms / 1e9 / PEAK_INT8_TOPS, 4),
+                     "shader_clock_GHz": round(cycles / (ms * 1e6), 3), "cycles_per_mfma": round(cycles / (iters * 64.0), 2)}
+    return out
+
+
 def time_row_kernels(torch, ffi, steps):
     """The HBM-bound kernels either side of the GEMM, each timed alone with HIP events on the launch stream: name,
     microseconds and algorithmic GB/s (bytes the call must read and write once)."""
@@ -279,7 +343,7 @@ def main():
         "config": {"workload": "image-DiT MLP up-projection W8A8 linear, bf16 activations M=%d K=%d -> N=%d, Hadamard "
                                "block %d, per-channel scales, bf16 bias and output" % (M, K, N, a.rotate),
                    "M": M, "K": K, "N": N, "rotate": a.rotate},
-        "roofline": {"bound": "mfma", "kernel": "int8_gemm_ring_kernel (gpu_int8_gemm: 256x256 tiles for the rows that fill whole rounds + 128x192 tiles for the rest)", "achieved": round(gemm_tops, 2),
+        "roofline": {"bound": "mfma", "kernel": "int8_gemm_pp_kernel (gpu_int8_gemm, one launch: 256x256 tiles for the rows that fill whole rounds, 128x256 tiles for the rest)", "achieved": round(gemm_tops, 2),
                      "peak": PEAK_INT8_TOPS, "unit": "TFLOP/s", "frac": round(gemm_tops / PEAK_INT8_TOPS, 4),
                      "traffic": traffic, "avg_launch_us": round(tg * 1e3, 2),
                      "algorithmic_ops": ops, "algorithmic_bytes": M * K + M * 4 + N * K + N * 4 + N * 2 + M * N * 2},
@@ -318,8 +382,17 @@ def main():
             w6.append({"name": name, "M": m, "K": k, "N": n, "kernel": "gpu_w6a8_group_gemm", "us": round(us, 1),
                        "TOPS": round(2.0 * m * n * k / us / 1e6, 1), "frac_int8_peak": round(2.0 * m * n * k / us / 1e6 / PEAK_INT8_TOPS, 4)})
         out["w6a8"] = w6
+        w6r = []
+        for (name, m, k, n) in (("h3 ffn gate+up", 8192, 5376, 28672), ("h3 ffn down", 8192, 14336, 5376)):
+            dec, lin = time_w6_reference_format(torch, ffi, m, k, n, few, 2)
+            w6r.append({"name": name, "M": m, "K": k, "N": n, "gpu_w6_decode_us": round(dec, 1),
+                        "gpu_w6_decode_GBs": round(n * k * 1.78125 / dec / 1e3, 1),
+                        "gpu_w6a8_gemm_us": round(lin, 1), "TOPS": round(2.0 * m * n * k / lin / 1e6, 1),
+                        "frac_int8_peak": round(2.0 * m * n * k / lin / 1e6 / PEAK_INT8_TOPS, 4)})
+        out["w6_reference_format"] = w6r
         out["row_kernels"] = time_row_kernels(torch, ffi, few)
         out["attention"] = time_attention(torch, ffi, few)
+    out["mfma_ceiling"] = time_mfma_ceiling(torch, ffi)
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(host, M, K, N, a.rotate, a.cpu_seconds)
     print(json.dumps(out))

@@ -1594,6 +1594,45 @@ __global__ void mfma_layout_probe_kernel(int* out) {
     for (int r = 0; r < 16; ++r) out[lane * 16 + r] = di[r] * 32 + dj[r];
 }
 
+// Nothing but v_mfma_i32_32x32x32_i8: four waves per CU, sixteen independent accumulator tiles per wave (the register
+// shape of the GEMM kernels), operands held in registers.  What this loop sustains is the matrix pipes' ceiling under
+// the chip's power management for the given operand bits; the shader-clock count per workgroup gives the clock.
+__global__ void __launch_bounds__(256, 1) mfma_ceiling_kernel(int iters, int random_bits, long long* cycles, int* sink) {
+    const uint32_t tid = threadIdx.x + blockIdx.x * 256u;
+    auto hash = [](uint32_t x) { x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16; return x; };
+    v4i a[4], b[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            a[i][r] = random_bits ? (int)hash(tid * 977u + i * 17u + r) : 0;
+            b[i][r] = random_bits ? (int)hash(tid * 613u + i * 29u + r + 99991u) : 0;
+        }
+    v16i acc[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][r] = 0;
+    const long long t0 = (long long)__builtin_readcyclecounter();
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(b[i >> 2], a[i & 3], acc[i], 0, 0, 0);
+                SCHED_FENCE();
+            }
+    }
+    const long long t1 = (long long)__builtin_readcyclecounter();
+    int s = 0;
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s += acc[i][r];
+    if (s == 0x7fffffff) sink[0] = s;   // keeps the accumulators alive
+    if (threadIdx.x == 0) cycles[blockIdx.x] = t1 - t0;
+}
+
 }  // namespace
 
 GPU_API int gpu_int8_gemm(const int8_t* A, const int8_t* W, const float* xs, const float* ws, const void* bias, void* D,
@@ -1646,6 +1685,14 @@ GPU_API int gpu_int8_gemm_acc(const int8_t* A, const int8_t* W, int32_t* acc, in
 // 6 = weight streaming; 7 = persistent ring, 128x192; -1 or anything else = automatic).
 GPU_API int gpu_int8_gemm_force_config(int cfg) {
     g_force_cfg.store(cfg, std::memory_order_relaxed);
+    return 0;
+}
+
+GPU_API int gpu_mfma_ceiling_probe(int iters, int random_bits, int64_t* cycles, int32_t* sink, void* stream) {
+    if (iters <= 0) return 0;
+    hipLaunchKernelGGL(mfma_ceiling_kernel, dim3((unsigned)device_cu_count()), dim3(256), 0, (hipStream_t)stream, iters, random_bits,
+                       (long long*)cycles, (int*)sink);
+    KCHECK();
     return 0;
 }
 

@@ -49,6 +49,7 @@ SIGNATURES = {
     "gpu_int8_gemm_force_config": [_I32],
     "gpu_act_tables_init": [],
     "gpu_mfma_layout_probe": [_P, _P],
+    "gpu_mfma_ceiling_probe": [_I32, _I32, _P, _P, _P],
 }
 
 
