@@ -1006,27 +1006,32 @@ __global__ void __launch_bounds__(PpL::NT, 1) int8_gemm_pp_kernel(GemmArgs main,
 
 // ---------------------------------------------------------------------------------------------------------------
 // Weight-streaming kernel for skinny M (M <= 256): one row of 256 x 96 tiles, every weight read from HBM exactly once.
-// An iteration of such a tile is short (24 MFMAs per wave) against the 44 DMA instructions that feed it, and a DMA
-// instruction holds its wave's issue port for about 70 cycles: in the ring kernel above, where the MFMA waves issue
-// their own DMA, a skinny launch spends as long issuing loads as multiplying.  Here the roles are split over eight waves:
-//   waves 0-3  multiply (64 x 96 each, MFMA + fragment reads only, no memory instruction in their K loop);
-//   wave  4    streams W: 12 DMA instructions per K tile into a ring of 5 stages, three K tiles ahead;
-//   waves 5-7  stream A (from L2: all CUs read the same 256 rows) into three stages, 10-11 instructions per K tile each.
-// Everybody meets at the ring kernel's two barriers per iteration, X (the stage of iteration g-1 is free) and Y (what
-// iteration g+1 needs has landed; the MFMA waves run three sub-steps before it and one after).  So that no wave makes
-// the others wait at a barrier, each producer splits its instructions between the two phases in the proportion of the
-// MFMA waves' work, three quarters before Y and one quarter after.  The counter a producer waits on retires in
-// order, which is why W has a wave to itself: its wait lets two and three quarter K tiles stay in flight.
+// An iteration of such a tile is short (24 MFMAs per wave, 768 cycles) against the 44 DMA instructions that feed it, and
+// a DMA instruction that hits the L2 keeps its wave busy for about 68 cycles: a wave that multiplies cannot also fetch.
+// The roles are split over twelve waves, three per SIMD:
+//   waves 0-3   multiply (64 x 96 each, MFMA + fragment reads only, no memory instruction in their K loop);
+//   waves 4-5   stream W: 6 DMA instructions per K tile each into a ring of 5 stages, three K tiles ahead;
+//   waves 6-11  stream A (from L2: all CUs read the same 256 rows) into three stages, 5-6 instructions per K tile each.
+// With three A waves (and eight waves in all) the A stream needed 11 x 68 cycles an iteration and set the pace; six keep
+// it near 400.  The price is the register budget of three waves per SIMD (168), which the multiplying waves meet by
+// keeping the epilogue's column constants in LDS.
+// Everybody meets at two barriers per iteration, X (the stage of iteration g-1 is free) and Y (what iteration g+1 needs
+// has landed; the MFMA waves run three sub-steps before it and one after).  Each producer splits its instructions
+// between the two phases roughly in the proportion of the MFMA waves' work.  The counter a producer waits on retires in
+// order, which is why W has waves to itself: their wait lets two and three quarter K tiles stay in flight.
 // Requires K % 128 == 0 and M*K, N*K < 2^32.
 // ---------------------------------------------------------------------------------------------------------------
 struct StreamCfg {
-    static constexpr int BM = 256, BN = 96, BK = 128, NT = 512, NSA = 3, NSW = 5;
+    static constexpr int BM = 256, BN = 96, BK = 128, NSA = 3, NSW = 5;
+    static constexpr int NWW = 2, NAW = 6, NT = 64 * (4 + NWW + NAW);   // W-stream waves, A-stream waves
     static constexpr int WTM = 64, WTN = 96, TM = 2, TN = 3, NM = TM * TN, NF = TM + TN;
     static constexpr int A_STAGE = BM * BK, W_STAGE = BN * BK, W_BASE = NSA * A_STAGE, SMEM = W_BASE + NSW * W_STAGE;
     static constexpr int A_BLK = BM / 8, W_BLK = BN / 8;    // 1 KB DMA blocks (8 rows) per stage
-    static constexpr int A_PER = (A_BLK + 2) / 3;           // per A wave: blocks ap, ap+3, ...
-    static constexpr int A_EARLY = 8, W_EARLY = 9;          // instructions a producer issues before barrier Y
-    static_assert(SMEM <= 160 * 1024 && (NSW - 3) * W_BLK + W_EARLY <= 63, "LDS budget; wait counts are 6-bit fields");
+    static constexpr int A_PER = (A_BLK + NAW - 1) / NAW;   // per A wave: blocks ap, ap + NAW, ...
+    static constexpr int W_PER = W_BLK / NWW;               // per W wave: blocks wp, wp + NWW, ...
+    static constexpr int A_EARLY = (3 * A_PER + 3) / 4, W_EARLY = (3 * W_PER + 3) / 4;   // issued before barrier Y
+    static_assert(W_BLK % NWW == 0 && NWW % 2 == 0, "whole blocks per W wave; block parity = wave parity for the swizzle");
+    static_assert(SMEM <= 160 * 1024 && (NSW - 3) * W_PER + W_EARLY <= 63, "LDS budget; wait counts are 6-bit fields");
 };
 
 template <int OUT_DT, int EPI>
@@ -1060,27 +1065,28 @@ __global__ void __launch_bounds__(StreamCfg::NT, 1) int8_gemm_stream_kernel(Gemm
     auto dma = [&](uint32_t dst, uint32_t off, const int8_t* base) {
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(off), "s"(base) : "memory", "m0");
     };
-
-    if (wave == 4) {
-        // ---- the W stream.  Block j is rows 8j..8j+7 of the tile; chunk swizzle (bits 1..3 of the row) on the global side.
-        uint32_t gw[C::W_BLK];
+    if (wave >= 4 && wave < 4 + C::NWW) {
+        // ---- the W stream: wave 4 + wp takes blocks wp, wp + NWW, ...  Block j is rows 8j..8j+7 of the tile; chunk
+        // swizzle (bits 1..3 of the row) on the global side.
+        const int wp = wave - 4;
+        uint32_t gw[C::W_PER];
         int w_tile = 0, w_kt = 0, w_stage = 0;
         auto set_w = [&](int i) {
             int m0, n0;
             tile_origin(i, m0, n0);
 #pragma unroll
-            for (int j = 0; j < C::W_BLK; ++j) {
-                const int row = j * 8 + lrow;
+            for (int j = 0; j < C::W_PER; ++j) {
+                const int row = (wp + C::NWW * j) * 8 + lrow;
                 const int gr = n0 + row < p.N ? n0 + row : p.N - 1;
-                gw[j] = (uint32_t)gr * (uint32_t)ld + (((lane & 7) ^ (((j & 1) << 2) | (lrow >> 1))) << 4);
+                gw[j] = (uint32_t)gr * (uint32_t)ld + (((lane & 7) ^ (((wp & 1) << 2) | (lrow >> 1))) << 4);
             }
         };
-        // blocks [j0, j1) of the stream's current K tile into the current stage
+        // instructions [j0, j1) of the stream's current K tile into the current stage
         auto fetch_w = [&](int j0, int j1) {
             const int8_t* base = p.W + k_lo + (int64_t)rk(w_kt) * BK;
 #pragma unroll
-            for (int j = 0; j < C::W_BLK; ++j)
-                if (j >= j0 && j < j1) dma(lds_base + C::W_BASE + w_stage * C::W_STAGE + j * 1024, gw[j], base);
+            for (int j = 0; j < C::W_PER; ++j)
+                if (j >= j0 && j < j1) dma(lds_base + C::W_BASE + w_stage * C::W_STAGE + (wp + C::NWW * j) * 1024, gw[j], base);
         };
         auto next_w = [&]() {   // the stream stops on its last K tile and keeps re-fetching it
             w_stage = w_stage == C::NSW - 1 ? 0 : w_stage + 1;
@@ -1089,16 +1095,16 @@ __global__ void __launch_bounds__(StreamCfg::NT, 1) int8_gemm_stream_kernel(Gemm
         };
         set_w(0);
 #pragma unroll
-        for (int i = 0; i < C::NSW - 1; ++i) { fetch_w(0, C::W_BLK); next_w(); }   // W(0) .. W(NSW-2)
-        wait_vmcnt<(C::NSW - 2) * C::W_BLK>();                                     // W(0) has landed
+        for (int i = 0; i < C::NSW - 1; ++i) { fetch_w(0, C::W_PER); next_w(); }   // W(0) .. W(NSW-2)
+        wait_vmcnt<(C::NSW - 2) * C::W_PER>();                                     // W(0) has landed
         wg_barrier();
         for (int ti = 0; ti < nt_b; ++ti) {
             for (int kt = 0; kt < nk; ++kt) {
                 wg_barrier();                                     // X: the stage of iteration g-1 is free
                 fetch_w(0, C::W_EARLY);                           // W(g + NSW - 1), first part
-                wait_vmcnt<(C::NSW - 3) * C::W_BLK + C::W_EARLY>();   // W(g + 1) has landed
+                wait_vmcnt<(C::NSW - 3) * C::W_PER + C::W_EARLY>();   // W(g + 1) has landed
                 wg_barrier();                                     // Y
-                fetch_w(C::W_EARLY, C::W_BLK);
+                fetch_w(C::W_EARLY, C::W_PER);
                 next_w();
             }
             wg_barrier();                                         // in front of the epilogue
@@ -1106,9 +1112,9 @@ __global__ void __launch_bounds__(StreamCfg::NT, 1) int8_gemm_stream_kernel(Gemm
         wait_vmcnt<0>();   // no DMA may still be writing this workgroup's LDS when it retires
         return;
     }
-    if (wave > 4) {
-        // ---- the A stream: wave 5 + ap takes blocks ap, ap + 3, ...
-        const int ap = wave - 5;
+    if (wave >= 4 + C::NWW) {
+        // ---- the A stream: wave 4 + NWW + ap takes blocks ap, ap + NAW, ...
+        const int ap = wave - 4 - C::NWW;
         uint32_t ga[C::A_PER];
         int a_tile = 0, a_kt = 0, a_stage = 0;
         auto set_a = [&](int i) {
@@ -1116,7 +1122,7 @@ __global__ void __launch_bounds__(StreamCfg::NT, 1) int8_gemm_stream_kernel(Gemm
             tile_origin(i, m0, n0);
 #pragma unroll
             for (int j = 0; j < C::A_PER; ++j) {
-                const int b = ap + 3 * j;
+                const int b = ap + C::NAW * j;
                 const int row = (b < C::A_BLK ? b : C::A_BLK - 1) * 8 + lrow;
                 const int gr = m0 + row < p.M ? m0 + row : p.M - 1;
                 ga[j] = (uint32_t)gr * (uint32_t)ld + (((lane & 7) ^ (((b & 1) << 2) | (lrow >> 1))) << 4);
@@ -1126,7 +1132,7 @@ __global__ void __launch_bounds__(StreamCfg::NT, 1) int8_gemm_stream_kernel(Gemm
             const int8_t* base = p.A + k_lo + (int64_t)rk(a_kt) * BK;
 #pragma unroll
             for (int j = 0; j < C::A_PER; ++j)
-                if (j >= j0 && j < j1 && ap + 3 * j < C::A_BLK) dma(lds_base + a_stage * C::A_STAGE + (ap + 3 * j) * 1024, ga[j], base);
+                if (j >= j0 && j < j1 && ap + C::NAW * j < C::A_BLK) dma(lds_base + a_stage * C::A_STAGE + (ap + C::NAW * j) * 1024, ga[j], base);
         };
         auto next_a = [&]() {
             a_stage = a_stage == C::NSA - 1 ? 0 : a_stage + 1;
@@ -1212,7 +1218,9 @@ __global__ void __launch_bounds__(StreamCfg::NT, 1) int8_gemm_stream_kernel(Gemm
         __syncthreads();   // every wave is done with the stage that becomes the shuffle scratch (8 KB per wave)
         constexpr int SZ = (EPI == EPI_ACC || OUT_DT == DT_F32) ? 4 : 2;
         // (The stage of A(g) is refilled with A(g+3), issued after barrier X of the next iteration: behind this epilogue.)
-        epilogue_shuffle<TM, TN, OUT_DT, EPI, 32, true>(p, acc, m0 + wm * C::WTM, n0, lane, smem + pa * C::A_STAGE + wave * 8192);
+        uint8_t* scratch = smem + pa * C::A_STAGE + wave * 8192;   // a 4 KB piece, then the wave's column constants
+        epilogue_shuffle<TM, TN, OUT_DT, EPI, 32, true, true>(p, acc, m0 + wm * C::WTM, n0, lane, scratch, nullptr,
+                                                              reinterpret_cast<float*>(scratch + 4096));
 #pragma unroll
         for (int j = 0; j < NF; ++j) f0[j] = frag(smem + ca * C::A_STAGE, smem + C::W_BASE + cw * C::W_STAGE, 0, j);
     }

@@ -349,18 +349,24 @@ __global__ void __launch_bounds__(512) quant_rows_kernel(QuantArgs p) {
                 } else {
                     t = x / st;
                 }
-                float r;
                 if (SR && (MODE == MODE_BF16 || MODE == MODE_F32)) {   // csrc/kernels.cu:1385-1388
                     const uint64_t key = (uint64_t)(m * (int64_t)p.K + e0 + 4 * i + j) + p.seed;
                     const float noise = (float)(pcg_hash((uint32_t)key ^ (uint32_t)(key >> 32)) >> 8) * 0x1.0p-24f;
-                    r = floorf(MODE == MODE_F32 ? t + noise : bf16_add_once(t, rnd_dt<DT_BF16>(noise)));
+                    const float r = floorf(MODE == MODE_F32 ? t + noise : bf16_add_once(t, rnd_dt<DT_BF16>(noise)));
+                    const int qi = (int)fminf(127.f, fmaxf(-128.f, r));
+                    acc |= ((uint32_t)qi & 0xffu) << (8 * j);
+                } else if (MODE == MODE_F32) {
+                    const int qi = (int)fminf(127.f, fmaxf(-128.f, nearbyintf(t)));
+                    acc |= ((uint32_t)qi & 0xffu) << (8 * j);
                 } else {
-                    r = nearbyintf(t);
+                    // clamp(rint(t), -128, 127) + 128 as one instruction: t is a 16-bit float, so t + 128 is exact
+                    // wherever t has a bit at 2^-16 or above set, and below that both t and t + 128 round to the
+                    // same integer; v_cvt_pk_u8_f32 rounds to nearest even, saturates to 0..255 (NaN to 0, which is
+                    // the -128 that fminf(127, fmaxf(-128, NaN)) gives) and drops the byte into place.
+                    acc = __builtin_amdgcn_cvt_pk_u8_f32(t + 128.f, j, acc);
                 }
-                const int qi = (int)fminf(127.f, fmaxf(-128.f, r));
-                acc |= ((uint32_t)qi & 0xffu) << (8 * j);
             }
-            w[i] = acc;
+            w[i] = (!SR && MODE != MODE_F32) ? acc ^ 0x80808080u : acc;
         }
         *reinterpret_cast<uint4*>(p.q + m * (int64_t)p.K + e0) = make_uint4(w[0], w[1], w[2], w[3]);
     }
