@@ -3,6 +3,7 @@
 // gpu_w6_requant, csrc/vendor/w6a8_requant.cu: same steps and float expressions (cited by line), one workgroup per row.
 // A load-time / LoRA-bake kernel: 1.5 B read + 0.78 B written per weight, bound by its arithmetic, not by HBM.
 #include "common.hpp"
+#include "convrot.hpp"
 
 namespace {
 
@@ -47,41 +48,42 @@ __device__ __forceinline__ int lower_bound(float t, float s, float inv_s) {     
     while (i < 63 && level(i, s) < t) ++i;
     return i;
 }
-__device__ __forceinline__ float h4(int d, float x0, float x1, float x2, float x3) {   // :154-156, csrc/common.cuh:99-106
-    switch (d) {
-        case 0: return 0.5f * (x0 + x1 + x2 - x3);
-        case 1: return 0.5f * (x0 + x1 - x2 + x3);
-        case 2: return 0.5f * (x0 - x1 + x2 + x3);
-        default: return 0.5f * (-x0 + x1 + x2 + x3);
-    }
-}
-
 __global__ void __launch_bounds__(256) w6_requant_kernel(const uint16_t* w, uint8_t* packed, uint8_t* s_rel, float* s_channel, int K,
                                                         uint64_t seed) {
-    extern __shared__ float smem[];
+    extern __shared__ __attribute__((aligned(16))) float smem[];
     __shared__ float red[4];
-    float* row = smem;              // [K]
-    float* gscale = smem + K;       // [K / 32]
+    float* row = smem;                                  // [K]
+    float* gscale = smem + K;                           // [K / 32]
+    float* tiles = smem + K + K / kG;                   // four wave-private rotation tiles, 16-byte aligned (K % 256 == 0)
     const int64_t n = blockIdx.x;
-    const int tid = threadIdx.x;
-    for (int k = tid; k < K; k += 256) row[k] = bf16_to_f(w[n * K + k]);
-    __syncthreads();
-    // ConvRot256: four radix-4 stages (strides 1, 4, 16, 64) per group of 256, :174-206
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // ConvRot256 (:174-206) as the row quantizer does it: a wave per chunk of 1024 values, 16 consecutive values per
+    // lane, strides 1 and 4 inside the lane and one trip through the wave's LDS tile for strides 16 and 64; the
+    // rotated row is kept in the weight dtype (:209-217).
+    for (int c = wave; c * convrot::kChunk < K; c += 4) {
+        const int e0 = c * convrot::kChunk + lane * 16;
+        float v[16];
+        if (e0 < K) {                                   // K % 256 == 0: a lane's 16 values are all in or all out
+            const uint4* src = reinterpret_cast<const uint4*>(w + n * K + e0);
+            const uint4 a = src[0], b = src[1];
+            const uint32_t ww[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
 #pragma unroll
-    for (int stage = 0; stage < 4; ++stage) {
-        const int s = 1 << (2 * stage);
-        for (int b = tid; b < (K >> 2); b += 256) {
-            const int g = b >> 6, r = b & 63;
-            const int i0 = (g << 8) + (r / s) * (s << 2) + (r % s);
-            const float x0 = row[i0], x1 = row[i0 + s], x2 = row[i0 + 2 * s], x3 = row[i0 + 3 * s];
-            row[i0] = h4(0, x0, x1, x2, x3);
-            row[i0 + s] = h4(1, x0, x1, x2, x3);
-            row[i0 + 2 * s] = h4(2, x0, x1, x2, x3);
-            row[i0 + 3 * s] = h4(3, x0, x1, x2, x3);
+            for (int i = 0; i < 8; ++i) {
+                v[2 * i] = u2f(ww[i] << 16);
+                v[2 * i + 1] = u2f(ww[i] & 0xffff0000u);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) v[i] = 0.f;
         }
-        __syncthreads();
+        convrot::rotate_chunk<256>(v, tiles + wave * convrot::kLdsPerWave, lane);
+        if (e0 < K) {
+#pragma unroll
+            for (int i = 0; i < 16; i += 4)
+                *reinterpret_cast<float4*>(row + e0 + i) = make_float4(rnd_dt<DT_BF16>(v[i]), rnd_dt<DT_BF16>(v[i + 1]),
+                                                                       rnd_dt<DT_BF16>(v[i + 2]), rnd_dt<DT_BF16>(v[i + 3]));
+        }
     }
-    for (int k = tid; k < K; k += 256) row[k] = rnd_dt<DT_BF16>(row[k]);          // the rotated row is kept in the weight dtype, :209-217
     __syncthreads();
 
     // phase 1: per-group step by two alternating-least-squares rounds; row maximum of the decoded weight, :94-120
@@ -148,7 +150,7 @@ __global__ void __launch_bounds__(256) w6_requant_kernel(const uint16_t* w, uint
 GPU_API int gpu_w6_requant(const void* weight, void* packed, void* s_rel, void* s_channel, int64_t N, int K, uint64_t seed,
                            void* stream) {
     if (K <= 0 || K % 256) return -1;
-    const size_t smem = (size_t)(K + K / kG) * sizeof(float);
+    const size_t smem = (size_t)(K + K / kG + 4 * convrot::kLdsPerWave) * sizeof(float);
     constexpr size_t kMaxDynamic = 160 * 1024 - 256;   // the kernel also has a few bytes of static LDS
     if (smem > kMaxDynamic || N > 0x7fffffff) return -2;
     if (N <= 0) return 0;
