@@ -35,6 +35,11 @@ struct AttnArgs {
     int64_t q_bs, q_rs, q_hs, k_bs, k_rs, k_hs, v_bs, v_rs, v_hs, o_bs, o_rs, o_hs;
     float sm, sink;
     int vec_ok, in_vec, v_vec, use_anchor;
+    // per-head RMSNorm (+ weight) and RoPE ahead of the quantizers (csrc/kernels.cu:482-540 through
+    // csrc/vendor/sage/quant_qk_int8.cu:160-291): q_norm / k_norm say which of Q and K take it
+    const float *qw, *kw, *rope;   // [128] or null (ones); rope [L][64] x (cos, sin) or null
+    float eps;
+    int q_norm, k_norm, rope_mode;
 };
 
 // fmaxf as the reference's device code uses it: a NaN operand is dropped.
@@ -104,6 +109,94 @@ __device__ __forceinline__ float max8(float m) {
     return fmax_nn(m, lane_xor4(m));
 }
 
+// Sum of squares of one 128-channel row in the order of the reference's warp of 32 lanes (csrc/kernels.cu:497-513,
+// csrc/common.cuh:30-34): lane L accumulates its four channels by fma in index order, then the lanes add pairwise at
+// distances 16, 8, 4, 2, 1.  Lane L owns channels 4L..4L+3, or, with split = rope_mode 2 (with or without a table),
+// channels 2L, 2L+1, 64+2L, 65+2L.  Here eight lanes hold sixteen adjacent channels each (o8 = lane within the eight),
+// so a lane carries four (eight, split) of the reference's lanes; all eight lanes get the sum.
+__device__ __forceinline__ float sumsq128(const float (&v)[16], int o8, bool split) {
+    if (!split) {
+        float s[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            s[i] = v[4 * i] * v[4 * i];
+            s[i] = __builtin_fmaf(v[4 * i + 1], v[4 * i + 1], s[i]);
+            s[i] = __builtin_fmaf(v[4 * i + 2], v[4 * i + 2], s[i]);
+            s[i] = __builtin_fmaf(v[4 * i + 3], v[4 * i + 3], s[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) s[i] += lane_xor4(s[i]);   // distance 16
+#pragma unroll
+        for (int i = 0; i < 4; ++i) s[i] += lane_xor2(s[i]);   // 8
+#pragma unroll
+        for (int i = 0; i < 4; ++i) s[i] += lane_xor1(s[i]);   // 4
+        return (s[0] + s[2]) + (s[1] + s[3]);                   // 2, then 1
+    }
+    // split: the lanes of the low half start each chain (channels 2L, 2L+1), the lanes of the high half finish it
+    float s[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float p = __builtin_fmaf(v[2 * i + 1], v[2 * i + 1], v[2 * i] * v[2 * i]);
+        const float q = lane_xor4(p);
+        s[i] = __builtin_fmaf(v[2 * i + 1], v[2 * i + 1], __builtin_fmaf(v[2 * i], v[2 * i], q));   // meaningful where o8 >= 4
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s[i] += lane_xor2(s[i]);       // distance 16
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s[i] += lane_xor1(s[i]);       // 8
+    const float t = ((s[0] + s[4]) + (s[2] + s[6])) + ((s[1] + s[5]) + (s[3] + s[7]));   // 4, 2, 1
+    const float u = lane_xor4(t);
+    return o8 >= 4 ? t : u;
+}
+
+// The same sum by one thread over a row in memory.
+__device__ inline float sumsq128_serial(const float* x, bool split) {
+    float s[32];
+    for (int l = 0; l < 32; ++l) {
+        const int i0 = split ? 2 * l : 4 * l, i2 = split ? 64 + 2 * l : 4 * l + 2;
+        float t = x[i0] * x[i0];
+        t = __builtin_fmaf(x[i0 + 1], x[i0 + 1], t);
+        t = __builtin_fmaf(x[i2], x[i2], t);
+        s[l] = __builtin_fmaf(x[i2 + 1], x[i2 + 1], t);
+    }
+    for (int o = 16; o > 0; o >>= 1)
+        for (int l = 0; l < o; ++l) s[l] += s[l + o];
+    return s[0];
+}
+
+// Per-head RMSNorm, weight and RoPE of one 128-channel row held by eight lanes (sixteen adjacent channels each), as the
+// reference applies them to q and k ahead of the quantizer (csrc/kernels.cu:482-540, csrc/vendor/sage/quant_qk_int8.cu:
+// 211-278): v = T((v * rstd) * w), rstd = 1/sqrt(mean(v^2) + eps) with the sum in the reference's order (sumsq128);
+// rope mode 1 turns the pairs (2p, 2p+1), mode 2 the pairs (j, j + 64), with (cos, sin) = rope_row[2p], rope_row[2p+1];
+// the result is rounded to bf16 again.  This build's definition of the two parts the reference leaves to its machine:
+// 1/sqrt is correctly rounded (the reference's rsqrtf is an approximation of up to two units in the last place), and
+// c*a - s*b, s*a + c*b contract to one fma each on their first product.  w == nullptr means ones; rope_row == nullptr
+// means no rotation.  All eight lanes must call it.
+__device__ __forceinline__ void norm_rope_row(float (&v)[16], int o8, const float* w, const float* rope_row, float eps, int mode) {
+    const float ss = sumsq128(v, o8, mode == 2);
+    const float rstd = (float)(1.0 / sqrt((double)(ss / 128.f + eps)));
+#pragma unroll
+    for (int e = 0; e < 16; ++e) v[e] = rnd_dt<DT_BF16>(v[e] * rstd * (w ? w[o8 * 16 + e] : 1.f));
+    if (!rope_row) return;
+    if (mode == 1) {
+#pragma unroll
+        for (int e = 0; e < 16; e += 2) {
+            const float c = rope_row[o8 * 16 + e], sn = rope_row[o8 * 16 + e + 1];
+            const float a = v[e], b = v[e + 1];
+            v[e] = rnd_dt<DT_BF16>(__builtin_fmaf(c, a, -(sn * b)));
+            v[e + 1] = rnd_dt<DT_BF16>(__builtin_fmaf(sn, a, c * b));
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const int j = (o8 & 3) * 16 + e;
+            const float c = rope_row[2 * j], sn = rope_row[2 * j + 1];
+            const float other = lane_xor4(v[e]);
+            v[e] = rnd_dt<DT_BF16>(o8 < 4 ? __builtin_fmaf(v[e], c, -(other * sn)) : __builtin_fmaf(v[e], c, other * sn));
+        }
+    }
+}
+
 __device__ __forceinline__ uint4 codes16(const float (&v)[16], float inv) {
     uint32_t w[4] = {0u, 0u, 0u, 0u};
 #pragma unroll
@@ -145,12 +238,49 @@ __device__ __forceinline__ void anchor_body(const AttnArgs& a, const int hi, con
         a.vmax[bh * D + c] = 0u;
         for (int t = 0; t < a.kb; ++t) a.vsum[(bh * a.kb + t) * D + c] = 0;
     }
+    if (a.k_norm) {
+        // the nine sampled keys as the K quantizer will see them: norm_rope_row's arithmetic with a thread per channel
+        __shared__ float rstd9[9];
+        __shared__ float nrm[9][D];
+#pragma unroll
+        for (int i = 0; i < 9; ++i) {
+            const int row = (int)((int64_t)i * (a.lk - 1) / 8);
+            s[i][c] = ld_dt<DT>(a.k, base + (int64_t)row * a.k_rs + c);
+        }
+        __syncthreads();
+        if (tid < 9) rstd9[tid] = (float)(1.0 / sqrt((double)(sumsq128_serial(s[tid], a.rope_mode == 2) / 128.f + a.eps)));
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 9; ++i) nrm[i][c] = rnd_dt<DT_BF16>(s[i][c] * rstd9[i] * (a.kw ? a.kw[c] : 1.f));
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 9; ++i) {
+            float x = nrm[i][c];
+            if (a.rope) {
+                const int row = (int)((int64_t)i * (a.lk - 1) / 8);
+                const float* r = a.rope + (int64_t)row * D;
+                if (a.rope_mode == 1) {
+                    const float cs = r[c & ~1], sn = r[c | 1], other = nrm[i][c ^ 1];
+                    x = rnd_dt<DT_BF16>((c & 1) ? __builtin_fmaf(sn, other, cs * x) : __builtin_fmaf(cs, x, -(sn * other)));
+                } else {
+                    const int j = c & 63;
+                    const float cs = r[2 * j], sn = r[2 * j + 1], other = nrm[i][c ^ 64];
+                    x = rnd_dt<DT_BF16>(c < 64 ? __builtin_fmaf(x, cs, -(other * sn)) : __builtin_fmaf(x, cs, other * sn));
+                }
+            }
+            s[i][c] = x;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 9; ++i) {
+            const int row = (int)((int64_t)i * (a.lk - 1) / 8);
+            s[i][c] = ld_dt<DT>(a.k, base + (int64_t)row * a.k_rs + c);
+        }
+    }
     float e = 0.f, m = 0.f, sum = 0.f;
 #pragma unroll
     for (int i = 0; i < 9; ++i) {
-        const int row = (int)((int64_t)i * (a.lk - 1) / 8);
-        const float x = ld_dt<DT>(a.k, base + (int64_t)row * a.k_rs + c);
-        s[i][c] = x;
+        const float x = s[i][c];
         e = fmaf(x, x, e);
         m = fmax_nn(m, fabsf(x));
         sum += x;
@@ -224,7 +354,9 @@ __device__ __forceinline__ void quant_q_body(const AttnArgs& a, const int hi, co
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const int row = t * 32 + g + 8 * j;
-        ld16_dt<DT>(a.q, base + (int64_t)(row < a.lq ? row : a.lq - 1) * a.q_rs, a.in_vec, v[j]);
+        const int rr = row < a.lq ? row : a.lq - 1;
+        ld16_dt<DT>(a.q, base + (int64_t)rr * a.q_rs, a.in_vec, v[j]);
+        if (a.q_norm) norm_rope_row(v[j], o8, a.qw, a.rope ? a.rope + (int64_t)rr * D : nullptr, a.eps, a.rope_mode);
     }
     float mx = 0.f;
 #pragma unroll
@@ -261,15 +393,19 @@ __device__ __forceinline__ void quant_k_body(const AttnArgs& a, const int hi, co
     float bias[16];
 #pragma unroll
     for (int e = 0; e < 16; ++e) bias[e] = 0.f;
-    if (anchor >= 0) ld16_dt<DT>(a.k, base + (int64_t)anchor * a.k_rs, a.in_vec, bias);
+    if (anchor >= 0) {
+        ld16_dt<DT>(a.k, base + (int64_t)anchor * a.k_rs, a.in_vec, bias);
+        if (a.k_norm) norm_rope_row(bias, o8, a.kw, a.rope ? a.rope + (int64_t)anchor * D : nullptr, a.eps, a.rope_mode);
+    }
     float v[R][16];
     int rt[R];
 #pragma unroll
     for (int j = 0; j < R; ++j) {
         const int i = sub * R + j;                  // index within the group
         rt[j] = (i / 2) * 8 + g * 2 + (i % 2);      // row within the tile
-        const int row = t * CK + rt[j];
-        ld16_dt<DT>(a.k, base + (int64_t)(row < a.lk ? row : a.lk - 1) * a.k_rs, a.in_vec, v[j]);
+        const int row = t * CK + rt[j], rr = row < a.lk ? row : a.lk - 1;
+        ld16_dt<DT>(a.k, base + (int64_t)rr * a.k_rs, a.in_vec, v[j]);
+        if (a.k_norm) norm_rope_row(v[j], o8, a.kw, a.rope ? a.rope + (int64_t)rr * D : nullptr, a.eps, a.rope_mode);
     }
     float mx = 0.f;
 #pragma unroll
@@ -648,11 +784,24 @@ int run(AttnArgs a, hipStream_t st) {
     return hipGetLastError() == hipSuccess ? 0 : -401;
 }
 
+// Per-head RMSNorm and RoPE for q and k, applied on the way into the quantizer (csrc/attn_int8.cu:69-76).  A null kw
+// takes K as it is (csrc/vendor/sage/quant_qk_int8.cu:1264-1268).
+struct QkNorm {
+    const float* qw;
+    const float* kw;
+    const float* rope;
+    float eps;
+    int rope_mode;
+};
+
 int int8_attn(const void* q, const void* k, const void* v, void* o, void* ws, int b, int lq, int lk, int h, int hk, int Dh,
               int64_t q_bs, int64_t q_rs, int64_t q_hs, int64_t k_bs, int64_t k_rs, int64_t k_hs, int64_t v_bs, int64_t v_rs,
-              int64_t v_hs, int64_t o_bs, int64_t o_rs, int64_t o_hs, float scale, int dt, void* stream, float sink = 0.f) {
+              int64_t v_hs, int64_t o_bs, int64_t o_rs, int64_t o_hs, float scale, int dt, void* stream, float sink = 0.f,
+              const QkNorm* norm = nullptr) {
     const char* why = nullptr;
     if (Dh != D) why = "only head dim 128 is built";
+    else if (norm && dt != DT_BF16) why = "fused q/k norm needs bf16 head dim 128";                     // csrc/attn_int8.cu:135
+    else if (norm && (norm->rope_mode < 0 || norm->rope_mode > 2)) why = "rope_mode must be 0, 1 or 2";   // quant_qk_int8.cu:1279
     else if (!q || !k || !v || !o || !ws) why = "null pointer";
     else if (b <= 0 || lq <= 0 || lk <= 0 || h <= 0 || hk <= 0 || h % hk != 0) why = "bad sizes";
     else if (b > 65535 || h > 65535 || lq > (1 << 20) || lk > (1 << 20)) why = "batch, head count or length beyond the grid limits";
@@ -678,6 +827,18 @@ int int8_attn(const void* q, const void* k, const void* v, void* o, void* ws, in
     a.vec_ok = ((o_bs | o_rs | o_hs) % 4 == 0 && ((uintptr_t)o & 7) == 0) ? 1 : 0;
     a.v_vec = ((v_bs | v_rs | v_hs) % 4 == 0 && ((uintptr_t)v & 7) == 0) ? 1 : 0;
     a.in_vec = ((q_bs | q_rs | q_hs | k_bs | k_rs | k_hs) % 4 == 0 && (((uintptr_t)q | (uintptr_t)k) & 7) == 0) ? 1 : 0;
+    a.qw = a.kw = a.rope = nullptr;
+    a.eps = 0.f;
+    a.q_norm = a.k_norm = a.rope_mode = 0;
+    if (norm) {
+        a.qw = norm->qw;
+        a.kw = norm->kw;
+        a.rope = (norm->rope && norm->rope_mode != 0) ? norm->rope : nullptr;
+        a.eps = norm->eps;
+        a.rope_mode = norm->rope_mode;
+        a.q_norm = 1;
+        a.k_norm = norm->kw ? 1 : 0;
+    }
     return dt == DT_F16 ? run<DT_F16>(a, (hipStream_t)stream) : run<DT_BF16>(a, (hipStream_t)stream);
 }
 
@@ -721,13 +882,21 @@ GPU_API int gpu_int8_attn_sink(const void* q, const void* k, const void* v, void
                                int hk, int64_t q_bs, int64_t q_rs, int64_t q_hs, int64_t k_bs, int64_t k_rs, int64_t k_hs,
                                int64_t v_bs, int64_t v_rs, int64_t v_hs, int64_t o_bs, int64_t o_rs, int64_t o_hs, float scale,
                                float sink, const float* qw, float eps, void* stream) {
-    (void)eps;
-    if (qw) {
-        fprintf(stderr, "int8 attention: the fused q norm of the sink form is not built\n");
-        return -400;
-    }
+    const QkNorm norm{qw, nullptr, nullptr, eps, 0};   // a non-null qw normalizes q; k is taken as it is (csrc/attn_int8.cu:198-201)
     return int8_attn(q, k, v, o, ws, b, lq, lk, h, hk, D, q_bs, q_rs, q_hs, k_bs, k_rs, k_hs, v_bs, v_rs, v_hs, o_bs, o_rs,
-                     o_hs, scale, DT_BF16, stream, sink);
+                     o_hs, scale, DT_BF16, stream, sink, qw ? &norm : nullptr);
+}
+
+// gpu_int8_attn with q and k taken through the per-head RMSNorm, weight and RoPE of gpu_qk_norm_rope first, inside the
+// quantizers; q and k in memory are left as they are (csrc/attn_int8.cu:163-174).  Head dim 128, bf16.
+GPU_API int gpu_int8_attn_norm_rope(const void* q, const void* k, const void* v, void* o, void* ws, int b, int lq, int lk,
+                                    int h, int hk, int64_t q_bs, int64_t q_rs, int64_t q_hs, int64_t k_bs, int64_t k_rs,
+                                    int64_t k_hs, int64_t v_bs, int64_t v_rs, int64_t v_hs, int64_t o_bs, int64_t o_rs,
+                                    int64_t o_hs, float scale, const float* qw, const float* kw, float eps,
+                                    const float* rope, int rope_mode, void* stream) {
+    const QkNorm norm{qw, kw, rope, eps, rope_mode};
+    return int8_attn(q, k, v, o, ws, b, lq, lk, h, hk, D, q_bs, q_rs, q_hs, k_bs, k_rs, k_hs, v_bs, v_rs, v_hs, o_bs, o_rs,
+                     o_hs, scale, DT_BF16, stream, 0.f, &norm);
 }
 
 // Test hook: y[i] = v_cvt_pk_u8_f32(x[i]) into byte 0 of zero, so that a test can hold the instruction to
@@ -741,6 +910,25 @@ __global__ void cvt_pk_u8_probe_kernel(const float* x, uint32_t* y, int n) {
 GPU_API int gpu_internal_cvt_pk_u8_probe(const float* x, uint32_t* y, int n, void* stream) {
     if (!x || !y || n <= 0) return -400;
     cvt_pk_u8_probe_kernel<<<dim3((n + 255) / 256), 256, 0, (hipStream_t)stream>>>(x, y, n);
+    return hipGetLastError() == hipSuccess ? 0 : -401;
+}
+
+// Test hook: the sum of squares of rows of 128 floats as the fused norm takes it (eight lanes per row, sumsq128) and as
+// the anchor search takes it (one thread, sumsq128_serial).  out[2 * row] and out[2 * row + 1]; rows a multiple of 8.
+namespace {
+__global__ void __launch_bounds__(64) sumsq_probe_kernel(const float* x, float* out, int split) {
+    const int lane = threadIdx.x, o8 = lane & 7, row = blockIdx.x * 8 + (lane >> 3);
+    float v[16];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) v[e] = x[row * 128 + o8 * 16 + e];
+    const float ss = sumsq128(v, o8, split != 0);
+    if (o8 == (row & 7)) out[2 * row] = ss;          // any of the eight lanes holds it: take a different one per row
+    if (o8 == 0) out[2 * row + 1] = sumsq128_serial(x + row * 128, split != 0);
+}
+}  // namespace
+GPU_API int gpu_internal_attn_sumsq_probe(const float* x, float* out, int rows, int split, void* stream) {
+    if (!x || !out || rows <= 0 || rows % 8) return -400;
+    sumsq_probe_kernel<<<dim3(rows / 8), 64, 0, (hipStream_t)stream>>>(x, out, split);
     return hipGetLastError() == hipSuccess ? 0 : -401;
 }
 

@@ -44,7 +44,9 @@ SIGNATURES = {
     "gpu_int8_attn_f16": [_P, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _I32, _I32] + [_I64] * 12 + [_F32, _P],
     "gpu_int8_attn": [_P, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _I32] + [_I64] * 12 + [_F32, _P],
     "gpu_int8_attn_sink": [_P, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _I32] + [_I64] * 12 + [_F32, _F32, _P, _F32, _P],
+    "gpu_int8_attn_norm_rope": [_P, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _I32] + [_I64] * 12 + [_F32, _P, _P, _F32, _P, _I32, _P],
     "gpu_internal_cvt_pk_u8_probe": [_P, _P, _I32, _P],
+    "gpu_internal_attn_sumsq_probe": [_P, _P, _I32, _I32, _P],
     "gpu_internal_attn_layout": [_I32, _I32, _I32, _I32, _I32, _P],
     "gpu_int8_gemm_force_config": [_I32],
     "gpu_act_tables_init": [],

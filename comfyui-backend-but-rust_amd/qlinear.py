@@ -275,8 +275,35 @@ def linear_w8a8(x, W, ws, bias=None, rotate=0, out_dtype=None):
     return int8_gemm(q, W, xs, ws, bias, x.dtype if out_dtype is None else out_dtype)
 
 
-def int8_attn_sink(q, k, v, scale, sink, ws=None):
-    """int8_attn over the keys given plus `sink` zero keys with zero values (bf16), csrc/attn_int8.cu:193-202."""
+def _f32_vec(t, n, what):
+    if t is None:
+        return None
+    if t.dtype != torch.float32 or not t.is_contiguous() or t.numel() < n:
+        raise ValueError("%s must be contiguous float32 with at least %d elements" % (what, n))
+    return _ptr(t)
+
+
+def int8_attn_norm_rope(q, k, v, scale, qw, kw, eps, rope, rope_mode, ws=None):
+    """int8_attn with per-head RMSNorm (weight qw / kw, float32 [128]) and RoPE (rope float32 [max(lq, lk), 64, 2] of
+    (cos, sin), rope_mode 1 interleaved pairs, 2 split halves, 0 none) applied to q, and to k when kw is given, inside the
+    quantizers; q and k are not written (csrc/attn_int8.cu:163-174, the DiT's call at src/dit.rs:575).  bf16."""
+    b, lq, h, D = q.shape
+    lk, hk = k.shape[1], k.shape[2]
+    assert q.dtype == torch.bfloat16 and D == 128
+    assert q.stride(3) == 1 and k.stride(3) == 1 and v.stride(3) == 1
+    if ws is None:
+        ws = torch.empty((ffi.lib.gpu_int8_attn_workspace(b, h, hk, lq, lk),), dtype=torch.uint8, device=q.device)
+    o = torch.empty((b, lq, h, D), dtype=q.dtype, device=q.device)
+    ffi.k("gpu_int8_attn_norm_rope", _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(ws), b, lq, lk, h, hk, q.stride(0), q.stride(1),
+          q.stride(2), k.stride(0), k.stride(1), k.stride(2), v.stride(0), v.stride(1), v.stride(2), o.stride(0), o.stride(1),
+          o.stride(2), float(scale), _f32_vec(qw, D, "qw"), _f32_vec(kw, D, "kw"), float(eps),
+          _f32_vec(rope, max(lq, lk) * D, "rope"), int(rope_mode), _stream())
+    return o
+
+
+def int8_attn_sink(q, k, v, scale, sink, ws=None, qw=None, eps=0.0):
+    """int8_attn over the keys given plus `sink` zero keys with zero values (bf16), csrc/attn_int8.cu:193-202.  qw
+    (float32 [128]): q is RMS-normalized with that weight first, k taken as it is."""
     b, lq, h, D = q.shape
     lk, hk = k.shape[1], k.shape[2]
     assert q.dtype == torch.bfloat16 and D == 128
@@ -285,7 +312,7 @@ def int8_attn_sink(q, k, v, scale, sink, ws=None):
     o = torch.empty((b, lq, h, D), dtype=q.dtype, device=q.device)
     ffi.k("gpu_int8_attn_sink", _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(ws), b, lq, lk, h, hk, q.stride(0), q.stride(1),
           q.stride(2), k.stride(0), k.stride(1), k.stride(2), v.stride(0), v.stride(1), v.stride(2), o.stride(0), o.stride(1),
-          o.stride(2), float(scale), float(sink), None, 0.0, _stream())
+          o.stride(2), float(scale), float(sink), _f32_vec(qw, D, "qw"), float(eps), _stream())
     return o
 
 

@@ -128,8 +128,15 @@ int gpu_w6_requant(const void* weight, void* packed, void* s_rel, void* s_channe
  * (launch failure), the reference's codes.
  * gpu_int8_attn_sink (csrc/attn_int8.cu:193-202): attention over lk keys plus `sink` more whose keys and values are
  * zero, which count in the softmax denominator only; the K anchor is off so that a zero key's score stays zero; bf16.
- * A non-null qw (q normalized first) is not built: -400.
- * Not built: gpu_int8_attn_norm_rope, gpu_int8_attn_key_bias (csrc/attn_int8.cu:166-191,204-223). */
+ * A non-null qw normalizes q first as gpu_int8_attn_norm_rope does (weight qw, eps, no rotation), k taken as it is.
+ * gpu_int8_attn_norm_rope (csrc/attn_int8.cu:163-174, bound at src/ffi.rs:66-68, called from src/dit.rs:575): per-head
+ * RMSNorm with weight qw [128] (null = ones) and rotary embedding applied to q inside its quantizer, and to k as well
+ * when kw is not null (a null kw leaves k as it is, whatever rope says); q and k in memory are not written.  rope:
+ * f32 [max(lq, lk)][64][2] = (cos, sin) per position and pair, or null; rope_mode 1 rotates channel pairs (2p, 2p+1),
+ * 2 the pairs (j, j + 64), 0 none; other values -400.  bf16 only.  The values the quantizer sees are those
+ * gpu_qk_norm_rope (csrc/kernels.cu:482-540) would have stored, with 1/sqrt correctly rounded where CUDA's rsqrtf
+ * approximates.
+ * Not built: gpu_int8_attn_key_bias (csrc/attn_int8.cu:204-223). */
 int64_t gpu_int8_attn_workspace_d(int b, int h, int hk, int lq, int lk, int head_dim);
 int64_t gpu_int8_attn_workspace(int b, int h, int hk, int lq, int lk);
 int gpu_int8_attn_d(const void* q, const void* k, const void* v, void* o, void* ws, int b, int lq, int lk, int h, int hk,
@@ -148,10 +155,19 @@ int gpu_int8_attn_sink(const void* q, const void* k, const void* v, void* o, voi
                        int64_t q_bs, int64_t q_rs, int64_t q_hs, int64_t k_bs, int64_t k_rs, int64_t k_hs, int64_t v_bs,
                        int64_t v_rs, int64_t v_hs, int64_t o_bs, int64_t o_rs, int64_t o_hs, float scale, float sink,
                        const float* qw, float eps, void* stream);
+int gpu_int8_attn_norm_rope(const void* q, const void* k, const void* v, void* o, void* ws, int b, int lq, int lk, int h,
+                            int hk, int64_t q_bs, int64_t q_rs, int64_t q_hs, int64_t k_bs, int64_t k_rs, int64_t k_hs,
+                            int64_t v_bs, int64_t v_rs, int64_t v_hs, int64_t o_bs, int64_t o_rs, int64_t o_hs, float scale,
+                            const float* qw, const float* kw, float eps, const float* rope, int rope_mode, void* stream);
 
 /* Test hook, no reference counterpart: y[i] = the gfx950 float -> u8 pack conversion of x[i] (byte 0), which the attention
  * kernel's probabilities rely on being round-to-nearest-even with saturation to 0..255. */
 int gpu_internal_cvt_pk_u8_probe(const float* x, uint32_t* y, int n, void* stream);
+
+/* Test hook, no reference counterpart: sums of squares of rows of 128 floats in the order the fused norm of
+ * gpu_int8_attn_norm_rope takes them; out[2r] from the quantizers' eight-lane form, out[2r+1] from the anchor search's
+ * one-thread form; split != 0 is rope_mode 2's lane layout.  rows % 8 == 0. */
+int gpu_internal_attn_sumsq_probe(const float* x, float* out, int rows, int split, void* stream);
 
 /* Test hook, no reference counterpart: byte offsets of the pieces of the attention workspace and its tiling,
  * out[0..9] = qi, ki, qs, ks, vt, vs, anchors, vsum, key tile length, key tiles. */

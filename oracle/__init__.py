@@ -60,6 +60,13 @@ def lib():
         L.orc_set_threads.restype = None; L.orc_set_threads.argtypes = [i32]
         L.orc_attn_rot128.restype = None; L.orc_attn_rot128.argtypes = [vp]
         L.orc_attn_quant_qk.restype = i32
+        L.orc_attn_quant_qk_norm.restype = i32
+        L.orc_attn_quant_qk_norm.argtypes = [i32, vp, vp, i32, i32, i32, i32, i32, i64, i64, i64, i64, i64, i64, i32, i32, vp, vp,
+                                             vp, vp, vp, i32, vp, vp, vp, C.c_float, i32]
+        L.orc_attn_sumsq128.restype = C.c_float
+        L.orc_attn_sumsq128.argtypes = [vp, i32]
+        L.orc_attn_norm_rope_row.restype = None
+        L.orc_attn_norm_rope_row.argtypes = [vp, vp, vp, C.c_float, i32]
         L.orc_attn_quant_qk.argtypes = [i32, vp, vp, i32, i32, i32, i32, i32, i64, i64, i64, i64, i64, i64, i32, i32, vp, vp, vp, vp, vp]
         L.orc_attn_quant_v.restype = i32; L.orc_attn_quant_v.argtypes = [i32, vp, i32, i32, i32, i64, i64, i64, vp, vp]
         L.orc_attn_int8.restype = i32
@@ -343,9 +350,29 @@ def attn_rot128(row):
     return r
 
 
-def attn_quant(dt, q, k, v, use_anchor=True):
+def attn_sumsq128(row, split):
+    """Sum of squares of a 128-channel float32 row in the reference's warp order (split: rope_mode 2's lane layout)."""
+    r = np.ascontiguousarray(row, dtype=np.float32)
+    assert r.shape == (128,)
+    return float(lib().orc_attn_sumsq128(_p(r), 1 if split else 0))
+
+
+def attn_norm_rope_row(row, w, rope_row, eps, rope_mode):
+    """RMSNorm, weight and RoPE of one 128-channel row of bf16 values given as float32; returns the new row."""
+    r = np.ascontiguousarray(row, dtype=np.float32).copy()
+    assert r.shape == (128,)
+    w = None if w is None else np.ascontiguousarray(w, dtype=np.float32)
+    rope_row = None if rope_row is None else np.ascontiguousarray(rope_row, dtype=np.float32)
+    lib().orc_attn_norm_rope_row(_p(r), None if w is None else _p(w), None if rope_row is None else _p(rope_row), float(eps),
+                                 int(rope_mode))
+    return r
+
+
+def attn_quant(dt, q, k, v, use_anchor=True, norm=None):
     """q [b,lq,h,128], k/v [b,lk,hk,128] contiguous (uint16 bits for bf16/f16).  Returns a dict with the int8 tensors
-    in [b,heads,len,128] order, the scales, the anchors and the key tile length."""
+    in [b,heads,len,128] order, the scales, the anchors and the key tile length.  norm = dict(qw, kw, rope, eps,
+    rope_mode): per-head RMSNorm (+ weight, + RoPE from rope [max(lq,lk), 64, 2] float32) of q, and of k when kw is
+    given, ahead of the quantizers."""
     b, lq, h, D = q.shape
     _, lk, hk, _ = k.shape
     assert D == 128 and v.shape == k.shape
@@ -356,21 +383,31 @@ def attn_quant(dt, q, k, v, use_anchor=True):
                ki=np.zeros((b, hk, lk, D), np.int8), ks=np.zeros((b, hk, kb * 4), np.float32),
                anchors=np.zeros((b, hk), np.int32), vi=np.zeros((b, hk, lk, D), np.int8),
                vs=np.zeros((b, hk, D), np.float32))
-    rc = lib().orc_attn_quant_qk(dt, _p(q), _p(k), b, lq, lk, h, hk, lq * h * D, h * D, D, lk * hk * D, hk * D, D, ck,
-                                 1 if use_anchor else 0, _p(out["qi"]), _p(out["qs"]), _p(out["ki"]), _p(out["ks"]),
-                                 _p(out["anchors"]))
-    assert rc == 0
+    if norm is None:
+        rc = lib().orc_attn_quant_qk(dt, _p(q), _p(k), b, lq, lk, h, hk, lq * h * D, h * D, D, lk * hk * D, hk * D, D, ck,
+                                     1 if use_anchor else 0, _p(out["qi"]), _p(out["qs"]), _p(out["ki"]), _p(out["ks"]),
+                                     _p(out["anchors"]))
+    else:
+        f = {n: (None if norm.get(n) is None else np.ascontiguousarray(norm[n], dtype=np.float32)) for n in ("qw", "kw", "rope")}
+        if f["rope"] is not None:
+            assert f["rope"].size >= max(lq, lk) * D
+        pp = {n: (None if a is None else _p(a)) for n, a in f.items()}
+        rc = lib().orc_attn_quant_qk_norm(dt, _p(q), _p(k), b, lq, lk, h, hk, lq * h * D, h * D, D, lk * hk * D, hk * D, D, ck,
+                                          1 if use_anchor else 0, _p(out["qi"]), _p(out["qs"]), _p(out["ki"]), _p(out["ks"]),
+                                          _p(out["anchors"]), 1, pp["qw"], pp["kw"], pp["rope"], float(norm["eps"]),
+                                          int(norm["rope_mode"]))
+    assert rc == 0, rc
     rc = lib().orc_attn_quant_v(dt, _p(v), b, lk, hk, lk * hk * D, hk * D, D, _p(out["vi"]), _p(out["vs"]))
     assert rc == 0
     return out
 
 
-def attn_int8(dt, q, k, v, scale, use_anchor=True, quant=None, sink=0.0):
+def attn_int8(dt, q, k, v, scale, use_anchor=True, quant=None, sink=0.0, norm=None):
     """The whole int8 attention: o [b,lq,h,128] in dtype dt (uint16 bits for bf16/f16).  sink: that many more keys of
     score zero and value zero in the denominator (callers pass use_anchor=False with it, as the reference does)."""
     b, lq, h, D = q.shape
     lk, hk = k.shape[1], k.shape[2]
-    z = quant if quant is not None else attn_quant(dt, q, k, v, use_anchor)
+    z = quant if quant is not None else attn_quant(dt, q, k, v, use_anchor, norm)
     o = np.zeros((b, lq, h, D), np.float32 if dt == F32 else np.uint16)
     rc = lib().orc_attn_int8(dt, _p(z["qi"]), _p(z["ki"]), _p(z["vi"]), _p(z["qs"]), _p(z["ks"]), _p(z["vs"]), b, lq, lk,
                              h, hk, z["ck"], float(scale), float(sink), _p(o), lq * h * D, h * D, D)

@@ -808,15 +808,68 @@ static float attn_tree_sum32(const float* x) {
     return t[0];
 }
 
+/* Per-head RMSNorm, weight and RoPE of a 128-channel row ahead of the quantizers: gpu_qk_norm_rope (csrc/kernels.cu:482-540)
+ * as the INT8 attention applies it in its quantizers (csrc/vendor/sage/quant_qk_int8.cu:160-291), bf16 rows.
+ * v = bf16((v * rstd) * w), rstd = 1/sqrt(mean(v^2) + eps); rope_mode 1 turns the pairs (2p, 2p+1), 2 the pairs
+ * (j, j+64), by (cos, sin) = rope_row[2p], rope_row[2p+1]; the result is rounded to bf16 again.
+ * The sum of squares follows the reference's lane order.  Where the reference depends on its machine this build
+ * defines: a correctly rounded 1/sqrt (CUDA's rsqrtf is an approximation, up to 2 ulp) and c*a - s*b / s*a + c*b
+ * contracted to one fma on their first product.  Against a run of the reference: parity unpinned for those two. */
+typedef struct { const float* w; const float* rope; float eps; int mode; int on; } attn_norm_t;
+
+/* Sum of squares of a 128-channel row in the order of the reference's warp: lane l accumulates its four channels by fma
+ * in order (nvcc contracts ss += v * v), then warp_sum adds lanes at distances 16, 8, 4, 2, 1 (csrc/common.cuh:30-34).
+ * Lane l owns channels 4l..4l+3, or with rope_mode 2 (split, with or without a table) 2l, 2l+1, 64+2l, 65+2l
+ * (csrc/kernels.cu:497-505). */
+ORC_API float orc_attn_sumsq128(const float* v, int split) {
+    float lane[32];
+    for (int l = 0; l < 32; ++l) {
+        const int i0 = split ? 2 * l : 4 * l, i2 = split ? 64 + 2 * l : 4 * l + 2;
+        float t = fmaf(v[i0], v[i0], 0.f);
+        t = fmaf(v[i0 + 1], v[i0 + 1], t);
+        t = fmaf(v[i2], v[i2], t);
+        lane[l] = fmaf(v[i2 + 1], v[i2 + 1], t);
+    }
+    for (int o = 16; o > 0; o >>= 1) {
+        float nx[32];
+        for (int l = 0; l < 32; ++l) nx[l] = lane[l] + lane[l ^ o];
+        memcpy(lane, nx, sizeof nx);
+    }
+    return lane[0];
+}
+
+static void attn_norm_rope_row(float* v, const attn_norm_t* nm, int row) {
+    const float rstd = (float)(1.0 / sqrt((double)(orc_attn_sumsq128(v, nm->mode == 2) / 128.f + nm->eps)));
+    for (int c = 0; c < ATTN_D; ++c) v[c] = rnd_t(ORC_BF16, v[c] * rstd * (nm->w ? nm->w[c] : 1.f));
+    if (!nm->rope || nm->mode == 0) return;
+    const float* r = nm->rope + (int64_t)row * ATTN_D;
+    if (nm->mode == 1) {
+        for (int p = 0; p < 64; ++p) {
+            const float c = r[2 * p], s = r[2 * p + 1], a = v[2 * p], b = v[2 * p + 1];
+            v[2 * p] = rnd_t(ORC_BF16, fmaf(c, a, -(s * b)));
+            v[2 * p + 1] = rnd_t(ORC_BF16, fmaf(s, a, c * b));
+        }
+    } else {
+        for (int j = 0; j < 64; ++j) {
+            const float c = r[2 * j], s = r[2 * j + 1], a = v[j], b = v[j + 64];
+            v[j] = rnd_t(ORC_BF16, fmaf(a, c, -(b * s)));
+            v[j + 64] = rnd_t(ORC_BF16, fmaf(b, c, a * s));
+        }
+    }
+}
+
+/* One row of q or k as the quantizer sees it. */
+static void attn_load_row(int dt, const void* x, int64_t base, int64_t stride_n, int row, const attn_norm_t* nm, float* out) {
+    for (int c = 0; c < ATTN_D; ++c) out[c] = ld_t(dt, x, base + (int64_t)row * stride_n + c);
+    if (nm && nm->on) attn_norm_rope_row(out, nm, row);
+}
+
 /* K anchor for one (batch, head): nine evenly spaced keys, the one closest to their mean, kept only when it lowers
  * the sampled energy without raising the sampled abs-max by more than 12.5 % (quant_qk_int8.cu:591-756, C = 128: one
  * channel per thread, four warps).  The distance 9*s - sum is taken as one fma, nvcc's default contraction. */
-static int attn_detect_anchor(int dt, const void* k, int64_t base, int64_t stride_n, int Lk) {
+static int attn_detect_anchor(int dt, const void* k, int64_t base, int64_t stride_n, int Lk, const attn_norm_t* nm) {
     float s[9][ATTN_D];
-    for (int i = 0; i < 9; ++i) {
-        const int row = (int)((int64_t)i * (Lk - 1) / 8);
-        for (int c = 0; c < ATTN_D; ++c) s[i][c] = ld_t(dt, k, base + (int64_t)row * stride_n + c);
-    }
+    for (int i = 0; i < 9; ++i) attn_load_row(dt, k, base, stride_n, (int)((int64_t)i * (Lk - 1) / 8), nm, s[i]);
     float energy[ATTN_D], amax[ATTN_D], dist[9][ATTN_D];
     for (int c = 0; c < ATTN_D; ++c) {
         float e = 0.f, m = 0.f, sum = 0.f;
@@ -862,15 +915,14 @@ static int attn_detect_anchor(int dt, const void* k, int64_t base, int64_t strid
  * rotated, abs-max over the group, scale = max/127 + 1e-7, codes = rn(v * (1/scale))
  * (quant_qk_int8.cu:296-413 for Q, :422-575 for K). */
 static void attn_quant_group(int dt, const void* x, int64_t base, int64_t stride_n, const int* rows, int n, int L,
-                             const float* bias, int8_t* out, float* scale) {
+                             const float* bias, const attn_norm_t* nm, int8_t* out, float* scale) {
     float buf[32][ATTN_D];
     float mx = 0.f;
     for (int i = 0; i < n; ++i) {
         if (rows[i] >= L) continue;
-        for (int c = 0; c < ATTN_D; ++c) {
-            buf[i][c] = ld_t(dt, x, base + (int64_t)rows[i] * stride_n + c);
-            if (bias) buf[i][c] -= bias[c];
-        }
+        attn_load_row(dt, x, base, stride_n, rows[i], nm, buf[i]);
+        if (bias)
+            for (int c = 0; c < ATTN_D; ++c) buf[i][c] -= bias[c];
         orc_attn_rot128(buf[i]);
         for (int c = 0; c < ATTN_D; ++c) mx = fmax_dev(mx, fabsf(buf[i][c]));
     }
@@ -885,10 +937,14 @@ static void attn_quant_group(int dt, const void* x, int64_t base, int64_t stride
 /* q [b, lq, h, 128], k [b, lk, hk, 128] through element strides (batch, row, head).  qi [b,h,lq,128],
  * qs [b,h,ceil(lq/128)*32] (eight groups per 32 rows: rows r, r+8, r+16, r+24), ki [b,hk,lk,128],
  * ks [b,hk,ceil(lk/ck)*4] (four groups per ck keys: keys with (key % 8) / 2 equal), anchors [b,hk]. */
-ORC_API int orc_attn_quant_qk(int dt, const void* q, const void* k, int b, int lq, int lk, int h, int hk, int64_t q_bs,
-                              int64_t q_rs, int64_t q_hs, int64_t k_bs, int64_t k_rs, int64_t k_hs, int ck, int use_anchor,
-                              int8_t* qi, float* qs, int8_t* ki, float* ks, int32_t* anchors) {
+/* norm != 0: q (always) and k (when kw is not null) go through attn_norm_rope_row first; rope may be null. */
+ORC_API int orc_attn_quant_qk_norm(int dt, const void* q, const void* k, int b, int lq, int lk, int h, int hk, int64_t q_bs,
+                                   int64_t q_rs, int64_t q_hs, int64_t k_bs, int64_t k_rs, int64_t k_hs, int ck, int use_anchor,
+                                   int8_t* qi, float* qs, int8_t* ki, float* ks, int32_t* anchors, int norm, const float* qw,
+                                   const float* kw, const float* rope, float eps, int rope_mode) {
     if (ck != 64 && ck != 128) return -1;
+    if (norm && dt != ORC_BF16) return -400;
+    const attn_norm_t qn = {qw, rope, eps, rope_mode, norm ? 1 : 0}, kn = {kw, rope, eps, rope_mode, (norm && kw) ? 1 : 0};
     const int qg = (lq + 127) / 128 * 4, kb = (lk + ck - 1) / ck;
     for (int bi = 0; bi < b; ++bi)
         for (int hi = 0; hi < h; ++hi)
@@ -897,27 +953,39 @@ ORC_API int orc_attn_quant_qk(int dt, const void* q, const void* k, int b, int l
                     int rows[4];
                     for (int j = 0; j < 4; ++j) rows[j] = t * 32 + g + 8 * j;
                     const int64_t bh = (int64_t)bi * h + hi;
-                    attn_quant_group(dt, q, bi * q_bs + hi * q_hs, q_rs, rows, 4, lq, NULL, qi + bh * lq * ATTN_D,
+                    attn_quant_group(dt, q, bi * q_bs + hi * q_hs, q_rs, rows, 4, lq, NULL, &qn, qi + bh * lq * ATTN_D,
                                      &qs[(bh * qg + t) * 8 + g]);
                 }
     for (int bi = 0; bi < b; ++bi)
         for (int hi = 0; hi < hk; ++hi) {
             const int64_t bh = (int64_t)bi * hk + hi, base = bi * k_bs + hi * k_hs;
-            const int anchor = use_anchor ? attn_detect_anchor(dt, k, base, k_rs, lk) : -1;
+            const int anchor = use_anchor ? attn_detect_anchor(dt, k, base, k_rs, lk, &kn) : -1;
             anchors[bh] = anchor;
             float bias[ATTN_D];
-            if (anchor >= 0)
-                for (int c = 0; c < ATTN_D; ++c) bias[c] = ld_t(dt, k, base + (int64_t)anchor * k_rs + c);
+            if (anchor >= 0) attn_load_row(dt, k, base, k_rs, anchor, &kn, bias);
             for (int t = 0; t < kb; ++t)
                 for (int g = 0; g < 4; ++g) {
                     int rows[32];
                     const int n = ck / 4;
                     for (int i = 0; i < n; ++i) rows[i] = t * ck + (i / 2) * 8 + g * 2 + (i % 2);
-                    attn_quant_group(dt, k, base, k_rs, rows, n, lk, anchor >= 0 ? bias : NULL, ki + bh * lk * ATTN_D,
+                    attn_quant_group(dt, k, base, k_rs, rows, n, lk, anchor >= 0 ? bias : NULL, &kn, ki + bh * lk * ATTN_D,
                                      &ks[(bh * kb + t) * 4 + g]);
                 }
         }
     return 0;
+}
+
+ORC_API int orc_attn_quant_qk(int dt, const void* q, const void* k, int b, int lq, int lk, int h, int hk, int64_t q_bs,
+                              int64_t q_rs, int64_t q_hs, int64_t k_bs, int64_t k_rs, int64_t k_hs, int ck, int use_anchor,
+                              int8_t* qi, float* qs, int8_t* ki, float* ks, int32_t* anchors) {
+    return orc_attn_quant_qk_norm(dt, q, k, b, lq, lk, h, hk, q_bs, q_rs, q_hs, k_bs, k_rs, k_hs, ck, use_anchor, qi, qs, ki, ks,
+                                  anchors, 0, NULL, NULL, NULL, 0.f, 0);
+}
+
+/* The row transform alone, for pins: v[128] float in place. */
+ORC_API void orc_attn_norm_rope_row(float* v, const float* w, const float* rope_row, float eps, int rope_mode) {
+    const attn_norm_t nm = {w, rope_row, eps, rope_mode, 1};
+    attn_norm_rope_row(v, &nm, 0);
 }
 
 /* v [b, lk, hk, 128] -> vi [b,hk,lk,128] (plain order; the reference stores it transposed and permuted for its MMA,

@@ -168,12 +168,172 @@ def test_attention_with_sink_keys(shape):
     cos = float((got * ex).sum() / np.sqrt((got * got).sum() * (ex * ex).sum()))
     assert cos > 0.9995, cos
     assert np.abs(got - ex).max() < 0.03
-    # the fused q norm of this form is not built
-    p = lambda t: C.c_void_p(t.data_ptr())
-    x = torch.zeros(1, 4, 1, 128, dtype=torch.bfloat16, device="cuda")
-    qw = torch.ones(128, device="cuda")
-    assert ffi.raw("gpu_int8_attn_sink", p(x), p(x), p(x), p(x), p(ws), 1, 4, 4, 1, 1, 512, 128, 128, 512, 128, 128, 512, 128,
-                   128, 512, 128, 128, 0.1, 4.0, p(qw), 1e-6, None) == -400
+
+
+def _rope_table(n, seed):
+    """[n, 64, 2] of (cos, sin) at angles that grow with position, as a rotary table does."""
+    g = torch.Generator().manual_seed(seed)
+    freq = torch.exp(-torch.rand(64, generator=g) * 6.0)
+    ang = torch.arange(n, dtype=torch.float32)[:, None] * freq[None, :]
+    return torch.stack([torch.cos(ang), torch.sin(ang)], -1).contiguous()
+
+
+def _norm_rope_f64(x, w, rope, eps, mode):
+    """The transform in float64 with one rounding to bf16 at the end: what the fused stage approximates."""
+    x = x.double()
+    y = x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps)
+    if w is not None:
+        y = y * w.double()
+    if rope is None or mode == 0:
+        return y
+    r = rope[: x.shape[1]].double()[None, :, None]          # [1, l, 1, 64, 2]
+    c, s = r[..., 0], r[..., 1]
+    if mode == 1:
+        a, b2 = y[..., 0::2], y[..., 1::2]
+        return torch.stack([c * a - s * b2, s * a + c * b2], -1).reshape(y.shape)
+    a, b2 = y[..., :64], y[..., 64:]
+    return torch.cat([a * c - b2 * s, b2 * c + a * s], -1)
+
+
+NORM_CASES = [
+    # b, lq, lk, h, hk, rope_mode, rope table, qw, kw, k_offset
+    (1, 150, 210, 2, 1, 1, True, True, True, 0.0),
+    (1, 150, 210, 2, 1, 2, True, True, True, 0.0),
+    (2, 77, 64, 2, 2, 0, False, True, True, 0.0),
+    (1, 65, 100, 2, 2, 2, False, True, True, 0.0),        # rope_mode 2 without a table: its lane order for the sum only
+    (1, 90, 130, 2, 2, 1, True, True, False, 3.0),         # kw null: k untouched (not even rotated), anchor on raw k
+    (1, 64, 1100, 2, 1, 2, True, False, True, 0.0),        # 128-key tiles, qw null (ones)
+    (1, 257, 95, 1, 1, 1, True, True, True, 0.0),
+]
+
+
+@pytest.mark.parametrize("case", NORM_CASES, ids=lambda c: "b%d_lq%d_lk%d_h%d_hk%d_mode%d_rope%d_qw%d_kw%d_off%g" % c)
+def test_attention_with_fused_norm_and_rope(case):
+    """gpu_int8_attn_norm_rope: Q/K codes, scales and anchors bit-exact against the oracle's restatement of the fused
+    stage, outputs within the attention tolerance, and the whole thing close to exact attention over q and k transformed
+    in float64."""
+    ql, ffi = _pkg()
+    b, lq, lk, h, hk, mode, has_rope, has_qw, has_kw, off = case
+    q, k, v = _inputs(b, lq, lk, h, hk, torch.bfloat16, seed=31 + lq + mode, k_offset=off)
+    q = q * 3.0                                             # a norm that has something to do
+    g = torch.Generator().manual_seed(lq)
+    qw = (1.0 + 0.3 * torch.randn(128, generator=g)) if has_qw else None
+    kw = (1.0 + 0.3 * torch.randn(128, generator=g)) if has_kw else None
+    rope = _rope_table(max(lq, lk), 3) if has_rope else None
+    eps, scale = 1e-6, 128 ** -0.5
+    norm = dict(qw=None if qw is None else qw.numpy(), kw=None if kw is None else kw.numpy(),
+                rope=None if rope is None else rope.numpy(), eps=eps, rope_mode=mode)
+    ref_q = oracle.attn_quant(oracle.BF16, _bits(q), _bits(k), _bits(v), norm=norm)
+    ref = _to_f32(oracle.attn_int8(oracle.BF16, _bits(q), _bits(k), _bits(v), scale, quant=ref_q), oracle.BF16)
+
+    ws = torch.zeros((ffi.lib.gpu_int8_attn_workspace(b, h, hk, lq, lk),), dtype=torch.uint8, device="cuda")
+    dev = lambda t: None if t is None else t.cuda()
+    qd, kd = q.cuda(), k.cuda()
+    q0, k0 = qd.clone(), kd.clone()
+    o = ql.int8_attn_norm_rope(qd, kd, v.cuda(), scale, dev(qw), dev(kw), eps, dev(rope), mode, ws=ws)
+    torch.cuda.synchronize()
+    assert torch.equal(qd, q0) and torch.equal(kd, k0), "q and k in memory are left as they were"
+    w = ws.cpu().numpy()
+    qi_o, ki_o, qs_o, ks_o, vt_o, vs_o, an_o, vsum_o, ck, kb = _layout(ffi, b, h, hk, lq, lk)
+
+    def take(at, n, dtp):
+        return w[at:at + n * np.dtype(dtp).itemsize].view(dtp)
+
+    assert np.array_equal(take(an_o, b * hk, np.int32).reshape(b, hk), ref_q["anchors"])
+    if off >= 2.0:
+        assert (ref_q["anchors"] >= 0).all()
+    assert np.array_equal(take(qi_o, b * h * lq * 128, np.int8).reshape(b, h, lq, 128), ref_q["qi"])
+    nblk = kb * (ck // 32)
+    ki = take(ki_o, b * hk * nblk * 32 * 128, np.int8).reshape(b, hk, nblk, 4, 2, 32, 16)
+    ki = ki.transpose(0, 1, 2, 5, 3, 4, 6).reshape(b, hk, nblk * 32, 128)[:, :, :lk]
+    assert np.array_equal(ki, ref_q["ki"])
+    own = np.zeros(ref_q["qs"].shape[-1], bool)
+    for r in range(lq):
+        own[(r // 32) * 8 + r % 8] = True
+    qs = take(qs_o, ref_q["qs"].size, np.float32).reshape(ref_q["qs"].shape)
+    assert np.array_equal(qs[..., own].view(np.uint32), ref_q["qs"][..., own].view(np.uint32))
+    assert np.array_equal(take(ks_o, ref_q["ks"].size, np.float32).view(np.uint32), ref_q["ks"].reshape(-1).view(np.uint32))
+
+    got = _to_f32(_bits(o), oracle.BF16)
+    vmax = float(v.float().abs().max())
+    tol = 2 * vmax / 255.0 + 2 * 2.0 ** -8 * np.abs(ref)
+    assert (np.abs(got - ref) <= tol).all()
+
+    qn = _norm_rope_f64(q, qw, rope, eps, mode).bfloat16()
+    kn = _norm_rope_f64(k, kw, rope, eps, mode).bfloat16() if has_kw else k
+    ex = _exact(qn, kn, v, scale)
+    cos = float((got * ex).sum() / np.sqrt((got * got).sum() * (ex * ex).sum()))
+    assert cos > 0.999, cos
+
+
+
+def test_fused_norm_sums_squares_in_the_reference_lane_order():
+    """Rows where the order of the fp32 additions shows (values of very different size, and random ones): both device
+    forms of the sum against the oracle's, whose order is pinned by hand-derived cases on the CPU."""
+    ql, ffi = _pkg()
+    g = torch.Generator().manual_seed(2)
+    rows = [torch.ones(128), torch.ones(128)]
+    rows[0][0] = 4096.0
+    rows[1][64] = 4096.0
+    x = torch.stack(rows + [torch.randn(128, generator=g) * (10.0 ** float(torch.randint(-3, 4, (1,), generator=g))) for _ in range(62)])
+    x[5] *= torch.exp(torch.randn(128, generator=g) * 4)
+    for split in (0, 1):
+        out = torch.zeros(2 * x.shape[0], device="cuda")
+        assert ffi.raw("gpu_internal_attn_sumsq_probe", C.c_void_p(x.cuda().data_ptr()), C.c_void_p(out.data_ptr()), x.shape[0], split, None) == 0
+        got = out.cpu().numpy().reshape(-1, 2)
+        want = np.array([oracle.attn_sumsq128(r.numpy(), split) for r in x], np.float32)
+        assert np.array_equal(got[:, 0].view(np.uint32), want.view(np.uint32))
+        assert np.array_equal(got[:, 1].view(np.uint32), want.view(np.uint32))
+
+
+def test_attention_norm_rope_equals_two_passes():
+    """The fused stage sees exactly the bf16 values a separate norm + rope pass would have stored: running the plain
+    entry point on q and k transformed row by row by the oracle gives the same workspace and the same output."""
+    ql, ffi = _pkg()
+    b, lq, lk, h, hk = 1, 70, 90, 2, 2
+    q, k, v = _inputs(b, lq, lk, h, hk, torch.bfloat16, seed=77)
+    g = torch.Generator().manual_seed(1)
+    qw, kw = 1.0 + 0.2 * torch.randn(128, generator=g), 1.0 + 0.2 * torch.randn(128, generator=g)
+    rope = _rope_table(max(lq, lk), 9)
+    scale, eps = 0.09, 1e-5
+    for mode in (1, 2):
+        def apply(x, w):
+            out = torch.empty_like(x)
+            xf = x.float().numpy()
+            for bi in range(x.shape[0]):
+                for r in range(x.shape[1]):
+                    for hh in range(x.shape[2]):
+                        out[bi, r, hh] = torch.from_numpy(oracle.attn_norm_rope_row(xf[bi, r, hh], w.numpy(), rope[r].numpy(), eps, mode)).bfloat16()
+            return out
+        q2, k2 = apply(q, qw), apply(k, kw)
+        ws1 = torch.zeros((ffi.lib.gpu_int8_attn_workspace(b, h, hk, lq, lk),), dtype=torch.uint8, device="cuda")
+        ws2 = torch.zeros_like(ws1)
+        o1 = ql.int8_attn_norm_rope(q.cuda(), k.cuda(), v.cuda(), scale, qw.cuda(), kw.cuda(), eps, rope.cuda(), mode, ws=ws1)
+        o2 = ql.int8_attn(q2.cuda(), k2.cuda(), v.cuda(), scale, ws=ws2)
+        assert torch.equal(ws1, ws2)
+        assert torch.equal(o1, o2)
+
+
+def test_attention_sink_with_q_norm():
+    """gpu_int8_attn_sink with qw: q normalized (weight, no rotation), k as it is, anchor off."""
+    ql, ffi = _pkg()
+    b, lq, lk, h, hk, sink = 1, 50, 180, 2, 1, 76.0
+    q, k, v = _inputs(b, lq, lk, h, hk, torch.bfloat16, seed=23)
+    qw = 1.0 + 0.25 * torch.randn(128, generator=torch.Generator().manual_seed(4))
+    scale, eps = 128 ** -0.5, 1e-6
+    norm = dict(qw=qw.numpy(), kw=None, rope=None, eps=eps, rope_mode=0)
+    ref_q = oracle.attn_quant(oracle.BF16, _bits(q), _bits(k), _bits(v), use_anchor=False, norm=norm)
+    ref = _to_f32(oracle.attn_int8(oracle.BF16, _bits(q), _bits(k), _bits(v), scale, quant=ref_q, sink=sink), oracle.BF16)
+    ws = torch.zeros((ffi.lib.gpu_int8_attn_workspace(b, h, hk, lq, lk),), dtype=torch.uint8, device="cuda")
+    o = ql.int8_attn_sink(q.cuda(), k.cuda(), v.cuda(), scale, sink, ws=ws, qw=qw.cuda(), eps=eps)
+    torch.cuda.synchronize()
+    lay = _layout(ffi, b, h, hk, lq, lk)
+    w = ws.cpu().numpy()
+    assert np.array_equal(w[lay[0]:lay[0] + b * h * lq * 128].view(np.int8).reshape(b, h, lq, 128), ref_q["qi"])
+    assert (w[lay[6]:lay[6] + 4 * b * hk].view(np.int32) == -1).all()
+    got = _to_f32(_bits(o), oracle.BF16)
+    tol = 2 * float(v.float().abs().max()) / 255.0 + 2 * 2.0 ** -8 * np.abs(ref)
+    assert (np.abs(got - ref) <= tol).all()
 
 
 def test_attention_unaligned_views_take_the_scalar_paths():

@@ -1019,3 +1019,103 @@ def test_attn_oracle_sink_equals_zero_keys_appended():
     # and it is not the plain attention: the sink takes a visible share of the weight
     plain = oracle.bf16_to_f32(oracle.attn_int8(oracle.BF16, bits(q), bits(k), bits(v), scale, use_anchor=False))
     assert np.abs(plain - got).max() > 0.01
+
+
+def test_attn_sumsq_lane_order_by_hand():
+    """orc_attn_sumsq128 against sums worked out by hand from the reference's order (csrc/kernels.cu:497-513: a lane's
+    four channels by fma in order, then lanes at distances 16, 8, 4, 2, 1).  One channel of 4096 among ones: 2^24 + 1
+    rounds back to 2^24 (tie to even), so each 1 added to that lane after the big square is lost, while the other 31
+    lanes' sums of 4 add exactly.
+      channel 0 big, 4 channels per lane: lane 0 = 2^24 (three ones lost), total 2^24 + 124.
+      channel 64 big, same layout: lane 16 holds 64..67, the same loss: 2^24 + 124.
+      channel 64 big, split layout (lane l: 2l, 2l+1, 64+2l, 65+2l): lane 0 = ((1 + 1) + 2^24) + 1 = 2^24 + 3 -> 2^24 + 4
+        (tie to even), total 2^24 + 128.
+      channel 1 big, split layout: lane 0 = 1, then + 2^24 -> 2^24, + 1 -> 2^24, + 1 -> 2^24: total 2^24 + 124.
+    A sequential fp32 sum would give 2^24 + {0..}, an fp64 sum 2^24 + 127 -> 2^24 + 128: every case separates at least
+    one plausible alternative."""
+    def row(big):
+        r = np.ones(128, np.float32)
+        r[big] = 4096.0
+        return r
+    assert oracle.attn_sumsq128(row(0), False) == 2.0 ** 24 + 124
+    assert oracle.attn_sumsq128(row(64), False) == 2.0 ** 24 + 124
+    assert oracle.attn_sumsq128(row(64), True) == 2.0 ** 24 + 128
+    assert oracle.attn_sumsq128(row(1), True) == 2.0 ** 24 + 124
+    # a tree, not a chain: 32 lanes of 2^22 + 1 ... each lane sums exactly; the tree's pair sums stay exact up to 2^24
+    r = np.zeros(128, np.float32)
+    r[0::4] = 2048.0                                  # one 2^22 per lane in the plain layout
+    r[1::4] = 1.0
+    # lanes: 2^22 + 1; distance 16: 2^23 + 2; 8: 2^24 + 4; 4: 2^25 + 8; 2: 2^26 + 16; 1: 2^27 + 32 (all exact)
+    assert oracle.attn_sumsq128(r, False) == 2.0 ** 27 + 32
+    # the same row in the split layout: lane l holds 2l, 2l+1, 64+2l, 65+2l = for even l (2048, 1, 2048, 1), for odd l
+    # (0, 0, 0, 0): even lanes 2^22 + 1 + 2^22 -> 2^23 + 1 exact, + 1 -> 2^23 + 2; 16 such lanes, all sums exact
+    assert oracle.attn_sumsq128(r, True) == 16 * (2.0 ** 23 + 2)
+
+
+def test_attn_norm_rope_row_special_cases_and_float64():
+    """The row transform against what the mathematics fixes: angle 0 is the identity on the normalized row, a quarter
+    turn maps (a, b) to (-b, a) exactly in both pairings, a constant row normalizes to +-weight, and random rows agree
+    with float64 within the two bf16 roundings."""
+    rng = np.random.default_rng(5)
+    bf = lambda a: oracle.bf16_to_f32(oracle.bf16_bits(np.asarray(a, np.float32)))
+    x = bf(rng.standard_normal(128) * 2)
+    w = bf(1 + 0.2 * rng.standard_normal(128))
+    ident = np.stack([np.ones(64), np.zeros(64)], -1).astype(np.float32)
+    quarter = np.stack([np.zeros(64), np.ones(64)], -1).astype(np.float32)
+    base = oracle.attn_norm_rope_row(x, w, None, 1e-6, 0)
+    assert np.array_equal(base, bf(base))
+    for mode in (1, 2):
+        got = oracle.attn_norm_rope_row(x, w, ident, 1e-6, mode)
+        assert np.array_equal(got + 0.0, base + 0.0)                       # +0.0 folds the sign of zero
+        got = oracle.attn_norm_rope_row(x, w, quarter, 1e-6, mode)
+        want = np.empty(128, np.float32)
+        if mode == 1:
+            want[0::2], want[1::2] = -base[1::2], base[0::2]
+        else:
+            want[:64], want[64:] = -base[64:], base[:64]
+        assert np.array_equal(got + 0.0, want + 0.0)
+    # rope_mode 0 ignores a table
+    assert np.array_equal(oracle.attn_norm_rope_row(x, w, quarter, 1e-6, 0), base)
+    # constant row c: mean square c^2, so the row becomes sign(c) * w up to the roundings of rstd (eps = 0)
+    c = oracle.attn_norm_rope_row(np.full(128, -3.0, np.float32), w, None, 0.0, 0)
+    assert np.abs(c + w).max() <= np.abs(w).max() * 2.0 ** -8
+    # random rows and angles against float64
+    for mode in (0, 1, 2):
+        ang = rng.random(64) * 6.28
+        rope = np.stack([np.cos(ang), np.sin(ang)], -1).astype(np.float32)
+        y = oracle.attn_norm_rope_row(x, w, rope, 1e-6, mode)
+        xd = x.astype(np.float64)
+        n = bf(xd / np.sqrt((xd * xd).mean() + 1e-6) * w).astype(np.float64)
+        cs, sn = rope[:, 0].astype(np.float64), rope[:, 1].astype(np.float64)
+        if mode == 1:
+            z = np.stack([cs * n[0::2] - sn * n[1::2], sn * n[0::2] + cs * n[1::2]], -1).reshape(-1)
+        elif mode == 2:
+            z = np.concatenate([n[:64] * cs - n[64:] * sn, n[64:] * cs + n[:64] * sn])
+        else:
+            z = n
+        assert np.abs(y - z).max() <= 2.0 ** -8 * np.abs(z).max() + 1e-6
+
+
+def test_attn_quant_with_norm_off_weights_is_the_plain_quantizer_on_transformed_rows():
+    """orc_attn_quant_qk_norm equals orc_attn_quant_qk run on rows transformed one by one, and a null kw leaves k alone."""
+    rng = np.random.default_rng(9)
+    b, lq, lk, h, hk = 1, 40, 70, 2, 1
+    bits = lambda a: oracle.bf16_bits(np.asarray(a, np.float32))
+    q, k, v = (bits(rng.standard_normal(s)) for s in ((b, lq, h, 128), (b, lk, hk, 128), (b, lk, hk, 128)))
+    qw, kw = (1 + 0.2 * rng.standard_normal(128)).astype(np.float32), (1 + 0.2 * rng.standard_normal(128)).astype(np.float32)
+    ang = rng.random((max(lq, lk), 64)) * 6.28
+    rope = np.stack([np.cos(ang), np.sin(ang)], -1).astype(np.float32)
+    for mode in (1, 2):
+        for use_kw in (True, False):
+            norm = dict(qw=qw, kw=kw if use_kw else None, rope=rope, eps=1e-6, rope_mode=mode)
+            fused = oracle.attn_quant(oracle.BF16, q, k, v, norm=norm)
+            def apply(x, w):
+                xf = oracle.bf16_to_f32(x)
+                out = np.empty_like(xf)
+                for r in range(x.shape[1]):
+                    for hh in range(x.shape[2]):
+                        out[0, r, hh] = oracle.attn_norm_rope_row(xf[0, r, hh], w, rope[r], 1e-6, mode)
+                return bits(out)
+            two = oracle.attn_quant(oracle.BF16, apply(q, qw), apply(k, kw) if use_kw else k, v)
+            for name in ("qi", "qs", "ki", "ks", "anchors"):
+                assert np.array_equal(fused[name], two[name]), name
