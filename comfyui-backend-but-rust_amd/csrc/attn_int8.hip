@@ -40,6 +40,9 @@ struct AttnArgs {
     const float *qw, *kw, *rope;   // [128] or null (ones); rope [L][64] x (cos, sin) or null
     float eps;
     int q_norm, k_norm, rope_mode;
+    const float* bias;    // per-key logit bias of the caller, f32 [lk], or null
+    float* kbias;         // prepared: bias * log2e per key of every tile (-inf: not kept / padding), then one value per tile
+    float* tbias;         // per tile: the bias all its keys share (times log2e), NaN when they differ, -inf when none is kept
 };
 
 // fmaxf as the reference's device code uses it: a NaN operand is dropped.
@@ -550,7 +553,7 @@ typedef const __attribute__((address_space(1))) void* glb_ptr_t;
 // The attention: a workgroup of four waves owns 128 query rows, a wave 32 of them.  The K tile, the V tile and the
 // tile's 128 x column sums are contiguous in the workspace, in the order the fragment reads want them, so the four waves
 // copy them global -> LDS with DMA loads (no registers) into one of two stages, a tile ahead; one barrier per tile.
-template <int OUT_DT, int CK>
+template <int OUT_DT, int CK, bool MASK = false>
 __global__ __launch_bounds__(256, 2) void attn_int8_kernel(AttnArgs a) {
     constexpr int NB = CK / 32, KV = CK * D, STAGE = 2 * KV + 512;
     extern __shared__ __align__(16) uint8_t smem[];
@@ -590,6 +593,8 @@ __global__ __launch_bounds__(256, 2) void attn_int8_kernel(AttnArgs a) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) ro[x][i] = 0.f;
     float m = -50000.f, dsum = 1.f;
+    float dsum2 = 1.f;   // the per-key mask route keeps the reference's four partial denominators per row: two per lane
+    bool kept = false;   // that route: some key of this lane was kept
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
@@ -615,42 +620,20 @@ __global__ __launch_bounds__(256, 2) void attn_int8_kernel(AttnArgs a) {
         const float* ksc = a.ks + (kvh * a.kb + t) * 4 + hh * 2;
         const float gs0 = a.sm * (q_scale * ksc[0]), gs1 = a.sm * (q_scale * ksc[1]);
 
-        // Group maxima on the integers (exact in fp32: |score| < 2^24).  Only the last tile can hold keys past lk; its
-        // maxima start at the reference's floor of -50000.
-        int i0, i1;
-        if constexpr (!last) {
-            i0 = i1 = INT_MIN;
-#pragma unroll
-            for (int blk = 0; blk < NB; ++blk)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    if ((i % 4) < 2) i0 = max(i0, S[blk][i]);
-                    else i1 = max(i1, S[blk][i]);
-                }
-        } else {
-            i0 = i1 = -50000;
-#pragma unroll
-            for (int blk = 0; blk < NB; ++blk)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const int key = key0 + blk * 32 + (i / 4) * 8 + hh * 4 + (i % 4);
-                    const int sv = key < a.lk ? S[blk][i] : INT_MIN;
-                    if ((i % 4) < 2) i0 = max(i0, sv);
-                    else i1 = max(i1, sv);
-                }
-        }
-        float tile_m = fmax_nn(fmaf((float)i0, gs0, -kU8Offset), fmaf((float)i1, gs1, -kU8Offset));
-        tile_m = fmax_nn(tile_m, __shfl_xor(tile_m, 32));
-        const float smaller = __builtin_amdgcn_exp2f(-fabsf(m - tile_m));
-        const float o_scale = m < tile_m ? smaller : 1.f, t_scale = tile_m < m ? smaller : 1.f;
-        m = fmax_nn(m, tile_m);
-        dsum *= o_scale;
-
-        // Probabilities: v_cvt_pk_u8_f32 rounds to nearest even, saturates to 0..255 and writes one byte of a dword, which
-        // is the reference's cvt.rni.sat.u8 plus the packing.  p - 128 as a signed byte is p ^ 0x80.
+        // Probabilities: v_cvt_pk_u8_f32 rounds to nearest even, saturates to 0..255 (NaN to 0) and writes one byte of a
+        // dword, which is the reference's cvt.rni.sat.u8 plus the packing.  p - 128 as a signed byte is p ^ 0x80.
         v4i pf[NB];
         uint32_t psum = 0;
-        auto probabilities = [&](auto masked) {
+        float tile_m, o_scale, t_scale;
+        auto rescale = [&]() {
+            tile_m = fmax_nn(tile_m, __shfl_xor(tile_m, 32));
+            const float smaller = __builtin_amdgcn_exp2f(-fabsf(m - tile_m));
+            o_scale = m < tile_m ? smaller : 1.f;
+            t_scale = tile_m < m ? smaller : 1.f;
+            m = fmax_nn(m, tile_m);
+        };
+        // integer route: exp2(fma(score, group scale, negm)), the unmasked path and a tile with one bias for all its keys
+        auto probabilities = [&](auto masked, const float negm) {
 #pragma unroll
             for (int blk = 0; blk < NB; ++blk) {
                 uint32_t w[4];
@@ -659,7 +642,7 @@ __global__ __launch_bounds__(256, 2) void attn_int8_kernel(AttnArgs a) {
                     uint32_t packed = 0u;
 #pragma unroll
                     for (int c = 0; c < 4; ++c) {
-                        float e = __builtin_amdgcn_exp2f(fmaf((float)S[blk][g4 * 4 + c], c < 2 ? gs0 : gs1, -tile_m));
+                        float e = __builtin_amdgcn_exp2f(fmaf((float)S[blk][g4 * 4 + c], c < 2 ? gs0 : gs1, negm));
                         if constexpr (decltype(masked)::value) {
                             const int key = key0 + blk * 32 + g4 * 8 + hh * 4 + c;
                             e = key < a.lk ? e : 0.f;
@@ -673,8 +656,130 @@ __global__ __launch_bounds__(256, 2) void attn_int8_kernel(AttnArgs a) {
                 __builtin_amdgcn_sched_barrier(0);   // one block at a time: the converted scores die here
             }
         };
-        probabilities(last_tag);
-        dsum += (float)psum * t_scale;
+        auto int_maxima = [&](int& i0, int& i1) {
+            i0 = i1 = INT_MIN;
+#pragma unroll
+            for (int blk = 0; blk < NB; ++blk)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    if ((i % 4) < 2) i0 = max(i0, S[blk][i]);
+                    else i1 = max(i1, S[blk][i]);
+                }
+        };
+        // float route of the masked forms: scores already carry scale and bias; exp2(score - tile_m)
+        float fsc[MASK ? NB : 1][16];
+        auto float_probabilities = [&](auto sum_floats) {
+#pragma unroll
+            for (int blk = 0; blk < NB; ++blk) {
+                uint32_t w[4];
+                float e[4][4];
+#pragma unroll
+                for (int g4 = 0; g4 < 4; ++g4) {
+                    uint32_t packed = 0u;
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        e[g4][c] = __builtin_amdgcn_exp2f(fsc[MASK ? blk : 0][g4 * 4 + c] + (-tile_m));
+                        packed = __builtin_amdgcn_cvt_pk_u8_f32(e[g4][c], c, packed);
+                    }
+                    psum = __builtin_amdgcn_sad_u8(packed, 0u, psum);
+                    w[g4] = packed ^ 0x80808080u;
+                }
+                if constexpr (decltype(sum_floats)::value) {
+                    // the reference's thread l of a row owns keys 2l, 2l+1, 8+2l, 9+2l of each 16: this lane carries
+                    // threads 2hh (c = 0, 1) and 2hh + 1 (c = 2, 3); a 16-key group is two g4 steps
+#pragma unroll
+                    for (int fk = 0; fk < 2; ++fk) {
+                        dsum += ((e[2 * fk][0] + e[2 * fk][1]) + (e[2 * fk + 1][0] + e[2 * fk + 1][1])) * t_scale;
+                        dsum2 += ((e[2 * fk][2] + e[2 * fk][3]) + (e[2 * fk + 1][2] + e[2 * fk + 1][3])) * t_scale;
+                    }
+                }
+                pf[blk] = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+
+        if constexpr (!MASK) {
+            // Group maxima on the integers (exact in fp32: |score| < 2^24).  Only the last tile can hold keys past lk; its
+            // maxima start at the reference's floor of -50000.
+            int i0, i1;
+            if constexpr (!last) {
+                int_maxima(i0, i1);
+            } else {
+                i0 = i1 = -50000;
+#pragma unroll
+                for (int blk = 0; blk < NB; ++blk)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const int key = key0 + blk * 32 + (i / 4) * 8 + hh * 4 + (i % 4);
+                        const int sv = key < a.lk ? S[blk][i] : INT_MIN;
+                        if ((i % 4) < 2) i0 = max(i0, sv);
+                        else i1 = max(i1, sv);
+                    }
+            }
+            tile_m = fmax_nn(fmaf((float)i0, gs0, -kU8Offset), fmaf((float)i1, gs1, -kU8Offset));
+            rescale();
+            dsum *= o_scale;
+            probabilities(last_tag, -tile_m);
+            dsum += (float)psum * t_scale;
+        } else {
+            // this lane's prepared biases: four consecutive keys per (blk, g4)
+            auto load_bias = [&](float (&bj)[NB][16]) {
+#pragma unroll
+                for (int blk = 0; blk < NB; ++blk)
+#pragma unroll
+                    for (int g4 = 0; g4 < 4; ++g4) {
+                        const float4 b4 = *reinterpret_cast<const float4*>(a.kbias + key0 + blk * 32 + g4 * 8 + hh * 4);
+                        bj[blk][g4 * 4] = b4.x; bj[blk][g4 * 4 + 1] = b4.y; bj[blk][g4 * 4 + 2] = b4.z; bj[blk][g4 * 4 + 3] = b4.w;
+                    }
+            };
+            if constexpr (CK == 64) {
+                // per-key mask: scaled score, plus the bias where the key is kept, -50000 elsewhere; the denominator sums
+                // the unrounded probabilities in the reference's per-thread partials
+                float bj[NB][16];
+                load_bias(bj);
+                float mx = -50000.f;
+#pragma unroll
+                for (int blk = 0; blk < NB; ++blk)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const bool keep = bj[blk][i] != -__builtin_inff();   // padding past lk is prepared as -inf too
+                        kept = kept || keep;
+                        const float rs = (float)S[blk][i] * ((i % 4) < 2 ? gs0 : gs1);
+                        fsc[MASK ? blk : 0][i] = keep ? rs + bj[blk][i] : -50000.f;
+                        mx = fmax_nn(mx, fsc[MASK ? blk : 0][i]);
+                    }
+                tile_m = mx - kU8Offset;
+                rescale();
+                dsum *= o_scale;
+                dsum2 *= o_scale;
+                float_probabilities(std::true_type{});
+            } else {
+                const float tb = a.tbias[t];   // uniform: a scalar branch
+                if (!last && __builtin_isfinite(tb)) {
+                    int i0, i1;
+                    int_maxima(i0, i1);
+                    tile_m = fmax_nn(fmaf((float)i0, gs0, -kU8Offset) + tb, fmaf((float)i1, gs1, -kU8Offset) + tb);
+                    rescale();
+                    probabilities(std::false_type{}, tb - tile_m);
+                } else {
+                    float bj[NB][16];
+                    load_bias(bj);
+                    float mx = -50000.f;
+#pragma unroll
+                    for (int blk = 0; blk < NB; ++blk)
+#pragma unroll
+                        for (int i = 0; i < 16; ++i) {
+                            fsc[MASK ? blk : 0][i] = fmaf((float)S[blk][i], (i % 4) < 2 ? gs0 : gs1, bj[blk][i]);
+                            mx = fmax_nn(mx, fsc[MASK ? blk : 0][i]);
+                        }
+                    tile_m = mx - kU8Offset;
+                    rescale();
+                    float_probabilities(std::false_type{});
+                }
+                dsum *= o_scale;
+                dsum += (float)psum * t_scale;
+            }
+        }
 
         // P.V: the four 32-channel blocks of the output keep their own accumulators (the scores are dead by now), key
         // blocks outside, so that consecutive MFMAs are independent here too.
@@ -708,7 +813,10 @@ __global__ __launch_bounds__(256, 2) void attn_int8_kernel(AttnArgs a) {
     for (int t = 0; t + 1 < a.kb; ++t) tile(t, std::false_type{});
     tile(a.kb - 1, std::true_type{});
 
+    if constexpr (MASK && CK == 64) dsum += dsum2;   // (d0 + d1) and (d2 + d3) of the reference's four threads
     float dtot = dsum + __shfl_xor(dsum, 32);
+    bool row_kept = true;
+    if constexpr (MASK && CK == 64) row_kept = (__shfl_xor((int)kept, 32) | (int)kept) != 0;   // a row with no kept key gives zeros
     // `sink` more keys of score zero and value zero: each adds exp2(0 - m) to the denominator, nothing to the output
     if (a.sink != 0.f) dtot = fmaf(a.sink, __builtin_amdgcn_exp2f(-m), dtot);
     const float rcp = 1.f / dtot;
@@ -722,6 +830,9 @@ __global__ __launch_bounds__(256, 2) void attn_int8_kernel(AttnArgs a) {
                 const float4 s4 = *reinterpret_cast<const float4*>(a.vs + kvh * D + d0);
                 float out[4] = {ro[x][g4 * 4] * rcp * s4.x, ro[x][g4 * 4 + 1] * rcp * s4.y, ro[x][g4 * 4 + 2] * rcp * s4.z,
                                 ro[x][g4 * 4 + 3] * rcp * s4.w};
+                if constexpr (MASK && CK == 64) {
+                    if (!row_kept) out[0] = out[1] = out[2] = out[3] = 0.f;
+                }
                 if (a.vec_ok) store4<OUT_DT>(a.o, ob + d0, out);
                 else
 #pragma unroll
@@ -731,6 +842,33 @@ __global__ __launch_bounds__(256, 2) void attn_int8_kernel(AttnArgs a) {
 }
 
 int cta_k_for(int lk, int d) { return lk > 1024 && d != 64 ? 128 : 64; }   // csrc/attn_int8.cu:56
+
+// The caller's per-key bias, prepared once per call (csrc/vendor/sage/sage_attn_launcher.cu:343-391; attn_utils.cuh:
+// 466-515 for the per-key form): bias * log2e per key of every tile, -inf where the bias is not finite and for the
+// padding past lk; for 128-key tiles also the value all keys of a tile share (times log2e), NaN when they differ.
+template <int CK>
+__global__ __launch_bounds__(CK) void attn_key_bias_kernel(const float* bias, int lk, float* kbias, float* tbias) {
+    __shared__ float lo_s[CK / 64], hi_s[CK / 64];
+    const int tid = threadIdx.x, key = blockIdx.x * CK + tid;
+    float raw = key < lk ? bias[key] : -__builtin_inff();
+    if (!__builtin_isfinite(raw)) raw = -__builtin_inff();
+    kbias[key] = raw * 1.44269504088896340736f;
+    if constexpr (CK == 128) {
+        float lo = raw, hi = raw;
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            lo = fminf(lo, __shfl_xor(lo, o));
+            hi = fmaxf(hi, __shfl_xor(hi, o));
+        }
+        if ((tid & 63) == 0) { lo_s[tid >> 6] = lo; hi_s[tid >> 6] = hi; }
+        __syncthreads();
+        if (tid == 0) {
+            lo = fminf(lo_s[0], lo_s[1]);
+            hi = fmaxf(hi_s[0], hi_s[1]);
+            tbias[blockIdx.x] = lo == hi ? hi * 1.44269504088896340736f : __builtin_nanf("");
+        }
+    }
+}
 
 struct Plan {
     int64_t qi, ki, qs, ks, vt, vs, anchors, vmax, vsum, total;
@@ -779,6 +917,23 @@ int run(AttnArgs a, hipStream_t st) {
             return -401;
         allowed[dev] = true;
     }
+    if (a.bias) {
+        static bool allowed_m[64] = {};
+        if (!allowed_m[dev]) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_int8_kernel<DT, 128, true>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, kLds128) != hipSuccess)
+                return -401;
+            allowed_m[dev] = true;
+        }
+        if (a.ck == 64) {
+            attn_key_bias_kernel<64><<<dim3(a.kb), 64, 0, st>>>(a.bias, a.lk, a.kbias, a.tbias);
+            attn_int8_kernel<DT, 64, true><<<grid, 256, kLds64, st>>>(a);
+        } else {
+            attn_key_bias_kernel<128><<<dim3(a.kb), 128, 0, st>>>(a.bias, a.lk, a.kbias, a.tbias);
+            attn_int8_kernel<DT, 128, true><<<grid, 256, kLds128, st>>>(a);
+        }
+        return hipGetLastError() == hipSuccess ? 0 : -401;
+    }
     if (a.ck == 64) attn_int8_kernel<DT, 64><<<grid, 256, kLds64, st>>>(a);
     else attn_int8_kernel<DT, 128><<<grid, 256, kLds128, st>>>(a);
     return hipGetLastError() == hipSuccess ? 0 : -401;
@@ -797,7 +952,7 @@ struct QkNorm {
 int int8_attn(const void* q, const void* k, const void* v, void* o, void* ws, int b, int lq, int lk, int h, int hk, int Dh,
               int64_t q_bs, int64_t q_rs, int64_t q_hs, int64_t k_bs, int64_t k_rs, int64_t k_hs, int64_t v_bs, int64_t v_rs,
               int64_t v_hs, int64_t o_bs, int64_t o_rs, int64_t o_hs, float scale, int dt, void* stream, float sink = 0.f,
-              const QkNorm* norm = nullptr) {
+              const QkNorm* norm = nullptr, const float* bias = nullptr) {
     const char* why = nullptr;
     if (Dh != D) why = "only head dim 128 is built";
     else if (norm && dt != DT_BF16) why = "fused q/k norm needs bf16 head dim 128";                     // csrc/attn_int8.cu:135
@@ -827,6 +982,9 @@ int int8_attn(const void* q, const void* k, const void* v, void* o, void* ws, in
     a.vec_ok = ((o_bs | o_rs | o_hs) % 4 == 0 && ((uintptr_t)o & 7) == 0) ? 1 : 0;
     a.v_vec = ((v_bs | v_rs | v_hs) % 4 == 0 && ((uintptr_t)v & 7) == 0) ? 1 : 0;
     a.in_vec = ((q_bs | q_rs | q_hs | k_bs | k_rs | k_hs) % 4 == 0 && (((uintptr_t)q | (uintptr_t)k) & 7) == 0) ? 1 : 0;
+    a.bias = bias;
+    a.kbias = (float*)(w + p.total);   // the key-bias form's workspace is this much longer
+    a.tbias = a.kbias + (int64_t)p.kb * p.ck;
     a.qw = a.kw = a.rope = nullptr;
     a.eps = 0.f;
     a.q_norm = a.k_norm = a.rope_mode = 0;
@@ -897,6 +1055,32 @@ GPU_API int gpu_int8_attn_norm_rope(const void* q, const void* k, const void* v,
     const QkNorm norm{qw, kw, rope, eps, rope_mode};
     return int8_attn(q, k, v, o, ws, b, lq, lk, h, hk, D, q_bs, q_rs, q_hs, k_bs, k_rs, k_hs, v_bs, v_rs, v_hs, o_bs, o_rs,
                      o_hs, scale, DT_BF16, stream, 0.f, &norm);
+}
+
+// sage's prepared key mask row for lk keys: each key's bias, then one value per 128-key tile (csrc/attn_int8.cu:178-182).
+// The layout kept here (bias * log2e per key of every tile, then one value per 128-key tile) fits the same size.
+static int64_t key_mask_width(int lk) {
+    const int64_t tiles = (lk + 127) / 128;
+    return (tiles * 129 + 3) / 4 * 4;
+}
+
+GPU_API int64_t gpu_int8_attn_key_bias_workspace(int b, int h, int hk, int lq, int lk) {
+    if (b <= 0 || h <= 0 || hk <= 0 || lq <= 0 || lk <= 0) return 0;
+    return gpu_int8_attn_workspace_d(b, h, hk, lq, lk, D) + (key_mask_width(lk) * 4 + 255) / 256 * 256;
+}
+
+// gpu_int8_attn with bias (f32 [lk], the same for every batch item, query and head) added to each key's logits, as an
+// additive attention mask; a bias that is not finite masks its key (csrc/attn_int8.cu:184-223).  bf16.
+GPU_API int gpu_int8_attn_key_bias(const void* q, const void* k, const void* v, void* o, void* ws, int b, int lq, int lk, int h,
+                                   int hk, int64_t q_bs, int64_t q_rs, int64_t q_hs, int64_t k_bs, int64_t k_rs, int64_t k_hs,
+                                   int64_t v_bs, int64_t v_rs, int64_t v_hs, int64_t o_bs, int64_t o_rs, int64_t o_hs, float scale,
+                                   const float* bias, void* stream) {
+    if (!bias) {
+        fprintf(stderr, "int8 attention: null key bias\n");
+        return -400;
+    }
+    return int8_attn(q, k, v, o, ws, b, lq, lk, h, hk, D, q_bs, q_rs, q_hs, k_bs, k_rs, k_hs, v_bs, v_rs, v_hs, o_bs, o_rs,
+                     o_hs, scale, DT_BF16, stream, 0.f, nullptr, bias);
 }
 
 // Test hook: y[i] = v_cvt_pk_u8_f32(x[i]) into byte 0 of zero, so that a test can hold the instruction to

@@ -45,6 +45,7 @@ SIGNATURES = {
     "gpu_int8_attn": [_P, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _I32] + [_I64] * 12 + [_F32, _P],
     "gpu_int8_attn_sink": [_P, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _I32] + [_I64] * 12 + [_F32, _F32, _P, _F32, _P],
     "gpu_int8_attn_norm_rope": [_P, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _I32] + [_I64] * 12 + [_F32, _P, _P, _F32, _P, _I32, _P],
+    "gpu_int8_attn_key_bias": [_P, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _I32] + [_I64] * 12 + [_F32, _P, _P],
     "gpu_internal_cvt_pk_u8_probe": [_P, _P, _I32, _P],
     "gpu_internal_attn_sumsq_probe": [_P, _P, _I32, _I32, _P],
     "gpu_internal_attn_layout": [_I32, _I32, _I32, _I32, _I32, _P],
@@ -68,6 +69,8 @@ def _load():
     lib.gpu_int8_attn_workspace_d.restype = _I64
     lib.gpu_int8_attn_workspace.argtypes = [_I32] * 5
     lib.gpu_int8_attn_workspace.restype = _I64
+    lib.gpu_int8_attn_key_bias_workspace.argtypes = [_I32] * 5
+    lib.gpu_int8_attn_key_bias_workspace.restype = _I64
     lib.gpu_int8_gemm_static_limit.argtypes = []
     lib.gpu_int8_gemm_static_limit.restype = _I64
     lib.gpu_kernels_build_info.restype = C.c_char_p

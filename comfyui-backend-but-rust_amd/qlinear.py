@@ -301,6 +301,22 @@ def int8_attn_norm_rope(q, k, v, scale, qw, kw, eps, rope, rope_mode, ws=None):
     return o
 
 
+def int8_attn_key_bias(q, k, v, scale, bias, ws=None):
+    """int8_attn with bias (float32 [lk], one row for every batch item, head and query) added to the logits of each key
+    (csrc/attn_int8.cu:184-223, the DiT's call at src/dit.rs:573).  bf16."""
+    b, lq, h, D = q.shape
+    lk, hk = k.shape[1], k.shape[2]
+    assert q.dtype == torch.bfloat16 and D == 128
+    assert q.stride(3) == 1 and k.stride(3) == 1 and v.stride(3) == 1
+    if ws is None:
+        ws = torch.empty((ffi.lib.gpu_int8_attn_key_bias_workspace(b, h, hk, lq, lk),), dtype=torch.uint8, device=q.device)
+    o = torch.empty((b, lq, h, D), dtype=q.dtype, device=q.device)
+    ffi.k("gpu_int8_attn_key_bias", _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(ws), b, lq, lk, h, hk, q.stride(0), q.stride(1),
+          q.stride(2), k.stride(0), k.stride(1), k.stride(2), v.stride(0), v.stride(1), v.stride(2), o.stride(0), o.stride(1),
+          o.stride(2), float(scale), _f32_vec(bias, lk, "bias"), _stream())
+    return o
+
+
 def int8_attn_sink(q, k, v, scale, sink, ws=None, qw=None, eps=0.0):
     """int8_attn over the keys given plus `sink` zero keys with zero values (bf16), csrc/attn_int8.cu:193-202.  qw
     (float32 [128]): q is RMS-normalized with that weight first, k taken as it is."""

@@ -136,7 +136,13 @@ int gpu_w6_requant(const void* weight, void* packed, void* s_rel, void* s_channe
  * 2 the pairs (j, j + 64), 0 none; other values -400.  bf16 only.  The values the quantizer sees are those
  * gpu_qk_norm_rope (csrc/kernels.cu:482-540) would have stored, with 1/sqrt correctly rounded where CUDA's rsqrtf
  * approximates.
- * Not built: gpu_int8_attn_key_bias (csrc/attn_int8.cu:204-223). */
+ * gpu_int8_attn_key_bias / gpu_int8_attn_key_bias_workspace (csrc/attn_int8.cu:184-223, bound at src/ffi.rs:196-199,
+ * called from src/dit.rs:519,573): bias f32 [lk], the same for every batch item, head and query, added to each key's
+ * logits (an additive attention mask; a bias that is not finite masks its key, a query row with every key masked gives
+ * zeros for lk <= 1024).  Its workspace is the plain one plus the prepared bias row, the reference's size.  bf16.  The
+ * two routes of the reference are kept: for lk <= 1024 (64-key tiles) the denominator sums the unrounded probabilities,
+ * for longer sequences (128-key tiles) the rounded ones, and a tile whose keys share one finite bias folds it into the
+ * exponent's constant. */
 int64_t gpu_int8_attn_workspace_d(int b, int h, int hk, int lq, int lk, int head_dim);
 int64_t gpu_int8_attn_workspace(int b, int h, int hk, int lq, int lk);
 int gpu_int8_attn_d(const void* q, const void* k, const void* v, void* o, void* ws, int b, int lq, int lk, int h, int hk,
@@ -159,6 +165,12 @@ int gpu_int8_attn_norm_rope(const void* q, const void* k, const void* v, void* o
                             int hk, int64_t q_bs, int64_t q_rs, int64_t q_hs, int64_t k_bs, int64_t k_rs, int64_t k_hs,
                             int64_t v_bs, int64_t v_rs, int64_t v_hs, int64_t o_bs, int64_t o_rs, int64_t o_hs, float scale,
                             const float* qw, const float* kw, float eps, const float* rope, int rope_mode, void* stream);
+
+int64_t gpu_int8_attn_key_bias_workspace(int b, int h, int hk, int lq, int lk);
+int gpu_int8_attn_key_bias(const void* q, const void* k, const void* v, void* o, void* ws, int b, int lq, int lk, int h,
+                           int hk, int64_t q_bs, int64_t q_rs, int64_t q_hs, int64_t k_bs, int64_t k_rs, int64_t k_hs,
+                           int64_t v_bs, int64_t v_rs, int64_t v_hs, int64_t o_bs, int64_t o_rs, int64_t o_hs, float scale,
+                           const float* bias, void* stream);
 
 /* Test hook, no reference counterpart: y[i] = the gfx950 float -> u8 pack conversion of x[i] (byte 0), which the attention
  * kernel's probabilities rely on being round-to-nearest-even with saturation to 0..255. */

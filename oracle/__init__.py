@@ -63,6 +63,8 @@ def lib():
         L.orc_attn_quant_qk_norm.restype = i32
         L.orc_attn_quant_qk_norm.argtypes = [i32, vp, vp, i32, i32, i32, i32, i32, i64, i64, i64, i64, i64, i64, i32, i32, vp, vp,
                                              vp, vp, vp, i32, vp, vp, vp, C.c_float, i32]
+        L.orc_attn_int8_bias.restype = i32
+        L.orc_attn_int8_bias.argtypes = [i32, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, C.c_float, vp, vp, i64, i64, i64]
         L.orc_attn_sumsq128.restype = C.c_float
         L.orc_attn_sumsq128.argtypes = [vp, i32]
         L.orc_attn_norm_rope_row.restype = None
@@ -400,6 +402,20 @@ def attn_quant(dt, q, k, v, use_anchor=True, norm=None):
     rc = lib().orc_attn_quant_v(dt, _p(v), b, lk, hk, lk * hk * D, hk * D, D, _p(out["vi"]), _p(out["vs"]))
     assert rc == 0
     return out
+
+
+def attn_int8_bias(dt, q, k, v, scale, bias, quant=None):
+    """attn_int8 with bias (float32 [lk]) added to each key's logits; a bias that is not finite masks its key."""
+    b, lq, h, D = q.shape
+    lk, hk = k.shape[1], k.shape[2]
+    z = quant if quant is not None else attn_quant(dt, q, k, v, True)
+    bias = np.ascontiguousarray(bias, dtype=np.float32)
+    assert bias.shape == (lk,)
+    o = np.zeros((b, lq, h, D), np.float32 if dt == F32 else np.uint16)
+    rc = lib().orc_attn_int8_bias(dt, _p(z["qi"]), _p(z["ki"]), _p(z["vi"]), _p(z["qs"]), _p(z["ks"]), _p(z["vs"]), b, lq, lk,
+                                  h, hk, z["ck"], float(scale), _p(bias), _p(o), lq * h * D, h * D, D)
+    assert rc == 0
+    return o
 
 
 def attn_int8(dt, q, k, v, scale, use_anchor=True, quant=None, sink=0.0, norm=None):

@@ -1080,5 +1080,149 @@ ORC_API int orc_attn_int8(int out_dt, const int8_t* qi, const int8_t* ki, const 
     return 0;
 }
 
+/* The same attention with an additive bias per key on the logits (gpu_int8_attn_key_bias, csrc/attn_int8.cu:204-223):
+ * bias f32 [lk], one row for every batch item, head and query.  The reference takes two routes by key tile length.
+ *
+ * ck = 64 (lk <= 1024), sage's per-key mask (mask mode kCustomKey: qk_int_sv_i8_cuda.cuh:637-700, attn_utils.cuh:466-515,
+ * 569-650, 862-880, 922-940): scores are scaled first, rs = float(S) * (sm * q_scale * k_scale); a key that is kept
+ * (inside lk, finite bias) becomes rs + bias * log2e (an fma with 1.0), any other -50000; the tile maximum starts at
+ * -50000 and has the u8 offset subtracted; probabilities exp2(rs - tile_max) are packed to u8 for P.V, but the
+ * DENOMINATOR sums the unrounded float probabilities: each of the four threads of a row keeps its own partial, adding per
+ * 16 keys ((p[2l] + p[2l+1]) + (p[8+2l] + p[8+2l+1])) * tile_scale, and the four are added pairwise at the end
+ * (attn_utils.cuh:1113-1122).  A row with no kept key at all gives zeros (qk_int_sv_i8_cuda.cuh:1031-1051).
+ *
+ * ck = 128 (lk > 1024), sage's prepared key mask (sage_attn_launcher.cu:343-391: non-finite biases and the padding past
+ * lk become -inf; a tile of 128 keys whose biases are all equal is marked with that value): a tile with a finite
+ * constant bias that is not the last takes the integer route with the bias added to the maximum and folded into the
+ * exponent's constant (attn_utils.cuh:719-790 with add_bias, qk_int_sv_i8_cuda.cuh:613-620); any other tile takes the
+ * float route, scores fma(float(S), scale, bias * log2e), maximum from -50000, probabilities exp2(score - tile_max)
+ * (:799-856).  Both sum the ROUNDED u8 probabilities into the denominator.  A tile whose biases are all -inf is skipped
+ * by the reference; the float route leaves m, d and the output as they were for it, so it is not special here.
+ * PARITY UNPINNED against a run of the reference for the same reasons as orc_attn_int8. */
+ORC_API int orc_attn_int8_bias(int out_dt, const int8_t* qi, const int8_t* ki, const int8_t* vi, const float* qs,
+                               const float* ks, const float* vs, int b, int lq, int lk, int h, int hk, int ck, float scale,
+                               const float* bias, void* o, int64_t o_bs, int64_t o_rs, int64_t o_hs) {
+    if ((ck != 64 && ck != 128) || hk <= 0 || h % hk != 0 || !bias) return -1;
+    const int qg = (lq + 127) / 128 * 4, kb = (lk + ck - 1) / ck, rep = h / hk;
+    const float log2e = 1.44269504088896340736f;
+    const float sm = scale * log2e;
+    /* prepared biases: bias * log2e, -inf for non-finite ones and for the padding */
+    float* bl = (float*)malloc(sizeof(float) * (size_t)kb * ck);
+    float* tb = (float*)malloc(sizeof(float) * (size_t)kb);
+    for (int j = 0; j < kb * ck; ++j) bl[j] = (j < lk && isfinite(bias[j])) ? bias[j] * log2e : -INFINITY;
+    for (int t = 0; t < kb; ++t) {
+        float lo = INFINITY, hi = -INFINITY;
+        for (int j = 0; j < ck; ++j) {
+            const int key = t * ck + j;
+            const float v = (key < lk && isfinite(bias[key])) ? bias[key] : -INFINITY;
+            lo = v < lo ? v : lo;
+            hi = v > hi ? v : hi;
+        }
+        tb[t] = lo == hi ? hi : NAN;
+    }
+    #pragma omp parallel for collapse(2) schedule(dynamic, 8)
+    for (int bh = 0; bh < b * h; ++bh)
+        for (int r = 0; r < lq; ++r) {
+            const int bi = bh / h, hi = bh % h;
+            const int64_t kvh = (int64_t)bi * hk + hi / rep;
+            const int8_t* qrow = qi + ((int64_t)bh * lq + r) * ATTN_D;
+            const float q_scale = qs[((int64_t)bh * qg + r / 32) * 8 + r % 8];
+            float m = -50000.f, ro[ATTN_D], d4[4] = {1.f, 1.f, 1.f, 1.f}, d = 1.f;
+            int valid = 0;
+            for (int c = 0; c < ATTN_D; ++c) ro[c] = 0.f;
+            int32_t s[128];
+            float f[128], pf[128];
+            for (int t = 0; t < kb; ++t) {
+                const int n = lk - t * ck < ck ? lk - t * ck : ck;
+                const int last = t == kb - 1;
+                float gs[4];
+                for (int g = 0; g < 4; ++g) gs[g] = sm * (q_scale * ks[(kvh * kb + t) * 4 + g]);
+                for (int j = 0; j < ck; ++j) {
+                    s[j] = 0;
+                    if (j >= n) continue;
+                    const int8_t* krow = ki + ((int64_t)kvh * lk + t * ck + j) * ATTN_D;
+                    int32_t acc = 0;
+                    for (int c = 0; c < ATTN_D; ++c) acc += (int32_t)qrow[c] * (int32_t)krow[c];
+                    s[j] = acc;
+                }
+                float tile_m, neg_m = 0.f;
+                int route;   /* 0: per-key mask (ck 64), 1: prepared, constant tile, 2: prepared, float route */
+                if (ck == 64) {
+                    route = 0;
+                    float mx = -50000.f;
+                    for (int j = 0; j < ck; ++j) {
+                        const float bj = bl[t * ck + j];
+                        const int keep = j < n && bj != -INFINITY;
+                        valid |= keep;
+                        const float rs = (float)s[j] * gs[(j % 8) / 2];
+                        f[j] = keep ? fmaf(rs, 1.0f, bj) : -50000.f;
+                        mx = f[j] > mx ? f[j] : mx;
+                    }
+                    tile_m = mx - ATTN_U8_OFFSET;
+                } else if (!last && isfinite(tb[t])) {
+                    route = 1;
+                    const float tbl = tb[t] * log2e;
+                    tile_m = -INFINITY;
+                    for (int g = 0; g < 4; ++g) {
+                        int32_t mg = INT32_MIN;
+                        for (int j = 0; j < ck; ++j)
+                            if ((j % 8) / 2 == g) mg = s[j] > mg ? s[j] : mg;
+                        const float cand = fmaf((float)mg, gs[g], -ATTN_U8_OFFSET) + tbl;
+                        tile_m = cand > tile_m ? cand : tile_m;
+                    }
+                    neg_m = tbl - tile_m;
+                } else {
+                    route = 2;
+                    float mx = -50000.f;
+                    for (int j = 0; j < ck; ++j) {
+                        f[j] = fmaf((float)s[j], gs[(j % 8) / 2], bl[t * ck + j]);
+                        mx = f[j] > mx ? f[j] : mx;
+                    }
+                    tile_m = mx - ATTN_U8_OFFSET;
+                }
+                const float smaller = attn_exp2(-fabsf(m - tile_m));
+                const float o_scale = m < tile_m ? smaller : 1.f, t_scale = tile_m < m ? smaller : 1.f;
+                m = m > tile_m ? m : tile_m;
+                int32_t pv[ATTN_D];
+                int32_t psum = 0;
+                for (int c = 0; c < ATTN_D; ++c) pv[c] = 0;
+                for (int j = 0; j < ck; ++j) {
+                    float p = route == 1 ? attn_exp2(fmaf((float)s[j], gs[(j % 8) / 2], neg_m)) : attn_exp2(f[j] + (-tile_m));
+                    pf[j] = p;
+                    p = p != p ? 0.f : p;                       /* the clamp maps NaN to 0 (mma.cuh:790-800) */
+                    p = rintf(p > 255.f ? 255.f : (p < 0.f ? 0.f : p));
+                    const int32_t pi = (int32_t)p;
+                    psum += pi;
+                    if (j >= n || pi == 0) continue;
+                    const int8_t* vrow = vi + ((int64_t)kvh * lk + t * ck + j) * ATTN_D;
+                    for (int c = 0; c < ATTN_D; ++c) pv[c] += pi * (int32_t)vrow[c];
+                }
+                if (route == 0) {
+                    for (int l = 0; l < 4; ++l) d4[l] *= o_scale;
+                    for (int fk = 0; fk < ck / 16; ++fk)
+                        for (int l = 0; l < 4; ++l) {
+                            const float* q4 = pf + fk * 16;
+                            const float tile_sum = (q4[2 * l] + q4[2 * l + 1]) + (q4[8 + 2 * l] + q4[8 + 2 * l + 1]);
+                            d4[l] += tile_sum * t_scale;
+                        }
+                } else {
+                    d *= o_scale;
+                    d += (float)psum * t_scale;
+                }
+                for (int c = 0; c < ATTN_D; ++c) ro[c] = fmaf((float)pv[c], t_scale, ro[c] * o_scale);
+            }
+            if (ck == 64) d = (d4[0] + d4[1]) + (d4[2] + d4[3]);
+            const float rcp = 1.f / d;
+            for (int c = 0; c < ATTN_D; ++c) {
+                float out = ro[c] * rcp;
+                if (ck == 64 && !valid) out = 0.f;
+                st_t(out_dt, o, bi * o_bs + (int64_t)r * o_rs + hi * o_hs + c, out * vs[kvh * ATTN_D + c]);
+            }
+        }
+    free(bl);
+    free(tb);
+    return 0;
+}
+
 /* csrc/attn_int8.cu:56 */
 ORC_API int orc_attn_cta_k(int lk, int d) { return lk > 1024 && d != 64 ? 128 : 64; }

@@ -444,3 +444,91 @@ def test_attention_dit_size_against_exact_attention():
     vc = torch.full_like(v, 0.75)
     oc = ql.int8_attn(q, k, vc, scale).float()
     assert float((oc - 0.75).abs().max()) <= 0.75 * 2 ** -7
+
+
+BIAS_CASES = [
+    # b, lq, lk, h, hk, kind
+    (1, 100, 150, 2, 1, "sparse"),        # 64-key tiles, ragged last tile
+    (2, 64, 64, 2, 2, "sparse"),
+    (1, 70, 1024, 2, 2, "sparse"),        # the longest sequence of the per-key route
+    (1, 90, 1100, 2, 1, "tiles"),         # 128-key tiles: constant tiles (zero and non-zero), varying tiles, ragged last
+    (1, 130, 1536, 4, 2, "tiles"),        # no ragged tail: the last tile still takes the float route
+    (1, 50, 1300, 1, 1, "masked"),        # -inf keys, one whole tile of them
+    (1, 60, 200, 2, 2, "masked"),
+    (1, 40, 300, 2, 1, "all_masked"),
+]
+
+
+def _bias_for(kind, lk, seed):
+    rng = np.random.default_rng(seed)
+    bias = np.zeros(lk, np.float32)
+    hot = rng.choice(lk, max(1, lk // 7), replace=False)
+    bias[hot] = rng.choice(np.array([0.6, 1.2, -1.5], np.float32), hot.size)
+    if kind == "tiles" or kind == "masked":
+        if lk > 1024:
+            bias[128:384] = 0.0
+            bias[512:640] = 0.75
+    if kind == "masked":
+        bias[rng.choice(lk, lk // 4, replace=False)] = -np.inf
+        if lk > 1024:
+            bias[640:768] = -np.inf
+    if kind == "all_masked":
+        bias[:] = -np.inf
+    return bias
+
+
+@pytest.mark.parametrize("case", BIAS_CASES, ids=lambda c: "b%d_lq%d_lk%d_h%d_hk%d_%s" % c)
+def test_attention_with_key_bias(case):
+    """gpu_int8_attn_key_bias against the oracle's restatement of the reference's two masked routes (quantizer stages
+    bit-exact as in the plain call, outputs within the attention tolerance) and against exact attention with the bias on
+    the logits."""
+    ql, ffi = _pkg()
+    b, lq, lk, h, hk, kind = case
+    q, k, v = _inputs(b, lq, lk, h, hk, torch.bfloat16, seed=lq + lk)
+    bias = _bias_for(kind, lk, lk)
+    scale = 128 ** -0.5
+    ref_q = oracle.attn_quant(oracle.BF16, _bits(q), _bits(k), _bits(v))
+    ref = _to_f32(oracle.attn_int8_bias(oracle.BF16, _bits(q), _bits(k), _bits(v), scale, bias, quant=ref_q), oracle.BF16)
+    n = ffi.lib.gpu_int8_attn_key_bias_workspace(b, h, hk, lq, lk)
+    assert n > ffi.lib.gpu_int8_attn_workspace(b, h, hk, lq, lk)
+    ws = torch.zeros((n,), dtype=torch.uint8, device="cuda")
+    o = ql.int8_attn_key_bias(q.cuda(), k.cuda(), v.cuda(), scale, torch.from_numpy(bias).cuda(), ws=ws)
+    torch.cuda.synchronize()
+    lay = _layout(ffi, b, h, hk, lq, lk)
+    w = ws.cpu().numpy()
+    assert np.array_equal(w[lay[0]:lay[0] + b * h * lq * 128].view(np.int8).reshape(b, h, lq, 128), ref_q["qi"])
+    assert np.array_equal(w[lay[6]:lay[6] + 4 * b * hk].view(np.int32).reshape(b, hk), ref_q["anchors"])
+    got = _to_f32(_bits(o), oracle.BF16)
+    assert np.isfinite(got).all()
+    if kind == "all_masked":
+        if lk <= 1024:
+            assert (got == 0).all()
+        return
+    vmax = float(v.float().abs().max())
+    tol = 2 * vmax / 255.0 + 2 * 2.0 ** -8 * np.abs(ref)
+    err = np.abs(got - ref)
+    assert (err <= tol).all(), "max excess %g" % float((err - tol).max())
+    assert (err <= 2.0 ** -8 * np.abs(ref) + 1e-30).mean() > 0.97
+
+    keep = np.isfinite(bias)
+    kk, vv = k[:, keep], v[:, keep]
+    hh, hkk = q.shape[2], k.shape[2]
+    qq = q.double().permute(0, 2, 1, 3)
+    kd = kk.double().permute(0, 2, 1, 3).repeat_interleave(hh // hkk, 1)
+    vd = vv.double().permute(0, 2, 1, 3).repeat_interleave(hh // hkk, 1)
+    logits = qq @ kd.transpose(-1, -2) * scale + torch.from_numpy(bias[keep]).double()
+    ex = (torch.softmax(logits, -1) @ vd).permute(0, 2, 1, 3).numpy()
+    cos = float((got * ex).sum() / np.sqrt((got * got).sum() * (ex * ex).sum()))
+    assert cos > 0.9995, cos
+
+
+def test_attention_key_bias_moves_weight_to_the_biased_keys():
+    """A large bias on one key makes every query attend to it: the output is that key's value row (to quantization)."""
+    ql, ffi = _pkg()
+    for lk in (200, 1200):
+        q, k, v = _inputs(1, 32, lk, 1, 1, torch.bfloat16, seed=3)
+        bias = torch.zeros(lk)
+        bias[lk // 2] = 60.0
+        o = ql.int8_attn_key_bias(q.cuda(), k.cuda(), v.cuda(), 128 ** -0.5, bias.cuda())
+        want = v[0, lk // 2, 0].float()
+        assert (o[0, :, 0].float().cpu() - want).abs().max() < 2 * float(v.float().abs().max()) / 127 + 0.02

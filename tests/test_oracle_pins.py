@@ -1119,3 +1119,64 @@ def test_attn_quant_with_norm_off_weights_is_the_plain_quantizer_on_transformed_
             two = oracle.attn_quant(oracle.BF16, apply(q, qw), apply(k, kw) if use_kw else k, v)
             for name in ("qi", "qs", "ki", "ks", "anchors"):
                 assert np.array_equal(fused[name], two[name]), name
+
+
+def _exact_attention(q, k, v, scale, bias=None):
+    """float64 softmax attention over bf16 bit tensors [b, l, h, 128]; bias [lk] added to the logits."""
+    qf, kf, vf = (oracle.bf16_to_f32(t).astype(np.float64) for t in (q, k, v))
+    rep = q.shape[2] // k.shape[2]
+    kf, vf = np.repeat(kf, rep, axis=2), np.repeat(vf, rep, axis=2)
+    logits = np.einsum("bqhd,bkhd->bhqk", qf, kf) * scale
+    if bias is not None:
+        logits = logits + np.asarray(bias, np.float64)[None, None, None, :]
+    logits -= logits.max(-1, keepdims=True)
+    p = np.exp(logits)
+    p /= p.sum(-1, keepdims=True)
+    return np.einsum("bhqk,bkhd->bqhd", p, vf)
+
+
+@pytest.mark.parametrize("lk", [150, 1100])
+def test_attn_key_bias_against_exact_attention_and_its_invariants(lk):
+    """orc_attn_int8_bias on both of the reference's routes (64-key tiles with the per-key mask, 128-key tiles with the
+    prepared mask): close to float64 attention with the bias on the logits; a bias of -inf removes its keys exactly as if
+    they were not there to attend to (same quantized tensors, so the comparison is within the attention tolerance);
+    adding one constant to every bias changes nothing beyond rounding; a zero bias agrees with the unbiased routine."""
+    rng = np.random.default_rng(lk)
+    b, lq, h, hk = 1, 40, 2, 1
+    bits = lambda a: oracle.bf16_bits(np.asarray(a, np.float32))
+    q, k, v = (bits(rng.standard_normal(s)) for s in ((b, lq, h, 128), (b, lk, hk, 128), (b, lk, hk, 128)))
+    scale = 128 ** -0.5
+    z = oracle.attn_quant(oracle.BF16, q, k, v)
+    f = lambda o: oracle.bf16_to_f32(o).astype(np.float64)
+    bias = np.zeros(lk, np.float32)
+    bias[rng.choice(lk, lk // 6, replace=False)] = rng.choice([0.6, 1.5, -2.0], lk // 6).astype(np.float32)
+    if lk > 1024:
+        bias[128:384] = 0.0            # two whole tiles of one bias: the constant-tile route
+        bias[512:640] = 0.75           # a tile with one non-zero bias
+    got = f(oracle.attn_int8_bias(oracle.BF16, q, k, v, scale, bias, quant=z))
+    ex = _exact_attention(q, k, v, scale, bias)
+    assert np.abs(got - ex).max() < 0.04
+    cos = (got * ex).sum() / np.sqrt((got * got).sum() * (ex * ex).sum())
+    assert cos > 0.9995
+    # zero bias against the unbiased routine (different denominators on the 64-key route: float sums against u8 sums)
+    plain = f(oracle.attn_int8(oracle.BF16, q, k, v, scale, quant=z))
+    zero = f(oracle.attn_int8_bias(oracle.BF16, q, k, v, scale, np.zeros(lk, np.float32), quant=z))
+    assert np.abs(zero - plain).max() <= 0.02
+    if lk > 1024:   # same u8 sums on this route: at most the last tile's float path differs
+        assert np.abs(zero - plain).max() <= 2.0 ** -7 * np.abs(plain).max()
+    # shift invariance
+    shifted = f(oracle.attn_int8_bias(oracle.BF16, q, k, v, scale, bias + 3.0, quant=z))
+    assert np.abs(shifted - got).max() <= 0.02
+    # -inf masks keys: equal to attention over the kept keys only
+    masked = bias.copy()
+    drop = rng.choice(lk, lk // 3, replace=False)
+    masked[drop] = -np.inf
+    got_m = f(oracle.attn_int8_bias(oracle.BF16, q, k, v, scale, masked, quant=z))
+    keep = np.setdiff1d(np.arange(lk), drop)
+    ex_m = _exact_attention(q, k[:, keep], v[:, keep], scale, bias[keep])
+    assert np.abs(got_m - ex_m).max() < 0.04
+    # every key masked: zeros on the 64-key route (the reference's row validity), finite output on the other
+    allm = f(oracle.attn_int8_bias(oracle.BF16, q, k, v, scale, np.full(lk, -np.inf, np.float32), quant=z))
+    assert np.isfinite(allm).all()
+    if lk <= 1024:
+        assert (allm == 0).all()
