@@ -35,6 +35,7 @@ struct AttnArgs {
     int64_t q_bs, q_rs, q_hs, k_bs, k_rs, k_hs, v_bs, v_rs, v_hs, o_bs, o_rs, o_hs;
     float sm, sink;
     int vec_ok, in_vec, v_vec, use_anchor;
+    int rot4;   // lk <= 256: the rotation is only the H4 on runs of four channels, without the sign diagonal
     // per-head RMSNorm (+ weight) and RoPE ahead of the quantizers (csrc/kernels.cu:482-540 through
     // csrc/vendor/sage/quant_qk_int8.cu:160-291): q_norm / k_norm say which of Q and K take it
     const float *qw, *kw, *rope;   // [128] or null (ones); rope [L][64] x (cos, sin) or null
@@ -104,6 +105,19 @@ __device__ __forceinline__ void rot128(float (&v)[16], int o8) {
     }
 #pragma unroll
     for (int e = 0; e < 16; ++e) v[e] *= 0.1767766952966369f;
+}
+
+// The rotation of sequences of at most 256 keys (csrc/vendor/sage/quant_qk_int8.cu:1160-1166, ROTATION 4): the
+// normalized H4 on each run of four adjacent channels and nothing else.
+__device__ __forceinline__ void rot4(float (&v)[16]) {
+#pragma unroll
+    for (int g = 0; g < 16; g += 4) {
+        const float a0 = v[g] + v[g + 1], a1 = v[g] - v[g + 1], a2 = v[g + 2] + v[g + 3], a3 = v[g + 2] - v[g + 3];
+        v[g] = (a0 + a2) * 0.5f;
+        v[g + 1] = (a1 + a3) * 0.5f;
+        v[g + 2] = (a0 - a2) * 0.5f;
+        v[g + 3] = (a1 - a3) * 0.5f;
+    }
 }
 
 __device__ __forceinline__ float max8(float m) {
@@ -364,7 +378,8 @@ __device__ __forceinline__ void quant_q_body(const AttnArgs& a, const int hi, co
     float mx = 0.f;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        rot128(v[j], o8);
+        if (a.rot4) rot4(v[j]);
+        else rot128(v[j], o8);
         if (t * 32 + g + 8 * j < a.lq) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) mx = fmax_nn(mx, fabsf(v[j][e]));
@@ -415,7 +430,8 @@ __device__ __forceinline__ void quant_k_body(const AttnArgs& a, const int hi, co
     for (int j = 0; j < R; ++j) {
 #pragma unroll
         for (int e = 0; e < 16; ++e) v[j][e] -= bias[e];
-        rot128(v[j], o8);
+        if (a.rot4) rot4(v[j]);
+        else rot128(v[j], o8);
         if (t * CK + rt[j] < a.lk) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) mx = fmax_nn(mx, fabsf(v[j][e]));
@@ -553,7 +569,11 @@ typedef const __attribute__((address_space(1))) void* glb_ptr_t;
 // The attention: a workgroup of four waves owns 128 query rows, a wave 32 of them.  The K tile, the V tile and the
 // tile's 128 x column sums are contiguous in the workspace, in the order the fragment reads want them, so the four waves
 // copy them global -> LDS with DMA loads (no registers) into one of two stages, a tile ahead; one barrier per tile.
-template <int OUT_DT, int CK, bool MASK = false>
+// FD (no mask, 64-key tiles): the reference's unfused probability path in every tile, which its build takes for f16
+// outputs and at most 512 keys (csrc/vendor/sage/sage_attn_launcher.cu:187-191, qk_int_sv_i8_cuda.cuh:132-139,637-700):
+// every tile's maximum starts at a raw score of -50000 and the denominator sums the unrounded probabilities in
+// per-thread partials (attn_utils.cuh:922-940).  Without FD only the last tile takes that form.
+template <int OUT_DT, int CK, bool MASK = false, bool FD = false>
 __global__ __launch_bounds__(256, 2) void attn_int8_kernel(AttnArgs a) {
     constexpr int NB = CK / 32, KV = CK * D, STAGE = 2 * KV + 512;
     extern __shared__ __align__(16) uint8_t smem[];
@@ -593,7 +613,7 @@ __global__ __launch_bounds__(256, 2) void attn_int8_kernel(AttnArgs a) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) ro[x][i] = 0.f;
     float m = -50000.f, dsum = 1.f;
-    float dsum2 = 1.f;   // the per-key mask route keeps the reference's four partial denominators per row: two per lane
+    float dsum2 = 0.f;   // the unfused and per-key mask routes keep the reference's four partial denominators per row: two per lane
     bool kept = false;   // that route: some key of this lane was kept
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
@@ -698,28 +718,62 @@ __global__ __launch_bounds__(256, 2) void attn_int8_kernel(AttnArgs a) {
             }
         };
 
-        if constexpr (!MASK) {
-            // Group maxima on the integers (exact in fp32: |score| < 2^24).  Only the last tile can hold keys past lk; its
-            // maxima start at the reference's floor of -50000.
-            int i0, i1;
-            if constexpr (!last) {
-                int_maxima(i0, i1);
-            } else {
-                i0 = i1 = -50000;
+        if constexpr (!MASK && (FD || last)) {
+            // The unfused form: every tile with FD, and the last tile always (the reference's last iteration has no fused
+            // variant, qk_int_sv_i8_cuda.cuh:956-1000).  Maxima start at a raw score of -50000, keys past lk drop out
+            // (-1e30 raw), and the denominator takes the unrounded probabilities, in the two per-thread partials of the
+            // reference that this lane carries (threads 2hh: c = 0, 1 and 2hh + 1: c = 2, 3 of each 16 keys).
+            int i0 = -50000, i1 = -50000;
 #pragma unroll
-                for (int blk = 0; blk < NB; ++blk)
+            for (int blk = 0; blk < NB; ++blk)
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) {
+                for (int i = 0; i < 16; ++i) {
+                    int sv = S[blk][i];
+                    if constexpr (last) {
                         const int key = key0 + blk * 32 + (i / 4) * 8 + hh * 4 + (i % 4);
-                        const int sv = key < a.lk ? S[blk][i] : INT_MIN;
-                        if ((i % 4) < 2) i0 = max(i0, sv);
-                        else i1 = max(i1, sv);
+                        sv = key < a.lk ? sv : INT_MIN;
                     }
-            }
+                    if ((i % 4) < 2) i0 = max(i0, sv);
+                    else i1 = max(i1, sv);
+                }
             tile_m = fmax_nn(fmaf((float)i0, gs0, -kU8Offset), fmaf((float)i1, gs1, -kU8Offset));
             rescale();
             dsum *= o_scale;
-            probabilities(last_tag, -tile_m);
+            dsum2 *= o_scale;
+#pragma unroll
+            for (int blk = 0; blk < NB; ++blk) {
+                uint32_t w[4];
+                float e[4][4];
+#pragma unroll
+                for (int g4 = 0; g4 < 4; ++g4) {
+                    uint32_t packed = 0u;
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        e[g4][c] = __builtin_amdgcn_exp2f(fmaf((float)S[blk][g4 * 4 + c], c < 2 ? gs0 : gs1, -tile_m));
+                        if constexpr (last) {
+                            const int key = key0 + blk * 32 + g4 * 8 + hh * 4 + c;
+                            e[g4][c] = key < a.lk ? e[g4][c] : 0.f;
+                        }
+                        packed = __builtin_amdgcn_cvt_pk_u8_f32(e[g4][c], c, packed);
+                    }
+                    w[g4] = packed ^ 0x80808080u;
+                }
+#pragma unroll
+                for (int fk = 0; fk < 2; ++fk) {
+                    dsum += ((e[2 * fk][0] + e[2 * fk][1]) + (e[2 * fk + 1][0] + e[2 * fk + 1][1])) * t_scale;
+                    dsum2 += ((e[2 * fk][2] + e[2 * fk][3]) + (e[2 * fk + 1][2] + e[2 * fk + 1][3])) * t_scale;
+                }
+                pf[blk] = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        } else if constexpr (!MASK) {
+            // Group maxima on the integers (exact in fp32: |score| < 2^24).
+            int i0, i1;
+            int_maxima(i0, i1);
+            tile_m = fmax_nn(fmaf((float)i0, gs0, -kU8Offset), fmaf((float)i1, gs1, -kU8Offset));
+            rescale();
+            dsum *= o_scale;
+            probabilities(std::false_type{}, -tile_m);
             dsum += (float)psum * t_scale;
         } else {
             // this lane's prepared biases: four consecutive keys per (blk, g4)
@@ -813,7 +867,7 @@ __global__ __launch_bounds__(256, 2) void attn_int8_kernel(AttnArgs a) {
     for (int t = 0; t + 1 < a.kb; ++t) tile(t, std::false_type{});
     tile(a.kb - 1, std::true_type{});
 
-    if constexpr (MASK && CK == 64) dsum += dsum2;   // (d0 + d1) and (d2 + d3) of the reference's four threads
+    dsum += dsum2;   // (d0 + d1) and (d2 + d3) of the reference's four threads
     float dtot = dsum + __shfl_xor(dsum, 32);
     bool row_kept = true;
     if constexpr (MASK && CK == 64) row_kept = (__shfl_xor((int)kept, 32) | (int)kept) != 0;   // a row with no kept key gives zeros
@@ -934,7 +988,8 @@ int run(AttnArgs a, hipStream_t st) {
         }
         return hipGetLastError() == hipSuccess ? 0 : -401;
     }
-    if (a.ck == 64) attn_int8_kernel<DT, 64><<<grid, 256, kLds64, st>>>(a);
+    if (DT == DT_F16 && a.lk <= 512 && a.ck == 64) attn_int8_kernel<DT_F16, 64, false, true><<<grid, 256, kLds64, st>>>(a);
+    else if (a.ck == 64) attn_int8_kernel<DT, 64><<<grid, 256, kLds64, st>>>(a);
     else attn_int8_kernel<DT, 128><<<grid, 256, kLds128, st>>>(a);
     return hipGetLastError() == hipSuccess ? 0 : -401;
 }
@@ -977,6 +1032,7 @@ int int8_attn(const void* q, const void* k, const void* v, void* o, void* ws, in
     a.q_bs = q_bs; a.q_rs = q_rs; a.q_hs = q_hs; a.k_bs = k_bs; a.k_rs = k_rs; a.k_hs = k_hs;
     a.v_bs = v_bs; a.v_rs = v_rs; a.v_hs = v_hs; a.o_bs = o_bs; a.o_rs = o_rs; a.o_hs = o_hs;
     a.sm = scale * 1.44269504088896340736f;
+    a.rot4 = lk <= 256 ? 1 : 0;
     a.sink = sink;
     a.use_anchor = sink == 0.f ? 1 : 0;   // with a sink a zero key's score must stay zero: no shift (csrc/attn_int8.cu:134-141)
     a.vec_ok = ((o_bs | o_rs | o_hs) % 4 == 0 && ((uintptr_t)o & 7) == 0) ? 1 : 0;
@@ -1003,7 +1059,7 @@ int int8_attn(const void* q, const void* k, const void* v, void* o, void* ws, in
 }  // namespace
 
 GPU_API int64_t gpu_int8_attn_workspace_d(int b, int h, int hk, int lq, int lk, int head_dim) {
-    (void)head_dim;
+    if (head_dim != D) return 0;   // only head dim 128 is built: no size that a caller could mistake for a usable one
     if (b <= 0 || h <= 0 || hk <= 0 || lq <= 0 || lk <= 0) return 0;
     return plan_for(b, h, hk, lq, lk).total;
 }

@@ -67,7 +67,9 @@ __device__ __forceinline__ void dma4(uint32_t lds_dst, uint32_t lane_off, const 
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds_dst), "v"(lane_off), "s"(base) : "memory", "m0");
 }
 
-template <int OUT_DT, bool DUMP>
+// ABL (measurement only, wrong results): bit 0 leaves out the fp32 fold, bit 1 the unpack, bit 2 the DMA of the MFMA
+// waves after the prologue; what remains shows what each part costs next to the MFMAs.
+template <int OUT_DT, bool DUMP, int ABL = 0>
 __global__ void __launch_bounds__(NT, 1) w6a8_group_gemm_kernel(W6Args p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -177,6 +179,10 @@ __global__ void __launch_bounds__(NT, 1) w6a8_group_gemm_kernel(W6Args p) {
 
     // fp32 fold of four values: register group q of tile im.  accf += float(part) * sw[n, g]
     auto fold = [&](int im, int q, const float4& s4) {
+        if (ABL & 1) {   // keep the partials alive with one operation per register group instead of eight
+            accf[0][im][4 * q] += __builtin_bit_cast(float, part[0][im][4 * q] ^ part[0][im][4 * q + 1] ^ part[0][im][4 * q + 2] ^ part[0][im][4 * q + 3]);
+            return;
+        }
         const float sv[4] = {s4.x, s4.y, s4.z, s4.w};
 #pragma unroll
         for (int c = 0; c < 4; ++c)
@@ -219,7 +225,8 @@ __global__ void __launch_bounds__(NT, 1) w6a8_group_gemm_kernel(W6Args p) {
 
         // The wave's own packed rows of group g+1 were the first two DMA instructions of the previous iteration; the
         // five issued after them may still be in flight.
-        wait_vmcnt_n<5>();
+        if (ABL & 4) wait_all_dma();
+        else wait_vmcnt_n<5>();
         // everything this iteration reads from LDS early: fragments of the first pair, the group's scales, packed words
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk) fw[kk] = *reinterpret_cast<const v4i*>(su + woff[kk]);
@@ -230,7 +237,8 @@ __global__ void __launch_bounds__(NT, 1) w6a8_group_gemm_kernel(W6Args p) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) sv[q] = *reinterpret_cast<const float4*>(sc + wn * 32 + 8 * q + 4 * fhalf);
 #pragma unroll
-        for (int i = 0; i < 2; ++i) raw_read(s ^ 1, i, raw[i]);
+        for (int i = 0; i < 2; ++i)
+            if (!(ABL & 2)) raw_read(s ^ 1, i, raw[i]);
         SCHED_FENCE();
         if (defer && g > 0) {   // the fold the previous iteration left over
 #pragma unroll
@@ -246,18 +254,24 @@ __global__ void __launch_bounds__(NT, 1) w6a8_group_gemm_kernel(W6Args p) {
         // group g-2, all of them last read before the barrier that ended iteration g-1.
         mma_pair(0, fa, [&](int i) {
             na[i & 1][i >> 1] = *reinterpret_cast<const v4i*>(sa + aoff[i >> 1] + (2 + (i & 1)) * 32 * BK);
-            if (i == 1) dma_raw(g + 2, s, 0);
-            if (i == 3) dma_raw(g + 2, s, 1);
-            if (i == 5) dma_a(g + 2, a_new, 0);
-            if (i == 7) dma_a(g + 2, a_new, 1);
-            if (i == 2) unpack_write(s ^ 1, 0, raw[0]);
-            if (i == 4) unpack_write(s ^ 1, 1, raw[1]);
+            if (!(ABL & 4)) {
+                if (i == 1) dma_raw(g + 2, s, 0);
+                if (i == 3) dma_raw(g + 2, s, 1);
+                if (i == 5) dma_a(g + 2, a_new, 0);
+                if (i == 7) dma_a(g + 2, a_new, 1);
+            }
+            if (!(ABL & 2)) {
+                if (i == 2) unpack_write(s ^ 1, 0, raw[0]);
+                if (i == 4) unpack_write(s ^ 1, 1, raw[1]);
+            }
         });
         mma_pair(2, na, [&](int i) {
             fold(i & 1, i >> 1, sv[i >> 1]);
-            if (i == 1) dma_a(g + 2, a_new, 2);
-            if (i == 3) dma_a(g + 2, a_new, 3);
-            if (i == 5) dma_scales(g + 2, s_new);
+            if (!(ABL & 4)) {
+                if (i == 1) dma_a(g + 2, a_new, 2);
+                if (i == 3) dma_a(g + 2, a_new, 3);
+                if (i == 5) dma_scales(g + 2, s_new);
+            }
         });
         if (!defer) {
 #pragma unroll
@@ -275,7 +289,8 @@ __global__ void __launch_bounds__(NT, 1) w6a8_group_gemm_kernel(W6Args p) {
                 }
             wait_all_dma();   // the dump's stores share the counter: drain it rather than count them
         }
-        wait_vmcnt_n<7>();   // everything older than this iteration's seven has landed: A and scales of group g+1
+        if (ABL & 4) wait_all_dma();
+        else wait_vmcnt_n<7>();   // everything older than this iteration's seven has landed: A and scales of group g+1
         __syncthreads();     // ... for every wave, and the expanded weights of group g+1 are written
         a_cur = a_cur == 2 ? 0 : a_cur + 1;
         s_cur = (s_cur + 1) & 3;
@@ -375,9 +390,9 @@ __global__ void __launch_bounds__(NT, 1) w6a8_group_gemm_kernel(W6Args p) {
     }
 }
 
-template <int OUT_DT, bool DUMP>
+template <int OUT_DT, bool DUMP, int ABL = 0>
 int launch(W6Args a, hipStream_t st) {
-    auto kern = w6a8_group_gemm_kernel<OUT_DT, DUMP>;
+    auto kern = w6a8_group_gemm_kernel<OUT_DT, DUMP, ABL>;
     static bool once = false;  // benign race: the attribute is idempotent
     if (!once) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
@@ -414,5 +429,27 @@ GPU_API int gpu_w6a8_group_gemm(const int8_t* A, const void* Wp, const float* xs
         case DT_F32: return launch_dt<DT_F32>(a, st);
         case DT_F16: return launch_dt<DT_F16>(a, st);
         default: return launch_dt<DT_BF16>(a, st);
+    }
+}
+
+// Measurement hook, no reference counterpart: gpu_w6a8_group_gemm (bf16 output) with parts of the kernel left out --
+// ablate bit 0 the fp32 fold, bit 1 the unpack, bit 2 the LDS-DMA after the prologue.  D receives meaningless values.
+GPU_API int gpu_internal_w6a8_group_gemm_ablate(int ablate, const int8_t* A, const void* Wp, const float* xs, const float* sw,
+                                                void* D, int64_t M, int64_t N, int64_t K, void* stream) {
+    if (K <= 0 || (K % 128) != 0 || M <= 0 || N <= 0 || M * K >= ((int64_t)1 << 32) || N * (K / 4 * 3) >= ((int64_t)1 << 32)) return -200;
+    W6Args a{A, (const uint8_t*)Wp, xs, sw, nullptr, D, nullptr, (int)M, (int)N, (int)K, (int)(K / 128), 0, 0};
+    a.tiles_m = (int)((M + BM - 1) / BM);
+    a.tiles_n = (int)((N + BN - 1) / BN);
+    hipStream_t st = (hipStream_t)stream;
+    switch (ablate) {
+        case 0: return launch<DT_BF16, false, 0>(a, st);
+        case 1: return launch<DT_BF16, false, 1>(a, st);
+        case 2: return launch<DT_BF16, false, 2>(a, st);
+        case 3: return launch<DT_BF16, false, 3>(a, st);
+        case 4: return launch<DT_BF16, false, 4>(a, st);
+        case 5: return launch<DT_BF16, false, 5>(a, st);
+        case 6: return launch<DT_BF16, false, 6>(a, st);
+        case 7: return launch<DT_BF16, false, 7>(a, st);
+        default: return -200;
     }
 }

@@ -48,6 +48,7 @@ SIGNATURES = {
     "gpu_int8_attn_key_bias": [_P, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _I32] + [_I64] * 12 + [_F32, _P, _P],
     "gpu_internal_cvt_pk_u8_probe": [_P, _P, _I32, _P],
     "gpu_internal_attn_sumsq_probe": [_P, _P, _I32, _I32, _P],
+    "gpu_internal_w6a8_group_gemm_ablate": [_I32, _P, _P, _P, _P, _P, _I64, _I64, _I64, _P],
     "gpu_internal_attn_layout": [_I32, _I32, _I32, _I32, _I32, _P],
     "gpu_int8_gemm_force_config": [_I32],
     "gpu_act_tables_init": [],

@@ -124,7 +124,8 @@ int gpu_w6_requant(const void* weight, void* packed, void* s_rel, void* s_channe
  * device scratch of gpu_int8_attn_workspace[_d] bytes, layout private to the library.
  * Replaces gpu_int8_attn_workspace_d / gpu_int8_attn_workspace (csrc/attn_int8.cu:62-82), gpu_int8_attn_d (:101-108),
  * gpu_int8_attn_f16 (:111-118), gpu_int8_attn (:225-231); src/ffi.rs binds them under the same names.
- * Returns 0, -400 (argument the library refuses: message on stderr; head dims other than 128 are not built) or -401
+ * Returns 0, -400 (argument the library refuses: message on stderr; head dims other than 128 are not built, and
+ * gpu_int8_attn_workspace_d returns 0 bytes for them) or -401
  * (launch failure), the reference's codes.
  * gpu_int8_attn_sink (csrc/attn_int8.cu:193-202): attention over lk keys plus `sink` more whose keys and values are
  * zero, which count in the softmax denominator only; the K anchor is off so that a zero key's score stays zero; bf16.
@@ -175,6 +176,12 @@ int gpu_int8_attn_key_bias(const void* q, const void* k, const void* v, void* o,
 /* Test hook, no reference counterpart: y[i] = the gfx950 float -> u8 pack conversion of x[i] (byte 0), which the attention
  * kernel's probabilities rely on being round-to-nearest-even with saturation to 0..255. */
 int gpu_internal_cvt_pk_u8_probe(const float* x, uint32_t* y, int n, void* stream);
+
+/* Measurement hook, no reference counterpart: gpu_w6a8_group_gemm (bf16 output, no bias) with parts of its kernel left
+ * out, to show what each costs next to the MFMAs: ablate bit 0 the fp32 fold, bit 1 the unpack, bit 2 the LDS-DMA after
+ * the prologue (0..7).  D receives meaningless values unless ablate is 0. */
+int gpu_internal_w6a8_group_gemm_ablate(int ablate, const int8_t* A, const void* Wp, const float* xs, const float* sw, void* D,
+                                        int64_t M, int64_t N, int64_t K, void* stream);
 
 /* Test hook, no reference counterpart: sums of squares of rows of 128 floats in the order the fused norm of
  * gpu_int8_attn_norm_rope takes them; out[2r] from the quantizers' eight-lane form, out[2r+1] from the anchor search's

@@ -65,6 +65,8 @@ def lib():
                                              vp, vp, vp, i32, vp, vp, vp, C.c_float, i32]
         L.orc_attn_int8_bias.restype = i32
         L.orc_attn_int8_bias.argtypes = [i32, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, C.c_float, vp, vp, i64, i64, i64]
+        L.orc_attn_rotate.restype = None
+        L.orc_attn_rotate.argtypes = [vp, i32]
         L.orc_attn_sumsq128.restype = C.c_float
         L.orc_attn_sumsq128.argtypes = [vp, i32]
         L.orc_attn_norm_rope_row.restype = None
@@ -72,7 +74,7 @@ def lib():
         L.orc_attn_quant_qk.argtypes = [i32, vp, vp, i32, i32, i32, i32, i32, i64, i64, i64, i64, i64, i64, i32, i32, vp, vp, vp, vp, vp]
         L.orc_attn_quant_v.restype = i32; L.orc_attn_quant_v.argtypes = [i32, vp, i32, i32, i32, i64, i64, i64, vp, vp]
         L.orc_attn_int8.restype = i32
-        L.orc_attn_int8.argtypes = [i32, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, f32, vp, i64, i64, i64]
+        L.orc_attn_int8.argtypes = [i32, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, f32, vp, i64, i64, i64, i32]
         L.orc_attn_cta_k.restype = i32; L.orc_attn_cta_k.argtypes = [i32, i32]
         _lib = L
     return _lib
@@ -370,6 +372,15 @@ def attn_norm_rope_row(row, w, rope_row, eps, rope_mode):
     return r
 
 
+def attn_rotate(row, lk):
+    """The rotation the Q/K quantizers apply for a sequence of lk keys: H4 on runs of four channels up to 256 keys, the
+    sign diagonal and H128 beyond."""
+    r = np.ascontiguousarray(row, dtype=np.float32).copy()
+    assert r.shape == (128,)
+    lib().orc_attn_rotate(_p(r), int(lk))
+    return r
+
+
 def attn_quant(dt, q, k, v, use_anchor=True, norm=None):
     """q [b,lq,h,128], k/v [b,lk,hk,128] contiguous (uint16 bits for bf16/f16).  Returns a dict with the int8 tensors
     in [b,heads,len,128] order, the scales, the anchors and the key tile length.  norm = dict(qw, kw, rope, eps,
@@ -426,6 +437,7 @@ def attn_int8(dt, q, k, v, scale, use_anchor=True, quant=None, sink=0.0, norm=No
     z = quant if quant is not None else attn_quant(dt, q, k, v, use_anchor, norm)
     o = np.zeros((b, lq, h, D), np.float32 if dt == F32 else np.uint16)
     rc = lib().orc_attn_int8(dt, _p(z["qi"]), _p(z["ki"]), _p(z["vi"]), _p(z["qs"]), _p(z["ks"]), _p(z["vs"]), b, lq, lk,
-                             h, hk, z["ck"], float(scale), float(sink), _p(o), lq * h * D, h * D, D)
+                             h, hk, z["ck"], float(scale), float(sink), _p(o), lq * h * D, h * D, D,
+                             1 if (dt == F16 and lk <= 512 and z["ck"] == 64) else 0)
     assert rc == 0
     return o

@@ -793,6 +793,23 @@ ORC_API void orc_attn_rot128(float* v) {
     for (int ch = 0; ch < ATTN_D; ++ch) v[ch] *= 0.1767766952966369f;
 }
 
+/* The rotation the quantizers apply, chosen by the key count (csrc/vendor/sage/quant_qk_int8.cu:1160-1166): sequences
+ * of at most 256 keys take only the normalized H4 on each run of four adjacent channels (ROTATION 4, convrot4 :72-85),
+ * longer ones the sign diagonal and H128. */
+ORC_API void orc_attn_rotate(float* v, int lk) {
+    if (lk > 256) {
+        orc_attn_rot128(v);
+        return;
+    }
+    for (int g = 0; g < ATTN_D; g += 4) {
+        const float a0 = v[g] + v[g + 1], a1 = v[g] - v[g + 1], a2 = v[g + 2] + v[g + 3], a3 = v[g + 2] - v[g + 3];
+        v[g] = (a0 + a2) * 0.5f;
+        v[g + 1] = (a1 + a3) * 0.5f;
+        v[g + 2] = (a0 - a2) * 0.5f;
+        v[g + 3] = (a1 - a3) * 0.5f;
+    }
+}
+
 static inline int8_t attn_rn_s8(float v) {                       /* cvt.rni.sat.s8.f32, float_utils.cuh:39-45 */
     if (isnan(v)) return 0;
     const float r = rintf(v);
@@ -915,7 +932,7 @@ static int attn_detect_anchor(int dt, const void* k, int64_t base, int64_t strid
  * rotated, abs-max over the group, scale = max/127 + 1e-7, codes = rn(v * (1/scale))
  * (quant_qk_int8.cu:296-413 for Q, :422-575 for K). */
 static void attn_quant_group(int dt, const void* x, int64_t base, int64_t stride_n, const int* rows, int n, int L,
-                             const float* bias, const attn_norm_t* nm, int8_t* out, float* scale) {
+                             const float* bias, const attn_norm_t* nm, int lk, int8_t* out, float* scale) {
     float buf[32][ATTN_D];
     float mx = 0.f;
     for (int i = 0; i < n; ++i) {
@@ -923,7 +940,7 @@ static void attn_quant_group(int dt, const void* x, int64_t base, int64_t stride
         attn_load_row(dt, x, base, stride_n, rows[i], nm, buf[i]);
         if (bias)
             for (int c = 0; c < ATTN_D; ++c) buf[i][c] -= bias[c];
-        orc_attn_rot128(buf[i]);
+        orc_attn_rotate(buf[i], lk);
         for (int c = 0; c < ATTN_D; ++c) mx = fmax_dev(mx, fabsf(buf[i][c]));
     }
     const float sc = mx / 127.f + 1e-7f, inv = 1.f / sc;
@@ -953,7 +970,7 @@ ORC_API int orc_attn_quant_qk_norm(int dt, const void* q, const void* k, int b, 
                     int rows[4];
                     for (int j = 0; j < 4; ++j) rows[j] = t * 32 + g + 8 * j;
                     const int64_t bh = (int64_t)bi * h + hi;
-                    attn_quant_group(dt, q, bi * q_bs + hi * q_hs, q_rs, rows, 4, lq, NULL, &qn, qi + bh * lq * ATTN_D,
+                    attn_quant_group(dt, q, bi * q_bs + hi * q_hs, q_rs, rows, 4, lq, NULL, &qn, lk, qi + bh * lq * ATTN_D,
                                      &qs[(bh * qg + t) * 8 + g]);
                 }
     for (int bi = 0; bi < b; ++bi)
@@ -968,7 +985,7 @@ ORC_API int orc_attn_quant_qk_norm(int dt, const void* q, const void* k, int b, 
                     int rows[32];
                     const int n = ck / 4;
                     for (int i = 0; i < n; ++i) rows[i] = t * ck + (i / 2) * 8 + g * 2 + (i % 2);
-                    attn_quant_group(dt, k, base, k_rs, rows, n, lk, anchor >= 0 ? bias : NULL, &kn, ki + bh * lk * ATTN_D,
+                    attn_quant_group(dt, k, base, k_rs, rows, n, lk, anchor >= 0 ? bias : NULL, &kn, lk, ki + bh * lk * ATTN_D,
                                      &ks[(bh * kb + t) * 4 + g]);
                 }
         }
@@ -1015,10 +1032,14 @@ static inline float attn_exp2(float x) { return (float)exp2((double)x); }
  * exp2(fma(score, scale, -tile_max)) rounded to u8 (:700-717, mma.cuh:793-804); denominators and outputs rescaled by
  * exp2(-|m_prev - tile_max|) on whichever side is smaller (:742-756); outputs += float(sum p*v) * tile_scale by fmaf
  * (:1254-1258); O = RO / d * v_scale (:1130-1146, qk_int_sv_i8_cuda.cuh:1056-1072).  The denominator is summed here
- * per row in key order; the reference keeps four per-thread partials. */
+ * per row in key order; the reference keeps four per-thread partials.
+ * The last tile always takes the reference's unfused form (qk_int_sv_i8_cuda.cuh:956-1000: maximum from a raw score
+ * of -50000, keys past lk at -1e30 raw, the denominator summing the UNROUNDED probabilities in the four per-thread
+ * partials of a row, attn_utils.cuh:922-940, :1113-1122).  unfused: every tile takes it, which is what the reference's
+ * build does for f16 outputs and at most 512 keys (sage_attn_launcher.cu:187-191, qk_int_sv_i8_cuda.cuh:132-139). */
 ORC_API int orc_attn_int8(int out_dt, const int8_t* qi, const int8_t* ki, const int8_t* vi, const float* qs,
                           const float* ks, const float* vs, int b, int lq, int lk, int h, int hk, int ck, float scale,
-                          float sink, void* o, int64_t o_bs, int64_t o_rs, int64_t o_hs) {
+                          float sink, void* o, int64_t o_bs, int64_t o_rs, int64_t o_hs, int unfused) {
     if ((ck != 64 && ck != 128) || hk <= 0 || h % hk != 0) return -1;
     const int qg = (lq + 127) / 128 * 4, kb = (lk + ck - 1) / ck, rep = h / hk;
     const float sm = scale * 1.44269504088896340736f;
@@ -1029,7 +1050,7 @@ ORC_API int orc_attn_int8(int out_dt, const int8_t* qi, const int8_t* ki, const 
             const int64_t kvh = (int64_t)bi * hk + hi / rep;
             const int8_t* qrow = qi + ((int64_t)bh * lq + r) * ATTN_D;
             const float q_scale = qs[((int64_t)bh * qg + r / 32) * 8 + r % 8];
-            float m = -50000.f, d = 1.f, ro[ATTN_D];
+            float m = -50000.f, d = 1.f, ro[ATTN_D], d4[4] = {0.f, 0.f, 0.f, 0.f}, pf[128];
             for (int c = 0; c < ATTN_D; ++c) ro[c] = 0.f;
             int32_t s[128];
             for (int t = 0; t < kb; ++t) {
@@ -1044,7 +1065,7 @@ ORC_API int orc_attn_int8(int out_dt, const int8_t* qi, const int8_t* ki, const 
                     s[j] = acc;
                 }
                 for (int g = 0; g < 4; ++g) {
-                    float mg = last ? -50000.f : -3.0e38f;
+                    float mg = (last || unfused) ? -50000.f : -3.0e38f;
                     int any = 0;
                     for (int j = 0; j < n; ++j)
                         if ((j % 8) / 2 == g) { mg = fmax_dev(mg, (float)s[j]); any = 1; }
@@ -1055,23 +1076,36 @@ ORC_API int orc_attn_int8(int out_dt, const int8_t* qi, const int8_t* ki, const 
                 const float smaller = attn_exp2(-fabsf(m - tile_m));
                 const float o_scale = m < tile_m ? smaller : 1.f, t_scale = tile_m < m ? smaller : 1.f;
                 m = m > tile_m ? m : tile_m;
-                d *= o_scale;
                 int32_t pv[ATTN_D];
                 int32_t psum = 0;
                 for (int c = 0; c < ATTN_D; ++c) pv[c] = 0;
+                for (int j = n; j < ck; ++j) pf[j] = 0.f;       /* keys past lk: -1e30 raw, probability zero */
                 for (int j = 0; j < n; ++j) {
                     float p = attn_exp2(fmaf((float)s[j], gs[(j % 8) / 2], -tile_m));
+                    pf[j] = p;
                     p = rintf(p > 255.f ? 255.f : p);
                     const int32_t pi = (int32_t)p;
                     psum += pi;
                     const int8_t* vrow = vi + ((int64_t)kvh * lk + t * ck + j) * ATTN_D;
                     for (int c = 0; c < ATTN_D; ++c) pv[c] += pi * (int32_t)vrow[c];
                 }
-                d += (float)psum * t_scale;
+                d *= o_scale;
+                for (int l = 0; l < 4; ++l) d4[l] *= o_scale;
+                if (unfused || last) {
+                    /* the unrounded probabilities in the four per-thread partials of a row */
+                    for (int fk = 0; fk < ck / 16; ++fk)
+                        for (int l = 0; l < 4; ++l) {
+                            const float* q4 = pf + fk * 16;
+                            d4[l] += ((q4[2 * l] + q4[2 * l + 1]) + (q4[8 + 2 * l] + q4[8 + 2 * l + 1])) * t_scale;
+                        }
+                } else {
+                    d += (float)psum * t_scale;
+                }
                 for (int c = 0; c < ATTN_D; ++c) ro[c] = fmaf((float)pv[c], t_scale, ro[c] * o_scale);
             }
             /* `sink` more keys of score zero and value zero: each adds exp2(0 - m) to the denominator and nothing to
              * the output (attn_utils.cuh:1122-1130, csrc/attn_int8.cu:193-197) */
+            d += (d4[0] + d4[1]) + (d4[2] + d4[3]);
             if (sink != 0.f) d = fmaf(sink, attn_exp2(-m), d);
             const float rcp = 1.f / d;
             for (int c = 0; c < ATTN_D; ++c)

@@ -421,6 +421,8 @@ def test_attention_refuses_what_it_does_not_build():
     p = lambda t: C.c_void_p(t.data_ptr())
     args = lambda D, h, hk: (p(x), p(x), p(x), p(x), p(ws), 1, 4, 4, h, hk, D, 512, 128, 128, 512, 128, 128, 512, 128, 128, 512, 128, 128, 0.1, None)
     assert ffi.raw("gpu_int8_attn_d", *args(64, 1, 1)) == -400
+    assert ffi.lib.gpu_int8_attn_workspace_d(1, 1, 1, 4, 4, 64) == 0 and ffi.lib.gpu_int8_attn_workspace_d(1, 1, 1, 4, 4, 256) == 0
+    assert ffi.lib.gpu_int8_attn_workspace_d(1, 1, 1, 4, 4, 128) > 0
     assert ffi.raw("gpu_int8_attn_d", *args(128, 3, 2)) == -400
     assert ffi.raw("gpu_int8_attn_d", *args(128, 1, 1)) == 0
     torch.cuda.synchronize()
@@ -532,3 +534,21 @@ def test_attention_key_bias_moves_weight_to_the_biased_keys():
         o = ql.int8_attn_key_bias(q.cuda(), k.cuda(), v.cuda(), 128 ** -0.5, bias.cuda())
         want = v[0, lk // 2, 0].float()
         assert (o[0, :, 0].float().cpu() - want).abs().max() < 2 * float(v.float().abs().max()) / 127 + 0.02
+
+
+@pytest.mark.parametrize("amp", [1.0, 1e-3])
+def test_attention_f16_short_sequences_take_the_unfused_path(amp):
+    """f16 with at most 512 keys: float denominators in every tile.  Against the oracle, which pins that path on the
+    CPU, and against exact attention (keys past lk weigh nothing, also with tiny q and k)."""
+    ql, ffi = _pkg()
+    b, lq, lk, h, hk = 1, 70, 100, 2, 1
+    q, k, v = _inputs(b, lq, lk, h, hk, torch.float32, seed=8)
+    q, k, v = (q * amp).half(), (k * amp).half(), v.half()
+    ref = _to_f32(oracle.attn_int8(oracle.F16, _bits(q), _bits(k), _bits(v), 0.088), oracle.F16)
+    got = _to_f32(_bits(ql.int8_attn(q.cuda(), k.cuda(), v.cuda(), 0.088)), oracle.F16)
+    vmax = float(v.float().abs().max())
+    tol = 2 * vmax / 255.0 + 2 * 2.0 ** -11 * np.abs(ref)
+    assert (np.abs(got - ref) <= tol).all()
+    ex = _exact(q, k, v, 0.088)
+    cos = float((got * ex).sum() / np.sqrt((got * got).sum() * (ex * ex).sum()))
+    assert cos > 0.9995, cos

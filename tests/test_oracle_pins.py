@@ -942,13 +942,19 @@ def _attn_case(b, lq, lk, h, hk, seed, k_offset=0.0):
     return q, k, v, bits
 
 
-def test_attn_quantizers_scale_groups_and_half_step_bound():
+@pytest.mark.parametrize("lk", [150, 300])
+def test_attn_quantizers_scale_groups_and_half_step_bound(lk):
     """Dequantized codes sit within half a step of the rotated rows, the step being the group's scale; the groups are the
-    ones the layout says (rows r, r+8, .. for Q; keys with equal (key % 8) / 2 per tile for K); V per channel."""
+    ones the layout says (rows r, r+8, .. for Q; keys with equal (key % 8) / 2 per tile for K); V per channel.  The
+    rotation is the one the key count selects: H4 blocks up to 256 keys, sign diagonal and H128 beyond."""
     import scipy.linalg
-    H = scipy.linalg.hadamard(128).astype(np.float64) / np.sqrt(128.0)
-    sg = _attn_sign_vector()
-    q, k, v, bits = _attn_case(1, 70, 150, 2, 1, seed=2)
+    if lk > 256:
+        H = scipy.linalg.hadamard(128).astype(np.float64) / np.sqrt(128.0)
+        sg = _attn_sign_vector()
+    else:
+        H = np.kron(np.eye(32), scipy.linalg.hadamard(4).astype(np.float64) * 0.5)
+        sg = np.ones(128)
+    q, k, v, bits = _attn_case(1, 70, lk, 2, 1, seed=2)
     z = oracle.attn_quant(oracle.BF16, bits(q), bits(k), bits(v), use_anchor=False)
     assert z["ck"] == 64 and oracle.lib().orc_attn_cta_k(1025, 128) == 128 and oracle.lib().orc_attn_cta_k(4096, 64) == 64
     rq = (q.double().numpy() * sg) @ H.T                                 # [1, lq, h, 128]
@@ -957,11 +963,11 @@ def test_attn_quantizers_scale_groups_and_half_step_bound():
         for hi in range(2):
             sc = z["qs"][0, hi, (r // 32) * 8 + r % 8]
             assert np.abs(z["qi"][0, hi, r] * np.float64(sc) - rq[0, r, hi]).max() <= 0.5 * sc * 1.0001 + 1e-6
-    for n in range(150):
+    for n in range(lk):
         sc = z["ks"][0, 0, (n // 64) * 4 + (n % 8) // 2]
         assert np.abs(z["ki"][0, 0, n] * np.float64(sc) - rk[0, n, 0]).max() <= 0.5 * sc * 1.0001 + 1e-6
     # every group's largest code reaches the ends of the int8 range: the scale is the group's abs-max / 127
-    grp = np.array([(n // 64) * 4 + (n % 8) // 2 for n in range(150)])
+    grp = np.array([(n // 64) * 4 + (n % 8) // 2 for n in range(lk)])
     for gi in np.unique(grp):
         assert np.abs(z["ki"][0, 0, grp == gi].astype(int)).max() in (126, 127)
     vs = z["vs"][0, 0]
@@ -1180,3 +1186,40 @@ def test_attn_key_bias_against_exact_attention_and_its_invariants(lk):
     assert np.isfinite(allm).all()
     if lk <= 1024:
         assert (allm == 0).all()
+
+
+def test_attn_rotation_is_chosen_by_the_key_count():
+    """Up to 256 keys the quantizers rotate with the normalized H4 on runs of four channels only (no sign diagonal);
+    beyond, with the sign diagonal and H128.  Against the dense matrices."""
+    import scipy.linalg
+    rng = np.random.default_rng(3)
+    x = rng.integers(-8, 9, 128).astype(np.float32)           # small integers: every sum is exact
+    h4 = np.kron(np.eye(32), scipy.linalg.hadamard(4) * 0.5)
+    for lk in (1, 64, 256):
+        assert np.array_equal(oracle.attn_rotate(x, lk), (h4 @ x).astype(np.float32))
+    for lk in (257, 5000):
+        assert np.array_equal(oracle.attn_rotate(x, lk), oracle.attn_rot128(x))
+    assert not np.array_equal(oracle.attn_rotate(x, 256), oracle.attn_rotate(x, 257))
+    # both are orthogonal: the row's energy is kept
+    y = rng.standard_normal(128).astype(np.float32)
+    for lk in (256, 257):
+        assert abs(float((oracle.attn_rotate(y, lk).astype(np.float64) ** 2).sum()) - float((y.astype(np.float64) ** 2).sum())) < 1e-3
+
+
+def test_attn_unfused_path_for_f16_short_sequences():
+    """f16 outputs with at most 512 keys take the reference's unfused probability path in every tile (float
+    denominators, maxima from a raw -50000): the same attention as float64 softmax to the usual tolerance, also with a
+    ragged last tile and with tiny scales (keys past lk weigh nothing)."""
+    rng = np.random.default_rng(12)
+    b, lq, h, hk = 1, 20, 1, 1
+    hb = lambda a: oracle.f16_bits(np.asarray(a, np.float32))
+    f = lambda o: oracle.f16_to_f32(o).astype(np.float64)
+    for lk, amp in ((128, 1.0), (100, 1.0), (100, 1e-3), (300, 1.0)):
+        q, k, v = (hb(rng.standard_normal(s) * amp) for s in ((b, lq, h, 128), (b, lk, hk, 128), (b, lk, hk, 128)))
+        z = oracle.attn_quant(oracle.F16, q, k, v)
+        got = f(oracle.attn_int8(oracle.F16, q, k, v, 0.088, quant=z))
+        qf, kf, vf = (oracle.f16_to_f32(t).astype(np.float64) for t in (q, k, v))
+        logits = np.einsum("bqhd,bkhd->bhqk", qf, kf) * 0.088
+        p = np.exp(logits - logits.max(-1, keepdims=True))
+        ex = np.einsum("bhqk,bkhd->bqhd", p / p.sum(-1, keepdims=True), vf)
+        assert np.abs(got - ex).max() < 0.04
