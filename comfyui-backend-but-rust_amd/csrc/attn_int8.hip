@@ -20,8 +20,11 @@
 
 namespace {
 
-constexpr int D = 128;
 constexpr float kU8Offset = 7.9943534f;
+// Head dims 64, 128 and 256 (csrc/attn_int8.cu:42-45).  A row's channels lie on D/16 consecutive lanes, sixteen channels
+// each; the Q quantizer's row block is 32 rows, 16 at head dim 256.
+constexpr int lanes_per_row(int D) { return D / 16; }
+constexpr int q_block_rows(int D) { return D == 256 ? 16 : 32; }
 
 struct AttnArgs {
     const void *q, *k, *v;
@@ -63,14 +66,20 @@ __device__ __forceinline__ float lane_xor1(float x) { return dpp_mov<0xB1>(x); }
 __device__ __forceinline__ float lane_xor2(float x) { return dpp_mov<0x4E>(x); }                   // quad_perm [2,3,0,1]
 __device__ __forceinline__ float lane_xor4(float x) { return dpp_mov<0x1B>(dpp_mov<0x141>(x)); }   // half-row mirror (xor 7), then quad reverse (xor 3)
 
-// Sign diagonal and normalized Walsh-Hadamard over the 128 channels of one row held by eight consecutive lanes, sixteen
-// adjacent channels per lane (o8 = lane within the eight).  Same operation order as the oracle: H4 on runs of four
-// channels, radix-2 butterflies over channel bits 2..6 (two in the lane, three across lanes), one scaling.
-__device__ __forceinline__ void rot128(float (&v)[16], int o8) {
-    const uint32_t word = (o8 >> 1) == 0 ? 0x1035997bu : (o8 >> 1) == 1 ? 0x8087f5eeu : (o8 >> 1) == 2 ? 0xee2e4e1au : 0x71132418u;
-    const uint32_t keep = word >> ((o8 & 1) * 16);
+__device__ __forceinline__ float lane_xor8(float x) { return dpp_mov<0x128>(x); }                  // row_ror:8 within a row of 16 lanes
+
+// Normalized Walsh-Hadamard over the 16 << LB channels of one row held by 1 << LB consecutive lanes, sixteen adjacent
+// channels per lane (ol = lane within the run), after the sign diagonal when SIGN (head dim 128 only).  Same operation
+// order as the oracle: H4 on runs of four channels, radix-2 butterflies over the higher channel bits in ascending order
+// (two in the lane, LB across lanes), one scaling.  LB = 3: H128 (the reference's convrot128 / convrot128_plain), LB = 2:
+// H64 (convrot64).
+template <int LB, bool SIGN> __device__ __forceinline__ void rot_wh(float (&v)[16], int ol) {
+    if (SIGN) {
+        const uint32_t word = (ol >> 1) == 0 ? 0x1035997bu : (ol >> 1) == 1 ? 0x8087f5eeu : (ol >> 1) == 2 ? 0xee2e4e1au : 0x71132418u;
+        const uint32_t keep = word >> ((ol & 1) * 16);
 #pragma unroll
-    for (int e = 0; e < 16; ++e) v[e] = u2f(f2u(v[e]) ^ ((((keep >> e) & 1u) ^ 1u) << 31));
+        for (int e = 0; e < 16; ++e) v[e] = u2f(f2u(v[e]) ^ ((((keep >> e) & 1u) ^ 1u) << 31));
+    }
 #pragma unroll
     for (int g = 0; g < 16; g += 4) {
         const float a0 = v[g] + v[g + 1], a1 = v[g] - v[g + 1], a2 = v[g + 2] + v[g + 3], a3 = v[g + 2] - v[g + 3];
@@ -91,20 +100,22 @@ __device__ __forceinline__ void rot128(float (&v)[16], int o8) {
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
         const float other = lane_xor1(v[e]);
-        v[e] = (o8 & 1) ? other - v[e] : v[e] + other;
+        v[e] = (ol & 1) ? other - v[e] : v[e] + other;
     }
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
         const float other = lane_xor2(v[e]);
-        v[e] = (o8 & 2) ? other - v[e] : v[e] + other;
+        v[e] = (ol & 2) ? other - v[e] : v[e] + other;
+    }
+    if (LB == 3) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const float other = lane_xor4(v[e]);
+            v[e] = (ol & 4) ? other - v[e] : v[e] + other;
+        }
     }
 #pragma unroll
-    for (int e = 0; e < 16; ++e) {
-        const float other = lane_xor4(v[e]);
-        v[e] = (o8 & 4) ? other - v[e] : v[e] + other;
-    }
-#pragma unroll
-    for (int e = 0; e < 16; ++e) v[e] *= 0.1767766952966369f;
+    for (int e = 0; e < 16; ++e) v[e] *= LB == 3 ? 0.1767766952966369f : 0.25f;
 }
 
 // The rotation of sequences of at most 256 keys (csrc/vendor/sage/quant_qk_int8.cu:1160-1166, ROTATION 4): the
@@ -120,10 +131,22 @@ __device__ __forceinline__ void rot4(float (&v)[16]) {
     }
 }
 
-__device__ __forceinline__ float max8(float m) {
+// The rotation the quantizers apply to a row of head dim D (csrc/vendor/sage/quant_qk_int8.cu:1150-1195): the H4 blocks
+// alone up to 256 keys, beyond that H64 at head dim 64, sign diagonal + H128 at 128, the plain H128 on each half at 256.
+template <int D> __device__ __forceinline__ void rotate_row(float (&v)[16], int ol, bool h4_only) {
+    if (h4_only) rot4(v);
+    else if (D == 64) rot_wh<2, false>(v, ol);
+    else if (D == 128) rot_wh<3, true>(v, ol);
+    else rot_wh<3, false>(v, ol & 7);
+}
+
+// Maximum over the lanes of a row.
+template <int D> __device__ __forceinline__ float max_row(float m) {
     m = fmax_nn(m, lane_xor1(m));
     m = fmax_nn(m, lane_xor2(m));
-    return fmax_nn(m, lane_xor4(m));
+    if (D >= 128) m = fmax_nn(m, lane_xor4(m));
+    if (D == 256) m = fmax_nn(m, lane_xor8(m));
+    return m;
 }
 
 // Sum of squares of one 128-channel row in the order of the reference's warp of 32 lanes (csrc/kernels.cu:497-513,
@@ -241,73 +264,90 @@ template <int DT> __device__ __forceinline__ void ld16_dt(const void* p, int64_t
     }
 }
 
-// The K anchor of one (kv head, batch): thread = channel (the workgroup has 256 threads; the upper half repeats the
-// lower half's work and writes the same values).  The shuffle trees of the reference are summed in their order.
-template <int DT>
+// The K anchor of one (kv head, batch).  The nine sampled keys go to LDS (a thread per channel); the sums then follow the
+// reference's block of 128 threads in four warps: thread t walks channels t and t + 128 with one set of accumulators
+// (head dim 256), threads past the head dim hold zeros (64), warps add by a shuffle-down tree and the four warps in
+// order (csrc/vendor/sage/quant_qk_int8.cu:640-756).
+template <int DT, int D>
 __device__ __forceinline__ void anchor_body(const AttnArgs& a, const int hi, const int bi) {
     __shared__ float s[9][D];
-    __shared__ float energy[D], best_energy[D], amax[D], bmax[D], dist[9][D];
+    __shared__ float energy[128], best_energy[128], amax[128], bmax[128], dist[9][128];
     __shared__ int chosen;
-    const int c = threadIdx.x & 127, tid = threadIdx.x;
+    const int tid = threadIdx.x, c = tid & (D - 1);
     const int64_t base = bi * a.k_bs + hi * a.k_hs;
-    {   // the V quantizer's accumulators for this (kv head, batch) start at zero
+    if (tid < D) {   // the V quantizer's accumulators for this (kv head, batch) start at zero
         const int64_t bh = (int64_t)bi * a.hk + hi;
         a.vmax[bh * D + c] = 0u;
         for (int t = 0; t < a.kb; ++t) a.vsum[(bh * a.kb + t) * D + c] = 0;
     }
-    if (a.k_norm) {
-        // the nine sampled keys as the K quantizer will see them: norm_rope_row's arithmetic with a thread per channel
-        __shared__ float rstd9[9];
-        __shared__ float nrm[9][D];
+    bool normed = false;
+    if constexpr (D == 128) {
+        if (a.k_norm) {
+            normed = true;
+            // the nine sampled keys as the K quantizer will see them: norm_rope_row's arithmetic with a thread per channel
+            __shared__ float rstd9[9];
+            __shared__ float nrm[9][D];
 #pragma unroll
-        for (int i = 0; i < 9; ++i) {
-            const int row = (int)((int64_t)i * (a.lk - 1) / 8);
-            s[i][c] = ld_dt<DT>(a.k, base + (int64_t)row * a.k_rs + c);
-        }
-        __syncthreads();
-        if (tid < 9) rstd9[tid] = (float)(1.0 / sqrt((double)(sumsq128_serial(s[tid], a.rope_mode == 2) / 128.f + a.eps)));
-        __syncthreads();
-#pragma unroll
-        for (int i = 0; i < 9; ++i) nrm[i][c] = rnd_dt<DT_BF16>(s[i][c] * rstd9[i] * (a.kw ? a.kw[c] : 1.f));
-        __syncthreads();
-#pragma unroll
-        for (int i = 0; i < 9; ++i) {
-            float x = nrm[i][c];
-            if (a.rope) {
+            for (int i = 0; i < 9; ++i) {
                 const int row = (int)((int64_t)i * (a.lk - 1) / 8);
-                const float* r = a.rope + (int64_t)row * D;
-                if (a.rope_mode == 1) {
-                    const float cs = r[c & ~1], sn = r[c | 1], other = nrm[i][c ^ 1];
-                    x = rnd_dt<DT_BF16>((c & 1) ? __builtin_fmaf(sn, other, cs * x) : __builtin_fmaf(cs, x, -(sn * other)));
-                } else {
-                    const int j = c & 63;
-                    const float cs = r[2 * j], sn = r[2 * j + 1], other = nrm[i][c ^ 64];
-                    x = rnd_dt<DT_BF16>(c < 64 ? __builtin_fmaf(x, cs, -(other * sn)) : __builtin_fmaf(x, cs, other * sn));
-                }
+                s[i][c] = ld_dt<DT>(a.k, base + (int64_t)row * a.k_rs + c);
             }
-            s[i][c] = x;
+            __syncthreads();
+            if (tid < 9) rstd9[tid] = (float)(1.0 / sqrt((double)(sumsq128_serial(s[tid], a.rope_mode == 2) / 128.f + a.eps)));
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < 9; ++i) nrm[i][c] = rnd_dt<DT_BF16>(s[i][c] * rstd9[i] * (a.kw ? a.kw[c] : 1.f));
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < 9; ++i) {
+                float x = nrm[i][c];
+                if (a.rope) {
+                    const int row = (int)((int64_t)i * (a.lk - 1) / 8);
+                    const float* r = a.rope + (int64_t)row * D;
+                    if (a.rope_mode == 1) {
+                        const float cs = r[c & ~1], sn = r[c | 1], other = nrm[i][c ^ 1];
+                        x = rnd_dt<DT_BF16>((c & 1) ? __builtin_fmaf(sn, other, cs * x) : __builtin_fmaf(cs, x, -(sn * other)));
+                    } else {
+                        const int j = c & 63;
+                        const float cs = r[2 * j], sn = r[2 * j + 1], other = nrm[i][c ^ 64];
+                        x = rnd_dt<DT_BF16>(c < 64 ? __builtin_fmaf(x, cs, -(other * sn)) : __builtin_fmaf(x, cs, other * sn));
+                    }
+                }
+                s[i][c] = x;
+            }
         }
-    } else {
+    }
+    if (!normed && tid < D) {
 #pragma unroll
         for (int i = 0; i < 9; ++i) {
             const int row = (int)((int64_t)i * (a.lk - 1) / 8);
             s[i][c] = ld_dt<DT>(a.k, base + (int64_t)row * a.k_rs + c);
         }
     }
-    float e = 0.f, m = 0.f, sum = 0.f;
+    __syncthreads();
+    if (tid < 128) {
+        float e = 0.f, m = 0.f, d9[9];
 #pragma unroll
-    for (int i = 0; i < 9; ++i) {
-        const float x = s[i][c];
-        e = fmaf(x, x, e);
-        m = fmax_nn(m, fabsf(x));
-        sum += x;
-    }
-    energy[c] = e;
-    amax[c] = m;
+        for (int i = 0; i < 9; ++i) d9[i] = 0.f;
+        for (int ch = tid; ch < D; ch += 128) {
+            float sum = 0.f;
 #pragma unroll
-    for (int i = 0; i < 9; ++i) {
-        const float d = fmaf(9.f, s[i][c], -sum);
-        dist[i][c] = fmaf(d, d, 0.f);
+            for (int i = 0; i < 9; ++i) {
+                const float x = s[i][ch];
+                e = fmaf(x, x, e);
+                m = fmax_nn(m, fabsf(x));
+                sum += x;
+            }
+#pragma unroll
+            for (int i = 0; i < 9; ++i) {
+                const float d = fmaf(9.f, s[i][ch], -sum);
+                d9[i] = fmaf(d, d, d9[i]);
+            }
+        }
+        energy[tid] = e;
+        amax[tid] = m;
+#pragma unroll
+        for (int i = 0; i < 9; ++i) dist[i][tid] = d9[i];
     }
     __syncthreads();
     auto tree = [](const float* x) {
@@ -333,15 +373,19 @@ __device__ __forceinline__ void anchor_body(const AttnArgs& a, const int hi, con
     }
     __syncthreads();
     const int best = chosen;
-    float be = 0.f, bm = 0.f;
+    if (tid < 128) {
+        float be = 0.f, bm = 0.f;
+        for (int ch = tid; ch < D; ch += 128) {
 #pragma unroll
-    for (int i = 0; i < 9; ++i) {
-        const float r = s[i][c] - s[best][c];
-        be = fmaf(r, r, be);
-        bm = fmax_nn(bm, fabsf(r));
+            for (int i = 0; i < 9; ++i) {
+                const float r = s[i][ch] - s[best][ch];
+                be = fmaf(r, r, be);
+                bm = fmax_nn(bm, fabsf(r));
+            }
+        }
+        best_energy[tid] = be;
+        bmax[tid] = bm;
     }
-    best_energy[c] = be;
-    bmax[c] = bm;
     __syncthreads();
     if (tid < 4) warp_sum[10][tid] = tree(&best_energy[tid * 32]);
     __syncthreads();
@@ -351,7 +395,7 @@ __device__ __forceinline__ void anchor_body(const AttnArgs& a, const int hi, con
             e0 += warp_sum[9][w];
             e1 += warp_sum[10][w];
         }
-        for (int i = 0; i < D; ++i) {
+        for (int i = 0; i < 128; ++i) {
             m0 = fmax_nn(m0, amax[i]);
             m1 = fmax_nn(m1, bmax[i]);
         }
@@ -359,61 +403,68 @@ __device__ __forceinline__ void anchor_body(const AttnArgs& a, const int hi, con
     }
 }
 
-// Q: a wave per 32 rows, four waves per workgroup; each run of eight lanes is one scale group (rows g, g+8, g+16, g+24),
-// a lane holding 16 channels of each of the four rows.
-template <int DT>
+// Q: every run of D/16 lanes is one scale group (rows g, g+8, .. of a block of 32 rows, 16 at head dim 256), a lane
+// holding 16 channels of each of the group's rows; a wave carries 64 / (D/16) groups, a workgroup four waves.
+template <int DT, int D>
 __device__ __forceinline__ void quant_q_body(const AttnArgs& a, const int hi, const int ty, const int bi) {
-    const int lane = threadIdx.x & 63, o8 = lane & 7, g = lane >> 3;
-    const int t = ty * 4 + (threadIdx.x >> 6);
-    if (t >= a.qg) return;
-    const int64_t bh = (int64_t)bi * a.h + hi, base = bi * a.q_bs + hi * a.q_hs + o8 * 16;
-    float v[4][16];
+    constexpr int LPR = lanes_per_row(D), GPW = 64 / LPR, WQ = q_block_rows(D), NR = WQ / 8;
+    const int lane = threadIdx.x & 63, ol = lane & (LPR - 1);
+    const int gid = (ty * 4 + (threadIdx.x >> 6)) * GPW + lane / LPR;   // scale group of the head: block * 8 + g
+    if (gid >= a.qg * 8) return;
+    const int t = gid >> 3, g = gid & 7;
+    const int64_t bh = (int64_t)bi * a.h + hi, base = bi * a.q_bs + hi * a.q_hs + ol * 16;
+    float v[NR][16];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int row = t * 32 + g + 8 * j;
+    for (int j = 0; j < NR; ++j) {
+        const int row = t * WQ + g + 8 * j;
         const int rr = row < a.lq ? row : a.lq - 1;
         ld16_dt<DT>(a.q, base + (int64_t)rr * a.q_rs, a.in_vec, v[j]);
-        if (a.q_norm) norm_rope_row(v[j], o8, a.qw, a.rope ? a.rope + (int64_t)rr * D : nullptr, a.eps, a.rope_mode);
+        if constexpr (D == 128) {
+            if (a.q_norm) norm_rope_row(v[j], ol, a.qw, a.rope ? a.rope + (int64_t)rr * D : nullptr, a.eps, a.rope_mode);
+        }
     }
     float mx = 0.f;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        if (a.rot4) rot4(v[j]);
-        else rot128(v[j], o8);
-        if (t * 32 + g + 8 * j < a.lq) {
+    for (int j = 0; j < NR; ++j) {
+        rotate_row<D>(v[j], ol, a.rot4);
+        if (t * WQ + g + 8 * j < a.lq) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) mx = fmax_nn(mx, fabsf(v[j][e]));
         }
     }
-    mx = max8(mx);
+    mx = max_row<D>(mx);
     const float sc = mx / 127.f + 1e-7f, inv = 1.f / sc;
-    if (o8 == 0) a.qs[(bh * a.qg + t) * 8 + g] = sc;
+    if (ol == 0) a.qs[bh * a.qg * 8 + gid] = sc;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int row = t * 32 + g + 8 * j;
-        if (row < a.lq) *reinterpret_cast<uint4*>(a.qi + (bh * a.lq + row) * D + o8 * 16) = codes16(v[j], inv);
+    for (int j = 0; j < NR; ++j) {
+        const int row = t * WQ + g + 8 * j;
+        if (row < a.lq) *reinterpret_cast<uint4*>(a.qi + (bh * a.lq + row) * D + ol * 16) = codes16(v[j], inv);
     }
 }
 
 // K: one workgroup of 256 threads per tile of CK keys.  A scale group is the keys with (key % 8) / 2 == g; its CK/4 rows
-// are shared out over eight runs of eight lanes, whose maxima meet in LDS.  The tile is assembled in LDS in fragment
-// order, [32-key block][channel step of 32][half of 16 channels][key][16 bytes] (the 64 lanes of the attention kernel
-// read one contiguous KB per load), and leaves as 16-byte stores over its contiguous CK * 128 bytes; keys past lk are
-// zeros.
-template <int DT, int CK>
+// are shared out over the runs of D/16 lanes that serve the group, whose maxima meet in LDS.  The tile is assembled in
+// LDS in fragment order, [32-key block][channel step of 32][half of 16 channels][key][16 bytes] (the 64 lanes of the
+// attention kernel read one contiguous KB per load), and leaves as 16-byte stores over its contiguous CK * D bytes;
+// keys past lk are zeros.
+template <int DT, int CK, int D>
 __device__ __forceinline__ void quant_k_body(const AttnArgs& a, const int hi, const int t, const int bi) {
-    constexpr int R = CK / 32;   // rows per run of eight lanes
-    __shared__ float omax[32];
+    constexpr int LPR = lanes_per_row(D), RUNS = 256 / LPR, NSUB = RUNS / 4;
+    constexpr int R = (CK / 4) / NSUB;   // rows per run
+    static_assert(R >= 1 && R * NSUB * 4 == CK, "rows of a group divide over its runs");
+    __shared__ float omax[RUNS];
     __shared__ __align__(16) uint8_t stage[CK * D];
-    const int o8 = threadIdx.x & 7, oct = threadIdx.x >> 3, g = oct & 3, sub = oct >> 2;
-    const int64_t bh = (int64_t)bi * a.hk + hi, base = bi * a.k_bs + hi * a.k_hs + o8 * 16;
+    const int ol = threadIdx.x & (LPR - 1), run = threadIdx.x / LPR, g = run & 3, sub = run >> 2;
+    const int64_t bh = (int64_t)bi * a.hk + hi, base = bi * a.k_bs + hi * a.k_hs + ol * 16;
     const int anchor = a.anchors[bh];
     float bias[16];
 #pragma unroll
     for (int e = 0; e < 16; ++e) bias[e] = 0.f;
     if (anchor >= 0) {
         ld16_dt<DT>(a.k, base + (int64_t)anchor * a.k_rs, a.in_vec, bias);
-        if (a.k_norm) norm_rope_row(bias, o8, a.kw, a.rope ? a.rope + (int64_t)anchor * D : nullptr, a.eps, a.rope_mode);
+        if constexpr (D == 128) {
+            if (a.k_norm) norm_rope_row(bias, ol, a.kw, a.rope ? a.rope + (int64_t)anchor * D : nullptr, a.eps, a.rope_mode);
+        }
     }
     float v[R][16];
     int rt[R];
@@ -423,36 +474,37 @@ __device__ __forceinline__ void quant_k_body(const AttnArgs& a, const int hi, co
         rt[j] = (i / 2) * 8 + g * 2 + (i % 2);      // row within the tile
         const int row = t * CK + rt[j], rr = row < a.lk ? row : a.lk - 1;
         ld16_dt<DT>(a.k, base + (int64_t)rr * a.k_rs, a.in_vec, v[j]);
-        if (a.k_norm) norm_rope_row(v[j], o8, a.kw, a.rope ? a.rope + (int64_t)rr * D : nullptr, a.eps, a.rope_mode);
+        if constexpr (D == 128) {
+            if (a.k_norm) norm_rope_row(v[j], ol, a.kw, a.rope ? a.rope + (int64_t)rr * D : nullptr, a.eps, a.rope_mode);
+        }
     }
     float mx = 0.f;
 #pragma unroll
     for (int j = 0; j < R; ++j) {
 #pragma unroll
         for (int e = 0; e < 16; ++e) v[j][e] -= bias[e];
-        if (a.rot4) rot4(v[j]);
-        else rot128(v[j], o8);
+        rotate_row<D>(v[j], ol, a.rot4);
         if (t * CK + rt[j] < a.lk) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) mx = fmax_nn(mx, fabsf(v[j][e]));
         }
     }
-    mx = max8(mx);
-    if (o8 == 0) omax[oct] = mx;
+    mx = max_row<D>(mx);
+    if (ol == 0) omax[run] = mx;
     __syncthreads();
     mx = 0.f;
 #pragma unroll
-    for (int x = 0; x < 8; ++x) mx = fmax_nn(mx, omax[x * 4 + g]);
+    for (int x = 0; x < NSUB; ++x) mx = fmax_nn(mx, omax[x * 4 + g]);
     const float sc = mx / 127.f + 1e-7f, inv = 1.f / sc;
-    if (sub == 0 && o8 == 0) a.ks[(bh * a.kb + t) * 4 + g] = sc;
+    if (sub == 0 && ol == 0) a.ks[(bh * a.kb + t) * 4 + g] = sc;
 #pragma unroll
     for (int j = 0; j < R; ++j) {
         uint4 w = make_uint4(0u, 0u, 0u, 0u);
         if (t * CK + rt[j] < a.lk) w = codes16(v[j], inv);
-        *reinterpret_cast<uint4*>(stage + (rt[j] / 32) * 4096 + (o8 >> 1) * 1024 + (o8 & 1) * 512 + (rt[j] % 32) * 16) = w;
+        *reinterpret_cast<uint4*>(stage + (rt[j] / 32) * (32 * D) + (ol >> 1) * 1024 + (ol & 1) * 512 + (rt[j] % 32) * 16) = w;
     }
     __syncthreads();
-    uint4* out = reinterpret_cast<uint4*>(a.ki + (bh * a.nblk + (int64_t)t * (CK / 32)) * 4096);
+    uint4* out = reinterpret_cast<uint4*>(a.ki + (bh * a.nblk + (int64_t)t * (CK / 32)) * (32 * D));
 #pragma unroll
     for (int i = 0; i < CK * D / 16 / 256; ++i)
         out[i * 256 + threadIdx.x] = *reinterpret_cast<const uint4*>(stage + (i * 256 + threadIdx.x) * 16);
@@ -460,16 +512,17 @@ __device__ __forceinline__ void quant_k_body(const AttnArgs& a, const int hi, co
 
 // V abs-max per channel: 256 threads take 128 rows of one (kv head, batch), four channels per thread; non-negative
 // floats order as their bits, so the workgroups combine with an integer atomic max.
-template <int DT>
+template <int DT, int D>
 __device__ __forceinline__ void v_absmax_body(const AttnArgs& a, const int hi, const int chunk, const int bi) {
-    __shared__ float red[8][D];
-    const int c4 = threadIdx.x & 31, rl = threadIdx.x >> 5;
+    constexpr int TPR = D / 4, RL = 256 / TPR;   // threads per row, rows per pass
+    __shared__ float red[RL][D];
+    const int c4 = threadIdx.x % TPR, rl = threadIdx.x / TPR;
     const int64_t base = bi * a.v_bs + hi * a.v_hs + c4 * 4;
     float mx[4] = {0.f, 0.f, 0.f, 0.f};
     const int r0 = chunk * 128;
 #pragma unroll 4
-    for (int i = 0; i < 16; ++i) {
-        const int r = r0 + rl + 8 * i;
+    for (int i = 0; i < 128 / RL; ++i) {
+        const int r = r0 + rl + RL * i;
         if (r < a.lk) {
             float x[4];
             ld4_dt<DT>(a.v, base + (int64_t)r * a.v_rs, a.v_vec, x);
@@ -483,7 +536,7 @@ __device__ __forceinline__ void v_absmax_body(const AttnArgs& a, const int hi, c
     if (threadIdx.x < D) {
         float m = 0.f;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) m = fmax_nn(m, red[i][threadIdx.x]);
+        for (int i = 0; i < RL; ++i) m = fmax_nn(m, red[i][threadIdx.x]);
         atomicMax(&a.vmax[((int64_t)bi * a.hk + hi) * D + threadIdx.x], f2u(m));
     }
 }
@@ -491,38 +544,40 @@ __device__ __forceinline__ void v_absmax_body(const AttnArgs& a, const int hi, c
 // Two launches carry the four bodies above: work that does not depend on each other shares a launch, heads fastest so
 // that neighbouring workgroups read neighbouring memory.  Stage 1: anchors (which also clear the V accumulators) and Q.
 // Stage 2: K (needs the anchors) and the V abs-max (needs the cleared accumulators).
-template <int DT>
+template <int DT, int D>
 __global__ __launch_bounds__(256) void attn_stage1_kernel(AttnArgs a) {
     int id = blockIdx.x;
     const int n_anchor = a.hk * a.b;
     if (id < n_anchor) {
-        anchor_body<DT>(a, id % a.hk, id / a.hk);
+        anchor_body<DT, D>(a, id % a.hk, id / a.hk);
         return;
     }
     id -= n_anchor;
-    const int ny = (a.qg + 3) / 4;
-    quant_q_body<DT>(a, id % a.h, (id / a.h) % ny, id / (a.h * ny));
+    constexpr int GPB = 4 * (64 / lanes_per_row(D));   // scale groups per workgroup
+    const int ny = (a.qg * 8 + GPB - 1) / GPB;
+    quant_q_body<DT, D>(a, id % a.h, (id / a.h) % ny, id / (a.h * ny));
 }
 
-template <int DT, int CK>
+template <int DT, int CK, int D>
 __global__ __launch_bounds__(256) void attn_stage2_kernel(AttnArgs a) {
     int id = blockIdx.x;
     const int n_k = a.hk * a.kb * a.b;
     if (id < n_k) {
-        quant_k_body<DT, CK>(a, id % a.hk, (id / a.hk) % a.kb, id / (a.hk * a.kb));
+        quant_k_body<DT, CK, D>(a, id % a.hk, (id / a.hk) % a.kb, id / (a.hk * a.kb));
         return;
     }
     id -= n_k;
     const int nc = (a.lk + 127) / 128;
-    v_absmax_body<DT>(a, id % a.hk, (id / a.hk) % nc, id / (a.hk * nc));
+    v_absmax_body<DT, D>(a, id % a.hk, (id / a.hk) % nc, id / (a.hk * nc));
 }
 
 // V codes: one workgroup per block of 32 keys.  Rows are read as they lie (a thread takes 16 channels of one key),
 // quantized and turned through LDS.  vt[(kv head, block)][d][32]: position h*16 + j of a row holds key
 // (j/4)*8 + h*4 + j%4 of the block, which is the order a lane of the attention kernel holds its 16 scores in.  Keys past
 // lk are zeros.  128 x the column sums go to vsum[(kv head, key tile)][d] by integer atomics.
-template <int DT>
+template <int DT, int D>
 __global__ __launch_bounds__(256) void attn_v_quant_kernel(AttnArgs a) {
+    constexpr int LPR = lanes_per_row(D), KPP = 256 / LPR;   // keys per pass of the read phase
     __shared__ float inv_s[D];
     __shared__ __align__(16) int8_t tile[32][D];
     const int hi = blockIdx.x, s = blockIdx.y, bi = blockIdx.z;
@@ -533,8 +588,10 @@ __global__ __launch_bounds__(256) void attn_v_quant_kernel(AttnArgs a) {
         inv_s[threadIdx.x] = 1.f / sc;
     }
     __syncthreads();
-    {
-        const int key = threadIdx.x >> 3, seg = threadIdx.x & 7;
+#pragma unroll
+    for (int pass = 0; pass < (32 + KPP - 1) / KPP; ++pass) {
+        const int key = pass * KPP + threadIdx.x / LPR, seg = threadIdx.x % LPR;
+        if (key >= 32) break;
         const int row = s * 32 + key;
         uint32_t w[4] = {0u, 0u, 0u, 0u};
         if (row < a.lk) {
@@ -550,17 +607,22 @@ __global__ __launch_bounds__(256) void attn_v_quant_kernel(AttnArgs a) {
         *reinterpret_cast<uint4*>(&tile[key][seg * 16]) = make_uint4(w[0], w[1], w[2], w[3]);
     }
     __syncthreads();
-    const int d = threadIdx.x & 127, hh = threadIdx.x >> 7;
-    uint32_t w[4] = {0u, 0u, 0u, 0u};
-    int sum = 0;
 #pragma unroll
-    for (int j = 0; j < 16; ++j) {
-        const int q = tile[(j / 4) * 8 + hh * 4 + (j % 4)][d];
-        sum += q;
-        w[j / 4] |= (uint32_t)(uint8_t)q << (8 * (j % 4));
+    for (int pass = 0; pass < (2 * D + 255) / 256; ++pass) {
+        const int id = pass * 256 + threadIdx.x;
+        if (id >= 2 * D) break;
+        const int d = id % D, hh = id / D;
+        uint32_t w[4] = {0u, 0u, 0u, 0u};
+        int sum = 0;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const int q = tile[(j / 4) * 8 + hh * 4 + (j % 4)][d];
+            sum += q;
+            w[j / 4] |= (uint32_t)(uint8_t)q << (8 * (j % 4));
+        }
+        *reinterpret_cast<uint4*>(a.vt + ((bh * a.nblk + s) * D + d) * 32 + hh * 16) = make_uint4(w[0], w[1], w[2], w[3]);
+        atomicAdd(&a.vsum[(bh * a.kb + s / (a.ck / 32)) * D + d], 128 * sum);
     }
-    *reinterpret_cast<uint4*>(a.vt + ((bh * a.nblk + s) * D + d) * 32 + hh * 16) = make_uint4(w[0], w[1], w[2], w[3]);
-    atomicAdd(&a.vsum[(bh * a.kb + s / (a.ck / 32)) * D + d], 128 * sum);
 }
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
@@ -573,9 +635,10 @@ typedef const __attribute__((address_space(1))) void* glb_ptr_t;
 // outputs and at most 512 keys (csrc/vendor/sage/sage_attn_launcher.cu:187-191, qk_int_sv_i8_cuda.cuh:132-139,637-700):
 // every tile's maximum starts at a raw score of -50000 and the denominator sums the unrounded probabilities in
 // per-thread partials (attn_utils.cuh:922-940).  Without FD only the last tile takes that form.
-template <int OUT_DT, int CK, bool MASK = false, bool FD = false>
-__global__ __launch_bounds__(256, 2) void attn_int8_kernel(AttnArgs a) {
-    constexpr int NB = CK / 32, KV = CK * D, STAGE = 2 * KV + 512;
+template <int OUT_DT, int CK, bool MASK = false, bool FD = false, int D = 128>
+__global__ __launch_bounds__(256, D == 256 ? 1 : 2) void attn_int8_kernel(AttnArgs a) {
+    constexpr int NB = CK / 32, NS = D / 32, KV = CK * D, STAGE = 2 * KV + D * 4, WQ = q_block_rows(D);
+    static_assert(!MASK || D == 128, "the key-bias form exists for head dim 128 only");
     extern __shared__ __align__(16) uint8_t smem[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int l32 = lane & 31, hh = lane >> 5;
@@ -587,29 +650,29 @@ __global__ __launch_bounds__(256, 2) void attn_int8_kernel(AttnArgs a) {
 
     auto fetch = [&](int t) {
         uint8_t* st = smem + (t & 1) * STAGE;
-        const int64_t tile = (kvh * a.nblk + (int64_t)t * NB) * 4096 + lane * 16;
+        const int64_t tile = (kvh * a.nblk + (int64_t)t * NB) * (32 * D) + lane * 16;
 #pragma unroll
         for (int j = 0; j < KV / 4096; ++j) {
             const int c = wave + 4 * j;
             __builtin_amdgcn_global_load_lds((glb_ptr_t)(a.ki + tile + c * 1024), (lds_ptr_t)(st + c * 1024), 16, 0, 0);
             __builtin_amdgcn_global_load_lds((glb_ptr_t)(a.vt + tile + c * 1024), (lds_ptr_t)(st + KV + c * 1024), 16, 0, 0);
         }
-        if (wave == 0 && lane < 32)
+        if (wave == 0 && lane < D / 4)
             __builtin_amdgcn_global_load_lds((glb_ptr_t)(a.vsum + (kvh * a.kb + t) * D + lane * 4), (lds_ptr_t)(st + 2 * KV), 16, 0, 0);
     };
     fetch(0);
 
-    v4i qf[4];
+    v4i qf[NS];
     {
         const int8_t* qrow = a.qi + (bh * a.lq + rc) * D + hh * 16;
 #pragma unroll
-        for (int s = 0; s < 4; ++s) qf[s] = *reinterpret_cast<const v4i*>(qrow + s * 32);
+        for (int s = 0; s < NS; ++s) qf[s] = *reinterpret_cast<const v4i*>(qrow + s * 32);
     }
-    const float q_scale = a.qs[(bh * a.qg + r / 32) * 8 + (r & 7)];
+    const float q_scale = a.qs[(bh * a.qg + r / WQ) * 8 + (r & 7)];
 
-    float ro[4][16];
+    float ro[NS][16];
 #pragma unroll
-    for (int x = 0; x < 4; ++x)
+    for (int x = 0; x < NS; ++x)
 #pragma unroll
         for (int i = 0; i < 16; ++i) ro[x][i] = 0.f;
     float m = -50000.f, dsum = 1.f;
@@ -630,10 +693,10 @@ __global__ __launch_bounds__(256, 2) void attn_int8_kernel(AttnArgs a) {
 #pragma unroll
         for (int blk = 0; blk < NB; ++blk) S[blk] = v16i{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-        for (int s = 0; s < 4; ++s)
+        for (int s = 0; s < NS; ++s)
 #pragma unroll
             for (int blk = 0; blk < NB; ++blk) {
-                const v4i kf = *reinterpret_cast<const v4i*>(st + blk * 4096 + s * 1024 + lane * 16);
+                const v4i kf = *reinterpret_cast<const v4i*>(st + blk * (32 * D) + s * 1024 + lane * 16);
                 S[blk] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf, qf[s], S[blk], 0, 0, 0);
             }
         if constexpr (!last) fetch(t + 1);   // the other stage: every wave left it at the barrier that ended the last tile
@@ -835,32 +898,36 @@ __global__ __launch_bounds__(256, 2) void attn_int8_kernel(AttnArgs a) {
             }
         }
 
-        // P.V: the four 32-channel blocks of the output keep their own accumulators (the scores are dead by now), key
-        // blocks outside, so that consecutive MFMAs are independent here too.
-        v16i acc[4];
+        // P.V: the 32-channel blocks of the output keep their own accumulators (the scores are dead by now), key blocks
+        // outside, so that consecutive MFMAs are independent here too; four output blocks at a time.
 #pragma unroll
-        for (int x = 0; x < 4; ++x) {
-            const int* vsp = reinterpret_cast<const int*>(st + 2 * KV) + x * 32 + hh * 4;
+        for (int x0 = 0; x0 < NS; x0 += 4) {
+            constexpr int NX = NS < 4 ? NS : 4;
+            v16i acc[NX];
 #pragma unroll
-            for (int g4 = 0; g4 < 4; ++g4) {
-                const v4i c4 = *reinterpret_cast<const v4i*>(vsp + g4 * 8);
-                acc[x][g4 * 4 + 0] = c4[0];
-                acc[x][g4 * 4 + 1] = c4[1];
-                acc[x][g4 * 4 + 2] = c4[2];
-                acc[x][g4 * 4 + 3] = c4[3];
+            for (int x = 0; x < NX; ++x) {
+                const int* vsp = reinterpret_cast<const int*>(st + 2 * KV) + (x0 + x) * 32 + hh * 4;
+#pragma unroll
+                for (int g4 = 0; g4 < 4; ++g4) {
+                    const v4i c4 = *reinterpret_cast<const v4i*>(vsp + g4 * 8);
+                    acc[x][g4 * 4 + 0] = c4[0];
+                    acc[x][g4 * 4 + 1] = c4[1];
+                    acc[x][g4 * 4 + 2] = c4[2];
+                    acc[x][g4 * 4 + 3] = c4[3];
+                }
             }
+#pragma unroll
+            for (int blk = 0; blk < NB; ++blk)
+#pragma unroll
+                for (int x = 0; x < NX; ++x) {
+                    const v4i vf = *reinterpret_cast<const v4i*>(st + KV + ((blk * D + (x0 + x) * 32 + l32) * 32 + hh * 16));
+                    acc[x] = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf, pf[blk], acc[x], 0, 0, 0);
+                }
+#pragma unroll
+            for (int x = 0; x < NX; ++x)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) ro[x0 + x][i] = fmaf((float)acc[x][i], t_scale, ro[x0 + x][i] * o_scale);
         }
-#pragma unroll
-        for (int blk = 0; blk < NB; ++blk)
-#pragma unroll
-            for (int x = 0; x < 4; ++x) {
-                const v4i vf = *reinterpret_cast<const v4i*>(st + KV + ((blk * D + x * 32 + l32) * 32 + hh * 16));
-                acc[x] = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf, pf[blk], acc[x], 0, 0, 0);
-            }
-#pragma unroll
-        for (int x = 0; x < 4; ++x)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) ro[x][i] = fmaf((float)acc[x][i], t_scale, ro[x][i] * o_scale);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wave's share of the next tile has landed
         __syncthreads();
     };
@@ -877,7 +944,7 @@ __global__ __launch_bounds__(256, 2) void attn_int8_kernel(AttnArgs a) {
     if (r < a.lq) {
         const int64_t ob = bi * a.o_bs + (int64_t)r * a.o_rs + hi * a.o_hs;
 #pragma unroll
-        for (int x = 0; x < 4; ++x)
+        for (int x = 0; x < NS; ++x)
 #pragma unroll
             for (int g4 = 0; g4 < 4; ++g4) {
                 const int d0 = x * 32 + g4 * 8 + hh * 4;
@@ -929,11 +996,11 @@ struct Plan {
     int ck, kb, qg, nblk;
 };
 
-Plan plan_for(int64_t b, int64_t h, int64_t hk, int64_t lq, int64_t lk) {
+Plan plan_for(int64_t b, int64_t h, int64_t hk, int64_t lq, int64_t lk, int D) {
     Plan p;
     p.ck = cta_k_for((int)lk, D);
     p.kb = (int)((lk + p.ck - 1) / p.ck);
-    p.qg = (int)((lq + 127) / 128 * 4);
+    p.qg = (int)((lq + 127) / 128 * (128 / q_block_rows(D)));   // row blocks of the Q quantizer, eight scale groups each
     p.nblk = p.kb * (p.ck / 32);
     int64_t n = 0;
     auto add = [&](int64_t bytes) { const int64_t at = n; n += (bytes + 255) / 256 * 256; return at; };
@@ -950,48 +1017,55 @@ Plan plan_for(int64_t b, int64_t h, int64_t hk, int64_t lq, int64_t lk) {
     return p;
 }
 
-template <int DT>
-int run(AttnArgs a, hipStream_t st) {
-    const int64_t n1 = (int64_t)a.hk * a.b + (int64_t)a.h * ((a.qg + 3) / 4) * a.b;
-    const int64_t n2 = (int64_t)a.hk * a.kb * a.b + (int64_t)a.hk * ((a.lk + 127) / 128) * a.b;
-    if (n1 > 0x7fffffff || n2 > 0x7fffffff) return -400;
-    attn_stage1_kernel<DT><<<dim3((unsigned)n1), 256, 0, st>>>(a);
-    if (a.ck == 64) attn_stage2_kernel<DT, 64><<<dim3((unsigned)n2), 256, 0, st>>>(a);
-    else attn_stage2_kernel<DT, 128><<<dim3((unsigned)n2), 256, 0, st>>>(a);
-    attn_v_quant_kernel<DT><<<dim3(a.hk, a.nblk, a.b), 256, 0, st>>>(a);
-    const dim3 grid((a.lq + 127) / 128, a.h, a.b);
-    constexpr int kLds64 = 2 * (2 * 64 * D + 512), kLds128 = 2 * (2 * 128 * D + 512);
-    // more than 64 KB of dynamic LDS has to be allowed once per device; a repeated set is harmless if two threads race
+// More than 64 KB of dynamic LDS has to be allowed once per kernel and device; a repeated set is harmless if two threads
+// race.
+template <class K> bool allow_lds(K kern, int bytes) {
     static bool allowed[64] = {};
     int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return -401;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
     if (!allowed[dev]) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_int8_kernel<DT, 128>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, kLds128) != hipSuccess)
-            return -401;
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess)
+            return false;
         allowed[dev] = true;
     }
-    if (a.bias) {
-        static bool allowed_m[64] = {};
-        if (!allowed_m[dev]) {
-            if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_int8_kernel<DT, 128, true>),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, kLds128) != hipSuccess)
-                return -401;
-            allowed_m[dev] = true;
-        }
-        if (a.ck == 64) {
-            attn_key_bias_kernel<64><<<dim3(a.kb), 64, 0, st>>>(a.bias, a.lk, a.kbias, a.tbias);
-            attn_int8_kernel<DT, 64, true><<<grid, 256, kLds64, st>>>(a);
-        } else {
-            attn_key_bias_kernel<128><<<dim3(a.kb), 128, 0, st>>>(a.bias, a.lk, a.kbias, a.tbias);
-            attn_int8_kernel<DT, 128, true><<<grid, 256, kLds128, st>>>(a);
-        }
-        return hipGetLastError() == hipSuccess ? 0 : -401;
-    }
-    if (DT == DT_F16 && a.lk <= 512 && a.ck == 64) attn_int8_kernel<DT_F16, 64, false, true><<<grid, 256, kLds64, st>>>(a);
-    else if (a.ck == 64) attn_int8_kernel<DT, 64><<<grid, 256, kLds64, st>>>(a);
-    else attn_int8_kernel<DT, 128><<<grid, 256, kLds128, st>>>(a);
+    return true;
+}
+
+template <int DT, int CK, bool MASK, bool FD, int D>
+int launch_attn(const AttnArgs& a, hipStream_t st) {
+    constexpr int kLds = 2 * (2 * CK * D + D * 4);
+    auto kern = attn_int8_kernel<DT, CK, MASK, FD, D>;
+    if (kLds > 64 * 1024 && !allow_lds(kern, kLds)) return -401;
+    kern<<<dim3((a.lq + 127) / 128, a.h, a.b), 256, kLds, st>>>(a);
     return hipGetLastError() == hipSuccess ? 0 : -401;
+}
+
+template <int DT, int D>
+int run(AttnArgs a, hipStream_t st) {
+    constexpr int GPB = 4 * (64 / lanes_per_row(D));   // scale groups per workgroup of the Q quantizer
+    const int64_t n1 = (int64_t)a.hk * a.b + (int64_t)a.h * ((a.qg * 8 + GPB - 1) / GPB) * a.b;
+    const int64_t n2 = (int64_t)a.hk * a.kb * a.b + (int64_t)a.hk * ((a.lk + 127) / 128) * a.b;
+    if (n1 > 0x7fffffff || n2 > 0x7fffffff) return -400;
+    attn_stage1_kernel<DT, D><<<dim3((unsigned)n1), 256, 0, st>>>(a);
+    if (a.ck == 64) attn_stage2_kernel<DT, 64, D><<<dim3((unsigned)n2), 256, 0, st>>>(a);
+    else if constexpr (D != 64) attn_stage2_kernel<DT, 128, D><<<dim3((unsigned)n2), 256, 0, st>>>(a);
+    attn_v_quant_kernel<DT, D><<<dim3(a.hk, a.nblk, a.b), 256, 0, st>>>(a);
+    if (hipGetLastError() != hipSuccess) return -401;
+    if constexpr (D == 128) {
+        if (a.bias) {
+            if (a.ck == 64) {
+                attn_key_bias_kernel<64><<<dim3(a.kb), 64, 0, st>>>(a.bias, a.lk, a.kbias, a.tbias);
+                return launch_attn<DT, 64, true, false, D>(a, st);
+            }
+            attn_key_bias_kernel<128><<<dim3(a.kb), 128, 0, st>>>(a.bias, a.lk, a.kbias, a.tbias);
+            return launch_attn<DT, 128, true, false, D>(a, st);
+        }
+    }
+    // f16 outputs with at most 512 keys: the reference's build takes its unfused probability path in every tile
+    if (DT == DT_F16 && a.lk <= 512 && a.ck == 64) return launch_attn<DT_F16, 64, false, true, D>(a, st);
+    if (a.ck == 64) return launch_attn<DT, 64, false, false, D>(a, st);
+    if constexpr (D != 64) return launch_attn<DT, 128, false, false, D>(a, st);
+    return -400;
 }
 
 // Per-head RMSNorm and RoPE for q and k, applied on the way into the quantizer (csrc/attn_int8.cu:69-76).  A null kw
@@ -1009,8 +1083,8 @@ int int8_attn(const void* q, const void* k, const void* v, void* o, void* ws, in
               int64_t v_hs, int64_t o_bs, int64_t o_rs, int64_t o_hs, float scale, int dt, void* stream, float sink = 0.f,
               const QkNorm* norm = nullptr, const float* bias = nullptr) {
     const char* why = nullptr;
-    if (Dh != D) why = "only head dim 128 is built";
-    else if (norm && dt != DT_BF16) why = "fused q/k norm needs bf16 head dim 128";                     // csrc/attn_int8.cu:135
+    if (Dh != 64 && Dh != 128 && Dh != 256) why = "head dim must be 64, 128 or 256";
+    else if ((norm || bias) && (dt != DT_BF16 || Dh != 128)) why = "fused q/k norm and key bias need bf16 head dim 128";   // csrc/attn_int8.cu:135
     else if (norm && (norm->rope_mode < 0 || norm->rope_mode > 2)) why = "rope_mode must be 0, 1 or 2";   // quant_qk_int8.cu:1279
     else if (!q || !k || !v || !o || !ws) why = "null pointer";
     else if (b <= 0 || lq <= 0 || lk <= 0 || h <= 0 || hk <= 0 || h % hk != 0) why = "bad sizes";
@@ -1020,7 +1094,7 @@ int int8_attn(const void* q, const void* k, const void* v, void* o, void* ws, in
         fprintf(stderr, "int8 attention: %s\n", why);
         return -400;
     }
-    const Plan p = plan_for(b, h, hk, lq, lk);
+    const Plan p = plan_for(b, h, hk, lq, lk, Dh);
     char* w = (char*)ws;
     AttnArgs a;
     a.q = q; a.k = k; a.v = v; a.o = o;
@@ -1053,19 +1127,22 @@ int int8_attn(const void* q, const void* k, const void* v, void* o, void* ws, in
         a.q_norm = 1;
         a.k_norm = norm->kw ? 1 : 0;
     }
-    return dt == DT_F16 ? run<DT_F16>(a, (hipStream_t)stream) : run<DT_BF16>(a, (hipStream_t)stream);
+    hipStream_t st = (hipStream_t)stream;
+    if (Dh == 64) return dt == DT_F16 ? run<DT_F16, 64>(a, st) : run<DT_BF16, 64>(a, st);
+    if (Dh == 256) return dt == DT_F16 ? run<DT_F16, 256>(a, st) : run<DT_BF16, 256>(a, st);
+    return dt == DT_F16 ? run<DT_F16, 128>(a, st) : run<DT_BF16, 128>(a, st);
 }
 
 }  // namespace
 
 GPU_API int64_t gpu_int8_attn_workspace_d(int b, int h, int hk, int lq, int lk, int head_dim) {
-    if (head_dim != D) return 0;   // only head dim 128 is built: no size that a caller could mistake for a usable one
+    if (head_dim != 64 && head_dim != 128 && head_dim != 256) return 0;
     if (b <= 0 || h <= 0 || hk <= 0 || lq <= 0 || lk <= 0) return 0;
-    return plan_for(b, h, hk, lq, lk).total;
+    return plan_for(b, h, hk, lq, lk, head_dim).total;
 }
 
 GPU_API int64_t gpu_int8_attn_workspace(int b, int h, int hk, int lq, int lk) {
-    return gpu_int8_attn_workspace_d(b, h, hk, lq, lk, D);
+    return gpu_int8_attn_workspace_d(b, h, hk, lq, lk, 128);
 }
 
 GPU_API int gpu_int8_attn_d(const void* q, const void* k, const void* v, void* o, void* ws, int b, int lq, int lk, int h,
@@ -1088,7 +1165,7 @@ GPU_API int gpu_int8_attn(const void* q, const void* k, const void* v, void* o, 
                           int hk, int64_t q_bs, int64_t q_rs, int64_t q_hs, int64_t k_bs, int64_t k_rs, int64_t k_hs,
                           int64_t v_bs, int64_t v_rs, int64_t v_hs, int64_t o_bs, int64_t o_rs, int64_t o_hs, float scale,
                           void* stream) {
-    return int8_attn(q, k, v, o, ws, b, lq, lk, h, hk, D, q_bs, q_rs, q_hs, k_bs, k_rs, k_hs, v_bs, v_rs, v_hs, o_bs, o_rs,
+    return int8_attn(q, k, v, o, ws, b, lq, lk, h, hk, 128, q_bs, q_rs, q_hs, k_bs, k_rs, k_hs, v_bs, v_rs, v_hs, o_bs, o_rs,
                      o_hs, scale, DT_BF16, stream);
 }
 
@@ -1097,7 +1174,7 @@ GPU_API int gpu_int8_attn_sink(const void* q, const void* k, const void* v, void
                                int64_t v_bs, int64_t v_rs, int64_t v_hs, int64_t o_bs, int64_t o_rs, int64_t o_hs, float scale,
                                float sink, const float* qw, float eps, void* stream) {
     const QkNorm norm{qw, nullptr, nullptr, eps, 0};   // a non-null qw normalizes q; k is taken as it is (csrc/attn_int8.cu:198-201)
-    return int8_attn(q, k, v, o, ws, b, lq, lk, h, hk, D, q_bs, q_rs, q_hs, k_bs, k_rs, k_hs, v_bs, v_rs, v_hs, o_bs, o_rs,
+    return int8_attn(q, k, v, o, ws, b, lq, lk, h, hk, 128, q_bs, q_rs, q_hs, k_bs, k_rs, k_hs, v_bs, v_rs, v_hs, o_bs, o_rs,
                      o_hs, scale, DT_BF16, stream, sink, qw ? &norm : nullptr);
 }
 
@@ -1109,7 +1186,7 @@ GPU_API int gpu_int8_attn_norm_rope(const void* q, const void* k, const void* v,
                                     int64_t o_hs, float scale, const float* qw, const float* kw, float eps,
                                     const float* rope, int rope_mode, void* stream) {
     const QkNorm norm{qw, kw, rope, eps, rope_mode};
-    return int8_attn(q, k, v, o, ws, b, lq, lk, h, hk, D, q_bs, q_rs, q_hs, k_bs, k_rs, k_hs, v_bs, v_rs, v_hs, o_bs, o_rs,
+    return int8_attn(q, k, v, o, ws, b, lq, lk, h, hk, 128, q_bs, q_rs, q_hs, k_bs, k_rs, k_hs, v_bs, v_rs, v_hs, o_bs, o_rs,
                      o_hs, scale, DT_BF16, stream, 0.f, &norm);
 }
 
@@ -1122,7 +1199,7 @@ static int64_t key_mask_width(int lk) {
 
 GPU_API int64_t gpu_int8_attn_key_bias_workspace(int b, int h, int hk, int lq, int lk) {
     if (b <= 0 || h <= 0 || hk <= 0 || lq <= 0 || lk <= 0) return 0;
-    return gpu_int8_attn_workspace_d(b, h, hk, lq, lk, D) + (key_mask_width(lk) * 4 + 255) / 256 * 256;
+    return gpu_int8_attn_workspace_d(b, h, hk, lq, lk, 128) + (key_mask_width(lk) * 4 + 255) / 256 * 256;
 }
 
 // gpu_int8_attn with bias (f32 [lk], the same for every batch item, query and head) added to each key's logits, as an
@@ -1135,7 +1212,7 @@ GPU_API int gpu_int8_attn_key_bias(const void* q, const void* k, const void* v, 
         fprintf(stderr, "int8 attention: null key bias\n");
         return -400;
     }
-    return int8_attn(q, k, v, o, ws, b, lq, lk, h, hk, D, q_bs, q_rs, q_hs, k_bs, k_rs, k_hs, v_bs, v_rs, v_hs, o_bs, o_rs,
+    return int8_attn(q, k, v, o, ws, b, lq, lk, h, hk, 128, q_bs, q_rs, q_hs, k_bs, k_rs, k_hs, v_bs, v_rs, v_hs, o_bs, o_rs,
                      o_hs, scale, DT_BF16, stream, 0.f, nullptr, bias);
 }
 
@@ -1174,10 +1251,13 @@ GPU_API int gpu_internal_attn_sumsq_probe(const float* x, float* out, int rows, 
 
 // Test hook: where the pieces of the workspace lie (byte offsets), and the tiling.  out[0..9] = qi, ki, qs, ks, vt, vs,
 // anchors, vsum, key tile length, key tiles.
-GPU_API int gpu_internal_attn_layout(int b, int h, int hk, int lq, int lk, int64_t* out) {
-    if (b <= 0 || h <= 0 || hk <= 0 || lq <= 0 || lk <= 0 || !out) return -400;
-    const Plan p = plan_for(b, h, hk, lq, lk);
+GPU_API int gpu_internal_attn_layout_d(int b, int h, int hk, int lq, int lk, int head_dim, int64_t* out) {
+    if (b <= 0 || h <= 0 || hk <= 0 || lq <= 0 || lk <= 0 || !out || (head_dim != 64 && head_dim != 128 && head_dim != 256)) return -400;
+    const Plan p = plan_for(b, h, hk, lq, lk, head_dim);
     const int64_t v[10] = {p.qi, p.ki, p.qs, p.ks, p.vt, p.vs, p.anchors, p.vsum, p.ck, p.kb};
     for (int i = 0; i < 10; ++i) out[i] = v[i];
     return 0;
+}
+GPU_API int gpu_internal_attn_layout(int b, int h, int hk, int lq, int lk, int64_t* out) {
+    return gpu_internal_attn_layout_d(b, h, hk, lq, lk, 128, out);
 }

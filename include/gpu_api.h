@@ -116,17 +116,18 @@ int gpu_convrot_requant(int dtype, const void* x, void* q, void* s, int64_t N, i
 int gpu_w6_requant(const void* weight, void* packed, void* s_rel, void* s_channel, int64_t N, int K, uint64_t seed,
                    void* stream);
 
-/* INT8 attention, head dim 128: o = softmax(q . k^T * scale) . v with q and k rotated (sign diagonal + Walsh-Hadamard
- * 128) and quantized per scale group (eight groups per 32 query rows, four per key tile), an optional K anchor
- * subtracted first, v quantized per channel, probabilities as u8 per key tile (64 keys, 128 beyond lk = 1024) and integer
- * P.V partials folded in fp32.  q/k/v/o: [b, seq, heads, 128] through element strides (batch, row, head), bf16
- * (gpu_int8_attn, gpu_int8_attn_d) or f16 (gpu_int8_attn_f16); h % hk == 0 (grouped-query heads); ws: 256-byte aligned
- * device scratch of gpu_int8_attn_workspace[_d] bytes, layout private to the library.
+/* INT8 attention, head dims 64, 128 and 256: o = softmax(q . k^T * scale) . v with q and k rotated and quantized per
+ * scale group (eight groups per block of 32 query rows, 16 at head dim 256; four per key tile), an optional K anchor
+ * subtracted first, v quantized per channel, probabilities as u8 per key tile (64 keys; 128 beyond lk = 1024 unless the
+ * head dim is 64) and integer P.V partials folded in fp32.  The rotation is the reference's choice by shape: up to 256
+ * keys H4 on runs of four channels only; beyond, H64 at head dim 64, sign diagonal + H128 at 128, H128 on each half at
+ * 256.  q/k/v/o: [b, seq, heads, head_dim] through element strides (batch, row, head), bf16 (gpu_int8_attn,
+ * gpu_int8_attn_d) or f16 (gpu_int8_attn_f16); h % hk == 0 (grouped-query heads); ws: 256-byte aligned device scratch of
+ * gpu_int8_attn_workspace[_d] bytes, layout private to the library.
  * Replaces gpu_int8_attn_workspace_d / gpu_int8_attn_workspace (csrc/attn_int8.cu:62-82), gpu_int8_attn_d (:101-108),
  * gpu_int8_attn_f16 (:111-118), gpu_int8_attn (:225-231); src/ffi.rs binds them under the same names.
- * Returns 0, -400 (argument the library refuses: message on stderr; head dims other than 128 are not built, and
- * gpu_int8_attn_workspace_d returns 0 bytes for them) or -401
- * (launch failure), the reference's codes.
+ * Returns 0, -400 (argument the library refuses: message on stderr; gpu_int8_attn_workspace_d returns 0 bytes for a
+ * head dim other than 64, 128, 256) or -401 (launch failure), the reference's codes.
  * gpu_int8_attn_sink (csrc/attn_int8.cu:193-202): attention over lk keys plus `sink` more whose keys and values are
  * zero, which count in the softmax denominator only; the K anchor is off so that a zero key's score stays zero; bf16.
  * A non-null qw normalizes q first as gpu_int8_attn_norm_rope does (weight qw, eps, no rotation), k taken as it is.
@@ -191,6 +192,7 @@ int gpu_internal_attn_sumsq_probe(const float* x, float* out, int rows, int spli
 /* Test hook, no reference counterpart: byte offsets of the pieces of the attention workspace and its tiling,
  * out[0..9] = qi, ki, qs, ks, vt, vs, anchors, vsum, key tile length, key tiles. */
 int gpu_internal_attn_layout(int b, int h, int hk, int lq, int lk, int64_t* out);
+int gpu_internal_attn_layout_d(int b, int h, int hk, int lq, int lk, int head_dim, int64_t* out);
 
 /* D[M,N] = Out((A[M,K] . W[N,K]^T) * xs[m] * ws[n] + bias[n]).
  * Replaces gpu_int8_gemm, src/ffi.rs:38 / csrc/gemm.cu:124-129.

@@ -65,6 +65,15 @@ def lib():
                                              vp, vp, vp, i32, vp, vp, vp, C.c_float, i32]
         L.orc_attn_int8_bias.restype = i32
         L.orc_attn_int8_bias.argtypes = [i32, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, C.c_float, vp, vp, i64, i64, i64]
+        L.orc_attn_quant_qk_d.restype = i32
+        L.orc_attn_quant_qk_d.argtypes = [i32, vp, vp, i32, i32, i32, i32, i32, i32, i64, i64, i64, i64, i64, i64, i32, i32, vp, vp,
+                                          vp, vp, vp, i32, vp, vp, vp, C.c_float, i32]
+        L.orc_attn_quant_v_d.restype = i32
+        L.orc_attn_quant_v_d.argtypes = [i32, vp, i32, i32, i32, i32, i64, i64, i64, vp, vp]
+        L.orc_attn_int8_d.restype = i32
+        L.orc_attn_int8_d.argtypes = [i32, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, f32, f32, vp, i64, i64, i64, i32]
+        L.orc_attn_rotate_d.restype = None
+        L.orc_attn_rotate_d.argtypes = [vp, i32, i32]
         L.orc_attn_rotate.restype = None
         L.orc_attn_rotate.argtypes = [vp, i32]
         L.orc_attn_sumsq128.restype = C.c_float
@@ -373,11 +382,11 @@ def attn_norm_rope_row(row, w, rope_row, eps, rope_mode):
 
 
 def attn_rotate(row, lk):
-    """The rotation the Q/K quantizers apply for a sequence of lk keys: H4 on runs of four channels up to 256 keys, the
-    sign diagonal and H128 beyond."""
+    """The rotation the Q/K quantizers apply to a row of 64, 128 or 256 channels for a sequence of lk keys: H4 on runs of
+    four channels up to 256 keys; beyond, H64 (head dim 64), the sign diagonal and H128 (128), H128 on each half (256)."""
     r = np.ascontiguousarray(row, dtype=np.float32).copy()
-    assert r.shape == (128,)
-    lib().orc_attn_rotate(_p(r), int(lk))
+    assert r.shape in ((64,), (128,), (256,))
+    lib().orc_attn_rotate_d(_p(r), r.shape[0], int(lk))
     return r
 
 
@@ -388,19 +397,20 @@ def attn_quant(dt, q, k, v, use_anchor=True, norm=None):
     given, ahead of the quantizers."""
     b, lq, h, D = q.shape
     _, lk, hk, _ = k.shape
-    assert D == 128 and v.shape == k.shape
+    assert D in (64, 128, 256) and v.shape == k.shape
     q, k, v = np.ascontiguousarray(q), np.ascontiguousarray(k), np.ascontiguousarray(v)
     ck = lib().orc_attn_cta_k(lk, D)
-    qg, kb = (lq + 127) // 128 * 4, (lk + ck - 1) // ck
+    qg, kb = (lq + 127) // 128 * (128 // (16 if D == 256 else 32)), (lk + ck - 1) // ck
     out = dict(ck=ck, qi=np.zeros((b, h, lq, D), np.int8), qs=np.zeros((b, h, qg * 8), np.float32),
                ki=np.zeros((b, hk, lk, D), np.int8), ks=np.zeros((b, hk, kb * 4), np.float32),
                anchors=np.zeros((b, hk), np.int32), vi=np.zeros((b, hk, lk, D), np.int8),
                vs=np.zeros((b, hk, D), np.float32))
     if norm is None:
-        rc = lib().orc_attn_quant_qk(dt, _p(q), _p(k), b, lq, lk, h, hk, lq * h * D, h * D, D, lk * hk * D, hk * D, D, ck,
-                                     1 if use_anchor else 0, _p(out["qi"]), _p(out["qs"]), _p(out["ki"]), _p(out["ks"]),
-                                     _p(out["anchors"]))
+        rc = lib().orc_attn_quant_qk_d(dt, _p(q), _p(k), b, lq, lk, h, hk, D, lq * h * D, h * D, D, lk * hk * D, hk * D, D, ck,
+                                       1 if use_anchor else 0, _p(out["qi"]), _p(out["qs"]), _p(out["ki"]), _p(out["ks"]),
+                                       _p(out["anchors"]), 0, None, None, None, 0.0, 0)
     else:
+        assert D == 128
         f = {n: (None if norm.get(n) is None else np.ascontiguousarray(norm[n], dtype=np.float32)) for n in ("qw", "kw", "rope")}
         if f["rope"] is not None:
             assert f["rope"].size >= max(lq, lk) * D
@@ -410,7 +420,7 @@ def attn_quant(dt, q, k, v, use_anchor=True, norm=None):
                                           _p(out["anchors"]), 1, pp["qw"], pp["kw"], pp["rope"], float(norm["eps"]),
                                           int(norm["rope_mode"]))
     assert rc == 0, rc
-    rc = lib().orc_attn_quant_v(dt, _p(v), b, lk, hk, lk * hk * D, hk * D, D, _p(out["vi"]), _p(out["vs"]))
+    rc = lib().orc_attn_quant_v_d(dt, _p(v), b, lk, hk, D, lk * hk * D, hk * D, D, _p(out["vi"]), _p(out["vs"]))
     assert rc == 0
     return out
 
@@ -436,8 +446,8 @@ def attn_int8(dt, q, k, v, scale, use_anchor=True, quant=None, sink=0.0, norm=No
     lk, hk = k.shape[1], k.shape[2]
     z = quant if quant is not None else attn_quant(dt, q, k, v, use_anchor, norm)
     o = np.zeros((b, lq, h, D), np.float32 if dt == F32 else np.uint16)
-    rc = lib().orc_attn_int8(dt, _p(z["qi"]), _p(z["ki"]), _p(z["vi"]), _p(z["qs"]), _p(z["ks"]), _p(z["vs"]), b, lq, lk,
-                             h, hk, z["ck"], float(scale), float(sink), _p(o), lq * h * D, h * D, D,
-                             1 if (dt == F16 and lk <= 512 and z["ck"] == 64) else 0)
+    rc = lib().orc_attn_int8_d(dt, _p(z["qi"]), _p(z["ki"]), _p(z["vi"]), _p(z["qs"]), _p(z["ks"]), _p(z["vs"]), b, lq, lk,
+                               h, hk, D, z["ck"], float(scale), float(sink), _p(o), lq * h * D, h * D, D,
+                               1 if (dt == F16 and lk <= 512 and z["ck"] == 64) else 0)
     assert rc == 0
     return o

@@ -762,27 +762,27 @@ ORC_API void orc_set_threads(int n) {
  * probabilities, integer P.V partials folded with fmaf) is pinned by the tests against a dense Hadamard matrix, the
  * quantizer's half-step bound and exact fp64 softmax attention.
  * ------------------------------------------------------------------------------------------- */
-#define ATTN_D 128
+#define ATTN_DMAX 256   /* head dims 64, 128, 256 (csrc/attn_int8.cu:42-45) */
 #define ATTN_U8_OFFSET 7.9943534f   /* csrc/vendor/sage/attn_utils.cuh:40 */
 
 /* Sign diagonal, then a normalized Walsh-Hadamard transform over 128 channels: H4 on each run of four channels, then
  * radix-2 butterflies over channel bits 2..6, then one scaling (csrc/vendor/sage/quant_qk_int8.cu:72-109,136-157). */
-ORC_API void orc_attn_rot128(float* v) {
-    static const uint32_t signs[4] = {0x1035997bu, 0x8087f5eeu, 0xee2e4e1au, 0x71132418u};
-    for (int ch = 0; ch < ATTN_D; ++ch) {
-        const int lane = ch >> 2, c = ch & 3;
-        const uint32_t flip = ((signs[lane >> 3] >> ((lane & 7) * 4 + c)) & 1u) ^ 1u;
-        v[ch] = u2f(f2u(v[ch]) ^ (flip << 31));
-    }
-    for (int g = 0; g < ATTN_D; g += 4) {
+/* The normalized H4 on each run of four adjacent channels (convrot4, quant_qk_int8.cu:72-85). */
+static void attn_h4(float* v, int n) {
+    for (int g = 0; g < n; g += 4) {
         const float a0 = v[g] + v[g + 1], a1 = v[g] - v[g + 1], a2 = v[g + 2] + v[g + 3], a3 = v[g + 2] - v[g + 3];
         v[g] = (a0 + a2) * 0.5f;
         v[g + 1] = (a1 + a3) * 0.5f;
         v[g + 2] = (a0 - a2) * 0.5f;
         v[g + 3] = (a1 - a3) * 0.5f;
     }
-    for (int bit = 1; bit < 32; bit <<= 1)
-        for (int lane = 0; lane < 32; ++lane) {
+}
+/* Walsh-Hadamard over n = 64 or 128 channels without the sign diagonal: H4, then radix-2 butterflies over the lane
+ * bits (channel bits 2 and up) in ascending order, then one scaling (convrot64 :111-133, convrot128_plain :136-157). */
+static void attn_h_plain(float* v, int n, float scale) {
+    attn_h4(v, n);
+    for (int bit = 1; bit < n / 4; bit <<= 1)
+        for (int lane = 0; lane < n / 4; ++lane) {
             if (lane & bit) continue;
             for (int c = 0; c < 4; ++c) {
                 const float lo = v[lane * 4 + c], hi = v[(lane | bit) * 4 + c];
@@ -790,25 +790,31 @@ ORC_API void orc_attn_rot128(float* v) {
                 v[(lane | bit) * 4 + c] = lo - hi;
             }
         }
-    for (int ch = 0; ch < ATTN_D; ++ch) v[ch] *= 0.1767766952966369f;
+    for (int ch = 0; ch < n; ++ch) v[ch] *= scale;
+}
+ORC_API void orc_attn_rot128(float* v) {
+    static const uint32_t signs[4] = {0x1035997bu, 0x8087f5eeu, 0xee2e4e1au, 0x71132418u};
+    for (int ch = 0; ch < 128; ++ch) {
+        const int lane = ch >> 2, c = ch & 3;
+        const uint32_t flip = ((signs[lane >> 3] >> ((lane & 7) * 4 + c)) & 1u) ^ 1u;
+        v[ch] = u2f(f2u(v[ch]) ^ (flip << 31));
+    }
+    attn_h_plain(v, 128, 0.1767766952966369f);
 }
 
-/* The rotation the quantizers apply, chosen by the key count (csrc/vendor/sage/quant_qk_int8.cu:1160-1166): sequences
- * of at most 256 keys take only the normalized H4 on each run of four adjacent channels (ROTATION 4, convrot4 :72-85),
- * longer ones the sign diagonal and H128. */
-ORC_API void orc_attn_rotate(float* v, int lk) {
-    if (lk > 256) {
-        orc_attn_rot128(v);
-        return;
-    }
-    for (int g = 0; g < ATTN_D; g += 4) {
-        const float a0 = v[g] + v[g + 1], a1 = v[g] - v[g + 1], a2 = v[g + 2] + v[g + 3], a3 = v[g + 2] - v[g + 3];
-        v[g] = (a0 + a2) * 0.5f;
-        v[g + 1] = (a1 + a3) * 0.5f;
-        v[g + 2] = (a0 - a2) * 0.5f;
-        v[g + 3] = (a1 - a3) * 0.5f;
+/* The rotation the quantizers apply, chosen by head dim and key count (quant_qk_int8.cu:1150-1195): sequences of at most
+ * 256 keys take only the H4 blocks (ROTATION 4); longer ones H64 at head dim 64, the sign diagonal and H128 at 128, and
+ * the plain H128 on each half at 256 (ROTATION 64, 128, 129). */
+ORC_API void orc_attn_rotate_d(float* v, int D, int lk) {
+    if (lk <= 256) attn_h4(v, D);
+    else if (D == 64) attn_h_plain(v, 64, 0.25f);
+    else if (D == 128) orc_attn_rot128(v);
+    else {
+        attn_h_plain(v, 128, 0.1767766952966369f);
+        attn_h_plain(v + 128, 128, 0.1767766952966369f);
     }
 }
+ORC_API void orc_attn_rotate(float* v, int lk) { orc_attn_rotate_d(v, 128, lk); }
 
 static inline int8_t attn_rn_s8(float v) {                       /* cvt.rni.sat.s8.f32, float_utils.cuh:39-45 */
     if (isnan(v)) return 0;
@@ -856,10 +862,11 @@ ORC_API float orc_attn_sumsq128(const float* v, int split) {
 }
 
 static void attn_norm_rope_row(float* v, const attn_norm_t* nm, int row) {
+    const int D = 128;   /* the fused norm exists for head dim 128 only (csrc/attn_int8.cu:135) */
     const float rstd = (float)(1.0 / sqrt((double)(orc_attn_sumsq128(v, nm->mode == 2) / 128.f + nm->eps)));
-    for (int c = 0; c < ATTN_D; ++c) v[c] = rnd_t(ORC_BF16, v[c] * rstd * (nm->w ? nm->w[c] : 1.f));
+    for (int c = 0; c < D; ++c) v[c] = rnd_t(ORC_BF16, v[c] * rstd * (nm->w ? nm->w[c] : 1.f));
     if (!nm->rope || nm->mode == 0) return;
-    const float* r = nm->rope + (int64_t)row * ATTN_D;
+    const float* r = nm->rope + (int64_t)row * D;
     if (nm->mode == 1) {
         for (int p = 0; p < 64; ++p) {
             const float c = r[2 * p], s = r[2 * p + 1], a = v[2 * p], b = v[2 * p + 1];
@@ -876,31 +883,36 @@ static void attn_norm_rope_row(float* v, const attn_norm_t* nm, int row) {
 }
 
 /* One row of q or k as the quantizer sees it. */
-static void attn_load_row(int dt, const void* x, int64_t base, int64_t stride_n, int row, const attn_norm_t* nm, float* out) {
-    for (int c = 0; c < ATTN_D; ++c) out[c] = ld_t(dt, x, base + (int64_t)row * stride_n + c);
+static void attn_load_row(int dt, const void* x, int64_t base, int64_t stride_n, int row, const attn_norm_t* nm, int D, float* out) {
+    for (int c = 0; c < D; ++c) out[c] = ld_t(dt, x, base + (int64_t)row * stride_n + c);
     if (nm && nm->on) attn_norm_rope_row(out, nm, row);
 }
 
 /* K anchor for one (batch, head): nine evenly spaced keys, the one closest to their mean, kept only when it lowers
- * the sampled energy without raising the sampled abs-max by more than 12.5 % (quant_qk_int8.cu:591-756, C = 128: one
- * channel per thread, four warps).  The distance 9*s - sum is taken as one fma, nvcc's default contraction. */
-static int attn_detect_anchor(int dt, const void* k, int64_t base, int64_t stride_n, int Lk, const attn_norm_t* nm) {
-    float s[9][ATTN_D];
-    for (int i = 0; i < 9; ++i) attn_load_row(dt, k, base, stride_n, (int)((int64_t)i * (Lk - 1) / 8), nm, s[i]);
-    float energy[ATTN_D], amax[ATTN_D], dist[9][ATTN_D];
-    for (int c = 0; c < ATTN_D; ++c) {
-        float e = 0.f, m = 0.f, sum = 0.f;
-        for (int i = 0; i < 9; ++i) {
-            e = fmaf(s[i][c], s[i][c], e);
-            m = fmax_dev(m, fabsf(s[i][c]));
-            sum += s[i][c];
+ * the sampled energy without raising the sampled abs-max by more than 12.5 % (quant_qk_int8.cu:591-756).  The
+ * reference's block has 128 threads in four warps; thread t walks channels t and t + 128 (head dim 256) with one set of
+ * accumulators, threads past the head dim (64) hold zeros; warps add by a shuffle-down tree, then the four warps in
+ * order.  The distance 9*s - sum is taken as one fma, nvcc's default contraction. */
+static int attn_detect_anchor(int dt, const void* k, int64_t base, int64_t stride_n, int Lk, const attn_norm_t* nm, int D) {
+    float s[9][ATTN_DMAX];
+    for (int i = 0; i < 9; ++i) attn_load_row(dt, k, base, stride_n, (int)((int64_t)i * (Lk - 1) / 8), nm, D, s[i]);
+    float energy[128], dist[9][128], amax = 0.f;
+    for (int t = 0; t < 128; ++t) {
+        float e = 0.f, d9[9] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        for (int c = t; c < D; c += 128) {
+            float sum = 0.f;
+            for (int i = 0; i < 9; ++i) {
+                e = fmaf(s[i][c], s[i][c], e);
+                amax = fmax_dev(amax, fabsf(s[i][c]));
+                sum += s[i][c];
+            }
+            for (int i = 0; i < 9; ++i) {
+                const float d = fmaf(9.f, s[i][c], -sum);
+                d9[i] = fmaf(d, d, d9[i]);
+            }
         }
-        energy[c] = e;
-        amax[c] = m;
-        for (int i = 0; i < 9; ++i) {
-            const float d = fmaf(9.f, s[i][c], -sum);
-            dist[i][c] = fmaf(d, d, 0.f);
-        }
+        energy[t] = e;
+        for (int i = 0; i < 9; ++i) dist[i][t] = d9[i];
     }
     int best = 0;
     float best_d = 3.402823466e+38F;
@@ -909,94 +921,105 @@ static int attn_detect_anchor(int dt, const void* k, int64_t base, int64_t strid
         for (int w = 0; w < 4; ++w) d += attn_tree_sum32(&dist[i][w * 32]);
         if (d < best_d) { best = i; best_d = d; }
     }
-    float e0 = 0.f, m0 = 0.f, e1 = 0.f, m1 = 0.f;
-    float be[ATTN_D];
-    for (int c = 0; c < ATTN_D; ++c) {
+    float e0 = 0.f, e1 = 0.f, m1 = 0.f;
+    float be[128];
+    for (int t = 0; t < 128; ++t) {
         float e = 0.f;
-        for (int i = 0; i < 9; ++i) {
-            const float r = s[i][c] - s[best][c];
-            e = fmaf(r, r, e);
-            m1 = fmax_dev(m1, fabsf(r));
-        }
-        be[c] = e;
-        m0 = fmax_dev(m0, amax[c]);
+        for (int c = t; c < D; c += 128)
+            for (int i = 0; i < 9; ++i) {
+                const float r = s[i][c] - s[best][c];
+                e = fmaf(r, r, e);
+                m1 = fmax_dev(m1, fabsf(r));
+            }
+        be[t] = e;
     }
     for (int w = 0; w < 4; ++w) {
         e0 += attn_tree_sum32(&energy[w * 32]);
         e1 += attn_tree_sum32(&be[w * 32]);
     }
-    return (e1 < e0 && m1 <= m0 * 1.125f) ? (int)((int64_t)best * (Lk - 1) / 8) : -1;
+    return (e1 < e0 && m1 <= amax * 1.125f) ? (int)((int64_t)best * (Lk - 1) / 8) : -1;
 }
 
 /* One scale group: rows[0..n) (absolute row numbers, those >= L skipped) of one head, minus `bias` when given,
  * rotated, abs-max over the group, scale = max/127 + 1e-7, codes = rn(v * (1/scale))
  * (quant_qk_int8.cu:296-413 for Q, :422-575 for K). */
 static void attn_quant_group(int dt, const void* x, int64_t base, int64_t stride_n, const int* rows, int n, int L,
-                             const float* bias, const attn_norm_t* nm, int lk, int8_t* out, float* scale) {
-    float buf[32][ATTN_D];
+                             const float* bias, const attn_norm_t* nm, int lk, int D, int8_t* out, float* scale) {
+    float buf[32][ATTN_DMAX];
     float mx = 0.f;
     for (int i = 0; i < n; ++i) {
         if (rows[i] >= L) continue;
-        attn_load_row(dt, x, base, stride_n, rows[i], nm, buf[i]);
+        attn_load_row(dt, x, base, stride_n, rows[i], nm, D, buf[i]);
         if (bias)
-            for (int c = 0; c < ATTN_D; ++c) buf[i][c] -= bias[c];
-        orc_attn_rotate(buf[i], lk);
-        for (int c = 0; c < ATTN_D; ++c) mx = fmax_dev(mx, fabsf(buf[i][c]));
+            for (int c = 0; c < D; ++c) buf[i][c] -= bias[c];
+        orc_attn_rotate_d(buf[i], D, lk);
+        for (int c = 0; c < D; ++c) mx = fmax_dev(mx, fabsf(buf[i][c]));
     }
     const float sc = mx / 127.f + 1e-7f, inv = 1.f / sc;
     *scale = sc;
     for (int i = 0; i < n; ++i) {
         if (rows[i] >= L) continue;
-        for (int c = 0; c < ATTN_D; ++c) out[(int64_t)rows[i] * ATTN_D + c] = attn_rn_s8(buf[i][c] * inv);
+        for (int c = 0; c < D; ++c) out[(int64_t)rows[i] * D + c] = attn_rn_s8(buf[i][c] * inv);
     }
 }
 
-/* q [b, lq, h, 128], k [b, lk, hk, 128] through element strides (batch, row, head).  qi [b,h,lq,128],
- * qs [b,h,ceil(lq/128)*32] (eight groups per 32 rows: rows r, r+8, r+16, r+24), ki [b,hk,lk,128],
- * ks [b,hk,ceil(lk/ck)*4] (four groups per ck keys: keys with (key % 8) / 2 equal), anchors [b,hk]. */
-/* norm != 0: q (always) and k (when kw is not null) go through attn_norm_rope_row first; rope may be null. */
-ORC_API int orc_attn_quant_qk_norm(int dt, const void* q, const void* k, int b, int lq, int lk, int h, int hk, int64_t q_bs,
-                                   int64_t q_rs, int64_t q_hs, int64_t k_bs, int64_t k_rs, int64_t k_hs, int ck, int use_anchor,
-                                   int8_t* qi, float* qs, int8_t* ki, float* ks, int32_t* anchors, int norm, const float* qw,
-                                   const float* kw, const float* rope, float eps, int rope_mode) {
+/* q [b, lq, h, D], k [b, lk, hk, D] through element strides (batch, row, head).  qi [b,h,lq,D];
+ * qs [b,h,ceil(lq/128)*(128/WQ)*8]: eight groups per WQ rows, group g of a block holding rows g, g+8, .. of it, WQ = 32
+ * rows (16 at head dim 256, csrc/attn_int8.cu:44); ki [b,hk,lk,D]; ks [b,hk,ceil(lk/ck)*4] (four groups per ck keys:
+ * keys with (key % 8) / 2 equal); anchors [b,hk].
+ * norm != 0 (head dim 128): q (always) and k (when kw is not null) go through attn_norm_rope_row first; rope may be null. */
+ORC_API int orc_attn_quant_qk_d(int dt, const void* q, const void* k, int b, int lq, int lk, int h, int hk, int D, int64_t q_bs,
+                                int64_t q_rs, int64_t q_hs, int64_t k_bs, int64_t k_rs, int64_t k_hs, int ck, int use_anchor,
+                                int8_t* qi, float* qs, int8_t* ki, float* ks, int32_t* anchors, int norm, const float* qw,
+                                const float* kw, const float* rope, float eps, int rope_mode) {
     if (ck != 64 && ck != 128) return -1;
-    if (norm && dt != ORC_BF16) return -400;
+    if (D != 64 && D != 128 && D != 256) return -1;
+    if (norm && (dt != ORC_BF16 || D != 128)) return -400;
     const attn_norm_t qn = {qw, rope, eps, rope_mode, norm ? 1 : 0}, kn = {kw, rope, eps, rope_mode, (norm && kw) ? 1 : 0};
-    const int qg = (lq + 127) / 128 * 4, kb = (lk + ck - 1) / ck;
+    const int wq = D == 256 ? 16 : 32, nr = wq / 8;
+    const int qg = (lq + 127) / 128 * (128 / wq), kb = (lk + ck - 1) / ck;
     for (int bi = 0; bi < b; ++bi)
         for (int hi = 0; hi < h; ++hi)
             for (int t = 0; t < qg; ++t)
                 for (int g = 0; g < 8; ++g) {
                     int rows[4];
-                    for (int j = 0; j < 4; ++j) rows[j] = t * 32 + g + 8 * j;
+                    for (int j = 0; j < nr; ++j) rows[j] = t * wq + g + 8 * j;
                     const int64_t bh = (int64_t)bi * h + hi;
-                    attn_quant_group(dt, q, bi * q_bs + hi * q_hs, q_rs, rows, 4, lq, NULL, &qn, lk, qi + bh * lq * ATTN_D,
+                    attn_quant_group(dt, q, bi * q_bs + hi * q_hs, q_rs, rows, nr, lq, NULL, &qn, lk, D, qi + bh * lq * D,
                                      &qs[(bh * qg + t) * 8 + g]);
                 }
     for (int bi = 0; bi < b; ++bi)
         for (int hi = 0; hi < hk; ++hi) {
             const int64_t bh = (int64_t)bi * hk + hi, base = bi * k_bs + hi * k_hs;
-            const int anchor = use_anchor ? attn_detect_anchor(dt, k, base, k_rs, lk, &kn) : -1;
+            const int anchor = use_anchor ? attn_detect_anchor(dt, k, base, k_rs, lk, &kn, D) : -1;
             anchors[bh] = anchor;
-            float bias[ATTN_D];
-            if (anchor >= 0) attn_load_row(dt, k, base, k_rs, anchor, &kn, bias);
+            float bias[ATTN_DMAX];
+            if (anchor >= 0) attn_load_row(dt, k, base, k_rs, anchor, &kn, D, bias);
             for (int t = 0; t < kb; ++t)
                 for (int g = 0; g < 4; ++g) {
                     int rows[32];
                     const int n = ck / 4;
                     for (int i = 0; i < n; ++i) rows[i] = t * ck + (i / 2) * 8 + g * 2 + (i % 2);
-                    attn_quant_group(dt, k, base, k_rs, rows, n, lk, anchor >= 0 ? bias : NULL, &kn, lk, ki + bh * lk * ATTN_D,
+                    attn_quant_group(dt, k, base, k_rs, rows, n, lk, anchor >= 0 ? bias : NULL, &kn, lk, D, ki + bh * lk * D,
                                      &ks[(bh * kb + t) * 4 + g]);
                 }
         }
     return 0;
 }
 
+ORC_API int orc_attn_quant_qk_norm(int dt, const void* q, const void* k, int b, int lq, int lk, int h, int hk, int64_t q_bs,
+                                   int64_t q_rs, int64_t q_hs, int64_t k_bs, int64_t k_rs, int64_t k_hs, int ck, int use_anchor,
+                                   int8_t* qi, float* qs, int8_t* ki, float* ks, int32_t* anchors, int norm, const float* qw,
+                                   const float* kw, const float* rope, float eps, int rope_mode) {
+    return orc_attn_quant_qk_d(dt, q, k, b, lq, lk, h, hk, 128, q_bs, q_rs, q_hs, k_bs, k_rs, k_hs, ck, use_anchor, qi, qs, ki, ks,
+                               anchors, norm, qw, kw, rope, eps, rope_mode);
+}
+
 ORC_API int orc_attn_quant_qk(int dt, const void* q, const void* k, int b, int lq, int lk, int h, int hk, int64_t q_bs,
                               int64_t q_rs, int64_t q_hs, int64_t k_bs, int64_t k_rs, int64_t k_hs, int ck, int use_anchor,
                               int8_t* qi, float* qs, int8_t* ki, float* ks, int32_t* anchors) {
-    return orc_attn_quant_qk_norm(dt, q, k, b, lq, lk, h, hk, q_bs, q_rs, q_hs, k_bs, k_rs, k_hs, ck, use_anchor, qi, qs, ki, ks,
-                                  anchors, 0, NULL, NULL, NULL, 0.f, 0);
+    return orc_attn_quant_qk_d(dt, q, k, b, lq, lk, h, hk, 128, q_bs, q_rs, q_hs, k_bs, k_rs, k_hs, ck, use_anchor, qi, qs, ki, ks,
+                               anchors, 0, NULL, NULL, NULL, 0.f, 0);
 }
 
 /* The row transform alone, for pins: v[128] float in place. */
@@ -1007,21 +1030,26 @@ ORC_API void orc_attn_norm_rope_row(float* v, const float* w, const float* rope_
 
 /* v [b, lk, hk, 128] -> vi [b,hk,lk,128] (plain order; the reference stores it transposed and permuted for its MMA,
  * quant_v_int8.cu:178-190), vs [b,hk,128]: scale = max(absmax/127 as a product with 1/127, 1e-12) (:163-168). */
-ORC_API int orc_attn_quant_v(int dt, const void* v, int b, int lk, int hk, int64_t v_bs, int64_t v_rs, int64_t v_hs,
-                             int8_t* vi, float* vs) {
+ORC_API int orc_attn_quant_v_d(int dt, const void* v, int b, int lk, int hk, int D, int64_t v_bs, int64_t v_rs, int64_t v_hs,
+                               int8_t* vi, float* vs) {
     for (int bi = 0; bi < b; ++bi)
         for (int hi = 0; hi < hk; ++hi) {
             const int64_t bh = (int64_t)bi * hk + hi, base = bi * v_bs + hi * v_hs;
-            for (int c = 0; c < ATTN_D; ++c) {
+            for (int c = 0; c < D; ++c) {
                 float mx = 0.f;
                 for (int n = 0; n < lk; ++n) mx = fmax_dev(mx, fabsf(ld_t(dt, v, base + (int64_t)n * v_rs + c)));
                 const float sc = fmax_dev(mx * (1.f / 127.f), 1e-12f), inv = 1.f / sc;
-                vs[bh * ATTN_D + c] = sc;
+                vs[bh * D + c] = sc;
                 for (int n = 0; n < lk; ++n)
-                    vi[(bh * lk + n) * ATTN_D + c] = attn_rn_s8(ld_t(dt, v, base + (int64_t)n * v_rs + c) * inv);
+                    vi[(bh * lk + n) * D + c] = attn_rn_s8(ld_t(dt, v, base + (int64_t)n * v_rs + c) * inv);
             }
         }
     return 0;
+}
+
+ORC_API int orc_attn_quant_v(int dt, const void* v, int b, int lk, int hk, int64_t v_bs, int64_t v_rs, int64_t v_hs,
+                             int8_t* vi, float* vs) {
+    return orc_attn_quant_v_d(dt, v, b, lk, hk, 128, v_bs, v_rs, v_hs, vi, vs);
 }
 
 static inline float attn_exp2(float x) { return (float)exp2((double)x); }
@@ -1037,21 +1065,22 @@ static inline float attn_exp2(float x) { return (float)exp2((double)x); }
  * of -50000, keys past lk at -1e30 raw, the denominator summing the UNROUNDED probabilities in the four per-thread
  * partials of a row, attn_utils.cuh:922-940, :1113-1122).  unfused: every tile takes it, which is what the reference's
  * build does for f16 outputs and at most 512 keys (sage_attn_launcher.cu:187-191, qk_int_sv_i8_cuda.cuh:132-139). */
-ORC_API int orc_attn_int8(int out_dt, const int8_t* qi, const int8_t* ki, const int8_t* vi, const float* qs,
-                          const float* ks, const float* vs, int b, int lq, int lk, int h, int hk, int ck, float scale,
-                          float sink, void* o, int64_t o_bs, int64_t o_rs, int64_t o_hs, int unfused) {
-    if ((ck != 64 && ck != 128) || hk <= 0 || h % hk != 0) return -1;
-    const int qg = (lq + 127) / 128 * 4, kb = (lk + ck - 1) / ck, rep = h / hk;
+ORC_API int orc_attn_int8_d(int out_dt, const int8_t* qi, const int8_t* ki, const int8_t* vi, const float* qs,
+                            const float* ks, const float* vs, int b, int lq, int lk, int h, int hk, int D, int ck, float scale,
+                            float sink, void* o, int64_t o_bs, int64_t o_rs, int64_t o_hs, int unfused) {
+    if ((ck != 64 && ck != 128) || hk <= 0 || h % hk != 0 || (D != 64 && D != 128 && D != 256)) return -1;
+    const int wq = D == 256 ? 16 : 32;
+    const int qg = (lq + 127) / 128 * (128 / wq), kb = (lk + ck - 1) / ck, rep = h / hk;
     const float sm = scale * 1.44269504088896340736f;
     #pragma omp parallel for collapse(2) schedule(dynamic, 8)
     for (int bh = 0; bh < b * h; ++bh)
         for (int r = 0; r < lq; ++r) {
             const int bi = bh / h, hi = bh % h;
             const int64_t kvh = (int64_t)bi * hk + hi / rep;
-            const int8_t* qrow = qi + ((int64_t)bh * lq + r) * ATTN_D;
-            const float q_scale = qs[((int64_t)bh * qg + r / 32) * 8 + r % 8];
-            float m = -50000.f, d = 1.f, ro[ATTN_D], d4[4] = {0.f, 0.f, 0.f, 0.f}, pf[128];
-            for (int c = 0; c < ATTN_D; ++c) ro[c] = 0.f;
+            const int8_t* qrow = qi + ((int64_t)bh * lq + r) * D;
+            const float q_scale = qs[((int64_t)bh * qg + r / wq) * 8 + r % 8];
+            float m = -50000.f, d = 1.f, ro[ATTN_DMAX], d4[4] = {0.f, 0.f, 0.f, 0.f}, pf[128];
+            for (int c = 0; c < D; ++c) ro[c] = 0.f;
             int32_t s[128];
             for (int t = 0; t < kb; ++t) {
                 const int n = lk - t * ck < ck ? lk - t * ck : ck;
@@ -1059,9 +1088,9 @@ ORC_API int orc_attn_int8(int out_dt, const int8_t* qi, const int8_t* ki, const 
                 float gs[4], tile_m = 0.f;
                 for (int g = 0; g < 4; ++g) gs[g] = sm * (q_scale * ks[(kvh * kb + t) * 4 + g]);
                 for (int j = 0; j < n; ++j) {
-                    const int8_t* krow = ki + ((int64_t)kvh * lk + t * ck + j) * ATTN_D;
+                    const int8_t* krow = ki + ((int64_t)kvh * lk + t * ck + j) * D;
                     int32_t acc = 0;
-                    for (int c = 0; c < ATTN_D; ++c) acc += (int32_t)qrow[c] * (int32_t)krow[c];
+                    for (int c = 0; c < D; ++c) acc += (int32_t)qrow[c] * (int32_t)krow[c];
                     s[j] = acc;
                 }
                 for (int g = 0; g < 4; ++g) {
@@ -1076,9 +1105,9 @@ ORC_API int orc_attn_int8(int out_dt, const int8_t* qi, const int8_t* ki, const 
                 const float smaller = attn_exp2(-fabsf(m - tile_m));
                 const float o_scale = m < tile_m ? smaller : 1.f, t_scale = tile_m < m ? smaller : 1.f;
                 m = m > tile_m ? m : tile_m;
-                int32_t pv[ATTN_D];
+                int32_t pv[ATTN_DMAX];
                 int32_t psum = 0;
-                for (int c = 0; c < ATTN_D; ++c) pv[c] = 0;
+                for (int c = 0; c < D; ++c) pv[c] = 0;
                 for (int j = n; j < ck; ++j) pf[j] = 0.f;       /* keys past lk: -1e30 raw, probability zero */
                 for (int j = 0; j < n; ++j) {
                     float p = attn_exp2(fmaf((float)s[j], gs[(j % 8) / 2], -tile_m));
@@ -1086,8 +1115,8 @@ ORC_API int orc_attn_int8(int out_dt, const int8_t* qi, const int8_t* ki, const 
                     p = rintf(p > 255.f ? 255.f : p);
                     const int32_t pi = (int32_t)p;
                     psum += pi;
-                    const int8_t* vrow = vi + ((int64_t)kvh * lk + t * ck + j) * ATTN_D;
-                    for (int c = 0; c < ATTN_D; ++c) pv[c] += pi * (int32_t)vrow[c];
+                    const int8_t* vrow = vi + ((int64_t)kvh * lk + t * ck + j) * D;
+                    for (int c = 0; c < D; ++c) pv[c] += pi * (int32_t)vrow[c];
                 }
                 d *= o_scale;
                 for (int l = 0; l < 4; ++l) d4[l] *= o_scale;
@@ -1101,17 +1130,23 @@ ORC_API int orc_attn_int8(int out_dt, const int8_t* qi, const int8_t* ki, const 
                 } else {
                     d += (float)psum * t_scale;
                 }
-                for (int c = 0; c < ATTN_D; ++c) ro[c] = fmaf((float)pv[c], t_scale, ro[c] * o_scale);
+                for (int c = 0; c < D; ++c) ro[c] = fmaf((float)pv[c], t_scale, ro[c] * o_scale);
             }
             /* `sink` more keys of score zero and value zero: each adds exp2(0 - m) to the denominator and nothing to
              * the output (attn_utils.cuh:1122-1130, csrc/attn_int8.cu:193-197) */
             d += (d4[0] + d4[1]) + (d4[2] + d4[3]);
             if (sink != 0.f) d = fmaf(sink, attn_exp2(-m), d);
             const float rcp = 1.f / d;
-            for (int c = 0; c < ATTN_D; ++c)
-                st_t(out_dt, o, bi * o_bs + (int64_t)r * o_rs + hi * o_hs + c, ro[c] * rcp * vs[kvh * ATTN_D + c]);
+            for (int c = 0; c < D; ++c)
+                st_t(out_dt, o, bi * o_bs + (int64_t)r * o_rs + hi * o_hs + c, ro[c] * rcp * vs[kvh * D + c]);
         }
     return 0;
+}
+
+ORC_API int orc_attn_int8(int out_dt, const int8_t* qi, const int8_t* ki, const int8_t* vi, const float* qs,
+                          const float* ks, const float* vs, int b, int lq, int lk, int h, int hk, int ck, float scale,
+                          float sink, void* o, int64_t o_bs, int64_t o_rs, int64_t o_hs, int unfused) {
+    return orc_attn_int8_d(out_dt, qi, ki, vi, qs, ks, vs, b, lq, lk, h, hk, 128, ck, scale, sink, o, o_bs, o_rs, o_hs, unfused);
 }
 
 /* The same attention with an additive bias per key on the logits (gpu_int8_attn_key_bias, csrc/attn_int8.cu:204-223):
@@ -1137,6 +1172,7 @@ ORC_API int orc_attn_int8_bias(int out_dt, const int8_t* qi, const int8_t* ki, c
                                const float* ks, const float* vs, int b, int lq, int lk, int h, int hk, int ck, float scale,
                                const float* bias, void* o, int64_t o_bs, int64_t o_rs, int64_t o_hs) {
     if ((ck != 64 && ck != 128) || hk <= 0 || h % hk != 0 || !bias) return -1;
+    const int D = 128;   /* the key-bias entry point exists for head dim 128 only (csrc/attn_int8.cu:191) */
     const int qg = (lq + 127) / 128 * 4, kb = (lk + ck - 1) / ck, rep = h / hk;
     const float log2e = 1.44269504088896340736f;
     const float sm = scale * log2e;
@@ -1159,11 +1195,11 @@ ORC_API int orc_attn_int8_bias(int out_dt, const int8_t* qi, const int8_t* ki, c
         for (int r = 0; r < lq; ++r) {
             const int bi = bh / h, hi = bh % h;
             const int64_t kvh = (int64_t)bi * hk + hi / rep;
-            const int8_t* qrow = qi + ((int64_t)bh * lq + r) * ATTN_D;
+            const int8_t* qrow = qi + ((int64_t)bh * lq + r) * D;
             const float q_scale = qs[((int64_t)bh * qg + r / 32) * 8 + r % 8];
-            float m = -50000.f, ro[ATTN_D], d4[4] = {1.f, 1.f, 1.f, 1.f}, d = 1.f;
+            float m = -50000.f, ro[ATTN_DMAX], d4[4] = {1.f, 1.f, 1.f, 1.f}, d = 1.f;
             int valid = 0;
-            for (int c = 0; c < ATTN_D; ++c) ro[c] = 0.f;
+            for (int c = 0; c < D; ++c) ro[c] = 0.f;
             int32_t s[128];
             float f[128], pf[128];
             for (int t = 0; t < kb; ++t) {
@@ -1174,9 +1210,9 @@ ORC_API int orc_attn_int8_bias(int out_dt, const int8_t* qi, const int8_t* ki, c
                 for (int j = 0; j < ck; ++j) {
                     s[j] = 0;
                     if (j >= n) continue;
-                    const int8_t* krow = ki + ((int64_t)kvh * lk + t * ck + j) * ATTN_D;
+                    const int8_t* krow = ki + ((int64_t)kvh * lk + t * ck + j) * D;
                     int32_t acc = 0;
-                    for (int c = 0; c < ATTN_D; ++c) acc += (int32_t)qrow[c] * (int32_t)krow[c];
+                    for (int c = 0; c < D; ++c) acc += (int32_t)qrow[c] * (int32_t)krow[c];
                     s[j] = acc;
                 }
                 float tile_m, neg_m = 0.f;
@@ -1217,9 +1253,9 @@ ORC_API int orc_attn_int8_bias(int out_dt, const int8_t* qi, const int8_t* ki, c
                 const float smaller = attn_exp2(-fabsf(m - tile_m));
                 const float o_scale = m < tile_m ? smaller : 1.f, t_scale = tile_m < m ? smaller : 1.f;
                 m = m > tile_m ? m : tile_m;
-                int32_t pv[ATTN_D];
+                int32_t pv[ATTN_DMAX];
                 int32_t psum = 0;
-                for (int c = 0; c < ATTN_D; ++c) pv[c] = 0;
+                for (int c = 0; c < D; ++c) pv[c] = 0;
                 for (int j = 0; j < ck; ++j) {
                     float p = route == 1 ? attn_exp2(fmaf((float)s[j], gs[(j % 8) / 2], neg_m)) : attn_exp2(f[j] + (-tile_m));
                     pf[j] = p;
@@ -1228,8 +1264,8 @@ ORC_API int orc_attn_int8_bias(int out_dt, const int8_t* qi, const int8_t* ki, c
                     const int32_t pi = (int32_t)p;
                     psum += pi;
                     if (j >= n || pi == 0) continue;
-                    const int8_t* vrow = vi + ((int64_t)kvh * lk + t * ck + j) * ATTN_D;
-                    for (int c = 0; c < ATTN_D; ++c) pv[c] += pi * (int32_t)vrow[c];
+                    const int8_t* vrow = vi + ((int64_t)kvh * lk + t * ck + j) * D;
+                    for (int c = 0; c < D; ++c) pv[c] += pi * (int32_t)vrow[c];
                 }
                 if (route == 0) {
                     for (int l = 0; l < 4; ++l) d4[l] *= o_scale;
@@ -1243,14 +1279,14 @@ ORC_API int orc_attn_int8_bias(int out_dt, const int8_t* qi, const int8_t* ki, c
                     d *= o_scale;
                     d += (float)psum * t_scale;
                 }
-                for (int c = 0; c < ATTN_D; ++c) ro[c] = fmaf((float)pv[c], t_scale, ro[c] * o_scale);
+                for (int c = 0; c < D; ++c) ro[c] = fmaf((float)pv[c], t_scale, ro[c] * o_scale);
             }
             if (ck == 64) d = (d4[0] + d4[1]) + (d4[2] + d4[3]);
             const float rcp = 1.f / d;
-            for (int c = 0; c < ATTN_D; ++c) {
+            for (int c = 0; c < D; ++c) {
                 float out = ro[c] * rcp;
                 if (ck == 64 && !valid) out = 0.f;
-                st_t(out_dt, o, bi * o_bs + (int64_t)r * o_rs + hi * o_hs + c, out * vs[kvh * ATTN_D + c]);
+                st_t(out_dt, o, bi * o_bs + (int64_t)r * o_rs + hi * o_hs + c, out * vs[kvh * D + c]);
             }
         }
     free(bl);

@@ -30,11 +30,11 @@ def _to_f32(bits, dt):
     return oracle.bf16_to_f32(bits) if dt == oracle.BF16 else oracle.f16_to_f32(bits)
 
 
-def _inputs(b, lq, lk, h, hk, dtype, seed, k_offset=0.0, v_scale=1.0):
+def _inputs(b, lq, lk, h, hk, dtype, seed, k_offset=0.0, v_scale=1.0, D=128):
     g = torch.Generator().manual_seed(seed)
-    q = torch.randn(b, lq, h, 128, generator=g)
-    k = torch.randn(b, lk, hk, 128, generator=g) + k_offset
-    v = torch.randn(b, lk, hk, 128, generator=g) * v_scale
+    q = torch.randn(b, lq, h, D, generator=g)
+    k = torch.randn(b, lk, hk, D, generator=g) + k_offset
+    v = torch.randn(b, lk, hk, D, generator=g) * v_scale
     return q.to(dtype), k.to(dtype), v.to(dtype)
 
 
@@ -420,9 +420,9 @@ def test_attention_refuses_what_it_does_not_build():
     ws = torch.zeros(1 << 16, dtype=torch.uint8, device="cuda")
     p = lambda t: C.c_void_p(t.data_ptr())
     args = lambda D, h, hk: (p(x), p(x), p(x), p(x), p(ws), 1, 4, 4, h, hk, D, 512, 128, 128, 512, 128, 128, 512, 128, 128, 512, 128, 128, 0.1, None)
-    assert ffi.raw("gpu_int8_attn_d", *args(64, 1, 1)) == -400
-    assert ffi.lib.gpu_int8_attn_workspace_d(1, 1, 1, 4, 4, 64) == 0 and ffi.lib.gpu_int8_attn_workspace_d(1, 1, 1, 4, 4, 256) == 0
-    assert ffi.lib.gpu_int8_attn_workspace_d(1, 1, 1, 4, 4, 128) > 0
+    assert ffi.raw("gpu_int8_attn_d", *args(96, 1, 1)) == -400
+    assert ffi.lib.gpu_int8_attn_workspace_d(1, 1, 1, 4, 4, 96) == 0 and ffi.lib.gpu_int8_attn_workspace_d(1, 1, 1, 4, 4, 512) == 0
+    assert ffi.lib.gpu_int8_attn_workspace_d(1, 1, 1, 4, 4, 128) > 0 and ffi.lib.gpu_int8_attn_workspace_d(1, 1, 1, 4, 4, 64) > 0
     assert ffi.raw("gpu_int8_attn_d", *args(128, 3, 2)) == -400
     assert ffi.raw("gpu_int8_attn_d", *args(128, 1, 1)) == 0
     torch.cuda.synchronize()
@@ -550,5 +550,79 @@ def test_attention_f16_short_sequences_take_the_unfused_path(amp):
     tol = 2 * vmax / 255.0 + 2 * 2.0 ** -11 * np.abs(ref)
     assert (np.abs(got - ref) <= tol).all()
     ex = _exact(q, k, v, 0.088)
+    cos = float((got * ex).sum() / np.sqrt((got * got).sum() * (ex * ex).sum()))
+    assert cos > 0.9995, cos
+
+
+HD_CASES = [
+    # D, b, lq, lk, h, hk, dtype, k_offset
+    (64, 1, 200, 300, 4, 2, torch.bfloat16, 0.0),
+    (64, 2, 77, 64, 2, 2, torch.float16, 0.0),        # f16, short: unfused path, H4 rotation
+    (64, 1, 129, 1500, 2, 1, torch.float16, 3.0),      # head dim 64 keeps 64-key tiles at any length; anchor on
+    (64, 1, 1, 1, 1, 1, torch.bfloat16, 0.0),
+    (256, 1, 100, 150, 2, 1, torch.bfloat16, 0.0),     # 16-row Q blocks, H4 rotation
+    (256, 1, 70, 400, 2, 2, torch.float16, 2.5),       # plain H128 per half, anchor on, unfused path
+    (256, 1, 150, 1100, 2, 1, torch.bfloat16, 0.0),    # 128-key tiles
+    (256, 1, 33, 1025, 1, 1, torch.float16, 0.0),
+]
+
+
+@pytest.mark.parametrize("case", HD_CASES, ids=lambda c: "D%d_b%d_lq%d_lk%d_h%d_hk%d_%s_off%g" % (c[:6] + (str(c[6])[6:], c[7])))
+def test_attention_head_dims_64_and_256(case):
+    """gpu_int8_attn_d / gpu_int8_attn_f16 at head dims 64 and 256: anchors, Q and K codes and scales, V scales bit-exact
+    against the oracle; outputs within the attention tolerance; close to exact attention."""
+    ql, ffi = _pkg()
+    D, b, lq, lk, h, hk, dtype, off = case
+    dt = oracle.BF16 if dtype == torch.bfloat16 else oracle.F16
+    q, k, v = _inputs(b, lq, lk, h, hk, dtype, seed=D + lq + lk, k_offset=off, D=D)
+    scale = D ** -0.5
+    ref_q = oracle.attn_quant(dt, _bits(q), _bits(k), _bits(v))
+    ref = _to_f32(oracle.attn_int8(dt, _bits(q), _bits(k), _bits(v), scale, quant=ref_q), dt)
+    ws_bytes = ffi.lib.gpu_int8_attn_workspace_d(b, h, hk, lq, lk, D)
+    assert ws_bytes > 0
+    ws = torch.zeros((ws_bytes,), dtype=torch.uint8, device="cuda")
+    o = ql.int8_attn(q.cuda(), k.cuda(), v.cuda(), scale, ws=ws)
+    torch.cuda.synchronize()
+    w = ws.cpu().numpy()
+    out = (C.c_int64 * 10)()
+    assert ffi.raw("gpu_internal_attn_layout_d", b, h, hk, lq, lk, D, C.cast(out, C.c_void_p)) == 0
+    qi_o, ki_o, qs_o, ks_o, vt_o, vs_o, an_o, vsum_o, ck, kb = list(out)
+    assert ck == ref_q["ck"]
+
+    def take(at, n, dtp):
+        return w[at:at + n * np.dtype(dtp).itemsize].view(dtp)
+
+    assert np.array_equal(take(an_o, b * hk, np.int32).reshape(b, hk), ref_q["anchors"])
+    if off >= 2.0:
+        assert (ref_q["anchors"] >= 0).all()
+    assert np.array_equal(take(qi_o, b * h * lq * D, np.int8).reshape(b, h, lq, D), ref_q["qi"])
+    nblk = kb * (ck // 32)
+    ki = take(ki_o, b * hk * nblk * 32 * D, np.int8).reshape(b, hk, nblk, D // 32, 2, 32, 16)
+    ki = ki.transpose(0, 1, 2, 5, 3, 4, 6).reshape(b, hk, nblk * 32, D)[:, :, :lk]
+    assert np.array_equal(ki, ref_q["ki"])
+    wq = 16 if D == 256 else 32
+    own = np.zeros(ref_q["qs"].shape[-1], bool)
+    for r in range(lq):
+        own[(r // wq) * 8 + r % 8] = True
+    qs = take(qs_o, ref_q["qs"].size, np.float32).reshape(ref_q["qs"].shape)
+    assert np.array_equal(qs[..., own].view(np.uint32), ref_q["qs"][..., own].view(np.uint32))
+    assert np.array_equal(take(ks_o, ref_q["ks"].size, np.float32).view(np.uint32), ref_q["ks"].reshape(-1).view(np.uint32))
+    assert np.array_equal(take(vs_o, b * hk * D, np.float32).view(np.uint32), ref_q["vs"].reshape(-1).view(np.uint32))
+    vt = take(vt_o, b * hk * nblk * D * 32, np.int8).reshape(b, hk, nblk, D, 32)
+    pos = np.arange(32)
+    key_of_pos = ((pos % 16) // 4) * 8 + (pos // 16) * 4 + pos % 4
+    vi_pad = np.zeros((b, hk, nblk * 32, D), np.int8)
+    vi_pad[:, :, :lk] = ref_q["vi"]
+    want_vt = vi_pad.reshape(b, hk, nblk, 32, D)[:, :, :, key_of_pos, :].transpose(0, 1, 2, 4, 3)
+    assert np.array_equal(vt, want_vt)
+
+    got = _to_f32(_bits(o), dt)
+    vmax = float(v.float().abs().max())
+    ulp = 2.0 ** (-8 if dt == oracle.BF16 else -11)
+    tol = 2 * vmax / 255.0 + 2 * ulp * np.abs(ref)
+    err = np.abs(got - ref)
+    assert (err <= tol).all(), "max excess %g" % float((err - tol).max())
+    assert (err <= ulp * np.abs(ref) + 1e-30).mean() > 0.97
+    ex = _exact(q, k, v, scale)
     cos = float((got * ex).sum() / np.sqrt((got * got).sum() * (ex * ex).sum()))
     assert cos > 0.9995, cos

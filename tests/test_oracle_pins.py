@@ -1223,3 +1223,66 @@ def test_attn_unfused_path_for_f16_short_sequences():
         p = np.exp(logits - logits.max(-1, keepdims=True))
         ex = np.einsum("bhqk,bkhd->bqhd", p / p.sum(-1, keepdims=True), vf)
         assert np.abs(got - ex).max() < 0.04
+
+
+@pytest.mark.parametrize("D", [64, 256])
+def test_attn_other_head_dims_rotation_groups_and_attention(D):
+    """Head dims 64 and 256: the rotation against dense matrices (H64 over the row; H128 on each half, no sign diagonal;
+    H4 blocks up to 256 keys), the Q scale groups (32-row blocks, 16-row blocks at 256) through the half-step bound of
+    every code with its group's scale, and the whole attention against float64 softmax."""
+    import scipy.linalg
+    rng = np.random.default_rng(D)
+    x = rng.integers(-8, 9, D).astype(np.float32)
+    if D == 64:
+        H = scipy.linalg.hadamard(64).astype(np.float64) / 8.0
+    else:
+        H = np.kron(np.eye(2), scipy.linalg.hadamard(128).astype(np.float64) / np.sqrt(128.0))
+    assert np.abs(oracle.attn_rotate(x, 300) - H @ x).max() < 2e-6
+    e = np.zeros(D, np.float32)
+    e[D - 3] = 1.0
+    assert np.array_equal(oracle.attn_rotate(e, 300), H[:, D - 3].astype(np.float32))
+    h4 = np.kron(np.eye(D // 4), scipy.linalg.hadamard(4) * 0.5)
+    assert np.array_equal(oracle.attn_rotate(x, 256), (h4 @ x).astype(np.float32))
+
+    b, lq, h, hk = 1, 50, 2, 1
+    wq = 16 if D == 256 else 32
+    for lk in (90, 300, 1100):
+        bits = lambda a: oracle.bf16_bits(np.asarray(a, np.float32))
+        q, k, v = (bits(rng.standard_normal(s)) for s in ((b, lq, h, D), (b, lk, hk, D), (b, lk, hk, D)))
+        z = oracle.attn_quant(oracle.BF16, q, k, v, use_anchor=False)
+        assert z["ck"] == (128 if (lk > 1024 and D != 64) else 64)
+        assert z["qs"].shape[-1] == (lq + 127) // 128 * (128 // wq) * 8
+        R = H if lk > 256 else h4
+        rq = oracle.bf16_to_f32(q).astype(np.float64) @ R.T
+        rk = oracle.bf16_to_f32(k).astype(np.float64) @ R.T
+        for r in range(lq):
+            for hi in range(h):
+                sc = z["qs"][0, hi, (r // wq) * 8 + r % 8]
+                assert np.abs(z["qi"][0, hi, r] * np.float64(sc) - rq[0, r, hi]).max() <= 0.5 * sc * 1.0001 + 1e-6
+        ck = z["ck"]
+        for n in range(lk):
+            sc = z["ks"][0, 0, (n // ck) * 4 + (n % 8) // 2]
+            assert np.abs(z["ki"][0, 0, n] * np.float64(sc) - rk[0, n, 0]).max() <= 0.5 * sc * 1.0001 + 1e-6
+        scale = D ** -0.5
+        got = oracle.bf16_to_f32(oracle.attn_int8(oracle.BF16, q, k, v, scale)).astype(np.float64)
+        ex = _exact_attention(q, k, v, scale)
+        assert np.abs(got - ex).max() < 0.04
+        assert (got * ex).sum() / np.sqrt((got * got).sum() * (ex * ex).sum()) > 0.9995
+
+
+@pytest.mark.parametrize("D", [64, 256])
+def test_attn_anchor_at_other_head_dims(D):
+    """The anchor search walks channels t and t + 128 per thread at head dim 256 and leaves threads idle at 64: it still
+    switches on for offset keys only, and the attention does not change beyond rounding."""
+    rng = np.random.default_rng(7)
+    bits = lambda a: oracle.bf16_bits(np.asarray(a, np.float32))
+    q = bits(rng.standard_normal((1, 20, 2, D)))
+    v = bits(rng.standard_normal((1, 150, 2, D)))
+    k0 = rng.standard_normal((1, 150, 2, D))
+    assert (oracle.attn_quant(oracle.BF16, q, bits(k0), v)["anchors"] == -1).all()
+    k1 = bits(k0 + 4.0)
+    z = oracle.attn_quant(oracle.BF16, q, k1, v)
+    assert (z["anchors"] >= 0).all()
+    a = oracle.bf16_to_f32(oracle.attn_int8(oracle.BF16, q, k1, v, D ** -0.5, quant=z)).astype(np.float64)
+    ex = _exact_attention(q, k1, v, D ** -0.5)
+    assert np.abs(a - ex).max() < 0.04
