@@ -245,20 +245,37 @@ def time_row_kernels(torch, ffi, steps):
 
 
 def time_attention(torch, ffi, steps):
-    """INT8 attention (quantizers + attention kernel, one call) at the image-DiT joint-attention shape, HIP events on
-    the launch stream.  ops = 4 * b * h * lq * lk * 128 (the two matrix products)."""
+    """INT8 attention (quantizers + attention kernel, one call), HIP events on the launch stream: the image-DiT joint
+    attention as the plain call, as the DiT issues it (fused q/k norm + RoPE) and with a per-key bias; a long video
+    shape; the SDXL UNet's head dim 64 in fp16.  ops = 4 * b * h * lq * lk * head_dim (the two matrix products)."""
     dev = "cuda:0"
     st = torch.cuda.current_stream()
     g = torch.Generator(device=dev).manual_seed(11)
     out = []
-    for (name, b, l, h, hk) in (("image-dit joint attention", 1, 4608, 24, 24), ("long video attention", 2, 8192, 16, 16)):
-        q, k, v = (torch.randn(b, l, hh, 128, device=dev, generator=g).to(torch.bfloat16) for hh in (h, hk, hk))
+    cases = (("image-dit joint attention", "gpu_int8_attn_d", 1, 4608, 24, 24, 128, torch.bfloat16),
+             ("image-dit joint attention, fused q/k norm + rope", "gpu_int8_attn_norm_rope", 1, 4608, 24, 24, 128, torch.bfloat16),
+             ("image-dit joint attention, per-key bias", "gpu_int8_attn_key_bias", 1, 4608, 24, 24, 128, torch.bfloat16),
+             ("long video attention", "gpu_int8_attn_d", 2, 8192, 16, 16, 128, torch.bfloat16),
+             ("sdxl self-attention 64x64 latent, 10 heads of 64", "gpu_int8_attn_f16", 2, 4096, 10, 10, 64, torch.float16))
+    for (name, entry, b, l, h, hk, hd, dtype) in cases:
+        q, k, v = (torch.randn(b, l, hh, hd, device=dev, generator=g).to(dtype) for hh in (h, hk, hk))
         o = torch.empty_like(q)
-        ws = torch.empty((ffi.lib.gpu_int8_attn_workspace_d(b, h, hk, l, l, 128),), dtype=torch.uint8, device=dev)
+        nws = ffi.lib.gpu_int8_attn_key_bias_workspace(b, h, hk, l, l) if entry.endswith("key_bias") else ffi.lib.gpu_int8_attn_workspace_d(b, h, hk, l, l, hd)
+        ws = torch.empty((nws,), dtype=torch.uint8, device=dev)
         sq, sk = q.stride(), k.stride()
-        call = lambda: ffi.k("gpu_int8_attn_d", q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), ws.data_ptr(), b, l, l, h,
-                             hk, 128, sq[0], sq[1], sq[2], sk[0], sk[1], sk[2], sk[0], sk[1], sk[2], sq[0], sq[1], sq[2],
-                             128 ** -0.5, st.cuda_stream)
+        head = (q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), ws.data_ptr(), b, l, l, h, hk)
+        strides = (sq[0], sq[1], sq[2], sk[0], sk[1], sk[2], sk[0], sk[1], sk[2], sq[0], sq[1], sq[2])
+        if entry == "gpu_int8_attn_norm_rope":
+            qw, kw = (1.0 + 0.1 * torch.randn(hd, device=dev, generator=g) for _ in range(2))
+            ang = torch.arange(l, device=dev, dtype=torch.float32)[:, None] * torch.exp(-6.0 * torch.rand(hd // 2, device=dev, generator=g))[None, :]
+            rope = torch.stack([torch.cos(ang), torch.sin(ang)], -1).contiguous()
+            call = lambda: ffi.k(entry, *head, *strides, hd ** -0.5, qw.data_ptr(), kw.data_ptr(), 1e-6, rope.data_ptr(), 1, st.cuda_stream)
+        elif entry == "gpu_int8_attn_key_bias":
+            bias = torch.zeros(l, device=dev)
+            bias[torch.randint(0, l, (l // 16,), device=dev, generator=g)] = 0.6
+            call = lambda: ffi.k(entry, *head, *strides, hd ** -0.5, bias.data_ptr(), st.cuda_stream)
+        else:
+            call = lambda: ffi.k(entry, *head, hd, *strides, hd ** -0.5, st.cuda_stream)
         for _ in range(3):
             call()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -269,8 +286,8 @@ def time_attention(torch, ffi, steps):
         e1.record(st)
         torch.cuda.synchronize()
         us = e0.elapsed_time(e1) * 1e3 / steps
-        ops = 4.0 * b * h * l * l * 128
-        out.append({"name": name, "b": b, "lq": l, "lk": l, "h": h, "hk": hk, "head_dim": 128, "kernel": "gpu_int8_attn_d",
+        ops = 4.0 * b * h * l * l * hd
+        out.append({"name": name, "b": b, "lq": l, "lk": l, "h": h, "hk": hk, "head_dim": hd, "kernel": entry,
                     "us": round(us, 1), "TOPS": round(ops / us / 1e6, 1), "frac_int8_peak": round(ops / us / 1e6 / PEAK_INT8_TOPS, 4)})
         del q, k, v, o, ws
     return out
