@@ -757,8 +757,12 @@ ORC_API void orc_set_threads(int n) {
  * INT8 attention, head dim 128 (csrc/attn_int8.cu:118-160 chains the three stages below).
  *
  * PARITY UNPINNED against a run of the reference: its exp2 and reciprocal are PTX approximations
- * (csrc/vendor/sage/math.cuh:54-58,111-115) and its build may pass --use_fast_math (build.rs:140); here exp2 is
- * fp64 libm rounded to fp32 and divisions are IEEE.  The structure (rotation, scale groups, anchor, tile maxima, u8
+ * (csrc/vendor/sage/math.cuh:54-58,111-115), and its build compiles the sage units (quant_qk_int8.cu, quant_v_int8.cu,
+ * sage_attn_launcher.cu with the attention kernel) with --use_fast_math (build.rs:84-86,139-141): approximate division,
+ * reciprocal and rsqrt, denormals flushed, so the scales mx / 127 + 1e-7 and 1 / scale can differ from IEEE in the last
+ * bit and a code that sits on a rounding boundary with them.  Here exp2 is fp64 libm rounded to fp32 and divisions are
+ * IEEE.  (The linear path's units -- kernels.cu, gemm.cu, sd.cu, h3.cu, cutlass_gemm_int8.cu -- are built without fast
+ * math, build.rs:69-81.)  The structure (rotation, scale groups, anchor, tile maxima, u8
  * probabilities, integer P.V partials folded with fmaf) is pinned by the tests against a dense Hadamard matrix, the
  * quantizer's half-step bound and exact fp64 softmax attention.
  * ------------------------------------------------------------------------------------------- */

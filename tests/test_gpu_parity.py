@@ -860,6 +860,9 @@ def test_w6a8_linear_matches_decode_then_gemm():
 W6G_CASES = [  # (M, N, K, out_dt, with_bias)
     (256, 128, 128, BF16, True), (100, 200, 256, BF16, False), (300, 136, 640, F32, True), (513, 260, 384, F16, True),
     (1, 8, 128, BF16, True), (777, 1000, 1280, BF16, True),
+    (2200, 4000, 256, BF16, True),     # 288 tiles: workgroups walk more than one tile, two groups each
+    (1500, 5300, 128, F16, False),     # 252 tiles of one group: the DMA stream is always a tile ahead
+    (2304, 4224, 384, F32, True),      # 297 tiles, whole tiles only
 ]
 
 
