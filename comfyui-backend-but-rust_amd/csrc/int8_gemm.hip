@@ -530,10 +530,9 @@ __device__ __forceinline__ void wait_lgkmcnt0() { asm volatile("s_waitcnt lgkmcn
 // ---------------------------------------------------------------------------------------------------------------
 template <int V> struct ic { static constexpr int value = V; };
 
-// BN: tile width; WGM x WGN: wave grid, four waves (one per SIMD, 128x128 wave tiles, up to 512 registers each) or eight
-// (two per SIMD, 256 registers each: while one wave of a SIMD issues DMA, waits at a barrier or runs the epilogue's vector
-// arithmetic, the other's MFMAs keep the matrix pipe busy); NSA: LDS stages of A (2 for the 256-wide tile, where 160 KB
-// of LDS leave no room for a third; 3 where a narrower tile leaves room).  W always has three stages.
+// BN: tile width; WGM x WGN: wave grid of four waves, one per SIMD (up to 512 registers each); NSA: LDS stages of A (2
+// when a 256-wide tile leaves no room for a third in 160 KB of LDS; 3 where a narrower tile does).  W always has three
+// stages.
 template <int BN_, int WGM_, int WGN_, int NSA_, int BM_ = 256>
 struct RingCfg {
     static constexpr int BM = BM_, BN = BN_, BK = 128, WGM = WGM_, WGN = WGN_, NW = WGM * WGN, NT = 64 * NW, NSA = NSA_, NSW = 3;
@@ -543,7 +542,7 @@ struct RingCfg {
     static constexpr int A_STAGE = BM * BK, W_STAGE = BN * BK;
     static constexpr int W_BASE = NSA * A_STAGE;
     static constexpr int SMEM = NSA * A_STAGE + NSW * W_STAGE;
-    static_assert((NW == 4 || NW == 8) && BM % (32 * WGM) == 0 && BN % (32 * WGN) == 0 && BN % 32 == 0, "tile shape");
+    static_assert(NW == 4 && BM % (32 * WGM) == 0 && BN % (32 * WGN) == 0 && BN % 32 == 0, "tile shape");
     static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "whole DMA blocks per wave");
     static_assert(NF <= NM && SMEM <= 160 * 1024, "fragment loads hide behind MFMAs; LDS fits");
     // Slot of the d-th DMA instruction of an iteration (A first, then W), as the number of the MFMA it follows; an
@@ -573,9 +572,8 @@ struct RingCfg {
     // per lane in flight between the read and the store half of a piece) where the wave tile's width allows
     static constexpr int piece_cols(int sz) { return WTN % (128 / sz) == 0 ? 128 / sz : 32; }
     // Epilogue scratch of one wave inside a stage that was just multiplied: a shuffle piece in each of an A and a W
-    // stage.  With four waves (128 columns each) the wave's column constants (2 x WTN floats) sit behind the piece in the
-    // W stage; with eight (64 columns each) they fit in registers.
-    static constexpr bool STAGED = NW == 4;
+    // stage; the wave's column constants (2 x WTN floats) sit behind the piece in the W stage.
+    static constexpr bool STAGED = true;
     static constexpr int A_REGION = A_STAGE / NW, W_REGION = W_STAGE / NW;
     static constexpr int piece_bytes(int sz) { return 32 * piece_cols(sz) * sz; }
     static constexpr bool scratch_ok(int sz) {
@@ -1309,9 +1307,7 @@ int launch_ring_cfg(GemmArgs a, int slices, hipStream_t st) {
     return 0;
 }
 
-using RingL = RingCfg<256, 2, 2, 2>;         // 256x256, waves 2x2 of 128x128: the compute-bound workhorse
-using RingL8 = RingCfg<256, 2, 4, 2>;        // 256x256, waves 2x4 of 128x64, two per SIMD
-using RingS = RingCfg<192, 2, 2, 3, 128>;    // 128x192, waves 2x2 of 64x96: re-tiles what the last round of RingL leaves
+using RingS = RingCfg<192, 2, 2, 3, 128>;    // 128x192, waves 2x2 of 64x96: shapes with too few 256x256 tiles for the CUs
 
 // Rows [row0, row0 + rows) of the problem as a problem of its own.
 template <int OUT_DT, int EPI>
@@ -1372,41 +1368,6 @@ int launch_pp(GemmArgs a, hipStream_t st) {
     return 0;
 }
 
-// The persistent kernel gives every CU whole 256x256 tiles: when the tile count is not a multiple of the CU count, the
-// last round keeps only some CUs busy for a full tile's time (864 tiles on 256 CUs: 96 busy, 160 idle, a sixth of the
-// launch).  The tile rows that fill whole rounds go to the 256x256 kernel; the rows left over are re-tiled 128x192 and
-// run as a second launch when that is estimated to be shorter (a small tile costs about 0.45 of a large one).
-template <int OUT_DT, int EPI>
-int launch_ring(GemmArgs a, hipStream_t st) {
-    bool vec_ok, aligned;
-    epilogue_alignment<OUT_DT, EPI>(a, vec_ok, aligned);
-    if (!aligned) return launch_cfg<CfgM, OUT_DT, EPI>(a, st);   // the ring kernel has only the coalesced epilogue
-    const int64_t G = device_cu_count();
-    const int64_t tm = (a.M + RingL::BM - 1) / RingL::BM, tn = (a.N + RingL::BN - 1) / RingL::BN;
-    const int64_t full = tm * tn / G, rem = tm * tn % G;
-    if (full >= 1 && rem > 0 && tm > 1) {
-        int64_t main_rows = full * G / tn;
-        if (main_rows >= tm) main_rows = tm - 1;
-        const int64_t m_main = main_rows * RingL::BM, m_rest = a.M - m_main;
-        const int64_t small = ((m_rest + RingS::BM - 1) / RingS::BM) * ((a.N + RingS::BN - 1) / RingS::BN);
-        const double split_cost = (double)((main_rows * tn + G - 1) / G) + 0.45 * (double)((small + G - 1) / G);
-        if (main_rows > 0 && split_cost < (double)(full + 1) - 0.1) {
-            const int rc = launch_ring_cfg<RingL, OUT_DT, EPI>(row_band<OUT_DT, EPI>(a, 0, m_main), 1, st);
-            if (rc) return rc;
-            return launch_ring_cfg<RingS, OUT_DT, EPI>(row_band<OUT_DT, EPI>(a, m_main, m_rest), 1, st);
-        }
-    }
-    return launch_ring_cfg<RingL, OUT_DT, EPI>(a, 1, st);
-}
-
-// The eight-wave 256x256 ring kernel on the whole problem.
-template <int OUT_DT, int EPI>
-int launch_ring8(GemmArgs a, hipStream_t st) {
-    bool vec_ok, aligned;
-    epilogue_alignment<OUT_DT, EPI>(a, vec_ok, aligned);
-    if (!aligned) return launch_cfg<CfgM, OUT_DT, EPI>(a, st);
-    return launch_ring_cfg<RingL8, OUT_DT, EPI>(a, 1, st);
-}
 
 // The 128x192 ring kernel on the whole problem: shapes with too few 256x256 tiles to fill the CUs.
 template <int OUT_DT, int EPI>
@@ -1548,7 +1509,7 @@ std::atomic<int> g_force_cfg{-1};
 int choose_cfg(int64_t M, int64_t N, int64_t K) {
     const int force = g_force_cfg.load(std::memory_order_relaxed);
     const bool dma_ok = M * K < ((int64_t)1 << 32) && N * K < ((int64_t)1 << 32);   // 32-bit lane offsets
-    if (force >= 5 && force <= 9) return (dma_ok && (K % 128) == 0) ? force : 1;
+    if (force == 6 || force == 7 || force == 9) return (dma_ok && (K % 128) == 0) ? force : 1;
     if (force == 1 || force == 2) return force;
     if (M <= 256 && N >= 1024 && (K % 128) == 0 && K >= 512 && dma_ok) return 6;
     const int64_t tiles_l = ((M + 255) / 256) * ((N + 255) / 256);
@@ -1564,10 +1525,8 @@ int choose_cfg(int64_t M, int64_t N, int64_t K) {
 template <int OUT_DT, int EPI>
 int dispatch_cfg(const GemmArgs& a, hipStream_t st) {
     switch (choose_cfg(a.M, a.N, a.K)) {
-        case 5: return launch_ring<OUT_DT, EPI>(a, st);
         case 6: return launch_skinny<OUT_DT, EPI>(a, st);
         case 7: return launch_ring_small<OUT_DT, EPI>(a, st);
-        case 8: return launch_ring8<OUT_DT, EPI>(a, st);
         case 9: return launch_pp<OUT_DT, EPI>(a, st);
         case 1: return launch_cfg<CfgM, OUT_DT, EPI>(a, st);
         default: return launch_cfg<CfgS, OUT_DT, EPI>(a, st);

@@ -257,11 +257,10 @@ int gpu_w6a8_gemm(const int8_t* A, const void* wq, const void* s_rel, int G, con
 int gpu_w6a8_group_gemm(const int8_t* A, const void* Wp, const float* xs, const float* sw, const void* bias, void* D,
                         int32_t* partials, int64_t M, int64_t N, int64_t K, int out_dt, void* stream);
 
-/* Test and tuning hook: force the GEMM kernel family.  1, 2 = 128x128 and 64x64 register-staged tiles; 5 = four-wave
- * persistent ring kernel (256x256 tiles, 128x192 for the rows that do not fill whole rounds, two launches); 6 =
- * weight-streaming kernel (256x96 tiles, split K when N is small) for M <= 256; 7 = ring kernel on 128x192 tiles; 8 = ring
- * kernel with eight waves; 9 = two-group kernel (256x256 and 128x256 tiles, one launch), the choice for large shapes;
- * -1 = automatic.  A shape a family cannot run falls back to 1. */
+/* Test and tuning hook: force the GEMM kernel family.  1, 2 = 128x128 and 64x64 register-staged tiles; 6 =
+ * weight-streaming kernel (256x96 tiles, split K when N is small) for M <= 256; 7 = four-wave persistent ring kernel on
+ * 128x192 tiles (shapes with few tiles); 9 = two-group kernel (256x256 and 128x256 tiles, one launch), the choice for
+ * large shapes; -1 = automatic.  A shape a family cannot run falls back to 1. */
 int gpu_int8_gemm_force_config(int cfg);
 
 /* Writes, for each of the 64 lanes and 16 accumulator registers of one v_mfma_i32_32x32x32_i8, the (row of src0,

@@ -645,7 +645,7 @@ ACC_CASES = [(1, 96, 256), (3, 32, 16), (64, 64, 64), (65, 72, 48), (100, 104, 3
              (77, 4096, 1280), (250, 25000, 128)]
 
 
-@pytest.mark.parametrize("cfg", [2, 1, 5, 6, 7, 8, 9])
+@pytest.mark.parametrize("cfg", [2, 1, 6, 7, 9])
 @pytest.mark.parametrize("M,N,K", ACC_CASES)
 def test_int8_gemm_acc_bit_exact(M, N, K, cfg):
     say("gemm_acc", M, N, K, "cfg", cfg)
@@ -712,7 +712,7 @@ def test_int8_gemm_epilogue(M, N, K, with_bias, out_dt):
     bias = tob(synth.normal(2, 5, N) * np.float32(0.02)) if with_bias else None
     want = oracle.int8_gemm(A, W, xs, ws, bias, out_dt, fma=1)
     loose = oracle.int8_gemm(A, W, xs, ws, bias, out_dt, fma=0)
-    for cfg in (-1, 1, 2, 5, 6, 7, 8, 9):
+    for cfg in (-1, 1, 2, 6, 7, 9):
         ffi.raw("gpu_int8_gemm_force_config", cfg)
         try:
             got = ql.int8_gemm(dev(A), dev(W), dev(xs), dev(ws), None if bias is None else dev_bits(bias, out_dt), TDT[out_dt])
@@ -758,7 +758,7 @@ def test_int8_gemm_residual_in_place(out_dt):
 RESID_CASES = [  # (M, N, K, kernel families that can run the shape)
     (200, 1024, 4096, (-1, 6, 1, 2)),          # skinny: split K, planes summed by the reduce kernel
     (256, 2400, 1024, (-1, 6, 1)),             # skinny: one K slice, the streaming kernel's own epilogue
-    (600, 768, 512, (-1, 1, 2, 5, 7, 8, 9)),   # tile kernels and every persistent kernel
+    (600, 768, 512, (-1, 1, 2, 7, 9)),         # tile kernels and the persistent kernels
 ]
 
 
@@ -938,7 +938,7 @@ def test_full_size_linear_rows_against_oracle(name, M, K, N, rotate, kind):
     got_rowsum = acc.to(torch.int64).sum(dim=1).cpu().numpy()
     assert np.array_equal(got_rowsum, want_rowsum)
     # every kernel family that can run the shape gives the same bits
-    for cfg in (1, 5, 8, 9) if M > 256 and M * N < 8192 * 5120 else (1,) if M > 256 else (6, 1):
+    for cfg in (1, 7, 9) if M > 256 and M * N < 8192 * 5120 else (1,) if M > 256 else (6, 1):
         ffi.raw("gpu_int8_gemm_force_config", cfg)
         try:
             d2 = ql.int8_gemm(qd, Wd, xsd, wsd, bd, torch.bfloat16)
