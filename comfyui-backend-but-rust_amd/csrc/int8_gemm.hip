@@ -529,6 +529,13 @@ __device__ __forceinline__ void wait_lgkmcnt0() { asm volatile("s_waitcnt lgkmcn
 // iteration g+1.  Requires K % 128 == 0 and M*K, N*K < 2^32.
 // ---------------------------------------------------------------------------------------------------------------
 template <int V> struct ic { static constexpr int value = V; };
+template <int N, int I = 0, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(ic<I>{});
+        static_for<N, I + 1>(f);
+    }
+}
 
 // BN: tile width; WGM x WGN: wave grid of four waves, one per SIMD (up to 512 registers each); NSA: LDS stages of A (2
 // when a 256-wide tile leaves no room for a third in 160 KB of LDS; 3 where a narrower tile does).  W always has three
@@ -1020,16 +1027,15 @@ __global__ void __launch_bounds__(PpL::NT, 1) int8_gemm_pp_kernel(GemmArgs main,
 // Requires K % 128 == 0 and M*K, N*K < 2^32.
 // ---------------------------------------------------------------------------------------------------------------
 struct StreamCfg {
-    static constexpr int BM = 256, BN = 96, BK = 128, NSA = 3, NSW = 5;
+    static constexpr int BM = 256, BN = 96, BK = 128, NSA = 4, NSW = 2, NPW = 5;
     static constexpr int NWW = 2, NAW = 6, NT = 64 * (4 + NWW + NAW);   // W-stream waves, A-stream waves
     static constexpr int WTM = 64, WTN = 96, TM = 2, TN = 3, NM = TM * TN, NF = TM + TN;
     static constexpr int A_STAGE = BM * BK, W_STAGE = BN * BK, W_BASE = NSA * A_STAGE, SMEM = W_BASE + NSW * W_STAGE;
     static constexpr int A_BLK = BM / 8, W_BLK = BN / 8;    // 1 KB DMA blocks (8 rows) per stage
     static constexpr int A_PER = (A_BLK + NAW - 1) / NAW;   // per A wave: blocks ap, ap + NAW, ...
     static constexpr int W_PER = W_BLK / NWW;               // per W wave: blocks wp, wp + NWW, ...
-    static constexpr int A_EARLY = (3 * A_PER + 3) / 4, W_EARLY = (3 * W_PER + 3) / 4;   // issued before barrier Y
     static_assert(W_BLK % NWW == 0 && NWW % 2 == 0, "whole blocks per W wave; block parity = wave parity for the swizzle");
-    static_assert(SMEM <= 160 * 1024 && (NSW - 3) * W_PER + W_EARLY <= 63, "LDS budget; wait counts are 6-bit fields");
+    static_assert(SMEM <= 160 * 1024 && A_PER * NAW - A_BLK < NAW, "LDS budget; an A wave has A_PER blocks or one fewer");
 };
 
 template <int OUT_DT, int EPI>
@@ -1065,10 +1071,13 @@ __global__ void __launch_bounds__(StreamCfg::NT, 1) int8_gemm_stream_kernel(Gemm
     };
     if (wave >= 4 && wave < 4 + C::NWW) {
         // ---- the W stream: wave 4 + wp takes blocks wp, wp + NWW, ...  Block j is rows 8j..8j+7 of the tile; chunk
-        // swizzle (bits 1..3 of the row) on the global side.
+        // swizzle (bits 1..3 of the row) on the global side.  The loads land in registers, NPW K tiles ahead of the
+        // multiply, and move into the LDS stage of K tile g+1 during iteration g: HBM latency is covered by registers
+        // of waves that have nothing else to hold, and LDS keeps its room for A.
         const int wp = wave - 4;
         uint32_t gw[C::W_PER];
-        int w_tile = 0, w_kt = 0, w_stage = 0;
+        v4i wr[C::NPW][C::W_PER];
+        int w_tile = 0, w_kt = 0;
         auto set_w = [&](int i) {
             int m0, n0;
             tile_origin(i, m0, n0);
@@ -1079,39 +1088,48 @@ __global__ void __launch_bounds__(StreamCfg::NT, 1) int8_gemm_stream_kernel(Gemm
                 gw[j] = (uint32_t)gr * (uint32_t)ld + (((lane & 7) ^ (((wp & 1) << 2) | (lrow >> 1))) << 4);
             }
         };
-        // instructions [j0, j1) of the stream's current K tile into the current stage
-        auto fetch_w = [&](int j0, int j1) {
+        // the stream's current K tile into register slot S, then on to the next K tile (the stream stops on its last K
+        // tile and keeps re-fetching it)
+        auto load_w = [&](auto S) {
             const int8_t* base = p.W + k_lo + (int64_t)rk(w_kt) * BK;
 #pragma unroll
-            for (int j = 0; j < C::W_PER; ++j)
-                if (j >= j0 && j < j1) dma(lds_base + C::W_BASE + w_stage * C::W_STAGE + (wp + C::NWW * j) * 1024, gw[j], base);
-        };
-        auto next_w = [&]() {   // the stream stops on its last K tile and keeps re-fetching it
-            w_stage = w_stage == C::NSW - 1 ? 0 : w_stage + 1;
+            for (int j = 0; j < C::W_PER; ++j) wr[decltype(S)::value][j] = *reinterpret_cast<const v4i*>(base + gw[j]);
             if (w_tile == nt_b - 1 && w_kt == nk - 1) return;
             if (++w_kt == nk) { w_kt = 0; set_w(++w_tile); }
         };
-        set_w(0);
+        auto store_w = [&](auto S, int stage) {
+            uint8_t* dst = smem + C::W_BASE + stage * C::W_STAGE + wp * 1024 + lane * 16;
 #pragma unroll
-        for (int i = 0; i < C::NSW - 1; ++i) { fetch_w(0, C::W_PER); next_w(); }   // W(0) .. W(NSW-2)
-        wait_vmcnt<(C::NSW - 2) * C::W_PER>();                                     // W(0) has landed
+            for (int j = 0; j < C::W_PER; ++j) *reinterpret_cast<v4i*>(dst + C::NWW * j * 1024) = wr[decltype(S)::value][j];
+        };
+        set_w(0);
+        load_w(ic<0>{});
+        store_w(ic<0>{}, 0);                                      // W(0)
+        static_for<C::NPW>([&](auto I) { load_w(ic<(decltype(I)::value + 1) % C::NPW>{}); });   // W(1) .. W(NPW)
+        wait_lgkmcnt0();
         wg_barrier();
-        for (int ti = 0; ti < nt_b; ++ti) {
-            for (int kt = 0; kt < nk; ++kt) {
-                wg_barrier();                                     // X: the stage of iteration g-1 is free
-                fetch_w(0, C::W_EARLY);                           // W(g + NSW - 1), first part
-                wait_vmcnt<(C::NSW - 3) * C::W_PER + C::W_EARLY>();   // W(g + 1) has landed
-                wg_barrier();                                     // Y
-                fetch_w(C::W_EARLY, C::W_PER);
-                next_w();
-            }
-            wg_barrier();                                         // in front of the epilogue
-        }
-        wait_vmcnt<0>();   // no DMA may still be writing this workgroup's LDS when it retires
+        int stage = 1, kt = 0;
+        // iteration g, g = S mod NPW: K tile g+1 leaves slot (S+1) mod NPW for LDS, K tile g+1+NPW takes the slot
+        auto iteration = [&](auto S) {
+            constexpr int SLOT = (decltype(S)::value + 1) % C::NPW;
+            wg_barrier();                                         // X: the stage of iteration g-1 is free
+            store_w(ic<SLOT>{}, stage);
+            load_w(ic<SLOT>{});
+            wait_lgkmcnt0();
+            wg_barrier();                                         // Y
+            stage = stage == C::NSW - 1 ? 0 : stage + 1;
+            if (++kt == nk) { kt = 0; wg_barrier(); }             // in front of the epilogue
+        };
+        const int total = nt_b * nk;
+        int g = 0;
+        for (; g + C::NPW <= total; g += C::NPW) static_for<C::NPW>([&](auto I) { iteration(I); });
+        static_for<C::NPW>([&](auto I) { if (g + decltype(I)::value < total) iteration(I); });
         return;
     }
     if (wave >= 4 + C::NWW) {
-        // ---- the A stream: wave 4 + NWW + ap takes blocks ap, ap + NAW, ...
+        // ---- the A stream: wave 4 + NWW + ap takes blocks ap, ap + NAW, ... (A_PER of them, or one fewer), NSA - 1 K
+        // tiles ahead.  A's lines come from L2, but a CU's loads return in issue order, behind the W loads that went to
+        // HBM: the lead in K tiles times the iteration time has to cover HBM's latency, not L2's.
         const int ap = wave - 4 - C::NWW;
         uint32_t ga[C::A_PER];
         int a_tile = 0, a_kt = 0, a_stage = 0;
@@ -1130,32 +1148,37 @@ __global__ void __launch_bounds__(StreamCfg::NT, 1) int8_gemm_stream_kernel(Gemm
             const int8_t* base = p.A + k_lo + (int64_t)rk(a_kt) * BK;
 #pragma unroll
             for (int j = 0; j < C::A_PER; ++j)
-                if (j >= j0 && j < j1 && ap + C::NAW * j < C::A_BLK) dma(lds_base + a_stage * C::A_STAGE + (ap + C::NAW * j) * 1024, ga[j], base);
+                if (j >= j0 && j < j1) dma(lds_base + a_stage * C::A_STAGE + (ap + C::NAW * j) * 1024, ga[j], base);
         };
         auto next_a = [&]() {
             a_stage = a_stage == C::NSA - 1 ? 0 : a_stage + 1;
             if (a_tile == nt_b - 1 && a_kt == nk - 1) return;
             if (++a_kt == nk) { a_kt = 0; set_a(++a_tile); }
         };
-        set_a(0);
-        fetch_a(0, C::A_PER);                                     // A(0)
-        next_a();
-        wait_vmcnt<0>();
-        fetch_a(0, C::A_PER);                                     // A(1)
-        next_a();
-        wg_barrier();
-        for (int ti = 0; ti < nt_b; ++ti) {
-            for (int kt = 0; kt < nk; ++kt) {
-                wg_barrier();                                     // X: the stage of iteration g-1 is free
-                fetch_a(0, C::A_EARLY);                           // A(g + 2), first part
-                wait_vmcnt<C::A_EARLY>();                         // A(g + 1) has landed
-                wg_barrier();                                     // Y
-                fetch_a(C::A_EARLY, C::A_PER);
-                next_a();
+        // PER: DMA instructions of this wave per K tile (the wait counts below are exact only for the wave's own count)
+        auto stream_a = [&](auto PER_) {
+            constexpr int PER = decltype(PER_)::value, EARLY = (3 * PER + 3) / 4;   // EARLY are issued before barrier Y
+            static_assert((C::NSA - 2) * PER + EARLY <= 63, "wait counts are 6-bit fields");
+            set_a(0);
+#pragma unroll
+            for (int i = 0; i < C::NSA - 1; ++i) { fetch_a(0, PER); next_a(); }   // A(0) .. A(NSA-2)
+            wait_vmcnt<(C::NSA - 2) * PER>();                                     // A(0) has landed
+            wg_barrier();
+            for (int ti = 0; ti < nt_b; ++ti) {
+                for (int kt = 0; kt < nk; ++kt) {
+                    wg_barrier();                                     // X: the stage of iteration g-1 is free
+                    fetch_a(0, EARLY);                                // A(g + NSA - 1), first part
+                    wait_vmcnt<(C::NSA - 3) * PER + EARLY>();         // A(g + 1) has landed
+                    wg_barrier();                                     // Y
+                    fetch_a(EARLY, PER);
+                    next_a();
+                }
+                wg_barrier();                                         // in front of the epilogue
             }
-            wg_barrier();                                         // in front of the epilogue
-        }
-        wait_vmcnt<0>();
+            wait_vmcnt<0>();   // no DMA may still be writing this workgroup's LDS when it retires
+        };
+        if (ap + C::NAW * (C::A_PER - 1) < C::A_BLK) stream_a(ic<C::A_PER>{});
+        else stream_a(ic<C::A_PER - 1>{});
         return;
     }
 
@@ -1544,8 +1567,52 @@ int dispatch_dt(const GemmArgs& a, int out_dt, hipStream_t st) {
 }
 
 bool shape_ok(int64_t M, int64_t N, int64_t K) {
-    return M <= 0x7fffffff && N <= 0x7fffffff && K <= 0x7fffffff && (K % 16) == 0 && M * N < (int64_t)1 << 40;
+    return M <= 0x7fffffff && N <= 0x7fffffff && K <= 0x7fffffff - 8 && (K % 8) == 0 && M * N < (int64_t)1 << 40;
 }
+
+// K % 16 == 8 (the reference's alignment-8 tile configurations, csrc/vendor/cutlass_gemm_int8.cu:191,237-247,265): the
+// kernels here read 16-byte vectors of K, so such a call runs on copies of A and W whose rows carry eight more zero
+// bytes, which leave every int32 sum as it was.  The copies live in one stream-ordered allocation for the length of
+// the call.  No model in the reference's tree has such a K; the path exists so that the call is not refused.
+__global__ void __launch_bounds__(256) pad_k_rows_kernel(const int8_t* src, int8_t* dst, int64_t rows, int k8) {
+    const int64_t n = rows * (k8 + 1);   // 8-byte pieces of the destination
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+        const int64_t r = i / (k8 + 1);
+        const int c = (int)(i - r * (k8 + 1));
+        uint2 v = make_uint2(0u, 0u);
+        if (c < k8) v = *reinterpret_cast<const uint2*>(src + (r * k8 + c) * 8);
+        *reinterpret_cast<uint2*>(dst + i * 8) = v;
+    }
+}
+
+struct PaddedK {
+    int8_t* buf = nullptr;
+    hipStream_t st;
+    int rc = 0;
+    // replaces A, W and K by the padded copies when K % 16 != 0
+    PaddedK(const int8_t*& A, const int8_t*& W, int64_t M, int64_t N, int64_t& K, hipStream_t stream) : st(stream) {
+        if ((K % 16) == 0) return;
+        if ((((uintptr_t)A | (uintptr_t)W) & 7) != 0) { rc = -1; return; }
+        const int64_t k16 = K + 8;
+        retain_pool_memory();
+        hipError_t e = hipMallocAsync((void**)&buf, (size_t)((M + N) * k16), st);
+        if (e != hipSuccess) { buf = nullptr; rc = (int)e; return; }
+        const int8_t* src[2] = {A, W};
+        int8_t* dst[2] = {buf, buf + M * k16};
+        const int64_t rows[2] = {M, N};
+        for (int i = 0; i < 2; ++i) {
+            const int64_t pieces = rows[i] * (k16 / 8);
+            const unsigned grid = (unsigned)((pieces + 255) / 256 < 8192 ? (pieces + 255) / 256 : 8192);
+            hipLaunchKernelGGL(pad_k_rows_kernel, dim3(grid), dim3(256), 0, st, src[i], dst[i], rows[i], (int)(K / 8));
+        }
+        hipError_t le = hipGetLastError();
+        if (le != hipSuccess) rc = (int)le;
+        A = dst[0];
+        W = dst[1];
+        K = k16;
+    }
+    ~PaddedK() { if (buf) (void)hipFreeAsync(buf, st); }
+};
 
 __global__ void mfma_layout_probe_kernel(int* out) {
     const int lane = threadIdx.x;
@@ -1606,6 +1673,8 @@ GPU_API int gpu_int8_gemm(const int8_t* A, const int8_t* W, const float* xs, con
                           int64_t M, int64_t N, int64_t K, int out_dt, void* stream) {
     if (M == 0 || N == 0 || K == 0) return 0;  // csrc/vendor/cutlass_gemm_int8.cu:377
     if (out_dt < DT_F32 || out_dt > DT_BF16 || M < 0 || N < 0 || K < 0 || !shape_ok(M, N, K)) return -200;
+    PaddedK pad(A, W, M, N, K, (hipStream_t)stream);
+    if (pad.rc != 0) return pad.rc < 0 ? -200 : pad.rc;
     GemmArgs a{A, W, xs, ws, bias, nullptr, nullptr, D, (int)M, (int)N, (int)K, 0, 0, 0};
     const int rc = dispatch_dt<EPI_PLAIN>(a, out_dt, (hipStream_t)stream);
     return rc < 0 ? -200 : rc;
@@ -1617,6 +1686,8 @@ GPU_API int gpu_int8_gemm_residual(const int8_t* A, const int8_t* W, const float
     if (M == 0 || N == 0) return 0;                       // csrc/vendor/cutlass_gemm_int8.cu:353
     if (K == 0 || !rscale || !resid) return -201;         // :355-357
     if (out_dt < DT_F32 || out_dt > DT_BF16 || M < 0 || N < 0 || K < 0 || !shape_ok(M, N, K)) return -201;
+    PaddedK pad(A, W, M, N, K, (hipStream_t)stream);
+    if (pad.rc != 0) return pad.rc < 0 ? -201 : pad.rc;
     GemmArgs a{A, W, xs, ws, bias, rscale, resid, D, (int)M, (int)N, (int)K, 0, 0, 0};
     const int rc = dispatch_dt<EPI_RESID>(a, out_dt, (hipStream_t)stream);
     return rc < 0 ? -201 : rc;
@@ -1626,6 +1697,7 @@ GPU_API int gpu_int8_gemm_static(const int8_t* A, const int8_t* W, const float* 
                                  int64_t M, int64_t N, int64_t K, int out_dt, void* stream) {
     if (M == 0 || N == 0 || K == 0) return 0;
     if (out_dt < DT_F32 || out_dt > DT_BF16 || M < 0 || N < 0 || K < 0 || !shape_ok(M, N, K)) return -200;
+    if ((K % 16) != 0) return -200;   // the K % 16 == 8 path allocates its padded copies
     int rc = 0;
     void* ptr = static_scratch(&rc);
     if (!ptr) return rc;
@@ -1643,13 +1715,15 @@ GPU_API int64_t gpu_int8_gemm_static_limit(void) { return (int64_t)kStaticScratc
 GPU_API int gpu_int8_gemm_acc(const int8_t* A, const int8_t* W, int32_t* acc, int64_t M, int64_t N, int64_t K, void* stream) {
     if (M == 0 || N == 0 || K == 0) return 0;
     if (M < 0 || N < 0 || K < 0 || !shape_ok(M, N, K)) return -200;
+    PaddedK pad(A, W, M, N, K, (hipStream_t)stream);
+    if (pad.rc != 0) return pad.rc < 0 ? -200 : pad.rc;
     GemmArgs a{A, W, nullptr, nullptr, nullptr, nullptr, nullptr, acc, (int)M, (int)N, (int)K, 0, 0, 0};
     const int rc = dispatch_cfg<DT_F32, EPI_ACC>(a, (hipStream_t)stream);
     return rc < 0 ? -200 : rc;
 }
 
-// Test hook: force a kernel family (1 = 128x128, 2 = 64x64 register-staged tiles; 5 = persistent ring, 256x256;
-// 6 = weight streaming; 7 = persistent ring, 128x192; -1 or anything else = automatic).
+// Test hook: force a kernel family (1 = 128x128, 2 = 64x64 register-staged tiles; 6 = weight streaming; 7 = persistent
+// ring, 128x192; 9 = two-group kernel; -1 or anything else = automatic).
 GPU_API int gpu_int8_gemm_force_config(int cfg) {
     g_force_cfg.store(cfg, std::memory_order_relaxed);
     return 0;

@@ -13,7 +13,7 @@
  * (hipGetErrorString names it); < 0 = the launcher refused the arguments, with the reference's codes:
  *   quantizers  -1 shape (K granularity), -2 row too long (K > 32768), -3 prologue id, -4 dtype
  *   int8 GEMM   -200 (plain) / -201 (residual): unknown out_dt, null rscale/resid, K == 0 for the residual form,
- *               or a shape the kernels cannot run (K % 16 != 0)
+ *               or a shape the kernels cannot run (K % 8 != 0; gpu_int8_gemm_static also refuses K % 16 != 0)
  *   w6 decode   -1 (K % 32 or G % 16)
  */
 #ifndef GPU_API_H
@@ -196,7 +196,10 @@ int gpu_internal_attn_layout_d(int b, int h, int hk, int lq, int lk, int head_di
 
 /* D[M,N] = Out((A[M,K] . W[N,K]^T) * xs[m] * ws[n] + bias[n]).
  * Replaces gpu_int8_gemm, src/ffi.rs:38 / csrc/gemm.cu:124-129.
- * A, W int8 row-major (K contiguous); xs f32 [M]; ws f32 [N]; bias Out[N] or null; D Out[M,N]; out_dt a DT_* code. */
+ * A, W int8 row-major (K contiguous); xs f32 [M]; ws f32 [N]; bias Out[N] or null; D Out[M,N]; out_dt a DT_* code.
+ * K % 16 == 0 is the fast path; K % 16 == 8 (the reference's alignment-8 tile configurations,
+ * csrc/vendor/cutlass_gemm_int8.cu:191,237-247) runs on zero-padded copies of A and W in a stream-ordered allocation
+ * (A and W 8-byte aligned); any other K is refused. */
 int gpu_int8_gemm(const int8_t* A, const int8_t* W, const float* xs, const float* ws, const void* bias, void* D,
                   int64_t M, int64_t N, int64_t K, int out_dt, void* stream);
 

@@ -663,6 +663,30 @@ def test_int8_gemm_acc_bit_exact(M, N, K, cfg):
     assert np.array_equal(got.cpu().numpy(), want)
 
 
+# K % 16 == 8: the reference's alignment-8 configurations (csrc/vendor/cutlass_gemm_int8.cu:191,237-247)
+@pytest.mark.parametrize("M,N,K", [(5, 40, 8), (130, 264, 136), (300, 1030, 1000), (64, 2048, 4104)])
+def test_int8_gemm_k_multiple_of_8_only(M, N, K):
+    say("gemm_k8", M, N, K)
+    A = rand_i8(6, 1, M, K)
+    W = rand_i8(6, 2, N, K)
+    xs = synth.uniform(6, 3, M, 0.005, 0.2)
+    ws = synth.uniform(6, 4, N, 1e-3, 1e-2)
+    bias = oracle.bf16_bits(synth.normal(6, 5, N) * np.float32(0.02))
+    rscale = oracle.bf16_bits(synth.normal(6, 6, N))
+    resid = oracle.bf16_bits(synth.normal(6, 7, M * N).reshape(M, N))
+    want = oracle.int8_gemm_acc(A, W)
+    Ad, Wd = dev(A), dev(W)
+    got = ql.int8_gemm_acc(Ad, Wd)
+    d = ql.int8_gemm(Ad, Wd, dev(xs), dev(ws), dev_bits(bias, BF16), torch.bfloat16)
+    r = ql.int8_gemm_residual(Ad, Wd, dev(xs), dev(ws), dev_bits(bias, BF16), dev_bits(rscale, BF16), dev_bits(resid, BF16))
+    torch.cuda.synchronize()
+    assert np.array_equal(got.cpu().numpy(), want)
+    assert np.array_equal(host_bits(d), oracle.epilogue(want, xs, ws, bias, BF16, fma=1))
+    assert np.array_equal(host_bits(r), oracle.epilogue_residual(want, xs, ws, bias, rscale, resid, BF16, fma=1))
+    # no tile configuration of the reference takes K % 8 != 0
+    assert ffi.raw("gpu_int8_gemm", Ad.data_ptr(), Wd.data_ptr(), 0, 0, 0, 0, M, N, K - 4, 2, 0) == -200
+
+
 # More 256x256 tiles than CUs, and not a multiple of the CU count: the persistent kernel's workgroups then own unequal
 # numbers of tiles, and every output form runs through its coalesced epilogue.
 MANY_TILE_CASES = [(4352, 4096, 256), (4100, 4400, 384), (2304, 8200, 640)]

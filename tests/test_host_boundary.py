@@ -89,7 +89,7 @@ def test_gemm_refusals_and_empty_shapes():
     g = lambda M, N, K, dt=2: ffi.raw("gpu_int8_gemm", 0, 0, 0, 0, 0, 0, M, N, K, dt, 0)
     assert g(0, 8, 16) == 0 and g(8, 0, 16) == 0 and g(8, 8, 0) == 0       # csrc/vendor/cutlass_gemm_int8.cu:377
     assert g(8, 8, 16, dt=5) == -200                                         # csrc/gemm.cu:126
-    assert g(8, 8, 24) == -200
+    assert g(8, 8, 20) == -200                                               # K % 8: no tile configuration takes it (:191, :237-247)
     r = lambda M, N, K, rs=1, res=1, dt=2: ffi.raw("gpu_int8_gemm_residual", 0, 0, 0, 0, 0, rs, res, 0, M, N, K, dt, 0)
     assert r(0, 8, 16) == 0 and r(8, 0, 16) == 0                             # :353
     assert r(8, 8, 0) == -201                                                # :355, csrc/gemm.cu:137
