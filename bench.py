@@ -75,7 +75,7 @@ def make_inputs(torch, synth, M, K, N, seed=0, dev="cuda:0", kind="t3"):
     return host, devs
 
 
-def time_linear(torch, ffi, d, M, K, N, rotate, steps, warmup, nbuf=1):
+def time_linear(torch, ffi, d, M, K, N, rotate, steps, warmup, nbuf=1, settled=True):
     """Times `steps` linears; returns (ms_total, ms_quant_avg, ms_gemm_avg).  nbuf > 1 rotates among copies of the
     weights so that a memory-bound shape cannot live in the 256 MB last-level cache."""
     st = torch.cuda.current_stream()
@@ -95,7 +95,8 @@ def time_linear(torch, ffi, d, M, K, N, rotate, steps, warmup, nbuf=1):
               D.data_ptr(), M, N, K, ffi.DT_BF16, s)
         if evs: evs[2].record(st)
 
-    settle(torch, lambda: step(0))
+    if settled:
+        settle(torch, lambda: step(0))
     for i in range(warmup):
         step(i)
     evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
@@ -367,6 +368,9 @@ def main():
         torch.cuda.synchronize()
         del src, dst
     host, d = make_inputs(torch, synth, M, K, N)
+    # the same loop from an idle GPU first (reported beside the headline, not as it), then from the settled power state
+    time.sleep(0.5)
+    _, cold_wall, cold_tq, cold_tg = time_linear(torch, ffi, d, M, K, N, a.rotate, min(a.steps, 50), min(a.warmup, 10), settled=False)
     gpu_ms, wall_ms, tq, tg = time_linear(torch, ffi, d, M, K, N, a.rotate, a.steps, a.warmup)
     ops = 2.0 * M * N * K
     ms_per_step = wall_ms / a.steps
@@ -394,6 +398,10 @@ def main():
                      "algorithmic_ops": ops, "algorithmic_bytes": M * K + M * 4 + N * K + N * 4 + N * 2 + M * N * 2},
         "kernels": {"quant_rows_us": round(tq * 1e3, 2), "quant_rows_GBs": round(quant_bytes / (tq * 1e-3) / 1e9, 1),
                     "int8_gemm_us": round(tg * 1e3, 2), "gpu_ms_total": round(gpu_ms, 4)},
+        "from_idle": {"steps": min(a.steps, 50), "warmup": min(a.warmup, 10), "ms_per_step": round(cold_wall / min(a.steps, 50), 5),
+                      "value": round(ops / (cold_wall / min(a.steps, 50) * 1e-3) / 1e12, 2), "quant_rows_us": round(cold_tq * 1e3, 2),
+                      "int8_gemm_us": round(cold_tg * 1e3, 2),
+                      "note": "the first steps after 0.5 s of idle, no settling load: the clock is still rising"},
     }
     if not a.no_skinny:
         sk = []
