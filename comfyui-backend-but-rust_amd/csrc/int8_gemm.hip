@@ -1011,19 +1011,22 @@ __global__ void __launch_bounds__(PpL::NT, 1) int8_gemm_pp_kernel(GemmArgs main,
 
 // ---------------------------------------------------------------------------------------------------------------
 // Weight-streaming kernel for skinny M (M <= 256): one row of 256 x 96 tiles, every weight read from HBM exactly once.
-// An iteration of such a tile is short (24 MFMAs per wave, 768 cycles) against the 44 DMA instructions that feed it, and
-// a DMA instruction that hits the L2 keeps its wave busy for about 68 cycles: a wave that multiplies cannot also fetch.
+// An iteration of such a tile is short (24 MFMAs per wave, 768 cycles) against the 44 KB that feed it, and a DMA
+// instruction that hits the L2 keeps its wave busy for about 68 cycles: a wave that multiplies cannot also fetch.
 // The roles are split over twelve waves, three per SIMD:
 //   waves 0-3   multiply (64 x 96 each, MFMA + fragment reads only, no memory instruction in their K loop);
-//   waves 4-5   stream W: 6 DMA instructions per K tile each into a ring of 5 stages, three K tiles ahead;
-//   waves 6-11  stream A (from L2: all CUs read the same 256 rows) into three stages, 5-6 instructions per K tile each.
+//   waves 4-5   stream W: 6 loads of 1 KB per K tile each into registers, NPW K tiles ahead, and 6 LDS stores of the
+//               K tile that is multiplied next into a ring of two stages;
+//   waves 6-11  stream A (from L2: all CUs read the same 256 rows) by DMA into four LDS stages, three K tiles ahead,
+//               5-6 instructions per K tile each.
+// A CU's loads return in issue order, so A's lines wait behind W loads that went to HBM: A needs the lead of an HBM
+// access, and W's flight time is spent in registers of waves that hold nothing else, which leaves the LDS to A.
 // With three A waves (and eight waves in all) the A stream needed 11 x 68 cycles an iteration and set the pace; six keep
 // it near 400.  The price is the register budget of three waves per SIMD (168), which the multiplying waves meet by
 // keeping the epilogue's column constants in LDS.
 // Everybody meets at two barriers per iteration, X (the stage of iteration g-1 is free) and Y (what iteration g+1 needs
-// has landed; the MFMA waves run three sub-steps before it and one after).  Each producer splits its instructions
-// between the two phases roughly in the proportion of the MFMA waves' work.  The counter a producer waits on retires in
-// order, which is why W has waves to itself: their wait lets two and three quarter K tiles stay in flight.
+// has landed; the MFMA waves run three sub-steps before it and one after).  An A wave splits its instructions
+// between the two phases roughly in the proportion of the MFMA waves' work.
 // Requires K % 128 == 0 and M*K, N*K < 2^32.
 // ---------------------------------------------------------------------------------------------------------------
 struct StreamCfg {
@@ -1238,7 +1241,7 @@ __global__ void __launch_bounds__(StreamCfg::NT, 1) int8_gemm_stream_kernel(Gemm
         }
         __syncthreads();   // every wave is done with the stage that becomes the shuffle scratch (8 KB per wave)
         constexpr int SZ = (EPI == EPI_ACC || OUT_DT == DT_F32) ? 4 : 2;
-        // (The stage of A(g) is refilled with A(g+3), issued after barrier X of the next iteration: behind this epilogue.)
+        // (The stage of A(g) is refilled with A(g+NSA), issued after barrier X of the next iteration: behind this epilogue.)
         uint8_t* scratch = smem + pa * C::A_STAGE + wave * 8192;   // a 4 KB piece, then the wave's column constants
         epilogue_shuffle<TM, TN, OUT_DT, EPI, 32, true, true>(p, acc, m0 + wm * C::WTM, n0, lane, scratch, nullptr,
                                                               reinterpret_cast<float*>(scratch + 4096));
