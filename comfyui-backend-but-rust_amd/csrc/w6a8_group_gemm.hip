@@ -23,6 +23,7 @@
 // four waves fold their second pair at the end of an iteration, the lower four at the start of the next, so that on
 // every SIMD one wave's VALU-only stretch meets the other's MFMAs.
 #include "common.hpp"
+#include <atomic>
 
 #define SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
 
@@ -31,6 +32,7 @@ namespace {
 struct W6Args {
     const int8_t* A;
     const uint8_t* Wp;
+    const int8_t* W8;   // the weights already expanded to int8 [N, K] (the W8 form of the kernel), or null
     const float* xs;
     const float* sw;
     const void* bias;
@@ -43,10 +45,16 @@ struct W6Args {
 constexpr int BM = 256, BN = 128, BK = 128, RAW_ROW = 96;
 constexpr int A_STAGE = BM * BK, U_STAGE = BN * BK, R_STAGE = BN * RAW_ROW, S_STAGE = BN * 4;
 constexpr int NSA = 3, NSS = 4;   // stages of A and of the scales (the deferred fold still reads group g-1 in iteration g)
-constexpr int U_BASE = NSA * A_STAGE, R_BASE = U_BASE + 2 * U_STAGE, S_BASE = R_BASE + 2 * R_STAGE;
-constexpr int SMEM = S_BASE + NSS * S_STAGE;
+constexpr int U_BASE = NSA * A_STAGE;
+// Fused unpack: two stages of expanded weights and two of packed ones.  W8 form (weights expanded beforehand, fetched
+// like A): three stages of expanded weights, none of packed ones.
+template <bool W8> struct Lay {
+    static constexpr int NSU = W8 ? 3 : 2;
+    static constexpr int R_BASE = U_BASE + NSU * U_STAGE, S_BASE = R_BASE + (W8 ? 0 : 2 * R_STAGE);
+    static constexpr int SMEM = S_BASE + NSS * S_STAGE;
+    static_assert(SMEM <= 160 * 1024, "LDS budget");
+};
 constexpr int RAW_WAVE = 16 * RAW_ROW;   // bytes of packed weights a wave owns per group: 16 rows
-static_assert(SMEM <= 160 * 1024, "LDS budget");
 constexpr int TM = 4, TN = 1;   // 32x32 MFMA tiles of one wave: 128 rows (m) x 32 columns (n)
 constexpr int NT = 512;         // eight waves, 2 (m) x 4 (n)
 
@@ -69,8 +77,9 @@ __device__ __forceinline__ void dma4(uint32_t lds_dst, uint32_t lane_off, const 
 
 // ABL (measurement only, wrong results): bit 0 leaves out the fp32 fold, bit 1 the unpack, bit 2 the DMA of the MFMA
 // waves after the prologue; what remains shows what each part costs next to the MFMAs.
-template <int OUT_DT, bool DUMP, int ABL = 0>
+template <int OUT_DT, bool DUMP, int ABL = 0, bool W8 = false>
 __global__ void __launch_bounds__(NT, 1) w6a8_group_gemm_kernel(W6Args p) {
+    constexpr int R_BASE = Lay<W8>::R_BASE, S_BASE = Lay<W8>::S_BASE;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -94,7 +103,14 @@ __global__ void __launch_bounds__(NT, 1) w6a8_group_gemm_kernel(W6Args p) {
     }
     const uint32_t wrow = (uint32_t)p.K / 4 * 3;                   // bytes per packed weight row
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {                                  // the wave's own 1.5 KB: one full and one half instruction
+    for (int j = 0; j < 2; ++j) {
+        if (W8) {                                                  // expanded weights: 8-row blocks wave, wave + 8, as for A
+            const int row = (wave + 8 * j) * 8 + lrow;
+            const int r = n0 + row < p.N ? n0 + row : p.N - 1;
+            gr[j] = (uint32_t)r * (uint32_t)p.K + lch;
+            continue;
+        }
+        // the wave's own 1.5 KB of packed weights: one full and one half instruction
         const int b = (64 * j + (j ? (lane & 31) : lane)) * 16;    // byte inside the wave's block of 16 rows x 96 bytes
         const int row = 16 * wave + b / RAW_ROW, col = b % RAW_ROW;
         const int r = n0 + row < p.N ? n0 + row : p.N - 1;
@@ -111,6 +127,10 @@ __global__ void __launch_bounds__(NT, 1) w6a8_group_gemm_kernel(W6Args p) {
         dma16(lds_base + stage * A_STAGE + (wave + 8 * j) * 1024, ga[j], p.A + (int64_t)(g < ng ? g : ng - 1) * BK);
     };
     auto dma_raw = [&](int g, int stage, int j) {
+        if (W8) {   // `stage` is then a stage of expanded weights
+            dma16(lds_base + U_BASE + stage * U_STAGE + (wave + 8 * j) * 1024, gr[j], p.W8 + (int64_t)(g < ng ? g : ng - 1) * BK);
+            return;
+        }
         const uint8_t* base = p.Wp + (int64_t)(g < ng ? g : ng - 1) * RAW_ROW;
         const uint32_t dst = lds_base + R_BASE + stage * R_STAGE + wave * RAW_WAVE + j * 1024;
         if (j == 0) dma16(dst, gr[0], base);
@@ -163,11 +183,13 @@ __global__ void __launch_bounds__(NT, 1) w6a8_group_gemm_kernel(W6Args p) {
         dma_scales(g, g);
     }
     wait_all_dma();
+    if (!W8) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        uint32_t d[3];
-        raw_read(0, i, d);
-        unpack_write(0, i, d);
+        for (int i = 0; i < 2; ++i) {
+            uint32_t d[3];
+            raw_read(0, i, d);
+            unpack_write(0, i, d);
+        }
     }
     __syncthreads();
 
@@ -191,11 +213,11 @@ __global__ void __launch_bounds__(NT, 1) w6a8_group_gemm_kernel(W6Args p) {
 
     int a_cur = 0, s_cur = 0;   // stages of group g: g mod 3 (A), g mod 4 (scales)
     for (int g = 0; g < ng; ++g) {
-        const int s = g & 1;
         const int a_new = a_cur == 0 ? 2 : a_cur - 1;                  // (g + 2) mod 3
+        const int s = W8 ? a_new : g & 1;                              // the stage dma_raw fills with group g+2
         const int s_new = (s_cur + 2) & 3, s_prev = (s_cur + 3) & 3;   // (g + 2) mod 4, (g - 1) mod 4
         const uint8_t* sa = smem + a_cur * A_STAGE;
-        const uint8_t* su = smem + U_BASE + s * U_STAGE;
+        const uint8_t* su = smem + U_BASE + (W8 ? a_cur : g & 1) * U_STAGE;
         const float* sc = reinterpret_cast<const float*>(smem + S_BASE + s_cur * S_STAGE);
         const float* sc_prev = reinterpret_cast<const float*>(smem + S_BASE + s_prev * S_STAGE);
 
@@ -226,7 +248,7 @@ __global__ void __launch_bounds__(NT, 1) w6a8_group_gemm_kernel(W6Args p) {
         // The wave's own packed rows of group g+1 were the first two DMA instructions of the previous iteration; the
         // five issued after them may still be in flight.
         if (ABL & 4) wait_all_dma();
-        else wait_vmcnt_n<5>();
+        else if (!W8) wait_vmcnt_n<5>();
         // everything this iteration reads from LDS early: fragments of the first pair, the group's scales, packed words
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk) fw[kk] = *reinterpret_cast<const v4i*>(su + woff[kk]);
@@ -238,7 +260,7 @@ __global__ void __launch_bounds__(NT, 1) w6a8_group_gemm_kernel(W6Args p) {
         for (int q = 0; q < 4; ++q) sv[q] = *reinterpret_cast<const float4*>(sc + wn * 32 + 8 * q + 4 * fhalf);
 #pragma unroll
         for (int i = 0; i < 2; ++i)
-            if (!(ABL & 2)) raw_read(s ^ 1, i, raw[i]);
+            if (!(ABL & 2) && !W8) raw_read(s ^ 1, i, raw[i]);
         SCHED_FENCE();
         if (defer && g > 0) {   // the fold the previous iteration left over
 #pragma unroll
@@ -260,7 +282,7 @@ __global__ void __launch_bounds__(NT, 1) w6a8_group_gemm_kernel(W6Args p) {
                 if (i == 5) dma_a(g + 2, a_new, 0);
                 if (i == 7) dma_a(g + 2, a_new, 1);
             }
-            if (!(ABL & 2)) {
+            if (!(ABL & 2) && !W8) {
                 if (i == 2) unpack_write(s ^ 1, 0, raw[0]);
                 if (i == 4) unpack_write(s ^ 1, 1, raw[1]);
             }
@@ -390,9 +412,10 @@ __global__ void __launch_bounds__(NT, 1) w6a8_group_gemm_kernel(W6Args p) {
     }
 }
 
-template <int OUT_DT, bool DUMP, int ABL = 0>
+template <int OUT_DT, bool DUMP, int ABL = 0, bool W8 = false>
 int launch(W6Args a, hipStream_t st) {
-    auto kern = w6a8_group_gemm_kernel<OUT_DT, DUMP, ABL>;
+    auto kern = w6a8_group_gemm_kernel<OUT_DT, DUMP, ABL, W8>;
+    constexpr int SMEM = Lay<W8>::SMEM;
     static bool once = false;  // benign race: the attribute is idempotent
     if (!once) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
@@ -406,8 +429,26 @@ int launch(W6Args a, hipStream_t st) {
 
 template <int OUT_DT>
 int launch_dt(const W6Args& a, hipStream_t st) {
+    if (a.W8) return a.partials ? launch<OUT_DT, true, 0, true>(a, st) : launch<OUT_DT, false, 0, true>(a, st);
     return a.partials ? launch<OUT_DT, true>(a, st) : launch<OUT_DT, false>(a, st);
 }
+
+// The packed weights expanded to int8 [N, K]: a thread turns one 12-byte piece into 16 codes.
+__global__ void __launch_bounds__(256) w6_words_to_int8_kernel(const uint8_t* Wp, int8_t* out, int64_t pieces) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < pieces; i += (int64_t)gridDim.x * 256) {
+        const uint32_t* src = reinterpret_cast<const uint32_t*>(Wp + i * 12);
+        const uint32_t d0 = src[0], d1 = src[1], d2 = src[2];
+        *reinterpret_cast<v4i*>(out + i * 16) = v4i{spread6(d0), spread6(__builtin_amdgcn_alignbit(d1, d0, 24)),
+                                                   spread6(__builtin_amdgcn_alignbit(d2, d1, 16)), spread6(d2 >> 8)};
+    }
+}
+
+// From this many rows of A on, the weights are expanded once into a stream-ordered scratch and the kernel fetches them
+// like A; below, every workgroup expands its own 128 columns as it goes.  Each weight is used by M / 256 workgroups:
+// expanding it that many times costs the large-M shapes more vector issue slots than the int8 round trip through HBM
+// costs them time (M = 8192: 9 % faster; M = 2048: 10 % slower, the expansion being a fixed 25-30 us).
+constexpr int64_t kExpandFirstRows = 4096;
+std::atomic<int> g_mode{-1};   // test hook: 0 = always fused, 1 = always expand first, -1 = by M
 
 }  // namespace
 
@@ -420,27 +461,52 @@ GPU_API int gpu_w6a8_group_gemm(const int8_t* A, const void* Wp, const float* xs
     if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff || M * K >= ((int64_t)1 << 32) || N * (K / 4 * 3) >= ((int64_t)1 << 32) ||
         N * (K / 128) * 4 >= ((int64_t)1 << 32))
         return -200;
-    W6Args a{A, (const uint8_t*)Wp, xs, sw, bias, D, partials, (int)M, (int)N, (int)K, (int)(K / 128), 0, 0};
+    W6Args a{A, (const uint8_t*)Wp, nullptr, xs, sw, bias, D, partials, (int)M, (int)N, (int)K, (int)(K / 128), 0, 0};
     a.tiles_m = (int)((M + BM - 1) / BM);
     a.tiles_n = (int)((N + BN - 1) / BN);
     if ((int64_t)a.tiles_m * a.tiles_n > 0x7fffffff || K == 0) return -200;
     hipStream_t st = (hipStream_t)stream;
-    switch (out_dt) {
-        case DT_F32: return launch_dt<DT_F32>(a, st);
-        case DT_F16: return launch_dt<DT_F16>(a, st);
-        default: return launch_dt<DT_BF16>(a, st);
+    const int mode = g_mode.load(std::memory_order_relaxed);
+    int8_t* w8 = nullptr;
+    if ((mode == 1 || (mode != 0 && M >= kExpandFirstRows)) && N * K < ((int64_t)1 << 32) && ((uintptr_t)Wp & 3) == 0) {
+        hipError_t e = hipMallocAsync((void**)&w8, (size_t)(N * K), st);
+        if (e != hipSuccess) return (int)e;
+        const int64_t pieces = N * K / 16;
+        const unsigned grid = (unsigned)((pieces + 255) / 256 < 256 * 32 ? (pieces + 255) / 256 : 256 * 32);
+        hipLaunchKernelGGL(w6_words_to_int8_kernel, dim3(grid), dim3(256), 0, st, (const uint8_t*)Wp, w8, pieces);
+        a.W8 = w8;
     }
+    int rc;
+    switch (out_dt) {
+        case DT_F32: rc = launch_dt<DT_F32>(a, st); break;
+        case DT_F16: rc = launch_dt<DT_F16>(a, st); break;
+        default: rc = launch_dt<DT_BF16>(a, st); break;
+    }
+    if (w8) {
+        hipError_t e = hipFreeAsync(w8, st);
+        if (rc == 0 && e != hipSuccess) rc = (int)e;
+    }
+    return rc;
+}
+
+// Test hook, no reference counterpart: 0 = gpu_w6a8_group_gemm always expands the weights inside the kernel, 1 = always
+// expands them first, -1 = chooses by M.
+GPU_API int gpu_internal_w6a8_group_gemm_mode(int mode) {
+    g_mode.store(mode, std::memory_order_relaxed);
+    return 0;
 }
 
 // Measurement hook, no reference counterpart: gpu_w6a8_group_gemm (bf16 output) with parts of the kernel left out --
-// ablate bit 0 the fp32 fold, bit 1 the unpack, bit 2 the LDS-DMA after the prologue.  D receives meaningless values.
+// ablate bit 0 the fp32 fold, bit 1 the unpack, bit 2 the LDS-DMA after the prologue; bit 3 (8, 9, 12, 13) the form that
+// fetches expanded weights, with Wp then pointing at int8 [N, K].  D receives meaningless values.
 GPU_API int gpu_internal_w6a8_group_gemm_ablate(int ablate, const int8_t* A, const void* Wp, const float* xs, const float* sw,
                                                 void* D, int64_t M, int64_t N, int64_t K, void* stream) {
     if (K <= 0 || (K % 128) != 0 || M <= 0 || N <= 0 || M * K >= ((int64_t)1 << 32) || N * (K / 4 * 3) >= ((int64_t)1 << 32)) return -200;
-    W6Args a{A, (const uint8_t*)Wp, xs, sw, nullptr, D, nullptr, (int)M, (int)N, (int)K, (int)(K / 128), 0, 0};
+    W6Args a{A, (const uint8_t*)Wp, nullptr, xs, sw, nullptr, D, nullptr, (int)M, (int)N, (int)K, (int)(K / 128), 0, 0};
     a.tiles_m = (int)((M + BM - 1) / BM);
     a.tiles_n = (int)((N + BN - 1) / BN);
     hipStream_t st = (hipStream_t)stream;
+    if (ablate & 8) a.W8 = (const int8_t*)Wp;   // the caller passes expanded weights, int8 [N, K]
     switch (ablate) {
         case 0: return launch<DT_BF16, false, 0>(a, st);
         case 1: return launch<DT_BF16, false, 1>(a, st);
@@ -450,6 +516,10 @@ GPU_API int gpu_internal_w6a8_group_gemm_ablate(int ablate, const int8_t* A, con
         case 5: return launch<DT_BF16, false, 5>(a, st);
         case 6: return launch<DT_BF16, false, 6>(a, st);
         case 7: return launch<DT_BF16, false, 7>(a, st);
+        case 8: return launch<DT_BF16, false, 0, true>(a, st);
+        case 9: return launch<DT_BF16, false, 1, true>(a, st);
+        case 12: return launch<DT_BF16, false, 4, true>(a, st);
+        case 13: return launch<DT_BF16, false, 5, true>(a, st);
         default: return -200;
     }
 }

@@ -49,6 +49,7 @@ SIGNATURES = {
     "gpu_internal_cvt_pk_u8_probe": [_P, _P, _I32, _P],
     "gpu_internal_attn_sumsq_probe": [_P, _P, _I32, _I32, _P],
     "gpu_internal_w6a8_group_gemm_ablate": [_I32, _P, _P, _P, _P, _P, _I64, _I64, _I64, _P],
+    "gpu_internal_w6a8_group_gemm_mode": [_I32],
     "gpu_internal_attn_layout": [_I32, _I32, _I32, _I32, _I32, _P],
     "gpu_internal_attn_layout_d": [_I32, _I32, _I32, _I32, _I32, _I32, _P],
     "gpu_int8_gemm_force_config": [_I32],

@@ -184,6 +184,11 @@ int gpu_internal_cvt_pk_u8_probe(const float* x, uint32_t* y, int n, void* strea
 int gpu_internal_w6a8_group_gemm_ablate(int ablate, const int8_t* A, const void* Wp, const float* xs, const float* sw, void* D,
                                         int64_t M, int64_t N, int64_t K, void* stream);
 
+/* Test hook, no reference counterpart: which form of gpu_w6a8_group_gemm runs.  0 = the weights are expanded to int8
+ * inside the kernel, per workgroup; 1 = they are expanded once into a stream-ordered scratch (N*K bytes) and the kernel
+ * fetches them like A; -1 = by M (the second form from 4096 rows on).  Both forms give the same bits. */
+int gpu_internal_w6a8_group_gemm_mode(int mode);
+
 /* Test hook, no reference counterpart: sums of squares of rows of 128 floats in the order the fused norm of
  * gpu_int8_attn_norm_rope takes them; out[2r] from the quantizers' eight-lane form, out[2r+1] from the anchor search's
  * one-thread form; split != 0 is rope_mode 2's lane layout.  rows % 8 == 0. */
@@ -247,8 +252,11 @@ int64_t gpu_int8_gemm_static_limit(void);
 int gpu_w6a8_gemm(const int8_t* A, const void* wq, const void* s_rel, int G, const float* xs, const float* s_channel,
                   const void* bias, void* D, int64_t M, int64_t N, int64_t K, int out_dt, void* stream);
 
-/* W6A8 linear with the unpack fused ahead of the MFMA, for this library's own packed format (no counterpart in the
- * reference, whose W6 weights are two-plane with e4m3 group factors: gpu_w6_decode / gpu_w6a8_gemm above).
+/* W6A8 linear with fp32 scales per group of 128 along K, for this library's own packed format (no counterpart in the
+ * reference, whose W6 weights are two-plane with e4m3 group factors: gpu_w6_decode / gpu_w6a8_gemm above).  Up to 4095
+ * rows of A the weights are expanded to int8 inside the GEMM kernel, ahead of the MFMA; from 4096 rows on they are
+ * expanded once into a stream-ordered scratch of N*K bytes (hipMallocAsync / hipFreeAsync on the call's stream) that
+ * the same kernel then fetches like A.  Same bits either way.
  *   Wp  uint8 [N, 3K/4]: codes u = q + 32 with q in [-32, 31]; every three bytes are the little-endian 24-bit word
  *       u0 | u1 << 6 | u2 << 12 | u3 << 18 of four consecutive k.
  *   sw  f32 [N, K/128]: one scale per output channel and group of 128 along K.

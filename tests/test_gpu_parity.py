@@ -890,10 +890,20 @@ W6G_CASES = [  # (M, N, K, out_dt, with_bias)
 ]
 
 
+@pytest.mark.parametrize("mode", [0, 1, -1])
 @pytest.mark.parametrize("M,N,K,out_dt,with_bias", W6G_CASES)
-def test_w6a8_group_gemm_matches_oracle(M, N, K, out_dt, with_bias):
-    """The fused-unpack kernel against the oracle: every int32 group partial and every output bit."""
-    say("w6a8_group", M, N, K, out_dt, with_bias)
+def test_w6a8_group_gemm_matches_oracle(M, N, K, out_dt, with_bias, mode):
+    """Both forms of the kernel (weights expanded inside it, mode 0; expanded once beforehand, mode 1; the library's own
+    choice by M, -1) against the oracle: every int32 group partial and every output bit."""
+    say("w6a8_group", M, N, K, out_dt, with_bias, "mode", mode)
+    ffi.raw("gpu_internal_w6a8_group_gemm_mode", mode)
+    try:
+        _w6a8_group_case(M, N, K, out_dt, with_bias)
+    finally:
+        ffi.raw("gpu_internal_w6a8_group_gemm_mode", -1)
+
+
+def _w6a8_group_case(M, N, K, out_dt, with_bias):
     A = rand_i8(9, 1, M, K, -127, 127)
     A[0, :] = -128
     qv = synth.w6_codes(9, N, K)
