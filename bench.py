@@ -113,8 +113,9 @@ def time_linear(torch, ffi, d, M, K, N, rotate, steps, warmup, nbuf=1, settled=T
 
 
 def time_w6a8(torch, ffi, M, K, N, steps, warmup):
-    """The fused-unpack W6A8 GEMM (24-bit words of four 6-bit codes, fp32 scales per 128 along K) on synthetic weights
-    with codes uniform in [-31, 31]; returns the average microseconds of gpu_w6a8_group_gemm."""
+    """The group-scaled W6A8 GEMM (24-bit words of four 6-bit codes, fp32 scales per 128 along K) on synthetic weights
+    with codes uniform in [-31, 31]; returns the average microseconds of gpu_w6a8_group_gemm (at these M the call
+    expands the weights into scratch first, then runs the GEMM kernel on them)."""
     g = torch.Generator(device="cuda:0").manual_seed(4)
     u = torch.randint(1, 64, (N, K // 4, 4), dtype=torch.int32, device="cuda:0", generator=g)   # u = q + 32
     w = u[..., 0] | (u[..., 1] << 6) | (u[..., 2] << 12) | (u[..., 3] << 18)
