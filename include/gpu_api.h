@@ -241,7 +241,8 @@ int gpu_int8_gemm_acc(const int8_t* A, const int8_t* W, int32_t* acc, int64_t M,
  * Every call on one GPU shares that GPU's array: calls that overlap in time on one GPU (two streams, two threads) race
  * on it and must be serialized by the caller.  Nothing in the array needs clearing between calls (every plane element
  * is written before it is read).  A shape whose planes would not fit returns -210 with a message on stderr;
- * gpu_int8_gemm_static_limit() returns the array's size in bytes.  Other return codes as gpu_int8_gemm. */
+ * gpu_int8_gemm_static_limit() returns the array's size in bytes.  K % 16 == 8, which gpu_int8_gemm serves from
+ * padded copies that it allocates, is refused here (-200).  Other return codes as gpu_int8_gemm. */
 int gpu_int8_gemm_static(const int8_t* A, const int8_t* W, const float* xs, const float* ws, const void* bias, void* D,
                          int64_t M, int64_t N, int64_t K, int out_dt, void* stream);
 int64_t gpu_int8_gemm_static_limit(void);

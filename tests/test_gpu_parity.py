@@ -880,6 +880,47 @@ def test_w6a8_linear_matches_decode_then_gemm():
     assert ffi.raw("gpu_w6a8_gemm", 0, 0, 0, 32, 0, 0, 0, 0, 4, 8, 48, 2, 0) == -1
 
 
+# ------------------------------------------------------------------------------------------------ graph capture
+@pytest.mark.parametrize("M,N,K,entry", [(4096, 4096, 256, "gpu_int8_gemm"),          # two-group kernel
+                                           (1024, 2304, 256, "gpu_int8_gemm"),          # ring kernel on 128x192 tiles
+                                           (256, 24576, 256, "gpu_int8_gemm"),          # stream kernel, whole K
+                                           (640, 1536, 512, "gpu_int8_gemm"),           # register-staged tiles
+                                           (256, 2048, 2048, "gpu_int8_gemm_static")])  # stream kernel, split K, static planes
+def test_linear_replays_from_a_captured_graph(M, N, K, entry):
+    """The quantizer and the GEMM allocate nothing on these routes (the split-K shape through the entry point with the
+    static planes), so one linear can be captured.  Three replays with new activations and eager work between them,
+    each against the oracle's linear on the same inputs."""
+    say("graph", M, N, K, entry)
+    W, ws, bias = synth.w8_weights(21, N, K)
+    bias = oracle.bf16_bits(bias)
+    Wd, wsd, bd = dev(W), dev(ws), dev_bits(bias, BF16)
+    x = torch.zeros((M, K), dtype=torch.bfloat16, device="cuda")
+    q = torch.empty((M, K), dtype=torch.int8, device="cuda")
+    xs = torch.empty((M,), dtype=torch.float32, device="cuda")
+    D = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+
+    def call():
+        s = torch.cuda.current_stream().cuda_stream
+        ffi.k("gpu_quant_rows", ffi.DT_BF16, ffi.PRO_PLAIN, x.data_ptr(), K, 0, 0, 0, 0, 0.0, 0, 0, q.data_ptr(), xs.data_ptr(), M, K, 128, s)
+        ffi.k(entry, q.data_ptr(), Wd.data_ptr(), xs.data_ptr(), wsd.data_ptr(), bd.data_ptr(), D.data_ptr(), M, N, K, ffi.DT_BF16, s)
+
+    call()                       # sets the kernels' LDS limits and, for the static entry point, finds its array
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()
+    for rep in range(3):
+        xb = synth.bf16_bits(synth.activations(30 + rep, M, K, "t3"))
+        x.copy_(dev_bits(xb, BF16))
+        D.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        rc, want, _ = oracle.linear_w8a8(BF16, xb, 128, W, ws, bias, BF16, threads=8)
+        assert rc == 0
+        assert np.array_equal(host_bits(D), want.view(np.uint16)), "replay %d" % rep
+        _ = (torch.randn(1024, device="cuda") * 2).sum().item()   # eager work between the replays
+
+
 # ------------------------------------------------------------------------- W6A8, packed words + fp32 group scales
 W6G_CASES = [  # (M, N, K, out_dt, with_bias)
     (256, 128, 128, BF16, True), (100, 200, 256, BF16, False), (300, 136, 640, F32, True), (513, 260, 384, F16, True),

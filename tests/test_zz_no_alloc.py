@@ -67,3 +67,19 @@ def test_static_entry_point_on_shapes_without_scratch():
     for (M, N, K) in [(300, 520, 256), (64, 64, 64)]:
         A, W, xs, ws, bias = _inputs(50, M, N, K)
         assert np.array_equal(_run("gpu_int8_gemm_static", A, W, xs, ws, bias), _run("gpu_int8_gemm", A, W, xs, ws, bias))
+
+
+def test_static_entry_point_refuses_what_would_need_an_allocation():
+    """K % 16 == 8 runs on padded copies that gpu_int8_gemm allocates; the entry point that may not allocate refuses it.
+    (The split-K planes of every M <= 256 shape fit the static array on a 256-CU device: slices * N <= 256 * 96.)"""
+    M, N, K = 64, 128, 136
+    A, W, xs, ws, bias = _inputs(60, M, N, K)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+    Ad, Wd, xsd, wsd, bd = t(A), t(W), t(xs), t(ws), t(bias.view(np.int16))
+    D = torch.zeros((M, N), dtype=torch.int16, device=DEV)
+    s = torch.cuda.current_stream().cuda_stream
+    args = (Ad.data_ptr(), Wd.data_ptr(), xsd.data_ptr(), wsd.data_ptr(), bd.data_ptr(), D.data_ptr(), M, N, K, ffi.DT_BF16, s)
+    assert ffi.raw("gpu_int8_gemm_static", *args) == -200
+    assert ffi.raw("gpu_int8_gemm", *args) == 0
+    torch.cuda.synchronize()
+    assert np.array_equal(D.cpu().numpy().view(np.uint16), oracle.int8_gemm(A, W, xs, ws, bias, oracle.BF16, fma=1).view(np.uint16))
