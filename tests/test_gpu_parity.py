@@ -880,6 +880,63 @@ def test_w6a8_linear_matches_decode_then_gemm():
     assert ffi.raw("gpu_w6a8_gemm", 0, 0, 0, 32, 0, 0, 0, 0, 4, 8, 48, 2, 0) == -1
 
 
+# A beyond 4 GiB: byte offsets into A no longer fit 32 bits, which the DMA kernels' lane offsets assume; the dispatcher has
+# to take the register-staged tiles with 64-bit addressing.  Checked on sampled rows against the oracle.
+def test_int8_gemm_with_operand_beyond_4_gib():
+    M, N, K = 66000, 96, 65536
+    say("gemm_4gib", M, N, K)
+    g = torch.Generator(device="cuda").manual_seed(77)
+    A = torch.randint(-128, 128, (M, K), dtype=torch.int8, device="cuda", generator=g)
+    W = torch.randint(-128, 128, (N, K), dtype=torch.int8, device="cuda", generator=g)
+    assert A.numel() > 1 << 32
+    acc = ql.int8_gemm_acc(A, W)
+    xs = dev(synth.uniform(8, 3, M, 0.005, 0.2))
+    ws = dev(synth.uniform(8, 4, N, 1e-3, 1e-2))
+    d = ql.int8_gemm(A, W, xs, ws, None, torch.float32)
+    torch.cuda.synchronize()
+    rows = sorted({0, 1, 255, 256, 32767, 32768, 65535, 65536, 65537, M - 2, M - 1} | {int(r) for r in synth.randint(8, 9, 24, 0, M - 1)})
+    idx = torch.tensor(rows, device="cuda")
+    Ah, Wh = A[idx].cpu().numpy(), W.cpu().numpy()
+    want = oracle.int8_gemm_acc(Ah, Wh)
+    assert np.array_equal(acc[idx].cpu().numpy(), want)
+    want_d = oracle.epilogue(want, xs[idx].cpu().numpy(), ws.cpu().numpy(), None, F32, fma=1)
+    assert np.array_equal(d[idx].cpu().numpy().view(np.uint32), want_d.view(np.uint32))
+    # every row: the checksum identity sum_n acc[m, n] = A[m, :] . sum_n W[n, :]
+    wsum = W.to(torch.int32).sum(0).to(torch.float64)
+    lhs = acc.to(torch.float64).sum(1)
+    rhs = torch.empty(M, dtype=torch.float64, device="cuda")
+    for r0 in range(0, M, 6000):
+        rhs[r0:r0 + 6000] = A[r0:r0 + 6000].to(torch.float64) @ wsum
+    assert torch.equal(lhs, rhs)
+
+
+@pytest.mark.parametrize("rotate", [128, 256])
+def test_quant_rows_with_more_than_2_to_the_31_elements(rotate):
+    """Element offsets past 2^31 and byte offsets past 2^32 (the longest row the reference takes, K = 32768, reduced over
+    eight waves): sampled rows against the oracle, and every row's scale against the maximum of |codes * scale|."""
+    M, K = 66000, 32768
+    say("quant_big", M, K, rotate)
+    g = torch.Generator(device="cuda").manual_seed(78)
+    x = torch.empty((M, K), dtype=torch.bfloat16, device="cuda")
+    for r0 in range(0, M, 6000):   # in slices: randn makes an fp32 temporary
+        x[r0:r0 + 6000] = (torch.randn((min(6000, M - r0), K), device="cuda", generator=g) * (1 + (r0 % 7))).to(torch.bfloat16)
+    assert x.numel() > 1 << 31
+    q, sc = ql.quant_rows(x, rotate)
+    torch.cuda.synchronize()
+    rows = sorted({0, 1, 32767, 32768, 65535, 65536, 65537, M - 1} | {int(r) for r in synth.randint(8, 19, 8, 0, M - 1)})
+    idx = torch.tensor(rows, device="cuda")
+    xb = x[idx].view(torch.int16).cpu().numpy().view(np.uint16)
+    rc, wq, wsc = oracle.quant_rows(BF16, xb, K, rotate)
+    assert rc == 0
+    assert np.array_equal(q[idx].cpu().numpy(), wq)
+    assert np.array_equal(sc[idx].cpu().numpy().view(np.uint32), wsc.view(np.uint32))
+    # every row was written: a code of magnitude 127 (the row maximum) in each, and a positive finite scale
+    amax = torch.empty(M, dtype=torch.int16, device="cuda")
+    for r0 in range(0, M, 6000):
+        amax[r0:r0 + 6000] = q[r0:r0 + 6000].to(torch.int16).abs().amax(1)
+    assert bool((amax >= 126).all()) and bool(torch.isfinite(sc).all()) and bool((sc > 0).all())
+
+
 # ------------------------------------------------------------------------------------------------ graph capture
 @pytest.mark.parametrize("M,N,K,entry", [(4096, 4096, 256, "gpu_int8_gemm"),          # two-group kernel
                                            (1024, 2304, 256, "gpu_int8_gemm"),          # ring kernel on 128x192 tiles
