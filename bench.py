@@ -187,8 +187,10 @@ def time_w6_reference_format(torch, ffi, M, K, N, steps, warmup):
 
 def time_mfma_ceiling(torch, ffi):
     """The matrix pipes alone: four waves per CU issuing nothing but v_mfma_i32_32x32x32_i8 on register operands, with
-    pseudo-random and with all-zero bits.  The chip's power management sets the clock by what the operands toggle, so
-    this is the ceiling any int8 GEMM on this part runs under; the kernel's own shader-clock counts give that clock."""
+    pseudo-random and with all-zero bits, and the same with v_mfma_i32_16x16x64_i8 (the form the large-shape GEMM uses:
+    the same operations per cycle, accumulators touched half as often).  The chip's power management sets the clock by
+    what the instructions toggle, so this is the ceiling any int8 GEMM on this part runs under; the kernel's own
+    shader-clock counts give that clock."""
     dev = "cuda:0"
     cu = torch.cuda.get_device_properties(0).multi_processor_count
     cyc = torch.zeros(cu, dtype=torch.int64, device=dev)
@@ -196,7 +198,7 @@ def time_mfma_ceiling(torch, ffi):
     st = torch.cuda.current_stream()
     iters, reps = 600, 10
     out = {"kernel": "gpu_mfma_ceiling_probe: %d workgroups x 4 waves x %d x 64 MFMA" % (cu, iters)}
-    for name, rnd in (("random_bits", 1), ("zero_bits", 0)):
+    for name, rnd in (("random_bits", 1), ("zero_bits", 0), ("random_bits_16x16x64", 3), ("zero_bits_16x16x64", 2)):
         run = lambda: ffi.k("gpu_mfma_ceiling_probe", iters, rnd, cyc.data_ptr(), sink.data_ptr(), st.cuda_stream)
         settle(torch, run)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -210,7 +212,7 @@ def time_mfma_ceiling(torch, ffi):
         ops = cu * 4.0 * iters * 64 * 65536
         cycles = float(cyc.double().mean().item())
         out[name] = {"TOPS": round(ops / ms / 1e9, 1), "frac_peak": round(ops / ms / 1e9 / PEAK_INT8_TOPS, 4),
-                     "shader_clock_GHz": round(cycles / (ms * 1e6), 3), "cycles_per_mfma": round(cycles / (iters * 64.0), 2)}
+                     "shader_clock_GHz": round(cycles / (ms * 1e6), 3), "cycles_per_mfma": round(cycles / (iters * (128.0 if rnd & 2 else 64.0)), 2)}
     return out
 
 

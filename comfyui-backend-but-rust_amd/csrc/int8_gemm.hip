@@ -138,8 +138,11 @@ __device__ __forceinline__ void epilogue_store(const GemmArgs& p, v16i (&acc)[TN
 // on the way out.  Needs row starts of D (and resid) 16-byte aligned; the caller falls back to epilogue_store otherwise.
 // STAGED: the per-column constants (ws and bias as floats, 2 x 32*TN values) are kept in the wave's LDS area `cst` and
 // read back per piece, instead of 96 registers that a persistent kernel cannot spare next to its pipeline state.
-template <int TM, int TN, int OUT_DT, int EPI, int PW = TN * 32, bool UNTRACKED = false, bool STAGED = false>
-__device__ __forceinline__ void epilogue_shuffle(const GemmArgs& p, v16i (&acc)[TN][TM], int mb, int nb, int lane, uint8_t* wl,
+// L: the MFMA shape the accumulators come from.  32: v16i acc[TN][TM], a lane holds row lane % 32 of a 32x32 tile and
+// the columns 8*rb + 4*(lane / 32) + j.  16: v4i acc[2*TN][2*TM] of 16x16 tiles, a lane holds row lane % 16 and the
+// columns 4*(lane / 16) + j; the 32x32 block (in, im) is then the four tiles (2*in + rb, 2*im + hm).
+template <int TM, int TN, int OUT_DT, int EPI, int PW = TN * 32, bool UNTRACKED = false, bool STAGED = false, int L = 32, class Acc>
+__device__ __forceinline__ void epilogue_shuffle(const GemmArgs& p, Acc& acc, int mb, int nb, int lane, uint8_t* wl,
                                                  uint8_t* wl2 = nullptr, float* cst = nullptr) {
     // a piece is 32 rows x PW columns of the wave tile: PW*SZ bytes per LDS row, 32*PW*SZ bytes per wave
     constexpr int SZ = (EPI == EPI_ACC || OUT_DT == DT_F32) ? 4 : 2;
@@ -153,13 +156,20 @@ __device__ __forceinline__ void epilogue_shuffle(const GemmArgs& p, v16i (&acc)[
     // of addresses out of the tile loop, keep them live across the K loop and spill them; the reloads then sit between
     // the stores, each behind a full memory wait.  Making the lane number opaque here keeps the address arithmetic local.
     asm volatile("" : "+v"(lane));
-    const int frow = lane & 31, fhalf = lane >> 5;
+    constexpr int NRB = L == 32 ? 4 : 2, NHM = L == 32 ? 1 : 2;   // column runs per 32 columns, row halves per 32 rows
+    const int frow = lane & (L - 1), fhalf = lane / L;            // row inside a tile; which four of every 8 (16) columns
+    // first column of run rb inside a 32-column block; value j of run rb of block (in, im), row half hm
+    auto run_col = [&](int rb) { return L == 32 ? rb * 8 + fhalf * 4 : rb * 16 + fhalf * 4; };
+    auto val = [&](int in, int im, int rb, int hm, int j) -> int {
+        if constexpr (L == 32) return acc[in][im][4 * rb + j];
+        else return acc[2 * in + rb][2 * im + hm][j];
+    };
 
     // per-lane column constants, loaded once and in one batch (no branches between the loads, so a single wait covers
     // them): ws and the raw bias words for the 4 n of every (in, rb).  Columns past N read the last valid vector.
     constexpr int BW = SZ == 4 ? 4 : 2;            // 32-bit words holding 4 bias values
-    float wsr[STAGED ? 1 : TN][4][4];
-    uint32_t braw[STAGED ? 1 : TN][4][BW];
+    float wsr[STAGED ? 1 : TN][NRB][4];
+    uint32_t braw[STAGED ? 1 : TN][NRB][BW];
     if (EPI != EPI_ACC && STAGED) {
         // two columns per lane and pass
 #pragma unroll
@@ -183,8 +193,8 @@ __device__ __forceinline__ void epilogue_shuffle(const GemmArgs& p, v16i (&acc)[
 #pragma unroll
         for (int in = 0; in < TN; ++in)
 #pragma unroll
-            for (int rb = 0; rb < 4; ++rb) {
-                int n = nb + in * 32 + rb * 8 + fhalf * 4;
+            for (int rb = 0; rb < NRB; ++rb) {
+                int n = nb + in * 32 + run_col(rb);
                 n = n < p.N ? n : p.N - 4;
                 const float4 w4 = *reinterpret_cast<const float4*>(p.ws + n);
                 wsr[in][rb][0] = w4.x; wsr[in][rb][1] = w4.y; wsr[in][rb][2] = w4.z; wsr[in][rb][3] = w4.w;
@@ -213,12 +223,14 @@ __device__ __forceinline__ void epilogue_shuffle(const GemmArgs& p, v16i (&acc)[
 
     // Every global load is issued ahead of the stores that precede its use: the memory counter retires in order, so a
     // load issued after a store cannot be waited for without also waiting for that store to reach memory.
-    float xsr[TM];
+    float xsr[TM][NHM];
 #pragma unroll
-    for (int im = 0; im < TM; ++im) {
-        const int mrow = mb + im * 32 + frow;
-        xsr[im] = (EPI == EPI_ACC || mrow >= p.M) ? 0.f : p.xs[mrow];
-    }
+    for (int im = 0; im < TM; ++im)
+#pragma unroll
+        for (int hm = 0; hm < NHM; ++hm) {
+            const int mrow = mb + im * 32 + hm * 16 + frow;
+            xsr[im][hm] = (EPI == EPI_ACC || mrow >= p.M) ? 0.f : p.xs[mrow];
+        }
     float rs[NP][EPC];
     if (EPI == EPI_RESID) {
 #pragma unroll
@@ -242,41 +254,45 @@ __device__ __forceinline__ void epilogue_shuffle(const GemmArgs& p, v16i (&acc)[
         }
     };
 
-    // write phase of piece (im, np): row frow of the piece into `buf`
+    // write phase of piece (im, np): this lane's rows of the piece into `buf`
     auto write_piece = [&](int im, int np, uint8_t* buf) {
-        const float xs = xsr[im];
 #pragma unroll
-        for (int ip = 0; ip < TNP; ++ip)
+        for (int hm = 0; hm < NHM; ++hm) {
+            const float xs = xsr[im][hm];
+            const int prow = hm * 16 + frow;   // row inside the 32-row piece
 #pragma unroll
-            for (int rb = 0; rb < 4; ++rb) {
-                const int in = np * TNP + ip;
-                const int byte = (ip * 32 + rb * 8 + fhalf * 4) * SZ;
-                uint8_t* dst = buf + frow * ROWB + ((((byte >> 4) ^ frow) & MASK) << 4) + (byte & 15);
-                if (EPI == EPI_ACC) {
-                    *reinterpret_cast<v4i*>(dst) = v4i{acc[in][im][4 * rb], acc[in][im][4 * rb + 1], acc[in][im][4 * rb + 2], acc[in][im][4 * rb + 3]};
-                } else {
-                    float o[4];
-                    if (STAGED) {
-                        const float4 w4 = *reinterpret_cast<const float4*>(cst + in * 32 + rb * 8 + fhalf * 4);
-                        const float4 b4 = *reinterpret_cast<const float4*>(cst + WTN + in * 32 + rb * 8 + fhalf * 4);
-                        o[0] = __builtin_fmaf((float)acc[in][im][4 * rb] * xs, w4.x, b4.x);
-                        o[1] = __builtin_fmaf((float)acc[in][im][4 * rb + 1] * xs, w4.y, b4.y);
-                        o[2] = __builtin_fmaf((float)acc[in][im][4 * rb + 2] * xs, w4.z, b4.z);
-                        o[3] = __builtin_fmaf((float)acc[in][im][4 * rb + 3] * xs, w4.w, b4.w);
+            for (int ip = 0; ip < TNP; ++ip)
+#pragma unroll
+                for (int rb = 0; rb < NRB; ++rb) {
+                    const int in = np * TNP + ip;
+                    const int byte = (ip * 32 + run_col(rb)) * SZ;
+                    uint8_t* dst = buf + prow * ROWB + ((((byte >> 4) ^ prow) & MASK) << 4) + (byte & 15);
+                    if (EPI == EPI_ACC) {
+                        *reinterpret_cast<v4i*>(dst) = v4i{val(in, im, rb, hm, 0), val(in, im, rb, hm, 1), val(in, im, rb, hm, 2), val(in, im, rb, hm, 3)};
                     } else {
+                        float o[4];
+                        if (STAGED) {
+                            const float4 w4 = *reinterpret_cast<const float4*>(cst + in * 32 + run_col(rb));
+                            const float4 b4 = *reinterpret_cast<const float4*>(cst + WTN + in * 32 + run_col(rb));
+                            o[0] = __builtin_fmaf((float)val(in, im, rb, hm, 0) * xs, w4.x, b4.x);
+                            o[1] = __builtin_fmaf((float)val(in, im, rb, hm, 1) * xs, w4.y, b4.y);
+                            o[2] = __builtin_fmaf((float)val(in, im, rb, hm, 2) * xs, w4.z, b4.z);
+                            o[3] = __builtin_fmaf((float)val(in, im, rb, hm, 3) * xs, w4.w, b4.w);
+                        } else {
 #pragma unroll
-                        for (int j = 0; j < 4; ++j) o[j] = __builtin_fmaf((float)acc[in][im][4 * rb + j] * xs, wsr[in][rb][j], bias_f(in, rb, j));
-                    }
-                    if (OUT_DT == DT_F32) {
-                        *reinterpret_cast<float4*>(dst) = make_float4(o[0], o[1], o[2], o[3]);
-                    } else if (OUT_DT == DT_BF16) {
-                        *reinterpret_cast<uint2*>(dst) = make_uint2(pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]));
-                    } else {
-                        *reinterpret_cast<uint2*>(dst) = make_uint2((uint32_t)f_to_f16(o[0]) | ((uint32_t)f_to_f16(o[1]) << 16),
-                                                                    (uint32_t)f_to_f16(o[2]) | ((uint32_t)f_to_f16(o[3]) << 16));
+                            for (int j = 0; j < 4; ++j) o[j] = __builtin_fmaf((float)val(in, im, rb, hm, j) * xs, wsr[in][rb][j], bias_f(in, rb, j));
+                        }
+                        if (OUT_DT == DT_F32) {
+                            *reinterpret_cast<float4*>(dst) = make_float4(o[0], o[1], o[2], o[3]);
+                        } else if (OUT_DT == DT_BF16) {
+                            *reinterpret_cast<uint2*>(dst) = make_uint2(pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]));
+                        } else {
+                            *reinterpret_cast<uint2*>(dst) = make_uint2((uint32_t)f_to_f16(o[0]) | ((uint32_t)f_to_f16(o[1]) << 16),
+                                                                        (uint32_t)f_to_f16(o[2]) | ((uint32_t)f_to_f16(o[3]) << 16));
+                        }
                     }
                 }
-            }
+        }
     };
     // read phase, first half: the piece's rows back from `buf`, 16 bytes per lane and pass, all passes in one batch
     auto read_piece = [&](const uint8_t* buf, uint4* v) {
@@ -791,7 +807,8 @@ __global__ void __launch_bounds__(C::NT, 1) int8_gemm_ring_kernel(GemmArgs p) {
 // for part of each one.  Here a workgroup has eight waves, two per SIMD, in two groups of four: group g owns rows
 // 128g..128g+127 of a 256x256 tile (wave tiles 128x64).  The groups alternate between two kinds of phase, with one
 // workgroup barrier between phases:
-//   compute: the 32 MFMAs of one 128-deep K step, on fragments already in registers, and nothing else;
+//   compute: the 64 MFMAs (16x16x64, 16 cycles each) of one 128-deep K step, on fragments already in registers, and
+//            nothing else;
 //   memory:  the 24 fragment reads of the group's next K step and 8 DMA instructions per wave.
 // While one wave of a SIMD is in its memory phase the other is in its compute phase, so the matrix pipe always has an
 // MFMA to run and no MFMA waits behind a DMA.
@@ -884,51 +901,46 @@ __device__ __forceinline__ void pp_gemm_tiles(const GemmArgs& p, uint8_t* smem, 
         if (++w_kt == nk) { w_kt = 0; set_w(++w_tile); }
     };
 
-    // fragment addresses inside a stage: row r at r*128, chunk c at slot c ^ ((r>>1)&7); K sub-step kk flips bits 5 and 6
-    v16i acc[TN][TM];
-    v4i f[4][TM + TN];
+    // The tiles are multiplied with v_mfma_i32_16x16x64_i8: as many operations per cycle as the 32x32x32 form and the same
+    // fragment bytes per K, but an accumulator is touched once per 64 K instead of once per 32.  On this power-limited
+    // part that is worth clock: a loop of nothing but MFMAs on random bits sustains 3.95 POP/s in this form against 3.4,
+    // and this kernel ran 9-11 % faster with it.  A wave tile is FM x FN tiles of 16 x 16, four accumulator registers each.
+    // Fragment addresses inside a stage: row r at r*128, chunk c at slot c ^ ((r>>1)&7); a lane reads row lane % 16,
+    // chunk 4*kk + lane / 16 of K half kk (which flips bit 6).
+    constexpr int FM = 2 * TM, FN = 2 * TN;
+    v4i acc[FN][FM];
+    v4i f[2][FM + FN];
     int ra_stage = 0, rw_stage = 0;   // stages this group's next fragments come from
     auto load_frags = [&]() {
         const int l = hw_lane();
-        const int frow = l & 31, fhalf = l >> 5;
-        const int x = frow * BK + ((fhalf ^ ((frow >> 1) & 7)) << 4);
+        const int frow = l & 15, fq = l >> 4;
+        const int x = frow * BK + ((fq ^ ((frow >> 1) & 7)) << 4);
         const uint8_t* sa = smem + C::A_BASE + (grp * C::NSA + ra_stage) * C::A_STAGE;
         const uint8_t* sw = smem + rw_stage * C::W_STAGE + wq * C::WTN * BK;
         ra_stage = ra_stage == C::NSA - 1 ? 0 : ra_stage + 1;
         rw_stage = rw_stage == C::NSW - 1 ? 0 : rw_stage + 1;
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
+        for (int kk = 0; kk < 2; ++kk) {
+            const int xk = x ^ (kk << 6);
 #pragma unroll
-            for (int j = 0; j < TM; ++j) f[kk][j] = *reinterpret_cast<const v4i*>(sa + (x ^ (kk << 5)) + j * 32 * BK);
+            for (int j = 0; j < FM; ++j) f[kk][j] = *reinterpret_cast<const v4i*>(sa + xk + j * 16 * BK);
 #pragma unroll
-            for (int j = 0; j < TN; ++j) f[kk][TM + j] = *reinterpret_cast<const v4i*>(sw + (x ^ (kk << 5)) + j * 32 * BK);
+            for (int j = 0; j < FN; ++j) f[kk][FM + j] = *reinterpret_cast<const v4i*>(sw + xk + j * 16 * BK);
         }
     };
+    // a tile's first MFMAs take C = 0 instead of cleared accumulators
     auto compute = [&](bool first) {
         __builtin_amdgcn_s_setprio(1);
-        if (first) {
 #pragma unroll
-            for (int in = 0; in < TN; ++in)
+        for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
-                for (int im = 0; im < TM; ++im) {
-                    v16i z;
+            for (int in = 0; in < FN; ++in)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) z[r] = 0;
-                    acc[in][im] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f[0][TM + in], f[0][im], z, 0, 0, 0);
+                for (int im = 0; im < FM; ++im) {
+                    const v4i c = (first && kk == 0) ? v4i{0, 0, 0, 0} : acc[in][im];
+                    acc[in][im] = __builtin_amdgcn_mfma_i32_16x16x64_i8(f[kk][FM + in], f[kk][im], c, 0, 0, 0);
                     SCHED_FENCE();
                 }
-        }
-#pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
-            if (first && kk == 0) continue;
-#pragma unroll
-            for (int in = 0; in < TN; ++in)
-#pragma unroll
-                for (int im = 0; im < TM; ++im) {
-                    acc[in][im] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f[kk][TM + in], f[kk][im], acc[in][im], 0, 0, 0);
-                    SCHED_FENCE();
-                }
-        }
         __builtin_amdgcn_s_setprio(0);
     };
     // memory phase before this group's next step
@@ -975,7 +987,7 @@ __device__ __forceinline__ void pp_gemm_tiles(const GemmArgs& p, uint8_t* smem, 
         int m0, n0;
         tile_origin(ti, m0, n0);
         uint8_t* scratch = smem + (s_last % C::NSW) * C::W_STAGE + wave * 4096;
-        epilogue_shuffle<TM, TN, OUT_DT, EPI, PW, true, false>(p, acc, m0 + grp * C::GM, n0 + wq * C::WTN, hw_lane(), scratch);
+        epilogue_shuffle<TM, TN, OUT_DT, EPI, PW, true, false, 16>(p, acc, m0 + grp * C::GM, n0 + wq * C::WTN, hw_lane(), scratch);
     };
 
     // Both groups run the same loop; group 1 is one phase behind (the barrier in front), multiplies its last step of a
@@ -1634,7 +1646,7 @@ __global__ void mfma_layout_probe_kernel(int* out) {
 // Nothing but v_mfma_i32_32x32x32_i8: four waves per CU, sixteen independent accumulator tiles per wave (the register
 // shape of the GEMM kernels), operands held in registers.  What this loop sustains is the matrix pipes' ceiling under
 // the chip's power management for the given operand bits; the shader-clock count per workgroup gives the clock.
-__global__ void __launch_bounds__(256, 1) mfma_ceiling_kernel(int iters, int random_bits, long long* cycles, int* sink) {
+__global__ void __launch_bounds__(256, 1) mfma_ceiling_kernel(int iters, int random_bits, int form, long long* cycles, int* sink) {
     const uint32_t tid = threadIdx.x + blockIdx.x * 256u;
     auto hash = [](uint32_t x) { x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16; return x; };
     v4i a[4], b[4];
@@ -1645,6 +1657,33 @@ __global__ void __launch_bounds__(256, 1) mfma_ceiling_kernel(int iters, int ran
             a[i][r] = random_bits ? (int)hash(tid * 977u + i * 17u + r) : 0;
             b[i][r] = random_bits ? (int)hash(tid * 613u + i * 29u + r + 99991u) : 0;
         }
+    if (form == 16) {   // v_mfma_i32_16x16x64_i8: 32 accumulator tiles with their own operand pairs, the same operations per iteration
+        v4i c4[32];
+        v4i a2[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) a2[i][r] = random_bits ? (int)hash(tid * 331u + i * 41u + r + 77777u) : 0;
+#pragma unroll
+        for (int i = 0; i < 32; ++i) c4[i] = v4i{0, 0, 0, 0};
+        const long long t0 = (long long)__builtin_readcyclecounter();
+        for (int it = 0; it < iters; ++it) {
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+                for (int i = 0; i < 32; ++i) {
+                    c4[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b[(i >> 2) & 3], i < 16 ? a[i & 3] : a2[i & 3], c4[i], 0, 0, 0);
+                    SCHED_FENCE();
+                }
+        }
+        const long long t1 = (long long)__builtin_readcyclecounter();
+        int s = 0;
+#pragma unroll
+        for (int i = 0; i < 32; ++i) s += c4[i][0] + c4[i][1] + c4[i][2] + c4[i][3];
+        if (s == 0x7fffffff) sink[0] = s;   // keeps the accumulators alive
+        if (threadIdx.x == 0) cycles[blockIdx.x] = t1 - t0;
+        return;
+    }
     v16i acc[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i)
@@ -1734,8 +1773,9 @@ GPU_API int gpu_int8_gemm_force_config(int cfg) {
 
 GPU_API int gpu_mfma_ceiling_probe(int iters, int random_bits, int64_t* cycles, int32_t* sink, void* stream) {
     if (iters <= 0) return 0;
-    hipLaunchKernelGGL(mfma_ceiling_kernel, dim3((unsigned)device_cu_count()), dim3(256), 0, (hipStream_t)stream, iters, random_bits,
-                       (long long*)cycles, (int*)sink);
+    // random_bits: 0 = zero operands, 1 = random; + 2 = the 16x16x64 form of the instruction instead of 32x32x32
+    hipLaunchKernelGGL(mfma_ceiling_kernel, dim3((unsigned)device_cu_count()), dim3(256), 0, (hipStream_t)stream, iters, random_bits & 1,
+                       (random_bits & 2) ? 16 : 32, (long long*)cycles, (int*)sink);
     KCHECK();
     return 0;
 }

@@ -280,8 +280,9 @@ int gpu_int8_gemm_force_config(int cfg);
  * layout the GEMM kernels assume; out is int32 [1024]. */
 int gpu_mfma_layout_probe(int32_t* out, void* stream);
 
-/* Measurement hook: one workgroup of four waves per CU runs iters * 64 v_mfma_i32_32x32x32_i8 per wave on operands held in
- * registers (all zero, or pseudo-random bits when random_bits != 0) and nothing else.  cycles[i] receives the
+/* Measurement hook: one workgroup of four waves per CU runs iters * 64 v_mfma_i32_32x32x32_i8 per wave (or, with bit 1 of
+ * random_bits set, iters * 128 v_mfma_i32_16x16x64_i8: the same operations) on operands held in registers (all zero,
+ * or pseudo-random bits when bit 0 of random_bits is set) and nothing else.  cycles[i] receives the
  * shader-clock count of workgroup i (one entry per CU, device int64); ops per launch = CUs * 4 * iters * 64 * 65536.
  * Timed from outside with events, this gives the matrix pipes' ceiling under the chip's power management and, from the
  * cycle counts, the shader clock it settles at.  sink: one device int32 (never written in practice). */
