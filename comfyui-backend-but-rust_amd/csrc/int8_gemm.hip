@@ -1057,7 +1057,7 @@ template <int OUT_DT, int EPI>
 __global__ void __launch_bounds__(StreamCfg::NT, 1) int8_gemm_stream_kernel(GemmArgs p) {
     using C = StreamCfg;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    constexpr int BK = C::BK, TM = C::TM, TN = C::TN, NM = C::NM, NF = C::NF;
+    constexpr int BK = C::BK, TM = C::TM, TN = C::TN;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int ld = p.K;
@@ -1197,68 +1197,77 @@ __global__ void __launch_bounds__(StreamCfg::NT, 1) int8_gemm_stream_kernel(Gemm
         return;
     }
 
-    // ---- the four MFMA waves: wave w multiplies rows 64w..64w+63 of the tile by all 96 columns
+    // ---- the four MFMA waves: wave w multiplies rows 64w..64w+63 of the tile by all 96 columns, with
+    // v_mfma_i32_16x16x64_i8 (4 x 6 tiles of 16 x 16; see the two-group kernel for why this form).  A K tile is two halves
+    // of 64; a half is six slots of four MFMAs that share one W fragment.  Fragments live in 40 registers: the A
+    // fragments of the current half and of the next one, and three rotating W fragments read two slots ahead.
     const int wm = wave;
-    const int frow = lane & 31, fhalf = lane >> 5;
-    const int fsw = (fhalf ^ ((frow >> 1) & 7)) << 4;
-    int aoff[4], woff[4];
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
-        aoff[kk] = ((wm * C::WTM + frow) * BK + fsw) ^ (kk << 5);
-        woff[kk] = (frow * BK + fsw) ^ (kk << 5);
-    }
-    auto frag = [&](const uint8_t* sa, const uint8_t* sw, int kk, int j) -> v4i {
-        if (j < TM) return *reinterpret_cast<const v4i*>(sa + aoff[kk] + j * 32 * BK);
-        return *reinterpret_cast<const v4i*>(sw + woff[kk] + (j - TM) * 32 * BK);
-    };
-    v16i acc[TN][TM];
-    v4i f0[NF], f1[NF];
-    auto substep = [&](v4i* cur, v4i* nxt, const uint8_t* sa_n, const uint8_t* sw_n, int kk_n) {
-#pragma unroll
-        for (int i = 0; i < NM; ++i) {
-            const int in = i / TM, im = i % TM;
-            acc[in][im] = __builtin_amdgcn_mfma_i32_32x32x32_i8(cur[TM + in], cur[im], acc[in][im], 0, 0, 0);
-            SCHED_FENCE();
-            if (i < NF) { nxt[i] = frag(sa_n, sw_n, kk_n, i); SCHED_FENCE(); }
-        }
-    };
+    const int frow = lane & 15, fq = lane >> 4;
+    const int fx = frow * BK + ((fq ^ ((frow >> 1) & 7)) << 4);   // row r at r*128, chunk c at slot c ^ ((r>>1)&7)
+    const int aoff = wm * C::WTM * BK + fx;
+    constexpr int FM = 2 * TM, FN = 2 * TN;   // 4 x 6 tiles of 16 x 16
+    auto a_frag = [&](const uint8_t* sa, int h, int j) -> v4i { return *reinterpret_cast<const v4i*>(sa + ((aoff + j * 16 * BK) ^ (h << 6))); };
+    auto w_frag = [&](const uint8_t* sw, int h, int in) -> v4i { return *reinterpret_cast<const v4i*>(sw + ((fx + in * 16 * BK) ^ (h << 6))); };
+    v4i acc[FN][FM];
+    v4i fa[2][FM], fw[3];
     wg_barrier();   // A(0) and W(0) have landed
+    auto first_frags = [&](const uint8_t* sa, const uint8_t* sw) {
 #pragma unroll
-    for (int j = 0; j < NF; ++j) f0[j] = frag(smem, smem + C::W_BASE, 0, j);
+        for (int j = 0; j < FM; ++j) fa[0][j] = a_frag(sa, 0, j);
+        fw[0] = w_frag(sw, 0, 0);
+        fw[1] = w_frag(sw, 0, 1);
+    };
+    first_frags(smem, smem + C::W_BASE);
     int ca = 0, cw = 0;   // stages of the iteration being multiplied
     for (int ti = 0; ti < nt_b; ++ti) {
 #pragma unroll
-        for (int in = 0; in < TN; ++in)
+        for (int in = 0; in < FN; ++in)
 #pragma unroll
-            for (int im = 0; im < TM; ++im)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) acc[in][im][r] = 0;
-        int pa = 0, pw = 0;
+            for (int im = 0; im < FM; ++im) acc[in][im] = v4i{0, 0, 0, 0};
+        int pa = 0;
         int m0, n0;
         tile_origin(ti, m0, n0);
         for (int kt = 0; kt < nk; ++kt) {
             const uint8_t* sa = smem + ca * C::A_STAGE;
             const uint8_t* sw = smem + C::W_BASE + cw * C::W_STAGE;
             const int na = ca == C::NSA - 1 ? 0 : ca + 1, nw = cw == C::NSW - 1 ? 0 : cw + 1;
+            const uint8_t* sa_n = smem + na * C::A_STAGE;
+            const uint8_t* sw_n = smem + C::W_BASE + nw * C::W_STAGE;
             wg_barrier();                                                   // X
-            substep(f0, f1, sa, sw, 1);
-            substep(f1, f0, sa, sw, 2);
-            substep(f0, f1, sa, sw, 3);
-            wg_barrier();                                                   // Y
-            substep(f1, f0, smem + na * C::A_STAGE, smem + C::W_BASE + nw * C::W_STAGE, 0);
+            // slot s = 6h + in: four MFMAs on W fragment fw[s % 3] and the A fragments of half h.  Behind its MFMAs a slot
+            // reads the W fragment of slot s + 2 and one A fragment of the next half; from slot 8 on those come from the next
+            // K tile's stages, so barrier Y (they have landed) sits in front of slot 8.
+#pragma unroll
+            for (int sl = 0; sl < 12; ++sl) {
+                const int h = sl / 6, in = sl % 6;
+                if (sl == 8) wg_barrier();                                  // Y
+#pragma unroll
+                for (int im = 0; im < FM; ++im) {
+                    acc[in][im] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fw[sl % 3], fa[h][im], acc[in][im], 0, 0, 0);
+                    SCHED_FENCE();
+                    if (im == 0) {
+                        const int s2 = sl + 2;   // the slot two ahead: this K tile's, or the next one's first two
+                        fw[s2 % 3] = s2 < 12 ? w_frag(sw, s2 / 6, s2 % 6) : w_frag(sw_n, 0, s2 - 12);
+                        SCHED_FENCE();
+                    }
+                    if (im == 2 && in >= 2) {   // slots 2..5 of a half: the next half's A fragments
+                        fa[h ^ 1][in - 2] = h == 0 ? a_frag(sa, 1, in - 2) : a_frag(sa_n, 0, in - 2);
+                        SCHED_FENCE();
+                    }
+                }
+            }
             pa = ca;
-            pw = cw;
             ca = na;
             cw = nw;
         }
         __syncthreads();   // every wave is done with the stage that becomes the shuffle scratch (8 KB per wave)
-        constexpr int SZ = (EPI == EPI_ACC || OUT_DT == DT_F32) ? 4 : 2;
         // (The stage of A(g) is refilled with A(g+NSA), issued after barrier X of the next iteration: behind this epilogue.)
         uint8_t* scratch = smem + pa * C::A_STAGE + wave * 8192;   // a 4 KB piece, then the wave's column constants
-        epilogue_shuffle<TM, TN, OUT_DT, EPI, 32, true, true>(p, acc, m0 + wm * C::WTM, n0, lane, scratch, nullptr,
-                                                              reinterpret_cast<float*>(scratch + 4096));
-#pragma unroll
-        for (int j = 0; j < NF; ++j) f0[j] = frag(smem + ca * C::A_STAGE, smem + C::W_BASE + cw * C::W_STAGE, 0, j);
+        epilogue_shuffle<TM, TN, OUT_DT, EPI, 32, true, true, 16>(p, acc, m0 + wm * C::WTM, n0, lane, scratch, nullptr,
+                                                                  reinterpret_cast<float*>(scratch + 4096));
+        // the first fragments of the next tile were prefetched by the last slots; fetching them again here instead of
+        // carrying them across the epilogue keeps the epilogue free of spills
+        first_frags(smem + ca * C::A_STAGE, smem + C::W_BASE + cw * C::W_STAGE);
     }
 }
 
