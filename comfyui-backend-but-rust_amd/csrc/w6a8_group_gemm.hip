@@ -16,11 +16,11 @@
 //   * the packed weights are wave-local: wave w fetches rows 16w..16w+15 itself (1.5 KB), waits for its own fetch, and
 //     expands its 128 twelve-byte pieces (two per lane) of group g+1 into 16 int8 each, written in the swizzled
 //     fragment layout (conflict-free both ways).  Only the expanded tile crosses waves, behind the iteration's barrier;
-//   * each wave (2 x 4 grid, 128 x 32 outputs, four MFMA tiles) multiplies group g in two pairs of tiles; the fp32
-//     fold of the first pair rides between the MFMAs of the second.
+//   * each wave (2 x 4 grid, 128 x 32 outputs, 8 x 2 tiles of v_mfma_i32_16x16x64_i8) multiplies group g in two halves
+//     of eight tiles; the fp32 fold of the first half rides between the MFMAs of the second.
 // The fold costs two VALU operations per output and group and the unpack about six per code word: together more issue
 // slots than the MFMAs, so the kernel is bound by VALU issue, not by the matrix pipe.  Two waves share a SIMD; the upper
-// four waves fold their second pair at the end of an iteration, the lower four at the start of the next, so that on
+// four waves fold their second half at the end of an iteration, the lower four at the start of the next, so that on
 // every SIMD one wave's VALU-only stretch meets the other's MFMAs.
 #include "common.hpp"
 #include <atomic>
@@ -55,7 +55,6 @@ template <bool W8> struct Lay {
     static_assert(SMEM <= 160 * 1024, "LDS budget");
 };
 constexpr int RAW_WAVE = 16 * RAW_ROW;   // bytes of packed weights a wave owns per group: 16 rows
-constexpr int TM = 4, TN = 1;   // 32x32 MFMA tiles of one wave: 128 rows (m) x 32 columns (n)
 constexpr int NT = 512;         // eight waves, 2 (m) x 4 (n)
 
 // Four 6-bit fields of a 24-bit word (bits above 23 are ignored) -> four int8 q = u - 32, one per byte.
@@ -154,24 +153,24 @@ __global__ void __launch_bounds__(NT, 1) w6a8_group_gemm_kernel(W6Args p) {
         *reinterpret_cast<v4i*>(smem + U_BASE + ustage * U_STAGE + r * BK + ((pc ^ ((r >> 1) & 7)) << 4)) = out;
     };
 
-    // fragment addresses inside a stage: row r at r*128, chunk c at slot c ^ ((r>>1)&7); K sub-step kk flips bits 5 and 6
-    const int frow = lane & 31, fhalf = lane >> 5;
-    const int fsw = (fhalf ^ ((frow >> 1) & 7)) << 4;
-    int aoff[4], woff[4];
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
-        aoff[kk] = ((wm * 128 + frow) * BK + fsw) ^ (kk << 5);
-        woff[kk] = ((wn * 32 + frow) * BK + fsw) ^ (kk << 5);
-    }
+    // The tiles are multiplied with v_mfma_i32_16x16x64_i8 (the same operations per cycle as the 32x32x32 form, less
+    // accumulator traffic per operation, which this power-limited part pays back as clock): a wave's 128 x 32 outputs are
+    // 8 x 2 tiles of 16 x 16, four registers each.  A lane holds row lane % 16 of a tile and columns 4*(lane / 16) + c.
+    // Fragment addresses inside a stage: row r at r*128, chunk c at slot c ^ ((r>>1)&7); a lane reads row lane % 16, chunk
+    // 4*h + lane / 16 of K half h (which flips bit 6).
+    const int frow = lane & 15, fq = lane >> 4;
+    const int fsw = (fq ^ ((frow >> 1) & 7)) << 4;
+    const int aoff = (wm * 128 + frow) * BK + fsw, woff = (wn * 32 + frow) * BK + fsw;
+    constexpr int FM = 8, FN = 2;
 
-    v16i part[TN][TM];      // int32 partial of the current group
-    float accf[TN][TM][16]; // fp32 accumulators
+    v4i part[FN][FM];        // int32 partial of the current group
+    float accf[FN][FM][4];   // fp32 accumulators
 #pragma unroll
-    for (int in = 0; in < TN; ++in)
+    for (int in = 0; in < FN; ++in)
 #pragma unroll
-        for (int im = 0; im < TM; ++im)
+        for (int im = 0; im < FM; ++im)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) accf[in][im][r] = 0.f;
+            for (int r = 0; r < 4; ++r) accf[in][im][r] = 0.f;
 
     // prologue: groups 0 and 1 of everything land; the wave's rows of group 0 are unpacked
 #pragma unroll
@@ -193,22 +192,21 @@ __global__ void __launch_bounds__(NT, 1) w6a8_group_gemm_kernel(W6Args p) {
     }
     __syncthreads();
 
-    const bool defer = wm == 0;   // these waves fold their second pair at the start of the next iteration
+    const bool defer = wm == 0;   // these waves fold their second half at the start of the next iteration
 #pragma unroll
-    for (int im = 0; im < TM; ++im)
+    for (int in = 0; in < FN; ++in)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) part[0][im][r] = 0;
+        for (int im = 0; im < FM; ++im) part[in][im] = v4i{0, 0, 0, 0};
 
-    // fp32 fold of four values: register group q of tile im.  accf += float(part) * sw[n, g]
-    auto fold = [&](int im, int q, const float4& s4) {
-        if (ABL & 1) {   // keep the partials alive with one operation per register group instead of eight
-            accf[0][im][4 * q] += __builtin_bit_cast(float, part[0][im][4 * q] ^ part[0][im][4 * q + 1] ^ part[0][im][4 * q + 2] ^ part[0][im][4 * q + 3]);
+    // fp32 fold of one tile's four values.  accf += float(part) * sw[n, g]
+    auto fold = [&](int in, int im, const float4& s4) {
+        if (ABL & 1) {   // keep the partials alive with one operation per tile instead of eight
+            accf[in][im][0] += __builtin_bit_cast(float, part[in][im][0] ^ part[in][im][1] ^ part[in][im][2] ^ part[in][im][3]);
             return;
         }
         const float sv[4] = {s4.x, s4.y, s4.z, s4.w};
 #pragma unroll
-        for (int c = 0; c < 4; ++c)
-            accf[0][im][4 * q + c] = __builtin_fmaf((float)part[0][im][4 * q + c], sv[c], accf[0][im][4 * q + c]);
+        for (int c = 0; c < 4; ++c) accf[in][im][c] = __builtin_fmaf((float)part[in][im][c], sv[c], accf[in][im][c]);
     };
 
     int a_cur = 0, s_cur = 0;   // stages of group g: g mod 3 (A), g mod 4 (scales)
@@ -221,26 +219,21 @@ __global__ void __launch_bounds__(NT, 1) w6a8_group_gemm_kernel(W6Args p) {
         const float* sc = reinterpret_cast<const float*>(smem + S_BASE + s_cur * S_STAGE);
         const float* sc_prev = reinterpret_cast<const float*>(smem + S_BASE + s_prev * S_STAGE);
 
-        v4i fa[2][4], fw[4], na[2][4];
-        float4 sv[4];
+        v4i fa[4][2], fw[FN][2], na[4][2];   // A fragments of row tiles 0..3 / 4..7 and W fragments, per K half
+        float4 sv[FN];
         uint32_t raw[2][3];
-        // Eight MFMAs of the pair (imb, imb+1), the two accumulation chains interleaved; between(i) is issued after the
-        // i-th of them.
-        auto mma_pair = [&](int imb, v4i (&a)[2][4], auto&& between) {
+        // Sixteen MFMAs of one half of the wave tile (row tiles imb .. imb+3, both column tiles, both K halves; a tile's two
+        // MFMAs are eight apart); between(i) is issued after the i-th of them.
+        auto mma_half = [&](int imb, v4i (&a)[4][2], auto&& between) {
 #pragma unroll
-            for (int kk = 0; kk < 4; ++kk)
+            for (int h = 0; h < 2; ++h)
 #pragma unroll
-                for (int t = 0; t < 2; ++t) {
-                    if (kk == 0) {
-                        v16i zero;
-#pragma unroll
-                        for (int r = 0; r < 16; ++r) zero[r] = 0;
-                        part[0][imb + t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fw[kk], a[t][kk], zero, 0, 0, 0);
-                    } else {
-                        part[0][imb + t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fw[kk], a[t][kk], part[0][imb + t], 0, 0, 0);
-                    }
+                for (int t = 0; t < 8; ++t) {
+                    const int in = t & 1, il = t >> 1;
+                    const v4i c = h == 0 ? v4i{0, 0, 0, 0} : part[in][imb + il];
+                    part[in][imb + il] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fw[in][h], a[il][h], c, 0, 0, 0);
                     SCHED_FENCE();
-                    between(kk * 2 + t);
+                    between(h * 8 + t);
                     SCHED_FENCE();
                 }
         };
@@ -249,66 +242,72 @@ __global__ void __launch_bounds__(NT, 1) w6a8_group_gemm_kernel(W6Args p) {
         // five issued after them may still be in flight.
         if (ABL & 4) wait_all_dma();
         else if (!W8) wait_vmcnt_n<5>();
-        // everything this iteration reads from LDS early: fragments of the first pair, the group's scales, packed words
+        // everything this iteration reads from LDS early: fragments of the first half, the group's scales, packed words
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) fw[kk] = *reinterpret_cast<const v4i*>(su + woff[kk]);
+        for (int in = 0; in < FN; ++in)
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
+            for (int h = 0; h < 2; ++h) fw[in][h] = *reinterpret_cast<const v4i*>(su + ((woff + in * 16 * BK) ^ (h << 6)));
 #pragma unroll
-            for (int kk = 0; kk < 4; ++kk) fa[t][kk] = *reinterpret_cast<const v4i*>(sa + aoff[kk] + t * 32 * BK);
+        for (int il = 0; il < 4; ++il)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) sv[q] = *reinterpret_cast<const float4*>(sc + wn * 32 + 8 * q + 4 * fhalf);
+            for (int h = 0; h < 2; ++h) fa[il][h] = *reinterpret_cast<const v4i*>(sa + ((aoff + il * 16 * BK) ^ (h << 6)));
+#pragma unroll
+        for (int in = 0; in < FN; ++in) sv[in] = *reinterpret_cast<const float4*>(sc + wn * 32 + 16 * in + 4 * fq);
 #pragma unroll
         for (int i = 0; i < 2; ++i)
             if (!(ABL & 2) && !W8) raw_read(s ^ 1, i, raw[i]);
         SCHED_FENCE();
         if (defer && g > 0) {   // the fold the previous iteration left over
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const float4 sp = *reinterpret_cast<const float4*>(sc_prev + wn * 32 + 8 * q + 4 * fhalf);
-                fold(2, q, sp);
-                fold(3, q, sp);
+            for (int in = 0; in < FN; ++in) {
+                const float4 sp = *reinterpret_cast<const float4*>(sc_prev + wn * 32 + 16 * in + 4 * fq);
+#pragma unroll
+                for (int il = 0; il < 4; ++il) fold(in, 4 + il, sp);
             }
             SCHED_FENCE();
         }
-        // The second pair's A fragments take over the registers of the first pair's as those are consumed.  DMA targets:
-        // the packed stage of group g (expanded during iteration g-1), the A stage of group g-1 and the scale stage of
-        // group g-2, all of them last read before the barrier that ended iteration g-1.
-        mma_pair(0, fa, [&](int i) {
-            na[i & 1][i >> 1] = *reinterpret_cast<const v4i*>(sa + aoff[i >> 1] + (2 + (i & 1)) * 32 * BK);
+        // The second half's A fragments are read while the first half is multiplied.  DMA targets: the packed stage of
+        // group g (expanded during iteration g-1) or the expanded stage of group g-1, the A stage of group g-1 and the scale
+        // stage of group g-2, all of them last read before the barrier that ended iteration g-1.
+        mma_half(0, fa, [&](int i) {
+            if (i < 8) na[i >> 1][i & 1] = *reinterpret_cast<const v4i*>(sa + ((aoff + (4 + (i >> 1)) * 16 * BK) ^ ((i & 1) << 6)));
             if (!(ABL & 4)) {
-                if (i == 1) dma_raw(g + 2, s, 0);
-                if (i == 3) dma_raw(g + 2, s, 1);
-                if (i == 5) dma_a(g + 2, a_new, 0);
-                if (i == 7) dma_a(g + 2, a_new, 1);
+                if (i == 2) dma_raw(g + 2, s, 0);
+                if (i == 6) dma_raw(g + 2, s, 1);
+                if (i == 10) dma_a(g + 2, a_new, 0);
+                if (i == 14) dma_a(g + 2, a_new, 1);
             }
             if (!(ABL & 2) && !W8) {
-                if (i == 2) unpack_write(s ^ 1, 0, raw[0]);
-                if (i == 4) unpack_write(s ^ 1, 1, raw[1]);
+                if (i == 4) unpack_write(s ^ 1, 0, raw[0]);
+                if (i == 8) unpack_write(s ^ 1, 1, raw[1]);
             }
         });
-        mma_pair(2, na, [&](int i) {
-            fold(i & 1, i >> 1, sv[i >> 1]);
+        mma_half(4, na, [&](int i) {
+            if (i & 1) fold((i >> 1) & 1, i >> 2, sv[(i >> 1) & 1]);   // the first half's eight tiles, one every other MFMA
             if (!(ABL & 4)) {
-                if (i == 1) dma_a(g + 2, a_new, 2);
-                if (i == 3) dma_a(g + 2, a_new, 3);
-                if (i == 5) dma_scales(g + 2, s_new);
+                if (i == 2) dma_a(g + 2, a_new, 2);
+                if (i == 6) dma_a(g + 2, a_new, 3);
+                if (i == 10) dma_scales(g + 2, s_new);
             }
         });
         if (!defer) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) fold(2 + (i & 1), i >> 1, sv[i >> 1]);
+            for (int in = 0; in < FN; ++in)
+#pragma unroll
+                for (int il = 0; il < 4; ++il) fold(in, 4 + il, sv[in]);
         }
 
         if (DUMP) {   // test hook: the exact int32 partials, [M, N, ng]
 #pragma unroll
-            for (int im = 0; im < TM; ++im)
+            for (int in = 0; in < FN; ++in)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int m = m0 + wm * 128 + im * 32 + frow;
-                    const int n = n0 + wn * 32 + 8 * (r >> 2) + 4 * fhalf + (r & 3);
-                    if (m < p.M && n < p.N) p.partials[((int64_t)m * p.N + n) * ng + g] = part[0][im][r];
-                }
+                for (int im = 0; im < FM; ++im)
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        const int m = m0 + wm * 128 + im * 16 + frow;
+                        const int n = n0 + wn * 32 + 16 * in + 4 * fq + c;
+                        if (m < p.M && n < p.N) p.partials[((int64_t)m * p.N + n) * ng + g] = part[in][im][c];
+                    }
             wait_all_dma();   // the dump's stores share the counter: drain it rather than count them
         }
         if (ABL & 4) wait_all_dma();
@@ -321,34 +320,34 @@ __global__ void __launch_bounds__(NT, 1) w6a8_group_gemm_kernel(W6Args p) {
     if (defer) {
         const float* sc_last = reinterpret_cast<const float*>(smem + S_BASE + ((s_cur + 3) & 3) * S_STAGE);
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const float4 sp = *reinterpret_cast<const float4*>(sc_last + wn * 32 + 8 * q + 4 * fhalf);
-            fold(2, q, sp);
-            fold(3, q, sp);
+        for (int in = 0; in < FN; ++in) {
+            const float4 sp = *reinterpret_cast<const float4*>(sc_last + wn * 32 + 16 * in + 4 * fq);
+#pragma unroll
+            for (int il = 0; il < 4; ++il) fold(in, 4 + il, sp);
         }
     }
     __syncthreads();   // every wave's DMA is drained before the epilogue reuses the stages
 
-    // Epilogue.  A lane holds one m and runs of four consecutive n, so storing straight from the registers would touch
-    // 32 rows per instruction.  When the rows of D are 16-byte aligned each wave instead passes its tile, 32 rows at a
-    // time, through a private 4 KB of LDS (16-byte chunks XOR-swizzled by row, conflict-free both ways) and writes whole
-    // row segments, 16 bytes per lane.
+    // Epilogue.  A lane holds one m per row tile and four consecutive n per column tile, so storing straight from the
+    // registers would touch 16 rows per instruction.  When the rows of D are 16-byte aligned each wave instead passes its
+    // tile, 32 rows at a time, through a private 4 KB of LDS (16-byte chunks XOR-swizzled by row) and writes whole row
+    // segments, 16 bytes per lane.
     constexpr int SZ = dt_size<OUT_DT>::value;
     const bool vec_ok = (p.N & 3) == 0 && ((uintptr_t)p.D & (4 * SZ - 1)) == 0 && ((uintptr_t)p.bias & (4 * SZ - 1)) == 0;
     const bool rows_ok = vec_ok && (((int64_t)p.N * SZ) & 15) == 0 && ((uintptr_t)p.D & 15) == 0;
     const int nb = n0 + wn * 32;
-    float bv[4][4];
+    float bv[FN][4];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        const int n = nb + 8 * q + 4 * fhalf;
+    for (int in = 0; in < FN; ++in) {
+        const int n = nb + 16 * in + 4 * fq;
 #pragma unroll
-        for (int c = 0; c < 4; ++c) bv[q][c] = 0.f;
+        for (int c = 0; c < 4; ++c) bv[in][c] = 0.f;
         if (p.bias && n < p.N) {
             if (vec_ok) {
-                load4<OUT_DT>(p.bias, n, bv[q]);
+                load4<OUT_DT>(p.bias, n, bv[in]);
             } else {
 #pragma unroll
-                for (int c = 0; c < 4; ++c) if (n + c < p.N) bv[q][c] = ld_dt<OUT_DT>(p.bias, n + c);
+                for (int c = 0; c < 4; ++c) if (n + c < p.N) bv[in][c] = ld_dt<OUT_DT>(p.bias, n + c);
             }
         }
     }
@@ -357,23 +356,27 @@ __global__ void __launch_bounds__(NT, 1) w6a8_group_gemm_kernel(W6Args p) {
         constexpr int RPI = 64 / CPR, NI = 32 / RPI;            // rows per store instruction, instructions per piece
         uint8_t* wl = smem + wave * 4096;                        // the stages are idle: the loop ended with a barrier
 #pragma unroll
-        for (int im = 0; im < TM; ++im) {
-            const int mb = m0 + wm * 128 + im * 32;
-            const float xs = p.xs[mb + frow < p.M ? mb + frow : p.M - 1];
+        for (int ip = 0; ip < FM / 2; ++ip) {                    // a piece: row tiles 2*ip and 2*ip + 1
+            const int mb = m0 + wm * 128 + ip * 32;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                float out[4];
+            for (int hm = 0; hm < 2; ++hm) {
+                const int prow = hm * 16 + frow;
+                const float xs = p.xs[mb + prow < p.M ? mb + prow : p.M - 1];
 #pragma unroll
-                for (int c = 0; c < 4; ++c) out[c] = __builtin_fmaf(accf[0][im][4 * q + c], xs, bv[q][c]);
-                const int byte = (8 * q + 4 * fhalf) * SZ;       // columns 8q + 4*fhalf .. +3 of row frow
-                uint8_t* dst = wl + frow * ROWB + ((((byte >> 4) ^ (frow & (CPR - 1))) << 4) | (byte & 15));
-                if (OUT_DT == DT_F32) {
-                    *reinterpret_cast<float4*>(dst) = make_float4(out[0], out[1], out[2], out[3]);
-                } else if (OUT_DT == DT_BF16) {
-                    *reinterpret_cast<uint2*>(dst) = make_uint2(pack_bf16x2(out[0], out[1]), pack_bf16x2(out[2], out[3]));
-                } else {
-                    *reinterpret_cast<uint2*>(dst) = make_uint2((uint32_t)f_to_f16(out[0]) | ((uint32_t)f_to_f16(out[1]) << 16),
-                                                                (uint32_t)f_to_f16(out[2]) | ((uint32_t)f_to_f16(out[3]) << 16));
+                for (int in = 0; in < FN; ++in) {
+                    float out[4];
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) out[c] = __builtin_fmaf(accf[in][2 * ip + hm][c], xs, bv[in][c]);
+                    const int byte = (16 * in + 4 * fq) * SZ;    // columns 16*in + 4*fq .. +3 of row prow
+                    uint8_t* dst = wl + prow * ROWB + ((((byte >> 4) ^ (prow & (CPR - 1))) << 4) | (byte & 15));
+                    if (OUT_DT == DT_F32) {
+                        *reinterpret_cast<float4*>(dst) = make_float4(out[0], out[1], out[2], out[3]);
+                    } else if (OUT_DT == DT_BF16) {
+                        *reinterpret_cast<uint2*>(dst) = make_uint2(pack_bf16x2(out[0], out[1]), pack_bf16x2(out[2], out[3]));
+                    } else {
+                        *reinterpret_cast<uint2*>(dst) = make_uint2((uint32_t)f_to_f16(out[0]) | ((uint32_t)f_to_f16(out[1]) << 16),
+                                                                    (uint32_t)f_to_f16(out[2]) | ((uint32_t)f_to_f16(out[3]) << 16));
+                    }
                 }
             }
             asm volatile("" ::: "memory");   // the wave's own LDS writes are ordered before its reads
@@ -388,20 +391,20 @@ __global__ void __launch_bounds__(NT, 1) w6a8_group_gemm_kernel(W6Args p) {
         }
         return;
     }
-    // fallback for unaligned rows: four consecutive n per lane and register group, straight from the accumulators
+    // fallback for unaligned rows: four consecutive n per lane and tile, straight from the accumulators
 #pragma unroll
-    for (int im = 0; im < TM; ++im) {
-        const int m = m0 + wm * 128 + im * 32 + frow;
+    for (int im = 0; im < FM; ++im) {
+        const int m = m0 + wm * 128 + im * 16 + frow;
         if (m >= p.M) continue;
         const float xs = p.xs[m];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const int n = nb + 8 * q + 4 * fhalf;
+        for (int in = 0; in < FN; ++in) {
+            const int n = nb + 16 * in + 4 * fq;
             if (n >= p.N) continue;
             const int64_t o = (int64_t)m * p.N + n;
             float out[4];
 #pragma unroll
-            for (int c = 0; c < 4; ++c) out[c] = __builtin_fmaf(accf[0][im][4 * q + c], xs, bv[q][c]);
+            for (int c = 0; c < 4; ++c) out[c] = __builtin_fmaf(accf[in][im][c], xs, bv[in][c]);
             if (vec_ok) {
                 store4<OUT_DT>(p.D, o, out);
             } else {
