@@ -395,7 +395,7 @@ def main():
         "config": {"workload": "image-DiT MLP up-projection W8A8 linear, bf16 activations M=%d K=%d -> N=%d, Hadamard "
                                "block %d, per-channel scales, bf16 bias and output" % (M, K, N, a.rotate),
                    "M": M, "K": K, "N": N, "rotate": a.rotate},
-        "roofline": {"bound": "mfma", "kernel": "int8_gemm_pp_kernel (gpu_int8_gemm, one launch: 256x256 tiles for the rows that fill whole rounds, 128x256 tiles for the rest)", "achieved": round(gemm_tops, 2),
+        "roofline": {"bound": "mfma", "kernel": "int8_gemm_pp_kernel (gpu_int8_gemm, one launch: 256x256 tiles for the rows that fill whole rounds, 128x256 tiles for the rest; v_mfma_i32_16x16x64_i8)", "achieved": round(gemm_tops, 2),
                      "peak": PEAK_INT8_TOPS, "unit": "TFLOP/s", "frac": round(gemm_tops / PEAK_INT8_TOPS, 4),
                      "traffic": traffic, "avg_launch_us": round(tg * 1e3, 2),
                      "algorithmic_ops": ops, "algorithmic_bytes": M * K + M * 4 + N * K + N * 4 + N * 2 + M * N * 2},
