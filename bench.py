@@ -85,6 +85,8 @@ def time_linear(torch, ffi, d, M, K, N, rotate, steps, warmup, nbuf=1, settled=T
     D = torch.empty((M, N), dtype=torch.bfloat16, device="cuda:0")
     Ws = [d["W"]] + [d["W"].clone() for _ in range(nbuf - 1)]
 
+    # Two events per step: one in front of the quantizer, one between the two launches; the event in front of the next
+    # step's quantizer (one more after the last step) closes the GEMM's interval.
     def step(i, evs=None):
         W = Ws[i % nbuf]
         if evs: evs[0].record(st)
@@ -93,22 +95,22 @@ def time_linear(torch, ffi, d, M, K, N, rotate, steps, warmup, nbuf=1, settled=T
         if evs: evs[1].record(st)
         ffi.k("gpu_int8_gemm", q.data_ptr(), W.data_ptr(), xs.data_ptr(), d["ws"].data_ptr(), d["bias"].data_ptr(),
               D.data_ptr(), M, N, K, ffi.DT_BF16, s)
-        if evs: evs[2].record(st)
 
     if settled:
         settle(torch, lambda: step(0))
     for i in range(warmup):
         step(i)
-    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(steps + 1)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(steps):
         step(i, evs[i])
+    evs[steps][0].record(st)
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
-    gpu_ms = evs[0][0].elapsed_time(evs[-1][2])
-    tq = sum(e[0].elapsed_time(e[1]) for e in evs) / steps
-    tg = sum(e[1].elapsed_time(e[2]) for e in evs) / steps
+    gpu_ms = evs[0][0].elapsed_time(evs[steps][0])
+    tq = sum(evs[i][0].elapsed_time(evs[i][1]) for i in range(steps)) / steps
+    tg = sum(evs[i][1].elapsed_time(evs[i + 1][0]) for i in range(steps)) / steps
     return max(gpu_ms, 0.0), wall_ms, tq, tg
 
 
