@@ -26,6 +26,48 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, 8 TB/s
 SETTLE_MS = 150.0         # untimed load before every timed loop, see settle()
 
 
+class StreamEvents:
+    """HIP timing events created with hipEventDisableSystemFence, recorded on the launch stream.  An event with the
+    default flags makes the command processor write back and invalidate the caches at system scope when it completes;
+    between two kernels that costs 1.5-2 us of the following kernel's interval each time.  The flag is the one the HIP
+    headers name for events that only measure time.  torch.cuda.Event has no way to pass it, so the three runtime calls
+    are made through ctypes on the HIP runtime the process has already loaded."""
+    DISABLE_SYSTEM_FENCE = 0x20000000
+
+    def __init__(self, n, stream):
+        import ctypes
+        self.c = ctypes
+        self.hip = ctypes.CDLL("libamdhip64.so")
+        self.hip.hipEventCreateWithFlags.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_uint]
+        self.hip.hipEventRecord.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+        self.hip.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
+        self.hip.hipEventDestroy.argtypes = [ctypes.c_void_p]
+        self.stream = ctypes.c_void_p(stream)
+        self.ev = []
+        for _ in range(n):
+            e = ctypes.c_void_p()
+            self._ok(self.hip.hipEventCreateWithFlags(ctypes.byref(e), self.DISABLE_SYSTEM_FENCE), "hipEventCreateWithFlags")
+            self.ev.append(e)
+
+    @staticmethod
+    def _ok(rc, what):
+        if rc != 0:
+            raise RuntimeError("%s failed with HIP error %d" % (what, rc))
+
+    def record(self, i):
+        self._ok(self.hip.hipEventRecord(self.ev[i], self.stream), "hipEventRecord")
+
+    def ms(self, i, j):
+        f = self.c.c_float()
+        self._ok(self.hip.hipEventElapsedTime(self.c.byref(f), self.ev[i], self.ev[j]), "hipEventElapsedTime")
+        return f.value
+
+    def close(self):
+        for e in self.ev:
+            self.hip.hipEventDestroy(e)
+        self.ev = []
+
+
 def settle(torch, fn, ms=SETTLE_MS):
     """Runs `fn` untimed for about `ms` milliseconds of GPU time.  After any idle gap (0.2 s is enough: host-side input
     generation between two measurements) the part's power management holds the shader clock down and lets it rise over
@@ -85,14 +127,14 @@ def time_linear(torch, ffi, d, M, K, N, rotate, steps, warmup, nbuf=1, settled=T
     D = torch.empty((M, N), dtype=torch.bfloat16, device="cuda:0")
     Ws = [d["W"]] + [d["W"].clone() for _ in range(nbuf - 1)]
 
-    # Two events per step: one in front of the quantizer, one between the two launches; the event in front of the next
-    # step's quantizer (one more after the last step) closes the GEMM's interval.
+    # Two events per step: one in front of the quantizer (event 2i), one between the two launches (2i+1); the event in
+    # front of the next step's quantizer (one more after the last step) closes the GEMM's interval.
     def step(i, evs=None):
         W = Ws[i % nbuf]
-        if evs: evs[0].record(st)
+        if evs: evs.record(2 * i)
         ffi.k("gpu_quant_rows", ffi.DT_BF16, ffi.PRO_PLAIN, d["x"].data_ptr(), K, 0, 0, 0, 0, 0.0, 0, 0, q.data_ptr(),
               xs.data_ptr(), M, K, rotate, s)
-        if evs: evs[1].record(st)
+        if evs: evs.record(2 * i + 1)
         ffi.k("gpu_int8_gemm", q.data_ptr(), W.data_ptr(), xs.data_ptr(), d["ws"].data_ptr(), d["bias"].data_ptr(),
               D.data_ptr(), M, N, K, ffi.DT_BF16, s)
 
@@ -100,17 +142,18 @@ def time_linear(torch, ffi, d, M, K, N, rotate, steps, warmup, nbuf=1, settled=T
         settle(torch, lambda: step(0))
     for i in range(warmup):
         step(i)
-    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(steps + 1)]
+    evs = StreamEvents(2 * steps + 1, s)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(steps):
-        step(i, evs[i])
-    evs[steps][0].record(st)
+        step(i, evs)
+    evs.record(2 * steps)
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
-    gpu_ms = evs[0][0].elapsed_time(evs[steps][0])
-    tq = sum(evs[i][0].elapsed_time(evs[i][1]) for i in range(steps)) / steps
-    tg = sum(evs[i][1].elapsed_time(evs[i + 1][0]) for i in range(steps)) / steps
+    gpu_ms = evs.ms(0, 2 * steps)
+    tq = sum(evs.ms(2 * i, 2 * i + 1) for i in range(steps)) / steps
+    tg = sum(evs.ms(2 * i + 1, 2 * i + 2) for i in range(steps)) / steps
+    evs.close()
     return max(gpu_ms, 0.0), wall_ms, tq, tg
 
 
