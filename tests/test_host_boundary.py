@@ -197,3 +197,33 @@ def test_makefile_and_build_script_list_the_same_units_and_flags():
     for src, extra in build.EXTRA.items():
         line = re.search(r"^csrc/%s\.o: FLAGS \+= (.+)$" % re.escape(src[:-4]), mk, re.M)
         assert line and line.group(1).split() == extra
+
+
+def test_rust_host_crate_follows_the_headers_and_the_build_script():
+    """rust/src/sys.rs is generated from the headers (same names, arity and scalar types as the ctypes table), and
+    rust/build.rs compiles the units and flags that build.py does.  No Rust toolchain is needed for either check."""
+    import importlib
+    import subprocess
+    import sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "rust", "gen_sys.py"), "--check"], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    text = open(os.path.join(ROOT, "rust", "src", "sys.rs")).read()
+    decls = {m.group(1): m.group(2) for m in re.finditer(r"pub fn (gpu_\w+)\(([^)]*)\)", text)}
+    assert set(decls) == set(header_functions()) | set(header_functions("gpu_blas_api.h"))
+    # c_uint64 and c_size_t are one ctypes class on this platform
+    kinds = {ffi._P: {"P", "PM"}, ffi._I64: {"i64"}, ffi._I32: {"i32"}, ffi._F32: {"f32"}, ffi._U64: {"u64", "usize"}}
+    for table in (ffi.SIGNATURES, ffi.BLAS_SIGNATURES):
+        for name, argtypes in table.items():
+            rust = [a.split(":")[1].strip() for a in " ".join(decls[name].split()).split(",") if a.strip()]
+            assert len(rust) == len(argtypes), name
+            for rt, ct in zip(rust, argtypes):
+                assert rt in kinds[ct], (name, rt, ct)
+    build = importlib.import_module("comfyui-backend-but-rust_amd.build")
+    rs = open(os.path.join(ROOT, "rust", "build.rs")).read()
+    units = re.findall(r'"(\w+\.hip)"', rs[rs.index("const UNITS"):rs.index("];")])
+    assert sorted(units) == sorted(build.SOURCES)
+    for flag in build.FLAGS:
+        if not flag.startswith("--offload-arch"):
+            assert '"%s"' % flag in rs, flag
+    for src, extra in build.EXTRA.items():
+        assert src in rs and all('"%s"' % e in rs for e in extra)
