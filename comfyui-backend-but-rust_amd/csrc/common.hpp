@@ -60,18 +60,34 @@ template <int DT> struct dt_size { static constexpr int value = DT == DT_F32 ? 4
 // Workgroup -> tile.  Workgroups are dealt round-robin to the 8 XCDs (each with its own L2), so first renumber them
 // XCD-contiguously, then walk tiles in panels of 4 tile rows so that the 32 workgroups an XCD runs at once cover a
 // 4 x 8 patch of tiles and share A rows / W rows in that XCD's L2.
-__device__ __forceinline__ void tile_of_block(int b, int nblocks, int tiles_m, int tiles_n, int& tm, int& tn) {
+// A persistent kernel calls this three times per tile (two operand streams and the epilogue), and two integer divisions
+// are about a hundred dependent scalar instructions each time, so the divisions are multiplications: `magic` =
+// panel_magic(tiles_m, tiles_n) from the host turns lin / (4 * tiles_n) into a multiply-high, and the rows of a panel
+// are 4, or 1..3 in the last one.  magic == 0 (shapes beyond the multiply's exact range) divides.
+__host__ __device__ inline uint32_t panel_magic(int tiles_m, int tiles_n) {
+    // floor(n / d) == (n * ceil(2^32 / d)) >> 32 for n, d <= 65536
+    const int64_t per_panel = 4 * (int64_t)tiles_n, ntiles = (int64_t)tiles_m * tiles_n;
+    if (per_panel > 65536 || ntiles > 65536) return 0;
+    return (uint32_t)(((1ull << 32) + (uint64_t)per_panel - 1) / (uint64_t)per_panel);
+}
+__device__ __forceinline__ void tile_of_block(int b, int nblocks, int tiles_m, int tiles_n, int& tm, int& tn, uint32_t magic = 0) {
     const int base = nblocks >> 3, rem = nblocks & 7;
     const int xcd = b & 7, idx = b >> 3;
     const int lin = xcd * base + (xcd < rem ? xcd : rem) + idx;
     constexpr int GM = 4;
     const int per_panel = GM * tiles_n;
-    const int panel = lin / per_panel;
+    const int panel = magic ? (int)__umulhi((uint32_t)lin, magic) : lin / per_panel;
     const int first_m = panel * GM;
     const int rows = tiles_m - first_m < GM ? tiles_m - first_m : GM;
     const int in_panel = lin - panel * per_panel;
-    tm = first_m + in_panel % rows;
-    tn = in_panel / rows;
+    int q;   // in_panel / rows
+    if (rows == 4) q = in_panel >> 2;
+    else if (rows == 2) q = in_panel >> 1;
+    else if (rows == 1) q = in_panel;
+    else if (magic) q = (int)__umulhi((uint32_t)in_panel, 0x55555556u);   // rows == 3, in_panel < 65536
+    else q = in_panel / rows;
+    tm = first_m + in_panel - q * rows;
+    tn = q;
 }
 
 

@@ -31,6 +31,7 @@ struct GemmArgs {
     void* D;
     int M, N, K;
     int tiles_m, tiles_n;
+    uint32_t magic;   // panel_magic(tiles_m, tiles_n), for tile_of_block
     int kslice;   // ring kernel only: K elements per split-K slice (a multiple of 128), 0 = no split
 };
 
@@ -407,7 +408,7 @@ __global__ void __launch_bounds__(C::NT, C::OCC) int8_gemm_kernel(GemmArgs p) {
     const int wm = wave / C::WGN, wn = wave % C::WGN;
 
     int tm, tn;
-    tile_of_block(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, tm, tn);
+    tile_of_block(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, tm, tn, p.magic);
     const int m0 = tm * BM, n0 = tn * BN;
     const int K = p.K;
 
@@ -625,7 +626,7 @@ __global__ void __launch_bounds__(C::NT, 1) int8_gemm_ring_kernel(GemmArgs p) {
 
     auto tile_origin = [&](int i, int& m0, int& n0) {
         int tm, tn;
-        tile_of_block((int)blockIdx.x + i * G, ntiles, p.tiles_m, p.tiles_n, tm, tn);
+        tile_of_block((int)blockIdx.x + i * G, ntiles, p.tiles_m, p.tiles_n, tm, tn, p.magic);
         m0 = tm * C::BM;
         n0 = tn * C::BN;
     };
@@ -855,7 +856,7 @@ __device__ __forceinline__ void pp_gemm_tiles(const GemmArgs& p, uint8_t* smem, 
     const int S = nt_b * nk;                             // steps of this workgroup
     auto tile_origin = [&](int i, int& m0, int& n0) {
         int tm, tn;
-        tile_of_block(bid + i * G, ntiles, p.tiles_m, p.tiles_n, tm, tn);
+        tile_of_block(bid + i * G, ntiles, p.tiles_m, p.tiles_n, tm, tn, p.magic);
         m0 = tm * C::BM;
         n0 = tn * C::BN;
     };
@@ -1070,7 +1071,7 @@ __global__ void __launch_bounds__(StreamCfg::NT, 1) int8_gemm_stream_kernel(Gemm
     const int nt_b = (ntiles - (int)blockIdx.x + G - 1) / G;   // tiles of this workgroup: blockIdx, blockIdx + G, ...
     auto tile_origin = [&](int i, int& m0, int& n0) {
         int tm, tn;
-        tile_of_block((int)blockIdx.x + i * G, ntiles, p.tiles_m, p.tiles_n, tm, tn);
+        tile_of_block((int)blockIdx.x + i * G, ntiles, p.tiles_m, p.tiles_n, tm, tn, p.magic);
         m0 = tm * C::BM;
         n0 = tn * C::BN;
     };
@@ -1305,6 +1306,7 @@ template <class C, int OUT_DT, int EPI>
 int launch_cfg(GemmArgs a, hipStream_t st) {
     a.tiles_m = (a.M + C::BM - 1) / C::BM;
     a.tiles_n = (a.N + C::BN - 1) / C::BN;
+    a.magic = panel_magic(a.tiles_m, a.tiles_n);
     const int64_t nblocks = (int64_t)a.tiles_m * a.tiles_n;
     if (nblocks > 0x7fffffff) return -1;
     auto kern = int8_gemm_kernel<C, OUT_DT, EPI>;
@@ -1337,6 +1339,7 @@ template <class C, int OUT_DT, int EPI>
 int launch_ring_cfg(GemmArgs a, int slices, hipStream_t st) {
     a.tiles_m = (a.M + C::BM - 1) / C::BM;
     a.tiles_n = (a.N + C::BN - 1) / C::BN;
+    a.magic = panel_magic(a.tiles_m, a.tiles_n);
     const int64_t ntiles = (int64_t)a.tiles_m * a.tiles_n;
     if (ntiles > 0x7fffffff) return -1;
     auto kern = int8_gemm_ring_kernel<C, OUT_DT, EPI>;
@@ -1402,6 +1405,8 @@ int launch_pp(GemmArgs a, hipStream_t st) {
     main.tiles_n = (int)tn;
     rest.tiles_m = (rest.M + PpS::BM - 1) / PpS::BM;
     rest.tiles_n = (int)tn;
+    main.magic = panel_magic(main.tiles_m, main.tiles_n);
+    rest.magic = panel_magic(rest.tiles_m, rest.tiles_n);
     const int g_main = (int)(n_main < G ? n_main : G), g_rest = (int)(n_rest < G ? n_rest : G);
     auto kern = int8_gemm_pp_kernel<OUT_DT, EPI>;
     static bool once = false;  // benign race: the attribute is idempotent
@@ -1480,6 +1485,7 @@ int launch_stream(GemmArgs a, int slices, hipStream_t st) {
     using C = StreamCfg;
     a.tiles_m = (a.M + C::BM - 1) / C::BM;
     a.tiles_n = (a.N + C::BN - 1) / C::BN;
+    a.magic = panel_magic(a.tiles_m, a.tiles_n);
     const int64_t ntiles = (int64_t)a.tiles_m * a.tiles_n;
     if (ntiles > 0x7fffffff) return -1;
     auto kern = int8_gemm_stream_kernel<OUT_DT, EPI>;
