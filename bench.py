@@ -24,6 +24,7 @@ sys.path.insert(0, ROOT)
 PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, 5.0 POP/s
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, 8 TB/s
 SETTLE_MS = 150.0         # untimed load before every timed loop, see settle()
+EVENT_KIND = [None]       # which kind of events the last time_linear() used
 
 
 class StreamEvents:
@@ -31,23 +32,37 @@ class StreamEvents:
     default flags makes the command processor write back and invalidate the caches at system scope when it completes;
     between two kernels that costs 1.5-2 us of the following kernel's interval each time.  The flag is the one the HIP
     headers name for events that only measure time.  torch.cuda.Event has no way to pass it, so the three runtime calls
-    are made through ctypes on the HIP runtime the process has already loaded."""
+    are made through ctypes on the HIP runtime the process has already loaded; if that runtime cannot be reached this
+    way, torch's default-flag events are used instead and `kind` says so."""
     DISABLE_SYSTEM_FENCE = 0x20000000
 
-    def __init__(self, n, stream):
-        import ctypes
-        self.c = ctypes
-        self.hip = ctypes.CDLL("libamdhip64.so")
-        self.hip.hipEventCreateWithFlags.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_uint]
-        self.hip.hipEventRecord.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
-        self.hip.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
-        self.hip.hipEventDestroy.argtypes = [ctypes.c_void_p]
-        self.stream = ctypes.c_void_p(stream)
+    def __init__(self, torch, n, stream):
+        self.kind = "hipEventDisableSystemFence"
         self.ev = []
-        for _ in range(n):
-            e = ctypes.c_void_p()
-            self._ok(self.hip.hipEventCreateWithFlags(ctypes.byref(e), self.DISABLE_SYSTEM_FENCE), "hipEventCreateWithFlags")
-            self.ev.append(e)
+        try:
+            import ctypes
+            self.c = ctypes
+            self.hip = ctypes.CDLL("libamdhip64.so")
+            self.hip.hipEventCreateWithFlags.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_uint]
+            self.hip.hipEventRecord.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+            self.hip.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
+            self.hip.hipEventDestroy.argtypes = [ctypes.c_void_p]
+            self.stream = ctypes.c_void_p(stream.cuda_stream)
+            for _ in range(n):
+                e = ctypes.c_void_p()
+                self._ok(self.hip.hipEventCreateWithFlags(ctypes.byref(e), self.DISABLE_SYSTEM_FENCE), "hipEventCreateWithFlags")
+                self.ev.append(e)
+            # one recorded pair must read back, or the runtime reached here is not the one torch launches on
+            self.record(0); self.record(1)
+            torch.cuda.synchronize()
+            self.ms(0, 1)
+        except (OSError, AttributeError, RuntimeError) as err:
+            print("bench.py: timing-only HIP events unavailable (%s); using torch's events" % err, file=sys.stderr)
+            self.close()
+            self.kind = "torch default flags"
+            self.hip = None
+            self.tstream = stream
+            self.ev = [torch.cuda.Event(enable_timing=True) for _ in range(n)]
 
     @staticmethod
     def _ok(rc, what):
@@ -55,16 +70,22 @@ class StreamEvents:
             raise RuntimeError("%s failed with HIP error %d" % (what, rc))
 
     def record(self, i):
-        self._ok(self.hip.hipEventRecord(self.ev[i], self.stream), "hipEventRecord")
+        if self.hip is None:
+            self.ev[i].record(self.tstream)
+        else:
+            self._ok(self.hip.hipEventRecord(self.ev[i], self.stream), "hipEventRecord")
 
     def ms(self, i, j):
+        if self.hip is None:
+            return self.ev[i].elapsed_time(self.ev[j])
         f = self.c.c_float()
         self._ok(self.hip.hipEventElapsedTime(self.c.byref(f), self.ev[i], self.ev[j]), "hipEventElapsedTime")
         return f.value
 
     def close(self):
-        for e in self.ev:
-            self.hip.hipEventDestroy(e)
+        if getattr(self, "hip", None) is not None:
+            for e in self.ev:
+                self.hip.hipEventDestroy(e)
         self.ev = []
 
 
@@ -142,7 +163,7 @@ def time_linear(torch, ffi, d, M, K, N, rotate, steps, warmup, nbuf=1, settled=T
         settle(torch, lambda: step(0))
     for i in range(warmup):
         step(i)
-    evs = StreamEvents(2 * steps + 1, s)
+    evs = StreamEvents(torch, 2 * steps + 1, st)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(steps):
@@ -153,6 +174,7 @@ def time_linear(torch, ffi, d, M, K, N, rotate, steps, warmup, nbuf=1, settled=T
     gpu_ms = evs.ms(0, 2 * steps)
     tq = sum(evs.ms(2 * i, 2 * i + 1) for i in range(steps)) / steps
     tg = sum(evs.ms(2 * i + 1, 2 * i + 2) for i in range(steps)) / steps
+    EVENT_KIND[0] = evs.kind
     evs.close()
     return max(gpu_ms, 0.0), wall_ms, tq, tg
 
@@ -436,7 +458,7 @@ def main():
         "metric": "W8A8 linear TOPS @M%d K%d N%d (quantize + int8 GEMM + dequant epilogue)" % (M, K, N),
         "value": round(value, 2), "unit": "TOPS", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "int8", "data": "synthetic", "settle_ms": SETTLE_MS,
+        "dtype": "int8", "data": "synthetic", "settle_ms": SETTLE_MS, "events": EVENT_KIND[0],
         "config": {"workload": "image-DiT MLP up-projection W8A8 linear, bf16 activations M=%d K=%d -> N=%d, Hadamard "
                                "block %d, per-channel scales, bf16 bias and output" % (M, K, N, a.rotate),
                    "M": M, "K": K, "N": N, "rotate": a.rotate},
