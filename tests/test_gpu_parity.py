@@ -1143,3 +1143,100 @@ def test_full_size_w6a8_group_gemm(name, M, K, N):
     assert np.array_equal(part.sum(axis=1), want_sum)
     rc, _, want_part = oracle.w6a8_group_gemm(A[r0:r0 + 4], packed, xs[r0:r0 + 4], sw, bias, BF16, want_partials=True)
     assert np.array_equal(part[:4].reshape(want_part.shape), want_part)
+
+
+# ------------------------------------------------------------------------------------------------ random shapes
+def _bits_of(x, dt):
+    return x.astype(np.float32) if dt == F32 else (oracle.bf16_bits(x) if dt == BF16 else oracle.f16_bits(x))
+
+
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_int8_gemm_random_shapes_bit_exact(seed):
+    """Forty shapes per seed drawn over the ranges that select every kernel family and every alignment class (skinny,
+    split K, K % 16 == 8, odd N, tails of every tile size), all three entry points, all output types."""
+    rng = np.random.default_rng(seed)
+    for it in range(40):
+        kind = int(rng.integers(0, 6))
+        if kind == 0:   M, N, K = int(rng.integers(1, 257)), int(rng.integers(1, 700)) * 8, int(rng.integers(1, 40)) * 128
+        elif kind == 1: M, N, K = int(rng.integers(257, 3000)), int(rng.integers(64, 500)) * 8, int(rng.integers(1, 12)) * 128
+        elif kind == 2: M, N, K = int(rng.integers(1, 1200)), int(rng.integers(1, 1500)), int(rng.integers(1, 80)) * 8
+        elif kind == 3: M, N, K = int(rng.integers(1500, 5200)), int(rng.integers(64, 640)) * 8, int(rng.integers(1, 5)) * 128
+        elif kind == 4: M, N, K = int(rng.integers(1, 600)), int(rng.integers(1, 300)) * 4, int(rng.integers(1, 60)) * 16
+        else:           M, N, K = int(rng.integers(200, 2600)), int(rng.integers(512, 3000)), int(rng.integers(2, 20)) * 64
+        while M * N * K > 2e9:
+            M = max(1, M // 2)
+        dt = [BF16, F16, F32][int(rng.integers(0, 3))]
+        with_bias = bool(rng.integers(0, 4))
+        say("gemm_random", seed, it, M, N, K, dt, with_bias)
+        A = rng.integers(-128, 128, (M, K), dtype=np.int8)
+        W = rng.integers(-128, 128, (N, K), dtype=np.int8)
+        xs = rng.uniform(0.005, 0.2, M).astype(np.float32)
+        ws = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+        bias = _bits_of(rng.normal(size=N).astype(np.float32) * np.float32(0.02), dt) if with_bias else None
+        rscale = _bits_of(rng.normal(size=N).astype(np.float32), dt)
+        resid = _bits_of(rng.normal(size=(M, N)).astype(np.float32), dt)
+        want = oracle.int8_gemm_acc(A, W)
+        Ad, Wd = dev(A), dev(W)
+        bd = dev_bits(bias, dt) if with_bias else None
+        got = ql.int8_gemm_acc(Ad, Wd)
+        d = ql.int8_gemm(Ad, Wd, dev(xs), dev(ws), bd, TDT[dt])
+        r = ql.int8_gemm_residual(Ad, Wd, dev(xs), dev(ws), bd, dev_bits(rscale, dt), dev_bits(resid, dt))
+        torch.cuda.synchronize()
+        assert np.array_equal(got.cpu().numpy(), want), (M, N, K)
+        assert np.array_equal(host_bits(d), oracle.epilogue(want, xs, ws, bias, dt, fma=1)), (M, N, K, dt)
+        assert np.array_equal(host_bits(r), oracle.epilogue_residual(want, xs, ws, bias, rscale, resid, dt, fma=1)), (M, N, K, dt)
+
+
+@pytest.mark.parametrize("seed", [21, 22])
+def test_quant_rows_random_shapes_and_data_bit_exact(seed):
+    """150 draws per seed over dtype (bf16, f32, the SD fp16 quantizer), row length up to 32768, every rotation width, row
+    strides wider than K, and data that is Gaussian, heavy-tailed, scaled by 1e-30 .. 1e30, mostly zero, or carries an
+    infinity, a NaN, 3e38 or 1e-38."""
+    rng = np.random.default_rng(seed)
+
+    def data(M, width):
+        k = int(rng.integers(0, 5))
+        if k == 0:
+            x = rng.normal(size=(M, width)).astype(np.float32)
+        elif k == 1:
+            x = (rng.standard_t(3, size=(M, width)) * 4).astype(np.float32)
+        elif k == 2:
+            x = (rng.normal(size=(M, width)) * 10.0 ** int(rng.integers(-30, 30))).astype(np.float32)
+        elif k == 3:
+            x = rng.normal(size=(M, width)).astype(np.float32)
+            x[rng.random((M, width)) < 0.7] = 0
+        else:
+            x = rng.normal(size=(M, width)).astype(np.float32)
+            x[int(rng.integers(0, M)), int(rng.integers(0, width))] = [np.inf, -np.inf, np.nan, 3e38, 1e-38][int(rng.integers(0, 5))]
+        if M > 1 and rng.random() < 0.3:
+            x[int(rng.integers(0, M))] = 0
+        return x
+
+    for it in range(150):
+        which = int(rng.integers(0, 3))
+        rotate = int([0, 1, 64, 128, 256][int(rng.integers(0, 5))])
+        if which == 2:   # gpu_sd_quant_rows takes 0, 64 or 256
+            rotate = {128: 64, 1: 256}.get(rotate, rotate)
+        gran = 256 if rotate in (1, 256) else 128 if rotate == 128 else 64
+        K = int(rng.integers(1, 32768 // gran + 1)) * gran
+        if rng.random() < 0.7:
+            K = int(rng.integers(1, max(2, 6144 // gran))) * gran
+        M = int(rng.integers(1, 70))
+        stride = K if (which == 2 or rng.random() < 0.6) else K + 8 * int(rng.integers(1, 40))
+        say("quant_random", seed, it, which, M, K, stride, rotate)
+        x = data(M, stride)
+        if which == 0:
+            xb = oracle.bf16_bits(x)
+            rc, q, s = oracle.quant_rows(BF16, xb, K, rotate, x_stride=stride)
+            qd, sd = ql.quant_rows(dev_bits(xb, BF16), rotate, K=K)
+        elif which == 1:
+            rc, q, s = oracle.quant_rows(F32, x, K, rotate, x_stride=stride)
+            qd, sd = ql.quant_rows(dev(x), rotate, K=K)
+        else:
+            xb = oracle.f16_bits(np.clip(x, -6e4, 6e4))
+            rc, q, s = oracle.sd_quant_rows(xb, K, rotate)
+            qd, sd = ql.sd_quant_rows(dev_bits(xb, F16), rotate)
+        torch.cuda.synchronize()
+        assert rc == 0
+        assert np.array_equal(sd.cpu().numpy().view(np.uint32), s.view(np.uint32)), (which, M, K, stride, rotate)
+        assert np.array_equal(qd.cpu().numpy(), q), (which, M, K, stride, rotate)
