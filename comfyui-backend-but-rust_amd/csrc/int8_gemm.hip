@@ -138,13 +138,15 @@ __device__ __forceinline__ void epilogue_store(const GemmArgs& p, v16i (&acc)[TN
 // holds z = Out(acc*xs*ws + bias), exactly the intermediate the reference rounds, and fma(z, rscale, resid) is applied
 // on the way out.  Needs row starts of D (and resid) 16-byte aligned; the caller falls back to epilogue_store otherwise.
 // STAGED: the per-column constants (ws and bias as floats, 2 x 32*TN values) are kept in the wave's LDS area `cst` and
-// read back per piece, instead of 96 registers that a persistent kernel cannot spare next to its pipeline state.
+// read back per piece, instead of 96 registers that a persistent kernel cannot spare next to its pipeline state.  1: this
+// function loads them into `cst` first; 2: the caller has put them there (stage_columns, long before, so that their
+// trip from memory is off the epilogue's path), and `xs_lds`, when given, holds the tile's row scales the same way.
 // L: the MFMA shape the accumulators come from.  32: v16i acc[TN][TM], a lane holds row lane % 32 of a 32x32 tile and
 // the columns 8*rb + 4*(lane / 32) + j.  16: v4i acc[2*TN][2*TM] of 16x16 tiles, a lane holds row lane % 16 and the
 // columns 4*(lane / 16) + j; the 32x32 block (in, im) is then the four tiles (2*in + rb, 2*im + hm).
-template <int TM, int TN, int OUT_DT, int EPI, int PW = TN * 32, bool UNTRACKED = false, bool STAGED = false, int L = 32, class Acc>
+template <int TM, int TN, int OUT_DT, int EPI, int PW = TN * 32, bool UNTRACKED = false, int STAGED = 0, int L = 32, class Acc>
 __device__ __forceinline__ void epilogue_shuffle(const GemmArgs& p, Acc& acc, int mb, int nb, int lane, uint8_t* wl,
-                                                 uint8_t* wl2 = nullptr, float* cst = nullptr) {
+                                                 uint8_t* wl2 = nullptr, float* cst = nullptr, const float* xs_lds = nullptr) {
     // a piece is 32 rows x PW columns of the wave tile: PW*SZ bytes per LDS row, 32*PW*SZ bytes per wave
     constexpr int SZ = (EPI == EPI_ACC || OUT_DT == DT_F32) ? 4 : 2;
     constexpr int WTN = TN * 32, NP = WTN / PW, TNP = PW / 32;
@@ -171,7 +173,7 @@ __device__ __forceinline__ void epilogue_shuffle(const GemmArgs& p, Acc& acc, in
     constexpr int BW = SZ == 4 ? 4 : 2;            // 32-bit words holding 4 bias values
     float wsr[STAGED ? 1 : TN][NRB][4];
     uint32_t braw[STAGED ? 1 : TN][NRB][BW];
-    if (EPI != EPI_ACC && STAGED) {
+    if (EPI != EPI_ACC && STAGED == 1) {
         // two columns per lane and pass
 #pragma unroll
         for (int c0 = 0; c0 < WTN; c0 += 128) {
@@ -230,7 +232,8 @@ __device__ __forceinline__ void epilogue_shuffle(const GemmArgs& p, Acc& acc, in
 #pragma unroll
         for (int hm = 0; hm < NHM; ++hm) {
             const int mrow = mb + im * 32 + hm * 16 + frow;
-            xsr[im][hm] = (EPI == EPI_ACC || mrow >= p.M) ? 0.f : p.xs[mrow];
+            if (xs_lds) xsr[im][hm] = EPI == EPI_ACC ? 0.f : xs_lds[im * 32 + hm * 16 + frow];
+            else xsr[im][hm] = (EPI == EPI_ACC || mrow >= p.M) ? 0.f : p.xs[mrow];
         }
     float rs[NP][EPC];
     if (EPI == EPI_RESID) {
@@ -1024,43 +1027,50 @@ __global__ void __launch_bounds__(PpL::NT, 1) int8_gemm_pp_kernel(GemmArgs main,
 
 // ---------------------------------------------------------------------------------------------------------------
 // Weight-streaming kernel for skinny M (M <= 256): one row of 256 x 96 tiles, every weight read from HBM exactly once.
-// An iteration of such a tile is short (24 MFMAs per wave, 768 cycles) against the 44 KB that feed it, and a DMA
-// instruction that hits the L2 keeps its wave busy for about 68 cycles: a wave that multiplies cannot also fetch.
-// The roles are split over twelve waves, three per SIMD:
-//   waves 0-3   multiply (64 x 96 each, MFMA + fragment reads only, no memory instruction in their K loop);
-//   waves 4-5   stream W: 6 loads of 1 KB per K tile each into registers, NPW K tiles ahead, and 6 LDS stores of the
-//               K tile that is multiplied next into a ring of two stages;
-//   waves 6-11  stream A (from L2: all CUs read the same 256 rows) by DMA into four LDS stages, three K tiles ahead,
-//               5-6 instructions per K tile each.
-// A CU's loads return in issue order, so A's lines wait behind W loads that went to HBM: A needs the lead of an HBM
-// access, and W's flight time is spent in registers of waves that hold nothing else, which leaves the LDS to A.
-// With three A waves (and eight waves in all) the A stream needed 11 x 68 cycles an iteration and set the pace; six keep
-// it near 400.  The price is the register budget of three waves per SIMD (168), which the multiplying waves meet by
-// keeping the epilogue's column constants in LDS.
-// Everybody meets at two barriers per iteration, X (the stage of iteration g-1 is free) and Y (what iteration g+1 needs
-// has landed; the MFMA waves run three sub-steps before it and one after).  An A wave splits its instructions
-// between the two phases roughly in the proportion of the MFMA waves' work.
-// Requires K % 128 == 0 and M*K, N*K < 2^32.
+// Eight waves form two groups of four (one wave of each group per SIMD), and group g multiplies the K tiles
+// t = g, g + 2, ... of the workgroup's K range, all 256 x 96 outputs of them (wave tile 64 x 96, 4 x 6 tiles of
+// v_mfma_i32_16x16x64_i8), into accumulators of its own.  The groups alternate between two kinds of phase, with one
+// workgroup barrier per phase:
+//   compute: the 48 MFMAs of the group's K tile; the six W fragments of the second 64 K bytes are read behind the
+//            first MFMAs, and the wave's three DMA instructions of W follow the last one;
+//   memory:  the other 14 fragment reads of the group's next K tile with the wave's eight DMA instructions of A spread
+//            between them.
+// A group fetches only the K tiles it multiplies itself, so every wait for data is a wait of a wave on its own memory
+// counter, placed at the end of its compute phase.
+//
+// LDS: A in three stages of 32 KB, W in five of 12 KB (K tile t sits in stage t % 3 and t % 5), 2 KB of constants for the
+// epilogue.  In its memory phase before K tile t a group fetches A(t+2) into the stage of K tile t-1, whose fragments
+// the other group read a phase earlier; after multiplying K tile t it fetches W(t+4) into the W stage of K tile t-1,
+// whose second half the other group read during that earlier phase.  W, which comes from HBM, has three phases to land;
+// A, which comes from L2 behind it in the CU's in-order return path, has one and a half.
+//
+// What bounds this tile is how much a CU can keep in flight: 44 KB enter it per K tile, a third of them at HBM's
+// latency, and a kernel of any structure built on this tile (separate loader waves in lock step or free-running on LDS
+// counters, loads in registers instead of DMA) ran its K tile in the same 1350-1450 cycles.
+//
+// At the end the two groups swap halves of their accumulators through the LDS (the ring is dead by then) and each
+// finishes 32 of a wave tile's 64 rows; the tile's column constants and row scales were requested at the start and wait
+// in LDS.  Requires K % 128 == 0 and M*K, N*K < 2^32.
 // ---------------------------------------------------------------------------------------------------------------
-struct StreamCfg {
-    static constexpr int BM = 256, BN = 96, BK = 128, NSA = 4, NSW = 2, NPW = 5;
-    static constexpr int NWW = 2, NAW = 6, NT = 64 * (4 + NWW + NAW);   // W-stream waves, A-stream waves
-    static constexpr int WTM = 64, WTN = 96, TM = 2, TN = 3, NM = TM * TN, NF = TM + TN;
-    static constexpr int A_STAGE = BM * BK, W_STAGE = BN * BK, W_BASE = NSA * A_STAGE, SMEM = W_BASE + NSW * W_STAGE;
-    static constexpr int A_BLK = BM / 8, W_BLK = BN / 8;    // 1 KB DMA blocks (8 rows) per stage
-    static constexpr int A_PER = (A_BLK + NAW - 1) / NAW;   // per A wave: blocks ap, ap + NAW, ...
-    static constexpr int W_PER = W_BLK / NWW;               // per W wave: blocks wp, wp + NWW, ...
-    static_assert(W_BLK % NWW == 0 && NWW % 2 == 0, "whole blocks per W wave; block parity = wave parity for the swizzle");
-    static_assert(SMEM <= 160 * 1024 && A_PER * NAW - A_BLK < NAW, "LDS budget; an A wave has A_PER blocks or one fewer");
+struct TurnCfg {
+    static constexpr int BM = 256, BN = 96, BK = 128, NSA = 3, NSW = 5, NT = 512;
+    static constexpr int TM = 2, TN = 3;                                       // wave tile 64 x 96 as 32 x 32 blocks
+    static constexpr int A_STAGE = BM * BK, W_STAGE = BN * BK, W_BASE = NSA * A_STAGE;
+    static constexpr int NLA = BM / 32, NLW = BN / 32;                         // DMA instructions (8 rows each) per wave and K tile
+    static constexpr int RING = W_BASE + NSW * W_STAGE;
+    static constexpr int CST_BASE = RING, CST_FLOATS = 2 * BN + BM, SMEM = RING + 2048;   // ws[96], bias[96], xs[256] as floats
+    static constexpr int HALF_ACC = 2 * TM * TN * 1024;                        // half of one wave's accumulators
+    static_assert(SMEM <= 160 * 1024 && CST_FLOATS * 4 <= 2048, "LDS budget");
+    static_assert(8 * HALF_ACC <= W_BASE && 8 * 4096 <= NSW * W_STAGE, "hand-over area and epilogue scratch fit the dead ring");
 };
 
 template <int OUT_DT, int EPI>
-__global__ void __launch_bounds__(StreamCfg::NT, 1) int8_gemm_stream_kernel(GemmArgs p) {
-    using C = StreamCfg;
+__global__ void __launch_bounds__(TurnCfg::NT, 1) int8_gemm_turn_kernel(GemmArgs p) {
+    using C = TurnCfg;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    constexpr int BK = C::BK, TM = C::TM, TN = C::TN;
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    constexpr int BK = C::BK, TM = C::TM, TN = C::TN, FM = 2 * TM, FN = 2 * TN;
+    const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+    const int grp = wave >> 2, wq = wave & 3;   // group; wave within the group = its 64-row quarter and its DMA blocks
     const int ld = p.K;
     // split K: workgroup row blockIdx.y multiplies K slice [k_lo, k_lo + nk*128) and writes its own int32 plane
     const int k_lo = p.kslice ? (int)blockIdx.y * p.kslice : 0;
@@ -1069,206 +1079,242 @@ __global__ void __launch_bounds__(StreamCfg::NT, 1) int8_gemm_stream_kernel(Gemm
     if (p.kslice) p.D = (uint8_t*)p.D + (int64_t)blockIdx.y * p.M * p.N * 4;
     const int G = gridDim.x, ntiles = p.tiles_m * p.tiles_n;
     const int nt_b = (ntiles - (int)blockIdx.x + G - 1) / G;   // tiles of this workgroup: blockIdx, blockIdx + G, ...
-    auto tile_origin = [&](int i, int& m0, int& n0) {
-        int tm, tn;
-        tile_of_block((int)blockIdx.x + i * G, ntiles, p.tiles_m, p.tiles_n, tm, tn, p.magic);
-        m0 = tm * C::BM;
-        n0 = tn * C::BN;
-    };
-    // The K tiles of a slice are walked from a start that differs between the workgroups of an XCD (the int32 sums do
-    // not depend on the order): otherwise all 32 of them ask that XCD's L2 for the same 256 lines of A at the same
-    // moment, and every weight stream sits at the same offset inside its 4 KB-apart rows.
+    // The K tiles are walked from a start that differs between the workgroups of an XCD (the int32 sums do not depend
+    // on the order), so that they do not all ask that XCD's L2 for the same lines of A at the same moment.
     const int rot = (int)(((blockIdx.x >> 3) & 31) * (unsigned)nk) >> 5;
-    auto rk = [&](int kt) { return kt + rot < nk ? kt + rot : kt + rot - nk; };
+    auto rk = [&](int kt) { kt = kt < nk ? kt : nk - 1; return kt + rot < nk ? kt + rot : kt + rot - nk; };
     const uint32_t lds_base = (uint32_t)(uintptr_t)smem;
-    const int lrow = lane >> 3;
     auto dma = [&](uint32_t dst, uint32_t off, const int8_t* base) {
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(off), "s"(base) : "memory", "m0");
     };
-    if (wave >= 4 && wave < 4 + C::NWW) {
-        // ---- the W stream: wave 4 + wp takes blocks wp, wp + NWW, ...  Block j is rows 8j..8j+7 of the tile; chunk
-        // swizzle (bits 1..3 of the row) on the global side.  The loads land in registers, NPW K tiles ahead of the
-        // multiply, and move into the LDS stage of K tile g+1 during iteration g: HBM latency is covered by registers
-        // of waves that have nothing else to hold, and LDS keeps its room for A.
-        const int wp = wave - 4;
-        uint32_t gw[C::W_PER];
-        v4i wr[C::NPW][C::W_PER];
-        int w_tile = 0, w_kt = 0;
-        auto set_w = [&](int i) {
-            int m0, n0;
-            tile_origin(i, m0, n0);
-#pragma unroll
-            for (int j = 0; j < C::W_PER; ++j) {
-                const int row = (wp + C::NWW * j) * 8 + lrow;
-                const int gr = n0 + row < p.N ? n0 + row : p.N - 1;
-                gw[j] = (uint32_t)gr * (uint32_t)ld + (((lane & 7) ^ (((wp & 1) << 2) | (lrow >> 1))) << 4);
-            }
-        };
-        // the stream's current K tile into register slot S, then on to the next K tile (the stream stops on its last K
-        // tile and keeps re-fetching it)
-        auto load_w = [&](auto S) {
-            const int8_t* base = p.W + k_lo + (int64_t)rk(w_kt) * BK;
-#pragma unroll
-            for (int j = 0; j < C::W_PER; ++j) wr[decltype(S)::value][j] = *reinterpret_cast<const v4i*>(base + gw[j]);
-            if (w_tile == nt_b - 1 && w_kt == nk - 1) return;
-            if (++w_kt == nk) { w_kt = 0; set_w(++w_tile); }
-        };
-        auto store_w = [&](auto S, int stage) {
-            uint8_t* dst = smem + C::W_BASE + stage * C::W_STAGE + wp * 1024 + lane * 16;
-#pragma unroll
-            for (int j = 0; j < C::W_PER; ++j) *reinterpret_cast<v4i*>(dst + C::NWW * j * 1024) = wr[decltype(S)::value][j];
-        };
-        set_w(0);
-        load_w(ic<0>{});
-        store_w(ic<0>{}, 0);                                      // W(0)
-        static_for<C::NPW>([&](auto I) { load_w(ic<(decltype(I)::value + 1) % C::NPW>{}); });   // W(1) .. W(NPW)
-        wait_lgkmcnt0();
-        wg_barrier();
-        int stage = 1, kt = 0;
-        // iteration g, g = S mod NPW: K tile g+1 leaves slot (S+1) mod NPW for LDS, K tile g+1+NPW takes the slot
-        auto iteration = [&](auto S) {
-            constexpr int SLOT = (decltype(S)::value + 1) % C::NPW;
-            wg_barrier();                                         // X: the stage of iteration g-1 is free
-            store_w(ic<SLOT>{}, stage);
-            load_w(ic<SLOT>{});
-            wait_lgkmcnt0();
-            wg_barrier();                                         // Y
-            stage = stage == C::NSW - 1 ? 0 : stage + 1;
-            if (++kt == nk) { kt = 0; wg_barrier(); }             // in front of the epilogue
-        };
-        const int total = nt_b * nk;
-        int g = 0;
-        for (; g + C::NPW <= total; g += C::NPW) static_for<C::NPW>([&](auto I) { iteration(I); });
-        static_for<C::NPW>([&](auto I) { if (g + decltype(I)::value < total) iteration(I); });
-        return;
-    }
-    if (wave >= 4 + C::NWW) {
-        // ---- the A stream: wave 4 + NWW + ap takes blocks ap, ap + NAW, ... (A_PER of them, or one fewer), NSA - 1 K
-        // tiles ahead.  A's lines come from L2, but a CU's loads return in issue order, behind the W loads that went to
-        // HBM: the lead in K tiles times the iteration time has to cover HBM's latency, not L2's.
-        const int ap = wave - 4 - C::NWW;
-        uint32_t ga[C::A_PER];
-        int a_tile = 0, a_kt = 0, a_stage = 0;
-        auto set_a = [&](int i) {
-            int m0, n0;
-            tile_origin(i, m0, n0);
-#pragma unroll
-            for (int j = 0; j < C::A_PER; ++j) {
-                const int b = ap + C::NAW * j;
-                const int row = (b < C::A_BLK ? b : C::A_BLK - 1) * 8 + lrow;
-                const int gr = m0 + row < p.M ? m0 + row : p.M - 1;
-                ga[j] = (uint32_t)gr * (uint32_t)ld + (((lane & 7) ^ (((b & 1) << 2) | (lrow >> 1))) << 4);
-            }
-        };
-        auto fetch_a = [&](int j0, int j1) {
-            const int8_t* base = p.A + k_lo + (int64_t)rk(a_kt) * BK;
-#pragma unroll
-            for (int j = 0; j < C::A_PER; ++j)
-                if (j >= j0 && j < j1) dma(lds_base + a_stage * C::A_STAGE + (ap + C::NAW * j) * 1024, ga[j], base);
-        };
-        auto next_a = [&]() {
-            a_stage = a_stage == C::NSA - 1 ? 0 : a_stage + 1;
-            if (a_tile == nt_b - 1 && a_kt == nk - 1) return;
-            if (++a_kt == nk) { a_kt = 0; set_a(++a_tile); }
-        };
-        // PER: DMA instructions of this wave per K tile (the wait counts below are exact only for the wave's own count)
-        auto stream_a = [&](auto PER_) {
-            constexpr int PER = decltype(PER_)::value, EARLY = (3 * PER + 3) / 4;   // EARLY are issued before barrier Y
-            static_assert((C::NSA - 2) * PER + EARLY <= 63, "wait counts are 6-bit fields");
-            set_a(0);
-#pragma unroll
-            for (int i = 0; i < C::NSA - 1; ++i) { fetch_a(0, PER); next_a(); }   // A(0) .. A(NSA-2)
-            wait_vmcnt<(C::NSA - 2) * PER>();                                     // A(0) has landed
-            wg_barrier();
-            for (int ti = 0; ti < nt_b; ++ti) {
-                for (int kt = 0; kt < nk; ++kt) {
-                    wg_barrier();                                     // X: the stage of iteration g-1 is free
-                    fetch_a(0, EARLY);                                // A(g + NSA - 1), first part
-                    wait_vmcnt<(C::NSA - 3) * PER + EARLY>();         // A(g + 1) has landed
-                    wg_barrier();                                     // Y
-                    fetch_a(EARLY, PER);
-                    next_a();
-                }
-                wg_barrier();                                         // in front of the epilogue
-            }
-            wait_vmcnt<0>();   // no DMA may still be writing this workgroup's LDS when it retires
-        };
-        if (ap + C::NAW * (C::A_PER - 1) < C::A_BLK) stream_a(ic<C::A_PER>{});
-        else stream_a(ic<C::A_PER - 1>{});
-        return;
-    }
 
-    // ---- the four MFMA waves: wave w multiplies rows 64w..64w+63 of the tile by all 96 columns, with
-    // v_mfma_i32_16x16x64_i8 (4 x 6 tiles of 16 x 16; see the two-group kernel for why this form).  A K tile is two halves
-    // of 64; a half is six slots of four MFMAs that share one W fragment.  Fragments live in 40 registers: the A
-    // fragments of the current half and of the next one, and three rotating W fragments read two slots ahead.
-    const int wm = wave;
-    const int frow = lane & 15, fq = lane >> 4;
-    const int fx = frow * BK + ((fq ^ ((frow >> 1) & 7)) << 4);   // row r at r*128, chunk c at slot c ^ ((r>>1)&7)
-    const int aoff = wm * C::WTM * BK + fx;
-    constexpr int FM = 2 * TM, FN = 2 * TN;   // 4 x 6 tiles of 16 x 16
-    auto a_frag = [&](const uint8_t* sa, int h, int j) -> v4i { return *reinterpret_cast<const v4i*>(sa + ((aoff + j * 16 * BK) ^ (h << 6))); };
-    auto w_frag = [&](const uint8_t* sw, int h, int in) -> v4i { return *reinterpret_cast<const v4i*>(sw + ((fx + in * 16 * BK) ^ (h << 6))); };
-    v4i acc[FN][FM];
-    v4i fa[2][FM], fw[3];
-    wg_barrier();   // A(0) and W(0) have landed
-    auto first_frags = [&](const uint8_t* sa, const uint8_t* sw) {
+    // DMA streams of this wave: 8-row blocks wq, wq + 4, ... of the A tile and of the W tile, of this group's K tiles.
+    // The chunk swizzle (bits 1..3 of the row) is applied on the global side; a block's parity is the wave's.
+    // (Giving W to one wave of the group and A to the other three, so that no wave's A loads queue behind its own W
+    // loads, was measured and is slower: what A waits behind is the CU's return path, not the wave's counter.)
+    uint32_t ga[C::NLA], gw[C::NLW];
+    auto set_rows = [&](int m0, int n0) {
+        const int l = hw_lane();
+        const int lr = l >> 3, lc = ((l & 7) ^ (((wq & 1) << 2) | (lr >> 1))) * 16;
 #pragma unroll
-        for (int j = 0; j < FM; ++j) fa[0][j] = a_frag(sa, 0, j);
-        fw[0] = w_frag(sw, 0, 0);
-        fw[1] = w_frag(sw, 0, 1);
+        for (int j = 0; j < C::NLA; ++j) {
+            const int row = m0 + (wq + 4 * j) * 8 + lr;
+            ga[j] = (uint32_t)(row < p.M ? row : p.M - 1) * (uint32_t)ld + lc;
+        }
+#pragma unroll
+        for (int j = 0; j < C::NLW; ++j) {
+            const int row = n0 + (wq + 4 * j) * 8 + lr;
+            gw[j] = (uint32_t)(row < p.N ? row : p.N - 1) * (uint32_t)ld + lc;
+        }
     };
-    first_frags(smem, smem + C::W_BASE);
-    int ca = 0, cw = 0;   // stages of the iteration being multiplied
+    // K tile and stage each stream fetches next (a stream past the last K tile re-fetches it, into a stage that nothing
+    // reads again: the number of instructions per phase, which the wait counts assume, stays fixed)
+    int a_t, a_st, w_t, w_st, r_sa, r_sw;
+    // source and destination of the A blocks a memory phase fetches
+    const int8_t* base_a;
+    uint32_t dst_a;
+    auto fetch_one = [&](auto D) { dma(dst_a + decltype(D)::value * 4096, ga[decltype(D)::value], base_a); };
+    auto fetch_w = [&]() {
+        const int8_t* base = p.W + k_lo + (int64_t)rk(w_t) * BK;
+        const uint32_t dst = lds_base + C::W_BASE + w_st * C::W_STAGE + wq * 1024;
+#pragma unroll
+        for (int j = 0; j < C::NLW; ++j) dma(dst + j * 4096, gw[j], base);
+        w_t += 2;
+        w_st = w_st >= 3 ? w_st - 3 : w_st + 2;
+    };
+    auto fetch_a = [&]() {
+        const int8_t* base = p.A + k_lo + (int64_t)rk(a_t) * BK;
+        const uint32_t dst = lds_base + a_st * C::A_STAGE + wq * 1024;
+#pragma unroll
+        for (int j = 0; j < C::NLA; ++j) dma(dst + j * 4096, ga[j], base);
+        a_t += 2;
+        a_st = a_st == 0 ? 2 : a_st - 1;
+    };
+
+    // Fragments: row r of a stage at r*128, chunk c at slot c ^ ((r>>1)&7); a lane reads row lane % 16, chunk
+    // 4*kk + lane / 16 of K half kk (which flips bit 6 of the address).
+    v4i acc[FN][FM];
+    v4i f[2][FM + FN];
+    // The memory phase: 14 fragment reads of the group's next K tile (all of A, and W for the first 64 K bytes) with the
+    // wave's 8 DMA instructions of A spread between them.  The six W fragments of the second 64 K bytes are read in the
+    // compute phase, behind the first MFMAs, and the three DMA instructions of W follow the last MFMA: a compute phase
+    // (768 cycles of MFMA) would otherwise be a third shorter than the memory phase beside it, whose reads return at the
+    // SIMD's pace of about 25 cycles each and whose DMA instructions hold the wave about 50 cycles each.  W can move
+    // because its ring has the room (a stage stays readable for one phase more), A cannot.
+    const uint8_t* sw_cur = smem;   // W stage of the K tile whose fragments are in registers (its second half still in LDS)
+    int fx = 0;
+    auto memory = [&]() {
+        constexpr int ND = C::NLA;
+        const int l = hw_lane();
+        const int frow = l & 15, fq = l >> 4;
+        const int x = frow * BK + ((fq ^ ((frow >> 1) & 7)) << 4);
+        const uint8_t* sa = smem + r_sa * C::A_STAGE + wq * 64 * BK;
+        const uint8_t* sw = smem + C::W_BASE + r_sw * C::W_STAGE;
+        sw_cur = sw;
+        fx = x ^ 64;
+        r_sa = r_sa == 0 ? 2 : r_sa - 1;
+        r_sw = r_sw >= 3 ? r_sw - 3 : r_sw + 2;
+        base_a = p.A + k_lo + (int64_t)rk(a_t) * BK;
+        dst_a = lds_base + a_st * C::A_STAGE + wq * 1024;
+        a_t += 2;
+        a_st = a_st == 0 ? 2 : a_st - 1;            // + 2 mod 3
+        constexpr int NF = 2 * FM + FN;
+        static_for<NF>([&](auto I) {
+            constexpr int i = decltype(I)::value;
+            if constexpr (i < FM) f[0][i] = *reinterpret_cast<const v4i*>(sa + x + i * 16 * BK);
+            else if constexpr (i < FM + FN) f[0][i] = *reinterpret_cast<const v4i*>(sw + x + (i - FM) * 16 * BK);
+            else f[1][i - FM - FN] = *reinterpret_cast<const v4i*>(sa + (x ^ 64) + (i - FM - FN) * 16 * BK);
+            SCHED_FENCE();
+            // DMA instruction d goes behind read (d * NF) / ND + 1
+            static_for<ND>([&](auto D) {
+                if constexpr ((decltype(D)::value * NF) / ND + 1 == i) { fetch_one(D); SCHED_FENCE(); }
+            });
+        });
+        static_for<ND>([&](auto D) {
+            if constexpr ((decltype(D)::value * NF) / ND + 1 >= NF) { fetch_one(D); SCHED_FENCE(); }
+        });
+    };
+    auto compute = [&]() {
+        __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+        for (int in = 0; in < FN; ++in)
+#pragma unroll
+            for (int im = 0; im < FM; ++im) {
+                acc[in][im] = __builtin_amdgcn_mfma_i32_16x16x64_i8(f[0][FM + in], f[0][im], acc[in][im], 0, 0, 0);
+                SCHED_FENCE();
+                if (im == 1) {   // one W fragment of the second half behind every fourth MFMA
+                    f[1][FM + in] = *reinterpret_cast<const v4i*>(sw_cur + fx + in * 16 * BK);
+                    SCHED_FENCE();
+                }
+            }
+#pragma unroll
+        for (int in = 0; in < FN; ++in)
+#pragma unroll
+            for (int im = 0; im < FM; ++im) {
+                acc[in][im] = __builtin_amdgcn_mfma_i32_16x16x64_i8(f[1][FM + in], f[1][im], acc[in][im], 0, 0, 0);
+                SCHED_FENCE();
+            }
+        __builtin_amdgcn_s_setprio(0);
+        fetch_w();                                 // W(t + 4), into the stage whose second half the other group read a phase ago
+    };
+
     for (int ti = 0; ti < nt_b; ++ti) {
+        int m0, n0;
+        {
+            int tm, tn;
+            tile_of_block((int)blockIdx.x + ti * G, ntiles, p.tiles_m, p.tiles_n, tm, tn, p.magic);
+            m0 = tm * C::BM;
+            n0 = tn * C::BN;
+        }
+        set_rows(m0, n0);
 #pragma unroll
         for (int in = 0; in < FN; ++in)
 #pragma unroll
             for (int im = 0; im < FM; ++im) acc[in][im] = v4i{0, 0, 0, 0};
-        int pa = 0;
-        int m0, n0;
-        tile_origin(ti, m0, n0);
-        for (int kt = 0; kt < nk; ++kt) {
-            const uint8_t* sa = smem + ca * C::A_STAGE;
-            const uint8_t* sw = smem + C::W_BASE + cw * C::W_STAGE;
-            const int na = ca == C::NSA - 1 ? 0 : ca + 1, nw = cw == C::NSW - 1 ? 0 : cw + 1;
-            const uint8_t* sa_n = smem + na * C::A_STAGE;
-            const uint8_t* sw_n = smem + C::W_BASE + nw * C::W_STAGE;
-            wg_barrier();                                                   // X
-            // slot s = 6h + in: four MFMAs on W fragment fw[s % 3] and the A fragments of half h.  Behind its MFMAs a slot
-            // reads the W fragment of slot s + 2 and one A fragment of the next half; from slot 8 on those come from the next
-            // K tile's stages, so barrier Y (they have landed) sits in front of slot 8.
-#pragma unroll
-            for (int sl = 0; sl < 12; ++sl) {
-                const int h = sl / 6, in = sl % 6;
-                if (sl == 8) wg_barrier();                                  // Y
-#pragma unroll
-                for (int im = 0; im < FM; ++im) {
-                    acc[in][im] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fw[sl % 3], fa[h][im], acc[in][im], 0, 0, 0);
-                    SCHED_FENCE();
-                    if (im == 0) {
-                        const int s2 = sl + 2;   // the slot two ahead: this K tile's, or the next one's first two
-                        fw[s2 % 3] = s2 < 12 ? w_frag(sw, s2 / 6, s2 % 6) : w_frag(sw_n, 0, s2 - 12);
-                        SCHED_FENCE();
-                    }
-                    if (im == 2 && in >= 2) {   // slots 2..5 of a half: the next half's A fragments
-                        fa[h ^ 1][in - 2] = h == 0 ? a_frag(sa, 1, in - 2) : a_frag(sa_n, 0, in - 2);
-                        SCHED_FENCE();
-                    }
+        // The column constants and row scales of the tile are requested now and parked in LDS at the end of the K loop, so
+        // that the epilogue finds them there instead of waiting for memory.
+        float2 c_ws = make_float2(0.f, 0.f), c_b = make_float2(0.f, 0.f);
+        float c_xs[4] = {0.f, 0.f, 0.f, 0.f};
+        const bool stager = EPI != EPI_ACC && wave == 7;
+        if (stager) {
+            const int l = hw_lane();
+            int n = n0 + 2 * l;
+            n = n < p.N ? n : p.N - 2;
+            if (2 * l < C::BN) {
+                c_ws = *reinterpret_cast<const float2*>(p.ws + n);
+                if (p.bias) {
+                    c_b.x = ld_dt<(EPI == EPI_ACC || OUT_DT == DT_F32) ? DT_F32 : OUT_DT>(p.bias, n);
+                    c_b.y = ld_dt<(EPI == EPI_ACC || OUT_DT == DT_F32) ? DT_F32 : OUT_DT>(p.bias, n + 1);
                 }
             }
-            pa = ca;
-            ca = na;
-            cw = nw;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) c_xs[j] = m0 + l + 64 * j < p.M ? p.xs[m0 + l + 64 * j] : 0.f;
         }
-        __syncthreads();   // every wave is done with the stage that becomes the shuffle scratch (8 KB per wave)
-        // (The stage of A(g) is refilled with A(g+NSA), issued after barrier X of the next iteration: behind this epilogue.)
-        uint8_t* scratch = smem + pa * C::A_STAGE + wave * 8192;   // a 4 KB piece, then the wave's column constants
-        epilogue_shuffle<TM, TN, OUT_DT, EPI, 32, true, true, 16>(p, acc, m0 + wm * C::WTM, n0, lane, scratch, nullptr,
-                                                                  reinterpret_cast<float*>(scratch + 4096));
-        // the first fragments of the next tile were prefetched by the last slots; fetching them again here instead of
-        // carrying them across the epilogue keeps the epilogue free of spills
-        first_frags(smem + ca * C::A_STAGE, smem + C::W_BASE + cw * C::W_STAGE);
+        // prologue.  Group 0 asks for its first K tile (W first: it has the longer way), then group 1 for its first, so
+        // that what the first compute phase needs is at the head of the CU's return path.
+        a_t = grp; w_t = grp;
+        a_st = grp; w_st = grp;
+        r_sa = grp; r_sw = grp;
+        if (grp == 0) {
+            fetch_w();
+            fetch_a();
+            wg_barrier();
+            fetch_w();
+            wait_vmcnt<C::NLW>();              // all but the second W tile
+        } else {
+            wg_barrier();
+            fetch_w();
+            fetch_a();
+            fetch_w();
+        }
+        wg_barrier();
+        if (grp == 1) wait_vmcnt<C::NLW>();
+        // Both groups run the same loop, group 1 one phase behind.
+        if (grp == 1) wg_barrier();
+        for (int t = grp; t < nk; t += 2) {
+            memory();                          // fragments of K tile t; A(t + 2)
+            wait_lgkmcnt0();
+            wg_barrier();
+            compute();                         // K tile t; W(t + 4)
+            wait_vmcnt<C::NLW>();              // everything but the W tile fetched last has landed
+            wg_barrier();
+        }
+        if ((nk & 1) == grp) wg_barrier();     // the group with fewer K tiles sits out the last phase
+        wait_vmcnt<0>();
+        if (stager) {
+            float* cst = reinterpret_cast<float*>(smem + C::CST_BASE);
+            const int l = hw_lane();
+            if (2 * l < C::BN) {
+                *reinterpret_cast<float2*>(cst + 2 * l) = c_ws;
+                *reinterpret_cast<float2*>(cst + C::BN + 2 * l) = c_b;
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) cst[2 * C::BN + l + 64 * j] = c_xs[j];
+        }
+        __syncthreads();                       // no DMA in flight, nobody reads fragments: the LDS is free
+        // Each group finishes half of every wave tile: group 0 the 16-row tiles 0 and 1 of its waves' 64 rows, group 1
+        // tiles 2 and 3.  A wave parks the other group's half of its accumulators in LDS and adds the half it is handed.
+        v4i fin[FN][2];
+        {
+            uint8_t* mine = smem + wave * C::HALF_ACC + hw_lane() * 16;
+            const uint8_t* theirs = smem + (wave ^ 4) * C::HALF_ACC + hw_lane() * 16;
+            if (nk > 1) {
+#pragma unroll
+                for (int in = 0; in < FN; ++in)
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) {
+                        *reinterpret_cast<v4i*>(mine + (in * 2 + h) * 1024) = grp == 0 ? acc[in][2 + h] : acc[in][h];
+                        fin[in][h] = grp == 0 ? acc[in][h] : acc[in][2 + h];
+                    }
+                __syncthreads();
+#pragma unroll
+                for (int in = 0; in < FN; ++in)
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) fin[in][h] += *reinterpret_cast<const v4i*>(theirs + (in * 2 + h) * 1024);
+            } else {   // one K tile: group 0 holds all of it and hands group 1 its half
+#pragma unroll
+                for (int in = 0; in < FN; ++in)
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) {
+                        if (grp == 0) *reinterpret_cast<v4i*>(mine + (in * 2 + h) * 1024) = acc[in][2 + h];
+                        fin[in][h] = acc[in][h];
+                    }
+                __syncthreads();
+                if (grp == 1) {
+#pragma unroll
+                    for (int in = 0; in < FN; ++in)
+#pragma unroll
+                        for (int h = 0; h < 2; ++h) fin[in][h] = *reinterpret_cast<const v4i*>(theirs + (in * 2 + h) * 1024);
+                }
+            }
+        }
+        {
+            uint8_t* scratch = smem + C::W_BASE + wave * 4096;   // a 4 KB shuffle piece per wave
+            float* cst = reinterpret_cast<float*>(smem + C::CST_BASE);
+            const int rows = wq * 64 + grp * 32;
+            epilogue_shuffle<1, TN, OUT_DT, EPI, 32, true, 2, 16>(p, fin, m0 + rows, n0, hw_lane(), scratch, nullptr, cst, cst + 2 * C::BN + rows);
+        }
+        if (ti + 1 < nt_b) __syncthreads();    // the next tile's prologue overwrites what the epilogue reads
     }
 }
 
@@ -1279,8 +1325,16 @@ __global__ void __launch_bounds__(256) splitk_epilogue_kernel(GemmArgs p, const 
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * 256) {
         const int64_t o = i * 4;
         const int m = (int)(o / p.N), n = (int)(o - (int64_t)m * p.N);
-        v4i acc = *reinterpret_cast<const v4i*>(planes + o);
-        for (int s = 1; s < slices; ++s) acc += *reinterpret_cast<const v4i*>(planes + s * plane + o);
+        // the planes' loads go out in batches of four with nothing between them: one trip to memory instead of `slices`
+        const int* src = planes + o;
+        v4i acc = *reinterpret_cast<const v4i*>(src);
+        int s = 1;
+        for (; s + 3 < slices; s += 4) {
+            const v4i a0 = *reinterpret_cast<const v4i*>(src + s * plane), a1 = *reinterpret_cast<const v4i*>(src + (s + 1) * plane);
+            const v4i a2 = *reinterpret_cast<const v4i*>(src + (s + 2) * plane), a3 = *reinterpret_cast<const v4i*>(src + (s + 3) * plane);
+            acc += (a0 + a1) + (a2 + a3);
+        }
+        for (; s < slices; ++s) acc += *reinterpret_cast<const v4i*>(src + s * plane);
         if (EPI == EPI_ACC) {   // the caller asked for the accumulators themselves: no scales to apply
             *reinterpret_cast<v4i*>((int*)p.D + o) = acc;
             continue;
@@ -1482,13 +1536,13 @@ void retain_pool_memory() {
 // the int32 planes.
 template <int OUT_DT, int EPI>
 int launch_stream(GemmArgs a, int slices, hipStream_t st) {
-    using C = StreamCfg;
+    using C = TurnCfg;
     a.tiles_m = (a.M + C::BM - 1) / C::BM;
     a.tiles_n = (a.N + C::BN - 1) / C::BN;
     a.magic = panel_magic(a.tiles_m, a.tiles_n);
     const int64_t ntiles = (int64_t)a.tiles_m * a.tiles_n;
     if (ntiles > 0x7fffffff) return -1;
-    auto kern = int8_gemm_stream_kernel<OUT_DT, EPI>;
+    auto kern = int8_gemm_turn_kernel<OUT_DT, EPI>;
     static bool once = false;  // benign race: the attribute is idempotent
     if (!once) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);

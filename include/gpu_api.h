@@ -270,7 +270,8 @@ int gpu_w6a8_group_gemm(const int8_t* A, const void* Wp, const float* xs, const 
                         int32_t* partials, int64_t M, int64_t N, int64_t K, int out_dt, void* stream);
 
 /* Test and tuning hook: force the GEMM kernel family.  1, 2 = 128x128 and 64x64 register-staged tiles; 6 =
- * weight-streaming kernel (256x96 tiles, split K when N is small) for M <= 256; 7 = four-wave persistent ring kernel on
+ * weight-streaming kernel (256x96 tiles, two groups of waves taking turns on the K tiles, split K when N is small) for
+ * M <= 256; 7 = four-wave persistent ring kernel on
  * 128x192 tiles (shapes with few tiles); 9 = two-group kernel (256x256 and 128x256 tiles, one launch), the choice for
  * large shapes; -1 = automatic.  A shape a family cannot run falls back to 1. */
 int gpu_int8_gemm_force_config(int cfg);
