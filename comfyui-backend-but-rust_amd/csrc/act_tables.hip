@@ -1,5 +1,6 @@
 #include "act_tables.hpp"
 
+#include <atomic>
 #include <mutex>
 
 #include "common.hpp"
@@ -24,19 +25,28 @@ __global__ void __launch_bounds__(256) fill_tables_kernel(uint16_t* h16, float* 
 constexpr int kMaxDevices = 16;
 std::mutex g_mu;
 ActTables g_tables[kMaxDevices];
-int g_state[kMaxDevices];   // 0 not built (yet), 1 built
+std::atomic<int> g_state[kMaxDevices];   // 0 not built (yet), 1 built; read without the lock, written under it
 
 }  // namespace
 
 const ActTables* act_tables(hipStream_t stream) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
-    std::lock_guard<std::mutex> hold(g_mu);
-    if (g_state[dev] == 1) return &g_tables[dev];
-    // Building allocates, launches on the null stream and synchronizes, none of which a stream capture survives: a
-    // call made while `stream` is being captured evaluates per element instead, and a later call builds the tables.
+    if (g_state[dev].load(std::memory_order_acquire) == 1) return &g_tables[dev];
+    // Building allocates and waits for a fill kernel, which a capture of `stream` does not survive: a call made while
+    // `stream` is being captured evaluates per element instead, and a later call builds the tables.  A capture on another
+    // stream (in the global mode every thread's allocations are illegal while it runs) is kept intact by switching this
+    // thread to the relaxed capture mode for the length of the build.
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
     if (stream && (hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone)) return nullptr;
+    std::lock_guard<std::mutex> hold(g_mu);
+    if (g_state[dev].load(std::memory_order_acquire) == 1) return &g_tables[dev];
+    struct RelaxedCapture {   // calls that are unsafe under another stream's capture become legal for this thread
+        hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
+        bool swapped;
+        RelaxedCapture() { swapped = hipThreadExchangeStreamCaptureMode(&mode) == hipSuccess; }
+        ~RelaxedCapture() { if (swapped) (void)hipThreadExchangeStreamCaptureMode(&mode); }
+    } relaxed;
     // A failure (a transient out-of-memory, say) leaves the state at "not built", so that the next call tries again.
     uint16_t* h16 = nullptr;
     float* f32 = nullptr;
@@ -46,14 +56,23 @@ const ActTables* act_tables(hipStream_t stream) {
         (void)hipFree(h16);
         return nullptr;
     }
-    hipLaunchKernelGGL(fill_tables_kernel, dim3(256), dim3(256), 0, 0, h16, f32);
-    if (hipGetLastError() != hipSuccess || hipDeviceSynchronize() != hipSuccess) {
+    // filled on a stream of its own that does not synchronize with the null stream, so that the work of other streams
+    // (one of which may be capturing) is neither waited for nor disturbed
+    hipStream_t fill = nullptr;
+    bool ok = hipStreamCreateWithFlags(&fill, hipStreamNonBlocking) == hipSuccess;
+    if (ok) {
+        hipLaunchKernelGGL(fill_tables_kernel, dim3(256), dim3(256), 0, fill, h16, f32);
+        ok = hipGetLastError() == hipSuccess && hipStreamSynchronize(fill) == hipSuccess;
+        (void)hipStreamDestroy(fill);
+    }
+    if (!ok) {
+        (void)hipGetLastError();
         (void)hipFree(h16);
         (void)hipFree(f32);
         return nullptr;
     }
     g_tables[dev] = ActTables{h16, h16 + 65536, h16 + 2 * 65536, h16 + 3 * 65536, f32, f32 + 65536, h16 + 4 * 65536};
-    g_state[dev] = 1;
+    g_state[dev].store(1, std::memory_order_release);
     return &g_tables[dev];
 }
 

@@ -1017,18 +1017,10 @@ Plan plan_for(int64_t b, int64_t h, int64_t hk, int64_t lq, int64_t lk, int D) {
     return p;
 }
 
-// More than 64 KB of dynamic LDS has to be allowed once per kernel and device; a repeated set is harmless if two threads
-// race.
+// More than 64 KB of dynamic LDS has to be allowed once per kernel and device.
 template <class K> bool allow_lds(K kern, int bytes) {
-    static bool allowed[64] = {};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
-    if (!allowed[dev]) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess)
-            return false;
-        allowed[dev] = true;
-    }
-    return true;
+    static PerDeviceOnce once;
+    return allow_dynamic_lds(reinterpret_cast<const void*>(kern), bytes, once) == 0;
 }
 
 template <int DT, int CK, bool MASK, bool FD, int D>

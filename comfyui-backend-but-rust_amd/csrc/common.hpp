@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/gpu_api.h"
 
 #define GPU_API extern "C" __attribute__((visibility("default")))
@@ -14,6 +16,28 @@
         hipError_t e__ = hipGetLastError();        \
         if (e__ != hipSuccess) return (int)e__;    \
     } while (0)
+
+// "Done once per device" flags for host-side set-up (a kernel's dynamic LDS limit, a memory pool attribute): one bit per
+// device ordinal, set after the call has succeeded on that device.  Two threads that race both make the call, which is
+// idempotent.  Devices past 63 are not remembered and make the call every time.
+struct PerDeviceOnce {
+    std::atomic<uint64_t> done{0};
+    static int current() {
+        int dev = 0;
+        return hipGetDevice(&dev) == hipSuccess ? dev : -1;
+    }
+    bool is_done(int dev) const { return dev >= 0 && dev < 64 && ((done.load(std::memory_order_acquire) >> dev) & 1u); }
+    void mark(int dev) { if (dev >= 0 && dev < 64) done.fetch_or((uint64_t)1 << dev, std::memory_order_release); }
+};
+// Raises a kernel's dynamic LDS limit on the current device, the first time it is asked for there.  0 or a hipError_t.
+inline int allow_dynamic_lds(const void* kern, int bytes, PerDeviceOnce& once) {
+    const int dev = PerDeviceOnce::current();
+    if (once.is_done(dev)) return 0;
+    const hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e != hipSuccess) return (int)e;
+    once.mark(dev);
+    return 0;
+}
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));

@@ -18,12 +18,16 @@ __device__ __forceinline__ int lds_pos(int e) {
 }
 
 // h4_row x 4 outputs with the reference's left-to-right adds, scaled by 0.5 (csrc/common.cuh:99-106,119-122).
-__device__ __forceinline__ void bfly4(float& a, float& b, float& c, float& d) {
+// HALVE = false leaves the scaling out: the 128-wide transform, which is this library's own definition, applies its three
+// halvings together with the closing 1/sqrt(2), in one multiplication per output (bit-identical to halving per stage
+// while every intermediate stays in the normal range, and four instructions per butterfly shorter).
+template <bool HALVE = true> __device__ __forceinline__ void bfly4(float& a, float& b, float& c, float& d) {
     const float x0 = a, x1 = b, x2 = c, x3 = d;
-    a = 0.5f * (x0 + x1 + x2 - x3);
-    b = 0.5f * (x0 + x1 - x2 + x3);
-    c = 0.5f * (x0 - x1 + x2 + x3);
-    d = 0.5f * (-x0 + x1 + x2 + x3);
+    const float h = HALVE ? 0.5f : 1.0f;
+    a = h * (x0 + x1 + x2 - x3);
+    b = h * (x0 + x1 - x2 + x3);
+    c = h * (x0 - x1 + x2 + x3);
+    d = h * (-x0 + x1 + x2 + x3);
 }
 
 // Rotate one chunk held as v[16] per lane (element 16*lane + i).  wl is the wave's LDS tile.
@@ -33,10 +37,11 @@ __device__ __forceinline__ void bfly4(float& a, float& b, float& c, float& d) {
 
 template <int G> __device__ __forceinline__ void rotate_chunk(float* v, float* wl, int lane) {
     // strides 1 and 4: inside the lane
+    constexpr bool HV = G != 128;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) bfly4(v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]);
+    for (int i = 0; i < 4; ++i) bfly4<HV>(v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) bfly4(v[j], v[j + 4], v[j + 8], v[j + 12]);
+    for (int j = 0; j < 4; ++j) bfly4<HV>(v[j], v[j + 4], v[j + 8], v[j + 12]);
     // to LDS in row order
 #pragma unroll
     for (int i = 0; i < 4; ++i)
@@ -68,7 +73,7 @@ template <int G> __device__ __forceinline__ void rotate_chunk(float* v, float* w
         for (int d = 0; d < 4; ++d) *reinterpret_cast<float4*>(wl + lds_pos(base + d * 16)) = w[d];
     } else {
         // G == 128: lane (O = lane/8, p = lane%8) takes O*128 + t*64 + d*16 + 2p + j: stride 16 (radix 4) and the
-        // closing radix-2 stage at stride 64, scaled by 1/sqrt(2)
+        // closing radix-2 stage at stride 64; every output is then scaled once, by fl(1/sqrt(2)) / 8
         const int base = (lane >> 3) * 128 + (lane & 7) * 2;
         float2 w[2][4];
 #pragma unroll
@@ -77,10 +82,10 @@ template <int G> __device__ __forceinline__ void rotate_chunk(float* v, float* w
             for (int d = 0; d < 4; ++d) w[t][d] = *reinterpret_cast<float2*>(wl + lds_pos(base + t * 64 + d * 16));
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-            bfly4(w[t][0].x, w[t][1].x, w[t][2].x, w[t][3].x);
-            bfly4(w[t][0].y, w[t][1].y, w[t][2].y, w[t][3].y);
+            bfly4<false>(w[t][0].x, w[t][1].x, w[t][2].x, w[t][3].x);
+            bfly4<false>(w[t][0].y, w[t][1].y, w[t][2].y, w[t][3].y);
         }
-        const float c = 0.70710678118654752f;
+        const float c = 0.70710678118654752f * 0.125f;
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
             const float ax = w[0][d].x, bx = w[1][d].x, ay = w[0][d].y, by = w[1][d].y;

@@ -1365,12 +1365,8 @@ int launch_cfg(GemmArgs a, hipStream_t st) {
     if (nblocks > 0x7fffffff) return -1;
     auto kern = int8_gemm_kernel<C, OUT_DT, EPI>;
     if (C::SMEM > 48 * 1024) {
-        static bool once = false;  // benign race: the attribute is idempotent
-        if (!once) {
-            hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
-            if (e != hipSuccess) return (int)e;
-            once = true;
-        }
+        static PerDeviceOnce once;
+        if (const int e = allow_dynamic_lds((const void*)kern, C::SMEM, once)) return e;
     }
     hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(C::NT), C::SMEM, st, a);
     KCHECK();
@@ -1378,13 +1374,14 @@ int launch_cfg(GemmArgs a, hipStream_t st) {
 }
 
 int device_cu_count() {
-    static int num_cu = 0;   // benign race: every thread computes the same value
-    if (num_cu == 0) {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-        num_cu = n;
-    }
-    return num_cu;
+    static std::atomic<int> cached[64];   // compute units per device ordinal, 0 = not asked yet
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 256;
+    const bool keep = dev >= 0 && dev < 64;
+    if (keep && (n = cached[dev].load(std::memory_order_relaxed)) > 0) return n;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 256;
+    if (keep) cached[dev].store(n, std::memory_order_relaxed);
+    return n;
 }
 
 // Launches the persistent ring kernel on `slices` K slices (1 = whole K).  With slices > 1, EPI must be EPI_ACC and
@@ -1397,12 +1394,8 @@ int launch_ring_cfg(GemmArgs a, int slices, hipStream_t st) {
     const int64_t ntiles = (int64_t)a.tiles_m * a.tiles_n;
     if (ntiles > 0x7fffffff) return -1;
     auto kern = int8_gemm_ring_kernel<C, OUT_DT, EPI>;
-    static bool once = false;  // benign race: the attribute is idempotent
-    if (!once) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
-        if (e != hipSuccess) return (int)e;
-        once = true;
-    }
+    static PerDeviceOnce once;
+    if (const int e = allow_dynamic_lds((const void*)kern, C::SMEM, once)) return e;
     const int num_cu = device_cu_count();
     const int64_t per_slice = slices > 1 ? (num_cu / slices > 0 ? num_cu / slices : 1) : num_cu;
     const unsigned grid = (unsigned)(ntiles < per_slice ? ntiles : per_slice);
@@ -1463,12 +1456,8 @@ int launch_pp(GemmArgs a, hipStream_t st) {
     rest.magic = panel_magic(rest.tiles_m, rest.tiles_n);
     const int g_main = (int)(n_main < G ? n_main : G), g_rest = (int)(n_rest < G ? n_rest : G);
     auto kern = int8_gemm_pp_kernel<OUT_DT, EPI>;
-    static bool once = false;  // benign race: the attribute is idempotent
-    if (!once) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, PpL::SMEM);
-        if (e != hipSuccess) return (int)e;
-        once = true;
-    }
+    static PerDeviceOnce once;
+    if (const int e = allow_dynamic_lds((const void*)kern, PpL::SMEM, once)) return e;
     hipLaunchKernelGGL(kern, dim3((unsigned)(g_main + g_rest)), dim3(PpL::NT), PpL::SMEM, st, main, rest, g_main);
     KCHECK();
     return 0;
@@ -1522,14 +1511,13 @@ thread_local size_t tl_scratch_bytes = 0;
 // the reference's runtime layer does at start-up (src/cuda.rs:88-97): otherwise each call that needs scratch pays a
 // fresh allocation.
 void retain_pool_memory() {
-    static bool pool_set = false;   // benign race: the attribute is idempotent
-    if (pool_set) return;
-    int dev = 0;
+    static PerDeviceOnce once;
+    const int dev = PerDeviceOnce::current();
+    if (dev < 0 || once.is_done(dev)) return;
     hipMemPool_t pool;
     uint64_t keep = ~(uint64_t)0;
-    if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetDefaultMemPool(&pool, dev) == hipSuccess)
-        (void)hipMemPoolSetAttribute(pool, hipMemPoolAttrReleaseThreshold, &keep);
-    pool_set = true;
+    if (hipDeviceGetDefaultMemPool(&pool, dev) == hipSuccess && hipMemPoolSetAttribute(pool, hipMemPoolAttrReleaseThreshold, &keep) == hipSuccess)
+        once.mark(dev);
 }
 
 // Launches the weight-streaming kernel on `slices` K slices (1 = whole K).  With slices > 1, EPI must be EPI_ACC and a.D
@@ -1543,12 +1531,8 @@ int launch_stream(GemmArgs a, int slices, hipStream_t st) {
     const int64_t ntiles = (int64_t)a.tiles_m * a.tiles_n;
     if (ntiles > 0x7fffffff) return -1;
     auto kern = int8_gemm_turn_kernel<OUT_DT, EPI>;
-    static bool once = false;  // benign race: the attribute is idempotent
-    if (!once) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM);
-        if (e != hipSuccess) return (int)e;
-        once = true;
-    }
+    static PerDeviceOnce once;
+    if (const int e = allow_dynamic_lds((const void*)kern, C::SMEM, once)) return e;
     const int num_cu = device_cu_count();
     const int64_t per_slice = slices > 1 ? (num_cu / slices > 0 ? num_cu / slices : 1) : num_cu;
     const unsigned grid = (unsigned)(ntiles < per_slice ? ntiles : per_slice);

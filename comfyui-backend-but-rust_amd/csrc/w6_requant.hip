@@ -154,12 +154,8 @@ GPU_API int gpu_w6_requant(const void* weight, void* packed, void* s_rel, void* 
     constexpr size_t kMaxDynamic = 160 * 1024 - 256;   // the kernel also has a few bytes of static LDS
     if (smem > kMaxDynamic || N > 0x7fffffff) return -2;
     if (N <= 0) return 0;
-    static bool once = false;   // benign race: the attribute is idempotent
-    if (!once) {
-        const hipError_t e = hipFuncSetAttribute((const void*)w6_requant_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxDynamic);
-        if (e != hipSuccess) return (int)e;
-        once = true;
-    }
+    static PerDeviceOnce once;
+    if (const int e = allow_dynamic_lds((const void*)w6_requant_kernel, (int)kMaxDynamic, once)) return e;
     hipLaunchKernelGGL(w6_requant_kernel, dim3((unsigned)N), dim3(256), smem, (hipStream_t)stream, (const uint16_t*)weight,
                        (uint8_t*)packed, (uint8_t*)s_rel, (float*)s_channel, K, seed);
     KCHECK();

@@ -419,12 +419,8 @@ template <int OUT_DT, bool DUMP, int ABL = 0, bool W8 = false>
 int launch(W6Args a, hipStream_t st) {
     auto kern = w6a8_group_gemm_kernel<OUT_DT, DUMP, ABL, W8>;
     constexpr int SMEM = Lay<W8>::SMEM;
-    static bool once = false;  // benign race: the attribute is idempotent
-    if (!once) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
-        if (e != hipSuccess) return (int)e;
-        once = true;
-    }
+    static PerDeviceOnce once;
+    if (const int e = allow_dynamic_lds((const void*)kern, SMEM, once)) return e;
     hipLaunchKernelGGL(kern, dim3((unsigned)(a.tiles_m * a.tiles_n)), dim3(NT), SMEM, st, a);
     KCHECK();
     return 0;
@@ -453,6 +449,13 @@ __global__ void __launch_bounds__(256) w6_words_to_int8_kernel(const uint8_t* Wp
 constexpr int64_t kExpandFirstRows = 4096;
 std::atomic<int> g_mode{-1};   // test hook: 0 = always fused, 1 = always expand first, -1 = by M
 
+// 32-bit DMA lane offsets into A, the packed weights and the scales; a tile count that fits the grid
+bool shape_fits(int64_t M, int64_t N, int64_t K) {
+    if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff) return false;
+    if (M * K >= ((int64_t)1 << 32) || N * (K / 4 * 3) >= ((int64_t)1 << 32) || N * (K / 128) * 4 >= ((int64_t)1 << 32)) return false;
+    return ((M + BM - 1) / BM) * ((N + BN - 1) / BN) <= 0x7fffffff;
+}
+
 }  // namespace
 
 GPU_API int gpu_w6a8_group_gemm(const int8_t* A, const void* Wp, const float* xs, const float* sw, const void* bias,
@@ -460,14 +463,10 @@ GPU_API int gpu_w6a8_group_gemm(const int8_t* A, const void* Wp, const float* xs
     if (K < 0 || (K % 128) != 0) return -1;
     if (out_dt < DT_F32 || out_dt > DT_BF16 || M < 0 || N < 0) return -200;
     if (M == 0 || N == 0) return 0;
-    // 32-bit DMA lane offsets and tile counts
-    if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff || M * K >= ((int64_t)1 << 32) || N * (K / 4 * 3) >= ((int64_t)1 << 32) ||
-        N * (K / 128) * 4 >= ((int64_t)1 << 32))
-        return -200;
+    if (K == 0 || !shape_fits(M, N, K)) return -200;
     W6Args a{A, (const uint8_t*)Wp, nullptr, xs, sw, bias, D, partials, (int)M, (int)N, (int)K, (int)(K / 128), 0, 0};
     a.tiles_m = (int)((M + BM - 1) / BM);
     a.tiles_n = (int)((N + BN - 1) / BN);
-    if ((int64_t)a.tiles_m * a.tiles_n > 0x7fffffff || K == 0) return -200;
     hipStream_t st = (hipStream_t)stream;
     const int mode = g_mode.load(std::memory_order_relaxed);
     int8_t* w8 = nullptr;
@@ -504,7 +503,8 @@ GPU_API int gpu_internal_w6a8_group_gemm_mode(int mode) {
 // fetches expanded weights, with Wp then pointing at int8 [N, K].  D receives meaningless values.
 GPU_API int gpu_internal_w6a8_group_gemm_ablate(int ablate, const int8_t* A, const void* Wp, const float* xs, const float* sw,
                                                 void* D, int64_t M, int64_t N, int64_t K, void* stream) {
-    if (K <= 0 || (K % 128) != 0 || M <= 0 || N <= 0 || M * K >= ((int64_t)1 << 32) || N * (K / 4 * 3) >= ((int64_t)1 << 32)) return -200;
+    if (K <= 0 || (K % 128) != 0 || M <= 0 || N <= 0 || !shape_fits(M, N, K)) return -200;
+    if ((ablate & 8) && N * K >= ((int64_t)1 << 32)) return -200;
     W6Args a{A, (const uint8_t*)Wp, nullptr, xs, sw, nullptr, D, nullptr, (int)M, (int)N, (int)K, (int)(K / 128), 0, 0};
     a.tiles_m = (int)((M + BM - 1) / BM);
     a.tiles_n = (int)((N + BN - 1) / BN);

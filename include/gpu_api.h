@@ -180,7 +180,9 @@ int gpu_internal_cvt_pk_u8_probe(const float* x, uint32_t* y, int n, void* strea
 
 /* Measurement hook, no reference counterpart: gpu_w6a8_group_gemm (bf16 output, no bias) with parts of its kernel left
  * out, to show what each costs next to the MFMAs: ablate bit 0 the fp32 fold, bit 1 the unpack, bit 2 the LDS-DMA after
- * the prologue (0..7).  D receives meaningless values unless ablate is 0. */
+ * the prologue (0..7).  With bit 3 set (8, 9, 12, 13 only) the kernel is the form that fetches weights already expanded
+ * to int8, and Wp must then point at int8 [N, K] (N*K bytes), not at the packed words.  Shapes are checked as in
+ * gpu_w6a8_group_gemm; any other value of ablate returns -200.  D receives meaningless values unless ablate is 0 or 8. */
 int gpu_internal_w6a8_group_gemm_ablate(int ablate, const int8_t* A, const void* Wp, const float* xs, const float* sw, void* D,
                                         int64_t M, int64_t N, int64_t K, void* stream);
 
@@ -224,9 +226,9 @@ int gpu_w6_decode(const void* q, const void* s_rel, void* out, int64_t N, int K,
 
 /* Builds, for the current device, the lookup tables that the prologues GATE / SWIGLU / SILU / GELU / GELU_TANH / SITU and
  * the SD GEGLU source use on 16-bit rows (all 65536 inputs of each activation, about 1.2 MB, held until the process
- * ends).  Optional: the first call with such a prologue builds them itself, with two device allocations, a launch on
- * the null stream and a device synchronization -- unless its stream is being captured, in which case that call
- * evaluates the activations per element (same bits, slower) and a later call builds the tables.  Call this once at
+ * ends).  Optional: the first call with such a prologue builds them itself, with two device allocations, a fill kernel
+ * on a stream of its own and a wait for it -- unless its stream is being captured, in which case that call evaluates
+ * the activations per element (same bits, slower) and a later call builds the tables.  Call this once at
  * start-up to keep every quantizer call asynchronous and capturable.  Returns 0, or -1 if the tables could not be
  * built (calls then evaluate per element, and a later call tries again). */
 int gpu_act_tables_init(void);
@@ -240,7 +242,10 @@ int gpu_int8_gemm_acc(const int8_t* A, const int8_t* W, int32_t* acc, int64_t M,
  * allocation, and the call makes no hipMalloc / hipFree of any kind.  No counterpart in the reference.
  * Every call on one GPU shares that GPU's array: calls that overlap in time on one GPU (two streams, two threads) race
  * on it and must be serialized by the caller.  Nothing in the array needs clearing between calls (every plane element
- * is written before it is read).  A shape whose planes would not fit returns -210 with a message on stderr;
+ * is written before it is read).  The first call on a device looks up the array's address and sets kernel attributes:
+ * make it once before capturing a graph that contains this call.  The array occupies its 24 MiB on every device the
+ * process uses, from the moment the library is loaded.  A shape whose planes would not fit returns -210 with a message on
+ * stderr (every shape the automatic choice splits fits; with gpu_int8_gemm_force_config(6), M > 256 can exceed it);
  * gpu_int8_gemm_static_limit() returns the array's size in bytes.  K % 16 == 8, which gpu_int8_gemm serves from
  * padded copies that it allocates, is refused here (-200).  Other return codes as gpu_int8_gemm. */
 int gpu_int8_gemm_static(const int8_t* A, const int8_t* W, const float* xs, const float* ws, const void* bias, void* D,

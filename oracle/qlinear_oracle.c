@@ -125,7 +125,12 @@ static inline float fmin_dev(float a, float b) { return isnan(a) ? b : isnan(b) 
  * ConvRot group transform.  h4_row: csrc/common.cuh:99-106 (left-to-right adds).  Staged order:
  * fht256_rows_smem csrc/common.cuh:110-126 (4 radix-4 stages, strides 1,4,16,64, each scaled by 0.5) and
  * fht64_rows_smem csrc/sd.cu:560-576 (3 stages).  g = 128 has no reference form: it is defined here as the three
- * radix-4 stages of each 64-block followed by one radix-2 stage at stride 64 scaled by 1/sqrt(2).
+ * radix-4 stages of each 64-block WITHOUT their halvings, then one radix-2 stage at stride 64, then one scaling of
+ * every output by fl(1/sqrt(2)) / 8 (the three halvings and the 1/sqrt(2) in one exactly representable constant).
+ * A halving is exact in fp32, so this equals "halve after every stage, scale the last by fl(1/sqrt(2))" bit for bit
+ * as long as no intermediate leaves the normal range; where they differ, this definition overflows to infinity once
+ * partial sums pass 3.4e38 (inputs beyond about 5e36 in a group of like signs; the halved form would hold out to
+ * 3.4e38) and keeps the low bits of results below 1.2e-38 that the halved form would round away.
  * ------------------------------------------------------------------------------------------- */
 static inline float h4_row(int d, float x0, float x1, float x2, float x3) {
     switch (d) {
@@ -146,14 +151,15 @@ ORC_API int orc_fht(float* row, int K, int g) {
             const int grp = b / (blk / 4), r = b % (blk / 4);
             const int i0 = grp * blk + (r / s) * (4 * s) + (r % s);
             const float x0 = row[i0], x1 = row[i0 + s], x2 = row[i0 + 2 * s], x3 = row[i0 + 3 * s];
-            row[i0] = 0.5f * h4_row(0, x0, x1, x2, x3);
-            row[i0 + s] = 0.5f * h4_row(1, x0, x1, x2, x3);
-            row[i0 + 2 * s] = 0.5f * h4_row(2, x0, x1, x2, x3);
-            row[i0 + 3 * s] = 0.5f * h4_row(3, x0, x1, x2, x3);
+            const float half = g == 128 ? 1.0f : 0.5f;
+            row[i0] = half * h4_row(0, x0, x1, x2, x3);
+            row[i0 + s] = half * h4_row(1, x0, x1, x2, x3);
+            row[i0 + 2 * s] = half * h4_row(2, x0, x1, x2, x3);
+            row[i0 + 3 * s] = half * h4_row(3, x0, x1, x2, x3);
         }
     }
     if (g == 128) {
-        const float c = 0.70710678118654752f;
+        const float c = 0.70710678118654752f * 0.125f;
         for (int base = 0; base < K; base += 128)
             for (int i = 0; i < 64; ++i) {
                 const float a = row[base + i], b = row[base + 64 + i];

@@ -1034,8 +1034,10 @@ def test_w6a8_group_gemm_argument_checks():
 FULL = [  # (name, M, K, N, rotate, kind)
     ("dit mlp up", 4608, 3072, 12288, 128, "t3"),
     ("dit mlp down", 4608, 12288, 3072, 1, "t3"),
+    ("dit mlp down, block 128", 4608, 12288, 3072, 128, "t3"),
     ("skinny gate+up", 256, 4096, 24576, 128, "normal"),
     ("skinny down", 256, 12288, 4096, 1, "normal"),
+    ("skinny down, block 128", 256, 12288, 4096, 128, "normal"),
     ("sdxl geglu", 8192, 640, 5120, 0, "normal"),
     ("dit qkv", 4608, 3072, 9216, 128, "t3"),
     ("dit out-proj", 4608, 3072, 3072, 128, "t3"),
@@ -1132,6 +1134,17 @@ def test_full_size_w6a8_group_gemm(name, M, K, N):
     rc, want, _ = oracle.w6a8_group_gemm(A[rows], packed, xs[rows], sw, bias, BF16)
     assert rc == 0
     assert np.array_equal(host_bits(got[torch.tensor(rows, device=DEV)]), want.view(np.uint16))
+    # both forms of the kernel at this size: 0 unpacks inside the GEMM in every workgroup, 1 expands the weights once first
+    # (what the call picks by itself from 4096 rows on)
+    for mode in (0, 1):
+        ffi.raw("gpu_internal_w6a8_group_gemm_mode", mode)
+        try:
+            forced = ql.w6a8_group_gemm(Ad, pd, xsd, swd, bd, torch.bfloat16)
+            torch.cuda.synchronize()
+        finally:
+            ffi.raw("gpu_internal_w6a8_group_gemm_mode", -1)
+        assert torch.equal(forced.view(torch.int16), got.view(torch.int16)), mode
+        assert np.array_equal(host_bits(forced[torch.tensor(rows, device=DEV)]), want.view(np.uint16)), mode
     # a band of rows that straddles a tile boundary, with the partials dumped
     r0, nr = 3 * 256 - 80, 160
     band, part = ql.w6a8_group_gemm(Ad[r0:r0 + nr].contiguous(), pd, xsd[r0:r0 + nr].contiguous(), swd, bd, torch.bfloat16, want_partials=True)

@@ -157,6 +157,34 @@ def test_fht128_is_orthonormal_h2_kron_h64():
     assert np.allclose(oracle.fht(y, 128), x, atol=2e-6)
 
 
+def test_fht128_one_scaling_equals_halving_per_stage():
+    """The 128-wide transform adds through its three radix-4 stages and its radix-2 stage and scales once, by
+    fl(1/sqrt(2)) / 8.  Halving is exact in float32, so on data whose intermediates stay in the normal range this must be,
+    bit for bit, the hand-staged form that halves after every radix-4 stage and scales the last stage by fl(1/sqrt(2));
+    small integers give the dense matrix exactly up to that one scaling; and the two places where the forms part are as
+    the oracle's header says: sums past 3.4e38 overflow here and not there, results below 1.2e-38 keep bits here."""
+    rng = np.random.default_rng(128)
+    c = np.float32(0.70710678118654752)
+    for trial in range(8):
+        x = (rng.normal(0, 1, 256) * rng.choice([1e-3, 1.0, 37.0, 1e20, 1e-20], 256)).astype(np.float32)
+        y = oracle.fht(x, 128)
+        st = _staged_h4(x, (1, 4, 16)).reshape(2, 2, 64)                  # halved per stage, on every 64-block
+        want = np.stack([(st[:, 0] + st[:, 1]) * c, (st[:, 0] - st[:, 1]) * c], axis=1).reshape(-1)
+        assert np.array_equal(y.view(np.uint32), want.view(np.uint32)), trial
+    # exact integers: y * sqrt(128) / (fl(1/sqrt 2) * sqrt 2) is the +-1 matrix product
+    xi = rng.integers(-8, 9, size=128).astype(np.float32)
+    Hpm = np.kron(np.array([[1, 1], [1, -1]], np.float64), kron_h(3) * 8.0)
+    assert np.array_equal(oracle.fht(xi, 128), ((Hpm @ xi.astype(np.float64)).astype(np.float32) * (c * np.float32(0.125))))
+    # where the forms differ
+    big = (np.float32(1e37) * np.sign(Hpm[0])).astype(np.float32)           # signs of the matrix's first row: every term adds
+    assert np.isinf(oracle.fht(big, 128)[0])                               # 128e37 overflows; halving per stage would give 1.13e38
+    assert np.isclose(oracle.fht((big * np.float32(0.01)).astype(np.float32), 128)[0], 1.28e37 / np.sqrt(128.0), rtol=1e-5)   # in range: finite
+    tiny = np.zeros(128, np.float32)
+    tiny[0] = np.float32(3e-38)
+    got = oracle.fht(tiny, 128)
+    assert got[0] == np.float32(3e-38) * (c * np.float32(0.125)) and got[0] != 0
+
+
 # ----------------------------------------------------------------------------------------------- quantizer
 def torch_quant_bf16(xbits):
     """The quantizer as PyTorch tensor arithmetic in bf16 (what the reference says it emulates, csrc/kernels.cu:3-4)."""
