@@ -825,8 +825,9 @@ __global__ void __launch_bounds__(C::NT, 1) int8_gemm_ring_kernel(GemmArgs p) {
 // only after the barrier that follows its last reader.  Steps run straight through tile boundaries.
 //
 // End of a tile: group 0 runs its epilogue while group 1 multiplies its last step and then runs its own; the shuffle
-// scratch is the W stage of that step (4 KB per wave), which no DMA in flight targets.  One barrier, then group 0's
-// first memory phase of the next tile (group 1 has nothing to do in it), and the alternation resumes.
+// scratch is the W stage of that step (4 KB per wave), which no DMA in flight targets.  Group 0 follows its epilogue with
+// the memory phase of the next tile's first step (under group 1's epilogue), one barrier, and the alternation resumes
+// with group 0 multiplying.
 // Requires K % 128 == 0, M*K and N*K < 2^32, and the coalesced epilogue's alignment.
 // ---------------------------------------------------------------------------------------------------------------
 // GM: rows of a group.  128 gives the 256x256 tile (wave tiles 128x64); 64 gives a 128x256 tile (wave tiles 64x64) for
@@ -994,9 +995,12 @@ __device__ __forceinline__ void pp_gemm_tiles(const GemmArgs& p, uint8_t* smem, 
         epilogue_shuffle<TM, TN, OUT_DT, EPI, PW, true, false, 16>(p, acc, m0 + grp * C::GM, n0 + wq * C::WTN, hw_lane(), scratch);
     };
 
-    // Both groups run the same loop; group 1 is one phase behind (the barrier in front), multiplies its last step of a
-    // tile in the phase in which group 0 already runs its epilogue, and has nothing to do while group 0 reads the first
-    // fragments of the next tile (the second barrier after its epilogue).
+    // Both groups run the same loop; group 1 is one phase behind (the barrier in front) and multiplies its last step of a
+    // tile in the phase in which group 0 already runs its epilogue.  Group 0 goes from its epilogue straight into the
+    // memory phase of the next tile's first step, while group 1 is still in its epilogue: what that phase reads landed
+    // before the tile's last compute phases, and what it fetches goes to stages that neither epilogue uses (group 1's A
+    // stage of the step before last, and the half of the last step's W stage that was group 0's own shuffle scratch).
+    // After the one barrier that follows the epilogues group 0 multiplies at once and the alternation is back.
     if (grp == 1) wg_barrier();
     int s = 0;
     for (int ti = 0; ti < nt_b; ++ti) {
@@ -1008,8 +1012,9 @@ __device__ __forceinline__ void pp_gemm_tiles(const GemmArgs& p, uint8_t* smem, 
             if (grp == 0 || kt + 1 < nk) wg_barrier();
         }
         run_epilogue(ti, s - 1);
-        wg_barrier();
-        if (grp == 1 && ti + 1 < nt_b) wg_barrier();
+        // the barrier behind the epilogues; group 0 meets it after the next tile's first memory phase (the loop's first
+        // barrier), so it skips this one when a tile follows
+        if (grp == 1 || ti + 1 == nt_b) wg_barrier();
     }
     wait_vmcnt<0>();   // no DMA may still be writing this workgroup's LDS when it retires
 }

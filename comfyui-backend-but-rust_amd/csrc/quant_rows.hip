@@ -409,7 +409,7 @@ int run_quant(QuantArgs a, int g, hipStream_t st) {
     // few rows: more waves per row (down to one chunk per wave) so that the launch has enough waves to hide latency
     while (wpr < 8 && wpr < nchunks && (int64_t)a.M * wpr < 2048) wpr *= 2;
     const int C = (nchunks + wpr - 1) / wpr;
-    const int nw = wpr < 4 ? 4 : wpr;
+    const int nw = wpr < 2 ? 2 : wpr;   // two rows per workgroup at least: small workgroups spread evenly over the CUs
     a.wpr = wpr;
     a.rpb = nw / wpr;
     switch (g) {
