@@ -886,7 +886,21 @@ __device__ __forceinline__ void pp_gemm_tiles(const GemmArgs& p, uint8_t* smem, 
         }
     };
     auto set_a = [&](int tile) { int m0, n0; tile_origin(tile, m0, n0); set_rows(ga, ic<C::NLA>{}, m0 + (grp ^ 1) * C::GM, p.M); };
-    auto set_w = [&](int tile) { int m0, n0; tile_origin(tile, m0, n0); set_rows(gw, ic<C::NLW>{}, n0 + grp * 128, p.N); };
+    // W: a wave fetches the four CONSECUTIVE 8-row blocks 4*wq .. 4*wq + 3 of its group's half, which are exactly the 4 KB
+    // of the stage that serve as this wave's shuffle scratch in the epilogue: group 0 may then refill the stage right
+    // after its own epilogue, while other waves are still in theirs.  (A block's parity, which the swizzle needs, is j's.)
+    auto set_w = [&](int tile) {
+        int m0, n0;
+        tile_origin(tile, m0, n0);
+        const int l = hw_lane();
+        const int lr = l >> 3;
+#pragma unroll
+        for (int j = 0; j < C::NLW; ++j) {
+            const int row = n0 + grp * 128 + (4 * wq + j) * 8 + lr;
+            const int lc = ((l & 7) ^ (((j & 1) << 2) | (lr >> 1))) * 16;
+            gw[j] = (uint32_t)(row < p.N ? row : p.N - 1) * (uint32_t)ld + lc;
+        }
+    };
     auto fetch_a = [&]() {
         const int8_t* base = p.A + (int64_t)a_kt * BK;
         const uint32_t dst = lds_base + C::A_BASE + ((grp ^ 1) * C::NSA + a_stage) * C::A_STAGE + wq * 1024;
@@ -898,9 +912,9 @@ __device__ __forceinline__ void pp_gemm_tiles(const GemmArgs& p, uint8_t* smem, 
     };
     auto fetch_w = [&]() {
         const int8_t* base = p.W + (int64_t)w_kt * BK;
-        const uint32_t dst = lds_base + w_stage * C::W_STAGE + grp * 128 * BK + wq * 1024;
+        const uint32_t dst = lds_base + w_stage * C::W_STAGE + grp * 128 * BK + wq * 4096;
 #pragma unroll
-        for (int j = 0; j < C::NLW; ++j) dma(dst + j * 4096, gw[j], base);
+        for (int j = 0; j < C::NLW; ++j) dma(dst + j * 1024, gw[j], base);
         w_stage = w_stage == C::NSW - 1 ? 0 : w_stage + 1;
         if (w_tile == nt_b - 1 && w_kt == nk - 1) return;
         if (++w_kt == nk) { w_kt = 0; set_w(++w_tile); }
