@@ -17,6 +17,13 @@
 namespace {
 
 __device__ __forceinline__ void store16_untracked(void* ptr, uint4 v);
+__device__ __forceinline__ void store16_untracked_at(const void* base, uint32_t off, uint4 v);
+// A 64-bit value that is the same in every lane, moved to scalar registers.
+__device__ __forceinline__ uint64_t uniform64(uint64_t v) {
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
+    return ((uint64_t)hi << 32) | lo;
+}
 
 enum { EPI_PLAIN = 0, EPI_RESID = 1, EPI_ACC = 2 };
 
@@ -223,6 +230,11 @@ __device__ __forceinline__ void epilogue_shuffle(const GemmArgs& p, Acc& acc, in
         return f16_to_f((uint16_t)((j & 1) ? (w >> 16) : (w & 0xffffu)));
     };
     const int rrow = lane / CPRW, rc = lane % CPRW;   // read phase: row within a pass, chunk
+    // uniform per wave: the wave tile is wholly inside the matrix; where it starts; bytes per output row
+    const bool full = __builtin_amdgcn_readfirstlane((int)(mb + TM * 32 <= p.M && nb + WTN <= p.N && p.N < (1 << 21))) != 0;
+    const uint64_t row_bytes = (uint64_t)p.N * SZ;
+    const uint64_t tile_base = uniform64((uint64_t)(uintptr_t)p.D + ((uint64_t)mb * p.N + nb) * SZ);
+    const uint32_t lane_off = __umul24((uint32_t)rrow, (uint32_t)row_bytes) + (uint32_t)(rc * 16);   // both factors < 2^24 when `full`
 
     // Every global load is issued ahead of the stores that precede its use: the memory counter retires in order, so a
     // load issued after a store cannot be waited for without also waiting for that store to reach memory.
@@ -306,42 +318,57 @@ __device__ __forceinline__ void epilogue_shuffle(const GemmArgs& p, Acc& acc, in
             v[t] = *reinterpret_cast<const uint4*>(buf + r * ROWB + (((rc ^ r) & MASK) << 4));
         }
     };
-    // read phase, second half: whole rows out
+    // read phase, second half: whole rows out.  A wave tile that lies wholly inside the matrix stores through one
+    // scalar base per pass plus a 32-bit lane offset: no per-pass compares, branches or 64-bit vector address arithmetic
+    // (a fifth of the vector instructions of an epilogue that is bound by them).
+    auto finish = [&](int np, const uint4& z, const uint4& r) -> uint4 {
+        if (EPI != EPI_RESID) return z;
+        const uint32_t zw[4] = {z.x, z.y, z.z, z.w}, rw[4] = {r.x, r.y, r.z, r.w};
+        uint32_t ow[4];
+        if (OUT_DT == DT_F32) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) ow[j] = f2u(__builtin_fmaf(u2f(zw[j]), rs[np][j], u2f(rw[j])));
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float z0, z1, r0, r1;
+                if (OUT_DT == DT_BF16) {
+                    z0 = u2f(zw[j] << 16); z1 = u2f(zw[j] & 0xffff0000u); r0 = u2f(rw[j] << 16); r1 = u2f(rw[j] & 0xffff0000u);
+                    ow[j] = pack_bf16x2(__builtin_fmaf(z0, rs[np][2 * j], r0), __builtin_fmaf(z1, rs[np][2 * j + 1], r1));
+                } else {
+                    z0 = f16_to_f((uint16_t)(zw[j] & 0xffffu)); z1 = f16_to_f((uint16_t)(zw[j] >> 16));
+                    r0 = f16_to_f((uint16_t)(rw[j] & 0xffffu)); r1 = f16_to_f((uint16_t)(rw[j] >> 16));
+                    ow[j] = (uint32_t)f_to_f16(__builtin_fmaf(z0, rs[np][2 * j], r0)) | ((uint32_t)f_to_f16(__builtin_fmaf(z1, rs[np][2 * j + 1], r1)) << 16);
+                }
+            }
+        }
+        return make_uint4(ow[0], ow[1], ow[2], ow[3]);
+    };
     auto store_piece = [&](int im, int np, const uint4* v, const uint4* rv) {
-        const int ncol = nb + np * PW + rc * EPC;
-        uint8_t* base = (uint8_t*)p.D + ((int64_t)(mb + im * 32 + rrow) * p.N + ncol) * SZ;
+        if (full) {
+            const uint64_t piece = tile_base + (uint64_t)(im * 32) * row_bytes + (uint64_t)(np * PW * SZ);
+#pragma unroll
+            for (int t = 0; t < PASSES; ++t) {
+                const uint64_t pass = piece + (uint64_t)(t * RPI) * row_bytes;
+                const uint4 o = finish(np, v[t], rv[t]);
+                if (UNTRACKED) store16_untracked_at((const void*)pass, lane_off, o);
+                else *reinterpret_cast<uint4*>((uint8_t*)pass + lane_off) = o;
+            }
+            return;
+        }
+        int l = lane;
+        asm volatile("" : "+v"(l));   // keeps this path's address arithmetic from being hoisted in front of the branch
+        const int row = l / CPRW, ncol = nb + np * PW + (l % CPRW) * EPC;
+        uint8_t* base = (uint8_t*)p.D + ((int64_t)(mb + im * 32 + row) * p.N + ncol) * SZ;
         const int64_t step = (int64_t)RPI * p.N * SZ;
 #pragma unroll
         for (int t = 0; t < PASSES; ++t) {
-            const int m = mb + im * 32 + t * RPI + rrow;
+            const int m = mb + im * 32 + t * RPI + row;
             if (m >= p.M || ncol >= p.N) continue;
             uint8_t* out = base + t * step;
-            if (EPI != EPI_RESID) {
-                if (UNTRACKED) store16_untracked(out, v[t]);
-                else *reinterpret_cast<uint4*>(out) = v[t];
-            } else {
-                const uint32_t zw[4] = {v[t].x, v[t].y, v[t].z, v[t].w}, rw[4] = {rv[t].x, rv[t].y, rv[t].z, rv[t].w};
-                uint32_t ow[4];
-                if (OUT_DT == DT_F32) {
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) ow[j] = f2u(__builtin_fmaf(u2f(zw[j]), rs[np][j], u2f(rw[j])));
-                } else {
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        float z0, z1, r0, r1;
-                        if (OUT_DT == DT_BF16) {
-                            z0 = u2f(zw[j] << 16); z1 = u2f(zw[j] & 0xffff0000u); r0 = u2f(rw[j] << 16); r1 = u2f(rw[j] & 0xffff0000u);
-                            ow[j] = pack_bf16x2(__builtin_fmaf(z0, rs[np][2 * j], r0), __builtin_fmaf(z1, rs[np][2 * j + 1], r1));
-                        } else {
-                            z0 = f16_to_f((uint16_t)(zw[j] & 0xffffu)); z1 = f16_to_f((uint16_t)(zw[j] >> 16));
-                            r0 = f16_to_f((uint16_t)(rw[j] & 0xffffu)); r1 = f16_to_f((uint16_t)(rw[j] >> 16));
-                            ow[j] = (uint32_t)f_to_f16(__builtin_fmaf(z0, rs[np][2 * j], r0)) | ((uint32_t)f_to_f16(__builtin_fmaf(z1, rs[np][2 * j + 1], r1)) << 16);
-                        }
-                    }
-                }
-                if (UNTRACKED) store16_untracked(out, make_uint4(ow[0], ow[1], ow[2], ow[3]));
-                else *reinterpret_cast<uint4*>(out) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
-            }
+            const uint4 o = finish(np, v[t], rv[t]);
+            if (UNTRACKED) store16_untracked(out, o);
+            else *reinterpret_cast<uint4*>(out) = o;
         }
     };
 
@@ -525,9 +552,14 @@ __global__ void __launch_bounds__(C::NT, C::OCC) int8_gemm_kernel(GemmArgs p) {
 // 16-byte global store the compiler's wait-count bookkeeping does not see (see the ring kernel's epilogue)
 __device__ __forceinline__ void store16_untracked(void* ptr, uint4 v) {
     const v4i d = v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w};
-    // The trailing s_nop is the wait state the hardware needs between a store of more than 8 bytes and a write to its
-    // data registers; the compiler inserts it for its own stores but cannot see into this one.
-    asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 0" ::"v"(ptr), "v"(d) : "memory");
+    // The trailing s_nop gives the two wait states this hardware needs between a store of more than 8 bytes and a
+    // vector write to its data registers; the compiler inserts them for its own stores but cannot see into this one.
+    asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 1" ::"v"(ptr), "v"(d) : "memory");
+}
+// The same with a scalar base and a 32-bit lane offset.
+__device__ __forceinline__ void store16_untracked_at(const void* base, uint32_t off, uint4 v) {
+    const v4i d = v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+    asm volatile("global_store_dwordx4 %0, %1, %2 nt\n\ts_nop 1" ::"v"(off), "v"(d), "s"(base) : "memory");
 }
 
 template <int N> __device__ __forceinline__ void wait_vmcnt() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
