@@ -118,6 +118,7 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-skinny", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the other linears of the model configurations and the W6A8 shapes")
+    ap.add_argument("--no-graph", action="store_true", help="skip the captured-graph replays of the linears")
     ap.add_argument("--attention-only", action="store_true",
                     help="time only the INT8 attention shapes and print them as one JSON line (for profiling that path alone)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
@@ -516,8 +517,9 @@ def main():
                       "int8_gemm_us": round(cold_tg * 1e3, 2),
                       "note": "the first steps after 0.5 s of idle, no settling load: the clock is still rising"},
     }
-    out["graph_replay"] = {"linear_us": round(time_linear_graph(torch, ffi, d, M, K, N, a.rotate, a.steps, 1), 2),
-                           "note": "quantizer + GEMM captured once into a HIP graph and replayed (gpu_int8_gemm_static inside the capture)"}
+    if not a.no_graph:
+        out["graph_replay"] = {"linear_us": round(time_linear_graph(torch, ffi, d, M, K, N, a.rotate, a.steps, 1), 2),
+                               "note": "quantizer + GEMM captured once into a HIP graph and replayed (gpu_int8_gemm_static inside the capture)"}
     if not a.no_skinny:
         sk = []
         for (m, k, n) in ((256, 4096, 24576), (256, 12288, 4096)):
@@ -526,14 +528,14 @@ def main():
             _, wall2, tq2, tg2 = time_linear(torch, ffi, d2, m, k, n, a.rotate, a.steps, a.warmup, nbuf=nbuf)
             gemm_bytes = m * k + m * 4 + n * k + n * 4 + n * 2 + m * n * 2
             sp2 = dict(LAST_SPREAD)
-            graph_us = time_linear_graph(torch, ffi, d2, m, k, n, a.rotate, a.steps, nbuf)
+            graph_us = None if a.no_graph else time_linear_graph(torch, ffi, d2, m, k, n, a.rotate, a.steps, nbuf)
             sk.append({"M": m, "K": k, "N": n, "int8_gemm_us": round(tg2 * 1e3, 2),
                        "GBs": round(gemm_bytes / (tg2 * 1e-3) / 1e9, 1),
                        "frac_hbm": round(gemm_bytes / (tg2 * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
                        "int8_gemm_us_median": sp2["int8_gemm_us_median"], "int8_gemm_us_min": sp2["int8_gemm_us_min"],
                        "frac_hbm_best": round(gemm_bytes / (sp2["int8_gemm_us_min"] * 1e-6) / 1e9 / PEAK_HBM_GBS, 4),
                        "quant_rows_us": round(tq2 * 1e3, 2), "linear_us_by_events": round((tq2 + tg2) * 1e3, 2),
-                       "linear_us_graph_replay": round(graph_us, 2), "weight_copies_rotated": nbuf})
+                       "linear_us_graph_replay": None if graph_us is None else round(graph_us, 2), "weight_copies_rotated": nbuf})
             del h2, d2
         out["skinny"] = sk
     if not a.no_extra:
