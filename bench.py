@@ -456,6 +456,29 @@ def cpu_baseline(host, M, K, N, rotate, target_s):
             "sample": "first %d of %d rows, whole linear (quantize + int32 GEMM + epilogue), %d passes of %.2f s" % (rows2, M, reps, dt)}
 
 
+def cpu_config0(synth, target_s=1.5):
+    """BASELINE.json's configuration 0 (M=256, K=1024, N=1024, no rotation) on the host's cores: the oracle's whole
+    linear timed in full, with one thread and with all of them."""
+    import oracle
+    M, K, N = 256, 1024, 1024
+    x = synth.bf16_bits(synth.activations(0, M, K, "normal"))
+    W, ws, bias = synth.w8_weights(0, N, K)
+    bias = synth.bf16_bits(bias)
+    out = {"M": M, "K": K, "N": N, "kind": "port", "unit": "TOPS"}
+    for label, threads in (("one_thread", 1), ("all_threads", min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16"))))):
+        t0 = time.perf_counter()
+        rc, _, used = oracle.linear_w8a8(oracle.BF16, x, 0, W, ws, bias, oracle.BF16, threads=threads)
+        assert rc == 0
+        reps = max(1, int(round(target_s / max(time.perf_counter() - t0, 1e-4))))
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            rc, _, used = oracle.linear_w8a8(oracle.BF16, x, 0, W, ws, bias, oracle.BF16, threads=threads)
+            assert rc == 0
+        dt = (time.perf_counter() - t0) / reps
+        out[label] = {"value": round(2.0 * M * N * K / dt / 1e12, 5), "ms": round(dt * 1e3, 3), "cores": used, "passes": reps}
+    return out
+
+
 def main():
     a = parse()
     if a.gpus != 1:
@@ -542,7 +565,7 @@ def main():
         # the other linears of the image-DiT block and the SDXL-UNet level, then the video-DiT W6A8 pair
         extra = []
         few = max(5, min(40, a.steps // 3))
-        for (name, m, k, n, rot) in (("dit qkv", 4608, 3072, 9216, a.rotate), ("dit out-proj", 4608, 3072, 3072, a.rotate),
+        for (name, m, k, n, rot) in (("config 0 anchor", 256, 1024, 1024, 0), ("dit qkv", 4608, 3072, 9216, a.rotate), ("dit out-proj", 4608, 3072, 3072, a.rotate),
                                      ("dit mlp down", 4608, 12288, 3072, a.rotate), ("sdxl attn proj", 8192, 640, 640, 0),
                                      ("sdxl geglu up", 8192, 640, 5120, 0), ("sdxl down", 8192, 2560, 640, 0)):
             h2, d2 = make_inputs(torch, synth, m, k, n, seed=2, kind="t3" if rot else "normal")
@@ -570,6 +593,7 @@ def main():
     out["mfma_ceiling"] = time_mfma_ceiling(torch, ffi)
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(host, M, K, N, a.rotate, a.cpu_seconds)
+        out["cpu_baseline_config0"] = cpu_config0(synth)
     print(json.dumps(out))
 
 
