@@ -222,8 +222,9 @@ def time_linear_graph(torch, ffi, d, M, K, N, rotate, steps, nbuf):
 
 def time_w6a8(torch, ffi, M, K, N, steps, warmup):
     """The group-scaled W6A8 GEMM (24-bit words of four 6-bit codes, fp32 scales per 128 along K) on synthetic weights
-    with codes uniform in [-31, 31]; returns the average microseconds of gpu_w6a8_group_gemm (at these M the call
-    expands the weights into scratch first, then runs the GEMM kernel on them)."""
+    with codes uniform in [-31, 31]; returns the average microseconds of gpu_w6a8_group_gemm as it dispatches by itself
+    (at these M the call expands the weights into scratch first, then runs the GEMM kernel on them), with the unpack
+    forced inside the GEMM kernel, and with the expansion forced."""
     g = torch.Generator(device="cuda:0").manual_seed(4)
     u = torch.randint(1, 64, (N, K // 4, 4), dtype=torch.int32, device="cuda:0", generator=g)   # u = q + 32
     w = u[..., 0] | (u[..., 1] << 6) | (u[..., 2] << 12) | (u[..., 3] << 18)
@@ -241,16 +242,21 @@ def time_w6a8(torch, ffi, M, K, N, steps, warmup):
               0, M, N, K, ffi.DT_BF16, st.cuda_stream)
 
     settle(torch, run)
-    for _ in range(warmup):
-        run()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    torch.cuda.synchronize()
-    e0.record(st)
-    for _ in range(steps):
-        run()
-    e1.record(st)
-    torch.cuda.synchronize()
-    return e0.elapsed_time(e1) / steps * 1e3
+    res = []
+    for mode in (-1, 0, 1):
+        ffi.raw("gpu_internal_w6a8_group_gemm_mode", mode)
+        for _ in range(warmup):
+            run()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record(st)
+        for _ in range(steps):
+            run()
+        e1.record(st)
+        torch.cuda.synchronize()
+        res.append(e0.elapsed_time(e1) / steps * 1e3)
+    ffi.raw("gpu_internal_w6a8_group_gemm_mode", -1)
+    return tuple(res)
 
 
 def time_w6_reference_format(torch, ffi, M, K, N, steps, warmup):
@@ -576,8 +582,9 @@ def main():
         out["linears"] = extra
         w6 = []
         for (name, m, k, n) in (("video-dit ffn up", 8192, 5120, 13824), ("video-dit ffn down", 8192, 13824, 5120)):
-            us = time_w6a8(torch, ffi, m, k, n, few, 2)
+            us, us_fused, us_expanded = time_w6a8(torch, ffi, m, k, n, few, 2)
             w6.append({"name": name, "M": m, "K": k, "N": n, "kernel": "gpu_w6a8_group_gemm", "us": round(us, 1),
+                       "us_unpack_inside_the_gemm": round(us_fused, 1), "us_expanded_once_into_scratch": round(us_expanded, 1),
                        "TOPS": round(2.0 * m * n * k / us / 1e6, 1), "frac_int8_peak": round(2.0 * m * n * k / us / 1e6 / PEAK_INT8_TOPS, 4)})
         out["w6a8"] = w6
         w6r = []

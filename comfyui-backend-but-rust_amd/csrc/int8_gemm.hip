@@ -8,6 +8,7 @@
 // stores 8-byte (bf16/f16) or 16-byte (f32) vectors straight from the accumulators.
 #include <atomic>
 #include <cstdio>
+#include <mutex>
 
 #include "common.hpp"
 
@@ -1571,6 +1572,43 @@ void retain_pool_memory() {
         once.mark(dev);
 }
 
+// Split-K planes of the allocating entry points: one buffer per (device, stream), made on that stream's first split
+// call and kept until the process ends.  Work on one stream is ordered, so its calls can share a buffer, and a
+// stream-ordered allocation per call costs about 7 us on the stream's timeline (measured: 31 against 24 us per call at
+// M=256, K=12288, N=4096).  The buffer has the one size every shape that the dispatcher splits fits into (slices *
+// column tiles <= CUs, so slices * N <= CUs * 96, times 256 rows of int32: 24 MiB on 256 CUs) and is never grown or
+// freed, so a captured graph that holds its address stays valid.  At most kStreamPlanes streams per process are served;
+// a call on any further stream, a first call made under capture, or a shape beyond the size (a forced configuration)
+// falls back to a stream-ordered allocation.  A stream handle that the runtime reuses after hipStreamDestroy inherits
+// the destroyed stream's buffer; work still queued on the destroyed stream at that moment would share it.
+struct StreamPlanes { int dev; hipStream_t st; void* ptr; size_t bytes; };
+constexpr int kStreamPlanes = 8;
+std::mutex g_planes_mu;
+StreamPlanes g_planes[kStreamPlanes];
+int g_planes_n = 0;
+
+void* stream_planes(hipStream_t st, size_t need, int num_cu) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+    std::lock_guard<std::mutex> lock(g_planes_mu);
+    for (int i = 0; i < g_planes_n; ++i)
+        if (g_planes[i].dev == dev && g_planes[i].st == st) return need <= g_planes[i].bytes ? g_planes[i].ptr : nullptr;
+    const size_t bytes = (size_t)num_cu * TurnCfg::BN * TurnCfg::BM * sizeof(int);
+    if (g_planes_n == kStreamPlanes || need > bytes) return nullptr;
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    void* ptr = nullptr;
+    if (hipMalloc(&ptr, bytes) != hipSuccess) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    g_planes[g_planes_n++] = StreamPlanes{dev, st, ptr, bytes};
+    return ptr;
+}
+
 // Launches the weight-streaming kernel on `slices` K slices (1 = whole K).  With slices > 1, EPI must be EPI_ACC and a.D
 // the int32 planes.
 template <int OUT_DT, int EPI>
@@ -1594,8 +1632,8 @@ int launch_stream(GemmArgs a, int slices, hipStream_t st) {
 
 // M <= 256: one row of 256 x 96 tiles, the weights are read once and the run is bound by how fast they stream.  When N
 // is too small to give every CU a column slab, K is split as well: each slice writes an int32 plane (exact, so the
-// order of the sum does not matter) into a stream-ordered scratch allocation and a second kernel adds the planes and
-// applies the epilogue.
+// order of the sum does not matter) into the stream's scratch buffer and a second kernel adds the planes and applies
+// the epilogue.
 template <int OUT_DT, int EPI>
 int launch_skinny(GemmArgs a, hipStream_t st) {
     bool vec_ok, aligned;
@@ -1613,11 +1651,15 @@ int launch_skinny(GemmArgs a, hipStream_t st) {
     const int per = (nk + slices - 1) / slices;
     const size_t need = (size_t)slices * a.M * a.N * sizeof(int);
     int* planes = nullptr;
-    const bool own = tl_scratch == nullptr;
-    if (own) {
-        retain_pool_memory();
-        hipError_t e = hipMallocAsync((void**)&planes, need, st);
-        if (e != hipSuccess) return (int)e;
+    bool own = false;   // planes come from the stream-ordered pool and go back to it
+    if (tl_scratch == nullptr) {
+        planes = (int*)stream_planes(st, need, num_cu);
+        if (!planes) {
+            own = true;
+            retain_pool_memory();
+            hipError_t e = hipMallocAsync((void**)&planes, need, st);
+            if (e != hipSuccess) return (int)e;
+        }
     } else {
         if (need > tl_scratch_bytes) {
             fprintf(stderr, "gpu_int8_gemm_static: M=%d N=%d K=%d needs %zu bytes of split-K scratch, the static buffer has %zu\n",
@@ -1653,7 +1695,16 @@ int choose_cfg(int64_t M, int64_t N, int64_t K) {
     const bool dma_ok = M * K < ((int64_t)1 << 32) && N * K < ((int64_t)1 << 32);   // 32-bit lane offsets
     if (force == 6 || force == 7 || force == 9) return (dma_ok && (K % 128) == 0) ? force : 1;
     if (force == 1 || force == 2) return force;
-    if (M <= 256 && N >= 1024 && (K % 128) == 0 && K >= 512 && dma_ok) return 6;
+    if (M <= 256 && N >= 1024 && (K % 128) == 0 && K >= 512 && dma_ok) {
+        // The weight-streaming kernel pays a fixed price per call (a prologue that waits for HBM, two launches when K
+        // is split), which long K repays and short K does not.  Measured with weights from HBM, M = 16..256, K =
+        // 1024..12288, N = 1024..24576: it wins from K = 3072 on at M > 128 and from K = 1536 on below; under that the
+        // 128 x 192 ring tiles win for M > 128 (all N at K >= 1536, N >= 8192 below) and the small register-staged
+        // tiles for the rest.
+        if (K >= (M > 128 ? 3072 : 1536)) return 6;
+        if (M > 128 && (K >= 1536 || N >= 8192)) return 7;
+        return 2;
+    }
     const int64_t tiles_l = ((M + 255) / 256) * ((N + 255) / 256);
     if (M >= 512 && N >= 512 && tiles_l >= 192) return (dma_ok && (K % 128) == 0) ? 9 : 1;
     // too few 256x256 tiles for the CUs: the persistent kernel on 128x192 tiles, where those fill at least a third of them

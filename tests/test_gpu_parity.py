@@ -940,9 +940,9 @@ def test_quant_rows_with_more_than_2_to_the_31_elements(rotate):
 # ------------------------------------------------------------------------------------------------ graph capture
 @pytest.mark.parametrize("M,N,K,entry", [(4096, 4096, 256, "gpu_int8_gemm"),          # two-group kernel
                                            (1024, 2304, 256, "gpu_int8_gemm"),          # ring kernel on 128x192 tiles
-                                           (256, 24576, 256, "gpu_int8_gemm"),          # stream kernel, whole K
+                                           (256, 24576, 3072, "gpu_int8_gemm"),         # weight-streaming kernel, whole K
                                            (640, 1536, 512, "gpu_int8_gemm"),           # register-staged tiles
-                                           (256, 2048, 2048, "gpu_int8_gemm_static")])  # stream kernel, split K, static planes
+                                           (256, 2048, 4096, "gpu_int8_gemm_static")])  # weight-streaming kernel, split K, static planes
 def test_linear_replays_from_a_captured_graph(M, N, K, entry):
     """The quantizer and the GEMM allocate nothing on these routes (the split-K shape through the entry point with the
     static planes), so one linear can be captured.  Three replays with new activations and eager work between them,

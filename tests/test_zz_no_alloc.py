@@ -46,7 +46,7 @@ def _run(name, A, W, xs, ws, bias):
 
 
 # split-K shapes of the skinny path (M <= 256, N too narrow to give every CU a column slab), larger first
-SHAPES = [(256, 4096, 4096), (100, 1024, 1024)]
+SHAPES = [(256, 4096, 4096), (100, 1024, 2048)]
 
 
 def test_static_entry_point_matches_allocating_one_twice_in_a_row():
