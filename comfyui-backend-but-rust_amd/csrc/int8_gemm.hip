@@ -1705,13 +1705,19 @@ int choose_cfg(int64_t M, int64_t N, int64_t K) {
         if (M > 128 && (K >= 1536 || N >= 8192)) return 7;
         return 2;
     }
-    const int64_t tiles_l = ((M + 255) / 256) * ((N + 255) / 256);
-    if (M >= 512 && N >= 512 && tiles_l >= 192) return (dma_ok && (K % 128) == 0) ? 9 : 1;
-    // too few 256x256 tiles for the CUs: the persistent kernel on 128x192 tiles, where those fill at least a third of them
+    // Everything below was chosen from measured grids of shapes (weights from HBM, every family forced in turn).  A
+    // round of 128 x 192 ring tiles costs about two thirds of a round of 256 x 256 two-group tiles, so the large tiles
+    // win as soon as the small ones need a second round, i.e. more than one per CU.
     const int64_t tiles_s = ((M + 127) / 128) * ((N + 191) / 192);
-    if (dma_ok && (K % 128) == 0 && M > 128 && N >= 192 && tiles_s >= 96) return 7;
+    if (M >= 512 && N >= 512 && tiles_s > device_cu_count()) return (dma_ok && (K % 128) == 0) ? 9 : 1;
+    if (dma_ok && (K % 128) == 0) {
+        // a few hundred rows, long K, few columns: the ring tiles leave most CUs idle, the weight-streaming kernel splits
+        // K over them (not for the entry point that may not allocate: its planes are sized for 256 rows)
+        if (M <= 512 && N >= 1024 && K >= 8192 && tiles_s <= 96 && tl_scratch == nullptr) return 6;
+        if (M > 128 && N >= 192 && (tiles_s >= 96 || (tiles_s >= 40 && K >= 2048))) return 7;
+    }
     const int64_t tiles_m = ((M + 127) / 128) * ((N + 127) / 128);
-    if (M > 64 && N > 64 && tiles_m >= 128) return 1;
+    if (M > 64 && N > 64 && tiles_m >= 256) return 1;
     return 2;
 }
 

@@ -4,10 +4,10 @@
  * The first block of entry points has the reference's names, argument order and C types, so the reference's Rust
  * declarations (src/ffi.rs) bind to this library unchanged; each prototype cites the declaration it replaces.
  * All pointers are device pointers unless stated; `stream` is a hipStream_t passed as void* (null = default stream).
- * Every call is asynchronous on `stream`, allocates nothing that outlives it and never throws.  State kept between
- * calls: cached device attributes; per device, the lookup tables of the prologue activations (see
- * gpu_act_tables_init); the kernel family forced by the test hook gpu_int8_gemm_force_config; the static scratch of
- * gpu_int8_gemm_static.
+ * Every call is asynchronous on `stream` and never throws.  State kept between calls, all of it until the process ends:
+ * cached device attributes; per device, the lookup tables of the prologue activations (see gpu_act_tables_init); per
+ * stream (the first eight that need it), 24 MiB for the int32 planes of gpu_int8_gemm's split-K shapes; the kernel
+ * family forced by the test hook gpu_int8_gemm_force_config; the static scratch of gpu_int8_gemm_static.
  *
  * Return convention (src/ffi.rs:336-344, csrc/common.cuh:128): 0 = ok; > 0 = a hipError_t from the launch
  * (hipGetErrorString names it); < 0 = the launcher refused the arguments, with the reference's codes:
@@ -206,7 +206,11 @@ int gpu_internal_attn_layout_d(int b, int h, int hk, int lq, int lk, int head_di
  * A, W int8 row-major (K contiguous); xs f32 [M]; ws f32 [N]; bias Out[N] or null; D Out[M,N]; out_dt a DT_* code.
  * K % 16 == 0 is the fast path; K % 16 == 8 (the reference's alignment-8 tile configurations,
  * csrc/vendor/cutlass_gemm_int8.cu:191,237-247) runs on zero-padded copies of A and W in a stream-ordered allocation
- * (A and W 8-byte aligned); any other K is refused. */
+ * (A and W 8-byte aligned); any other K is refused.
+ * M <= 256 with long K and few output columns splits K; the int32 planes of the slices go to a 24 MiB buffer that the
+ * first such call on a stream allocates (hipMalloc) and the library keeps for that stream.  That first call should be
+ * made outside graph capture; under capture, or on a ninth stream, the call uses hipMallocAsync / hipFreeAsync on
+ * `stream` instead, as does a shape forced onto that kernel whose planes exceed the buffer. */
 int gpu_int8_gemm(const int8_t* A, const int8_t* W, const float* xs, const float* ws, const void* bias, void* D,
                   int64_t M, int64_t N, int64_t K, int out_dt, void* stream);
 
@@ -238,8 +242,8 @@ int gpu_int8_gemm_acc(const int8_t* A, const int8_t* W, int32_t* acc, int64_t M,
 
 /* gpu_int8_gemm for callers that cannot allocate device memory (code under HIP graph capture, serving loops and
  * harnesses that forbid hipMalloc): same arguments, same results bit for bit, but the int32 planes of a split-K run
- * (M <= 256 with a narrow N) live in a fixed 24 MiB device array inside the library instead of a stream-ordered
- * allocation, and the call makes no hipMalloc / hipFree of any kind.  No counterpart in the reference.
+ * (M <= 256 with a narrow N) live in a fixed 24 MiB device array inside the library instead of a buffer allocated
+ * for the stream, and the call makes no hipMalloc / hipFree of any kind, first call included.  No counterpart in the reference.
  * Every call on one GPU shares that GPU's array: calls that overlap in time on one GPU (two streams, two threads) race
  * on it and must be serialized by the caller.  Nothing in the array needs clearing between calls (every plane element
  * is written before it is read).  The first call on a device looks up the array's address and sets kernel attributes:
