@@ -689,7 +689,13 @@ def test_int8_gemm_k_multiple_of_8_only(M, N, K):
 
 # More 256x256 tiles than CUs, and not a multiple of the CU count: the persistent kernel's workgroups then own unequal
 # numbers of tiles, and every output form runs through its coalesced epilogue.
-MANY_TILE_CASES = [(4352, 4096, 256), (4100, 4400, 384), (2304, 8200, 640)]
+MANY_TILE_CASES = [(4352, 4096, 256), (4100, 4400, 384), (2304, 8200, 640),
+                   # either side of the dispatcher's thresholds: two row tiles of the weight-streaming kernel with K split
+                   # (planes beyond the per-stream buffer), ring tiles for few tiles and long K, short K at M <= 256 on
+                   # the register-staged and ring tiles, M <= 128 with K = 1536 on the weight-streaming kernel, and a
+                   # shape where the two-group tiles cover half of the CUs
+                   (384, 1056, 8192), (512, 4096, 2048), (256, 1024, 1024), (256, 12288, 1024), (200, 2048, 2048),
+                   (100, 3008, 1536), (2048, 2048, 512)]
 
 
 @pytest.mark.parametrize("M,N,K", MANY_TILE_CASES)
