@@ -1579,7 +1579,8 @@ void retain_pool_memory() {
 // column tiles <= CUs, so slices * N <= CUs * 96, times 256 rows of int32: 24 MiB on 256 CUs) and is never grown or
 // freed, so a captured graph that holds its address stays valid.  At most kStreamPlanes streams per process are served;
 // a call on any further stream, a first call made under capture, or a shape beyond the size (a forced configuration)
-// falls back to a stream-ordered allocation.  A stream handle that the runtime reuses after hipStreamDestroy inherits
+// falls back to a stream-ordered allocation, and so does hipStreamPerThread (one handle for a different stream in every
+// thread).  A stream handle that the runtime reuses after hipStreamDestroy inherits
 // the destroyed stream's buffer; work still queued on the destroyed stream at that moment would share it.
 struct StreamPlanes { int dev; hipStream_t st; void* ptr; size_t bytes; };
 constexpr int kStreamPlanes = 8;
@@ -1588,6 +1589,7 @@ StreamPlanes g_planes[kStreamPlanes];
 int g_planes_n = 0;
 
 void* stream_planes(hipStream_t st, size_t need, int num_cu) {
+    if (st == hipStreamPerThread) return nullptr;   // one handle, a different stream in every thread: nothing to key on
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) return nullptr;
     std::lock_guard<std::mutex> lock(g_planes_mu);

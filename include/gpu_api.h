@@ -209,8 +209,8 @@ int gpu_internal_attn_layout_d(int b, int h, int hk, int lq, int lk, int head_di
  * (A and W 8-byte aligned); any other K is refused.
  * M <= 256 with long K and few output columns splits K; the int32 planes of the slices go to a 24 MiB buffer that the
  * first such call on a stream allocates (hipMalloc) and the library keeps for that stream.  That first call should be
- * made outside graph capture; under capture, or on a ninth stream, the call uses hipMallocAsync / hipFreeAsync on
- * `stream` instead, as does a shape forced onto that kernel whose planes exceed the buffer. */
+ * made outside graph capture; under capture, on a ninth stream or on hipStreamPerThread the call uses hipMallocAsync /
+ * hipFreeAsync on `stream` instead, as does a shape whose planes exceed the buffer (more than 256 rows). */
 int gpu_int8_gemm(const int8_t* A, const int8_t* W, const float* xs, const float* ws, const void* bias, void* D,
                   int64_t M, int64_t N, int64_t K, int out_dt, void* stream);
 
